@@ -1,0 +1,341 @@
+"""CPU restatement of the reference's torch implementations of the FP8 quantized
+linear path (activation quantizers, 128x128 weight quantizer, block-scaled GEMM,
+per-token/per-channel scaled GEMM).
+
+TEST INFRASTRUCTURE. Only tests/, __graft_entry__.smoke() and bench.py's
+cpu_baseline leg may import this module.  The product (flaggems_amd) never
+imports it and has no CPU fallback.
+
+Every function restates one torch-native reference function that the reference
+repository keeps in its test/benchmark files, and cites it.  All functions run
+on CPU tensors with plain torch ops; nothing here touches a GPU.
+
+Pinning status (what checks each function against something other than itself;
+the checks live in tests/test_oracle_*.py):
+
+* act_quant_ref, per_token_group_quant_fp8_ref, per_token_group_quant_fp8_div_ref,
+  per_block_cast_to_fp8_ref, per_token_cast_to_fp8_ref -- pinned by a brute-force
+  numpy quantizer built on the bit-level E4M3 encoder of oracle/e4m3.py (itself
+  pinned against ``tensor.to(torch.float8_e4m3fn)`` on all 65 536 bf16 patterns
+  and against a nearest-value search), by the invariants "max |x| of a group
+  encodes to +-448", "codes(-x) = sign-flipped codes(x)", "ue8m0 scale is the
+  power of two in [s, 2s)", and by hand-worked special cases (all-zero group,
+  NaN, Inf, a lone huge element).
+* block_fp8_matmul_dequant_ref, block_fp8_matmul_tiled_ref -- pinned against each
+  other (two different algorithms from two reference files), a float64 triple
+  loop on tiny shapes, and closed forms (unit scales -> plain matmul, one-hot
+  rows pick scaled weight rows exactly, power-of-two scales are exact).
+* scaled_mm_ref, scaled_mm_ref_postscale -- pinned against each other, a float64
+  loop, and the unit-scale/zero-bias closed form.
+
+No function here is "parity unpinned".
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Tuple
+
+import torch
+
+FP8_DTYPE = torch.float8_e4m3fn
+FP8_MAX = 448.0
+
+
+# --------------------------------------------------------------------------------------
+# Activation quantizers
+# --------------------------------------------------------------------------------------
+def act_quant_ref(
+    x: torch.Tensor, block_size: int = 128, scale_fmt: Optional[str] = None
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Restates ``torch_act_quant`` (reference tests/test_act_quant.py:48-98).
+
+    fp32 amax per ``block_size`` group, floor 1e-4, scale = amax * fp32(1/448);
+    with ``scale_fmt`` set the scale is rounded up to a power of two by the
+    exponent/mantissa bit test of tests/test_act_quant.py:73-85; codes =
+    clamp(x * (1/scale), +-448) cast to e4m3fn (round-to-nearest-even).
+    """
+    assert x.is_contiguous(), "Input tensor must be contiguous"
+    assert x.size(-1) % block_size == 0, "Last dim must be divisible by block_size"
+    fp8_max_inv = 1.0 / 448.0
+    n = x.size(-1)
+    x_2d = x.view(-1, n)
+    m = x_2d.size(0)
+    n_blocks = n // block_size
+    xb = x_2d.view(m, n_blocks, block_size).float()
+    amax = xb.abs().amax(dim=-1)
+    amax = torch.clamp(amax, min=1e-4)
+    if scale_fmt is not None:
+        scale_raw = amax * fp8_max_inv
+        bits = scale_raw.view(torch.int32)
+        exp_x = (bits >> 23) & 0xFF
+        man = bits & ((1 << 23) - 1)
+        log2_ceil = (exp_x - 127 + (man != 0).int()).int()
+        scale = ((log2_ceil + 127) << 23).view(torch.float32)
+    else:
+        scale = amax * fp8_max_inv
+    yb = xb * (1.0 / scale.unsqueeze(-1))
+    yb = torch.clamp(yb, -FP8_MAX, FP8_MAX)
+    y = yb.view(m, n).to(FP8_DTYPE).view(x.shape)
+    s = scale.to(torch.float32).view(*x.shape[:-1], n_blocks)
+    return y, s
+
+
+def per_token_group_quant_fp8_ref(
+    x: torch.Tensor,
+    group_size: int,
+    eps: float = 1e-10,
+    dtype: torch.dtype = FP8_DTYPE,
+    scale_ue8m0: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Restates ``native_per_token_group_quant_fp8``
+    (reference tests/test_per_token_group_quant_fp8.py:23-48).
+
+    abs/max/clamp(eps) are done in x's own dtype, then widened to fp32;
+    scale = amax * fp32(1/448); optional exp2(ceil(log2(max(|s|,1e-10))));
+    codes = clamp(x / scale, +-448) with a true fp32 division.
+    """
+    assert x.shape[-1] % group_size == 0
+    assert x.is_contiguous(), "`x` is not contiguous"
+    finfo = torch.finfo(dtype)
+    x_ = x.reshape(x.numel() // group_size, group_size)
+    amax = x_.abs().max(dim=-1, keepdim=True)[0].clamp(min=eps).to(torch.float32)
+    x_s = amax * torch.tensor(1.0 / finfo.max, dtype=torch.float32)
+    if scale_ue8m0:
+        min_val = torch.tensor(1e-10, dtype=x_s.dtype)
+        x_s = torch.exp2(torch.ceil(torch.log2(torch.maximum(x_s.abs(), min_val))))
+    x_q = (x_ / x_s).clamp(min=finfo.min, max=finfo.max).to(dtype)
+    x_q = x_q.reshape(x.shape)
+    x_s = x_s.reshape(x.shape[:-1] + (x.shape[-1] // group_size,))
+    return x_q, x_s
+
+
+def per_token_group_quant_fp8_div_ref(
+    x: torch.Tensor, group_size: int, eps: float = 1e-10, dtype: torch.dtype = FP8_DTYPE
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Restates ``torch_per_token_group_quant_fp8``
+    (reference tests/test_fused_experts_impl.py:582-601): as above but the scale
+    is the true quotient amax / 448 (the form the reference's device kernel and
+    its MoE fallback use, src/flag_gems/fused/fused_moe.py:664-668)."""
+    assert x.shape[-1] % group_size == 0
+    assert x.is_contiguous()
+    finfo = torch.finfo(dtype)
+    xr = x.reshape(x.numel() // group_size, group_size)
+    amax = xr.abs().max(dim=-1, keepdim=True)[0].clamp(min=eps).to(torch.float32)
+    x_scales = amax / finfo.max
+    x_quant = (xr / x_scales).clamp(min=finfo.min, max=finfo.max).to(dtype)
+    x_quant = x_quant.reshape(x.shape)
+    x_scales = x_scales.reshape(x.shape[:-1] + (x.shape[-1] // group_size,))
+    return x_quant, x_scales
+
+
+# --------------------------------------------------------------------------------------
+# DeepGEMM-style casts used to prepare weights (128x128 blocks) and activations
+# --------------------------------------------------------------------------------------
+def _ceil_to_ue8m0(x: torch.Tensor) -> torch.Tensor:
+    """reference tests/test_fp8_einsum.py:63-67."""
+    bits = x.abs().float().view(torch.int32)
+    exp = ((bits >> 23) & 0xFF) + (bits & 0x7FFFFF).bool().int()
+    return (exp.clamp(1, 254) << 23).view(torch.float32)
+
+
+def per_token_cast_to_fp8_ref(
+    x: torch.Tensor, use_ue8m0: bool = False, gran_k: int = 128
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Restates ``per_token_cast_to_fp8`` (reference tests/test_fp8_einsum.py:70-86)."""
+    assert x.dim() == 2
+    m, n = x.shape
+    padded_n = math.ceil(n / gran_k) * gran_k
+    x_padded = torch.zeros((m, padded_n), dtype=x.dtype)
+    x_padded[:, :n] = x
+    x_view = x_padded.view(m, padded_n // gran_k, gran_k)
+    x_amax = x_view.abs().float().amax(dim=2).view(m, padded_n // gran_k).clamp(1e-4)
+    sf = x_amax / 448.0
+    sf = _ceil_to_ue8m0(sf) if use_ue8m0 else sf
+    x_fp8 = (
+        (x_view * (1.0 / sf.unsqueeze(2)))
+        .to(FP8_DTYPE)
+        .view(m, padded_n)[:, :n]
+        .contiguous()
+    )
+    return x_fp8, sf
+
+
+def per_block_cast_to_fp8_ref(
+    x: torch.Tensor, use_ue8m0: bool = False, gran_k: int = 128
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Restates ``per_block_cast_to_fp8`` (reference tests/test_fp8_einsum.py:89-103):
+    zero-pad to multiples of 128, amax over each (128,128) block in fp32, floor 1e-4,
+    sf = amax / 448, codes = x * (1/sf) cast to e4m3fn (no clamp)."""
+    assert x.dim() == 2
+    m, n = x.shape
+    padded_m = math.ceil(m / gran_k) * gran_k
+    padded_n = math.ceil(n / gran_k) * gran_k
+    x_padded = torch.zeros((padded_m, padded_n), dtype=x.dtype)
+    x_padded[:m, :n] = x
+    x_view = x_padded.view(-1, gran_k, x_padded.size(1) // gran_k, gran_k)
+    x_amax = x_view.abs().float().amax(dim=(1, 3), keepdim=True).clamp(1e-4)
+    sf = x_amax / 448.0
+    sf = _ceil_to_ue8m0(sf) if use_ue8m0 else sf
+    x_scaled = (x_view * (1.0 / sf)).to(FP8_DTYPE)
+    return (
+        x_scaled.view_as(x_padded)[:m, :n].contiguous(),
+        sf.view(x_view.size(0), x_view.size(2)),
+    )
+
+
+# --------------------------------------------------------------------------------------
+# Block-scaled GEMM
+# --------------------------------------------------------------------------------------
+def block_fp8_matmul_dequant_ref(
+    A: torch.Tensor,
+    B: torch.Tensor,
+    As: torch.Tensor,
+    Bs: torch.Tensor,
+    block_size: List[int],
+    output_dtype: torch.dtype = torch.float32,
+    compute_dtype: torch.dtype = torch.float32,
+) -> torch.Tensor:
+    """Restates the reference check of tests/test_w8a8_block_fp8_matmul.py:76-100:
+    dequantise A per (row, K-block) and B per (N-block, K-block) in fp32, then one
+    ``matmul(A_scaled, B_scaled.T)``.  ``compute_dtype=float64`` gives the
+    reference's ``--ref cpu`` mode (tests/accuracy_utils.py:287-302)."""
+    block_n, block_k = block_size
+    k = A.shape[-1]
+    n = B.shape[0]
+    a2 = A.reshape(-1, k).to(torch.float32)
+    as2 = As.reshape(a2.shape[0], -1).to(torch.float32)
+    b2 = B.to(torch.float32)
+    bs2 = Bs.to(torch.float32)
+    num_k_groups = (k + block_k - 1) // block_k
+    num_n_groups = (n + block_n - 1) // block_n
+    a_scaled = torch.zeros_like(a2)
+    for kg in range(num_k_groups):
+        ks, ke = kg * block_k, min((kg + 1) * block_k, k)
+        a_scaled[:, ks:ke] = a2[:, ks:ke] * as2[:, kg : kg + 1]
+    b_scaled = torch.zeros_like(b2)
+    for ng in range(num_n_groups):
+        ns, ne = ng * block_n, min((ng + 1) * block_n, n)
+        for kg in range(num_k_groups):
+            ks, ke = kg * block_k, min((kg + 1) * block_k, k)
+            b_scaled[ns:ne, ks:ke] = b2[ns:ne, ks:ke] * bs2[ng, kg]
+    out = torch.matmul(a_scaled.to(compute_dtype), b_scaled.to(compute_dtype).T)
+    return out.reshape(A.shape[:-1] + (n,)).to(output_dtype)
+
+
+def block_fp8_matmul_tiled_ref(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    a_scales: torch.Tensor,
+    b_scales: torch.Tensor,
+    block_size: List[int],
+    output_dtype: torch.dtype = torch.float32,
+    compute_type: torch.dtype = torch.float32,
+) -> torch.Tensor:
+    """Restates ``torch_w8a8_block_matmul`` (reference
+    tests/test_fused_experts_impl.py:531-579): per (K-tile, N-tile) unscaled
+    ``matmul`` accumulated into C after multiplying by a_scale[:,kt]*b_scale[nt,kt].
+    This is the order of operations of the device kernel
+    (src/flag_gems/ops/w8a8_block_fp8_matmul.py:99-109)."""
+    a = a.to(compute_type)
+    b = b.to(compute_type)
+    assert a.shape[-1] == b.shape[-1]
+    assert b.ndim == 2 and b_scales.ndim == 2
+    block_n, block_k = block_size
+    assert (a.shape[-1] + block_k - 1) // block_k == a_scales.shape[-1]
+    assert a.shape[:-1] == a_scales.shape[:-1]
+    m = a.numel() // a.shape[-1]
+    n, k = b.shape
+    origin_c_shape = a.shape[:-1] + (n,)
+    a = a.reshape(m, a.shape[-1])
+    a_scales = a_scales.reshape(m, a_scales.shape[-1]).to(compute_type)
+    b_scales = b_scales.to(compute_type)
+    n_tiles = (n + block_n - 1) // block_n
+    k_tiles = (k + block_k - 1) // block_k
+    assert n_tiles == b_scales.shape[0] and k_tiles == b_scales.shape[1]
+    c = torch.zeros((m, n), dtype=compute_type)
+    for i in range(k_tiles):
+        a_t = a[:, i * block_k : min((i + 1) * block_k, k)]
+        for j in range(n_tiles):
+            b_t = b[j * block_n : min((j + 1) * block_n, n), i * block_k : min((i + 1) * block_k, k)]
+            scale = a_scales[:, i : i + 1] * b_scales[j][i]
+            c[:, j * block_n : min((j + 1) * block_n, n)] += torch.matmul(a_t, b_t.t()) * scale
+    return c.reshape(origin_c_shape).to(output_dtype)
+
+
+# --------------------------------------------------------------------------------------
+# Per-tensor / per-token x per-channel scaled GEMM
+# --------------------------------------------------------------------------------------
+def scaled_mm_ref(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    scale_a: torch.Tensor,
+    scale_b: torch.Tensor,
+    out_dtype: torch.dtype,
+    bias: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Restates ``baseline_scaled_mm`` (reference tests/test_cutlass_scaled_mm.py:154-187)
+    for scalar / per-row ``scale_a`` ([M,1] or [1]) and scalar / per-column ``scale_b``
+    ([1,N] or [1]): scale the operands in fp32, one fp32 ``mm``, cast to ``out_dtype``,
+    then add the bias in ``out_dtype``."""
+    sa = scale_a.reshape(-1, 1) if scale_a.numel() > 1 else scale_a.reshape(1, 1)
+    sb = scale_b.reshape(1, -1) if scale_b.numel() > 1 else scale_b.reshape(1, 1)
+    lhs = sa * a.to(torch.float32)
+    rhs = sb * b.to(torch.float32)
+    output = torch.mm(lhs, rhs).to(out_dtype)
+    if bias is not None:
+        output = output + bias
+    return output
+
+
+def scaled_mm_ref_postscale(
+    mat1: torch.Tensor,
+    mat2: torch.Tensor,
+    scale_a: torch.Tensor,
+    scale_b: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    out_dtype: Optional[torch.dtype],
+    compute_dtype: torch.dtype = torch.float64,
+) -> torch.Tensor:
+    """Restates ``_reference_scaled_mm`` (reference tests/test_scaled_mm.py:111-124):
+    ``mm`` first (in the reference's float64 "to_reference" precision), then the two
+    scales, then the bias, one final cast."""
+    rows, cols = mat1.shape[0], mat2.shape[1]
+
+    def shaped(scale, is_left):
+        if scale.numel() == 1:
+            return scale
+        if scale.ndim == 1:
+            if is_left and scale.shape[0] == rows:
+                return scale.reshape(rows, 1)
+            if not is_left and scale.shape[0] == cols:
+                return scale.reshape(1, cols)
+        return scale
+
+    ref = mat1.to(compute_dtype).mm(mat2.to(compute_dtype))
+    ref = ref * shaped(scale_a.to(compute_dtype), True)
+    ref = ref * shaped(scale_b.to(compute_dtype), False)
+    if bias is not None:
+        ref = ref + bias.to(compute_dtype)
+    return ref.to(out_dtype or mat1.dtype)
+
+
+# --------------------------------------------------------------------------------------
+# Synthetic inputs of the benchmark configurations
+# --------------------------------------------------------------------------------------
+def make_config1(seed: int = 0):
+    """BASELINE config 1: X bf16 [64,1024] ~N(0,1), W bf16 [512,1024] ~N(0,0.02),
+    generator order X then W, one ``torch.manual_seed(seed)``."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(64, 1024, generator=g).bfloat16()
+    w = (0.02 * torch.randn(512, 1024, generator=g)).bfloat16()
+    return x, w
+
+
+def run_config1(seed: int = 0):
+    """Full CPU reference path of config 1: act_quant -> 128x128 weight quant ->
+    block-scaled matmul -> bf16 [64,512]."""
+    x, w = make_config1(seed)
+    xq, xs = act_quant_ref(x, 128)
+    wq, ws = per_block_cast_to_fp8_ref(w, use_ue8m0=False)
+    c = block_fp8_matmul_tiled_ref(xq, wq, xs, ws, [128, 128], torch.bfloat16)
+    return dict(x=x, w=w, xq=xq, xs=xs, wq=wq, ws=ws, c=c)

@@ -1,0 +1,156 @@
+"""Pins the GEMM functions of oracle/fp8_linear_oracle.py: two independent
+algorithms against each other, a float64 triple loop on tiny shapes, and closed
+forms a wrong index / dropped scale / transposed operand would break."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import e4m3
+from oracle import fp8_linear_oracle as O
+
+FP8 = torch.float8_e4m3fn
+
+
+def _inputs(m, n, k, seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(m, k, generator=g).to(FP8)
+    b = torch.randn(n, k, generator=g).to(FP8)
+    kb, nb = (k + 127) // 128, (n + 127) // 128
+    a_s = 0.01 * torch.rand(m, kb, generator=g) + 0.005
+    b_s = 0.01 * torch.rand(nb, kb, generator=g) + 0.005
+    return a, b, a_s, b_s
+
+
+def _loop_f64(a, b, a_s, b_s):
+    dec = e4m3.decode_table().astype(np.float64)
+    an = dec[a.view(torch.uint8).numpy()]
+    bn = dec[b.view(torch.uint8).numpy()]
+    m, k = an.shape
+    n = bn.shape[0]
+    out = np.zeros((m, n))
+    for i in range(m):
+        for j in range(n):
+            acc = 0.0
+            for kk in range(k):
+                acc += an[i, kk] * bn[j, kk] * float(a_s[i, kk // 128]) * float(b_s[j // 128, kk // 128])
+            out[i, j] = acc
+    return out
+
+
+@pytest.mark.parametrize("shape", [(3, 5, 128), (4, 130, 200), (2, 7, 300)])
+def test_block_matmul_refs_vs_f64_loop(shape):
+    m, n, k = shape
+    a, b, a_s, b_s = _inputs(m, n, k, 11)
+    want = _loop_f64(a, b, a_s, b_s)
+    for fn in (O.block_fp8_matmul_dequant_ref, O.block_fp8_matmul_tiled_ref):
+        got = fn(a, b, a_s, b_s, [128, 128], torch.float32).double().numpy()
+        np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("shape", [(64, 512, 1024), (83, 260, 3884 // 4), (17, 2112, 512)])
+def test_two_block_matmul_algorithms_agree(shape):
+    m, n, k = shape
+    a, b, a_s, b_s = _inputs(m, n, k, 12)
+    x = O.block_fp8_matmul_dequant_ref(a, b, a_s, b_s, [128, 128], torch.float32)
+    y = O.block_fp8_matmul_tiled_ref(a, b, a_s, b_s, [128, 128], torch.float32)
+    z = O.block_fp8_matmul_dequant_ref(a, b, a_s, b_s, [128, 128], torch.float64, torch.float64)
+    torch.testing.assert_close(x, y, rtol=1e-4, atol=1e-6)
+    torch.testing.assert_close(x.double(), z, rtol=1e-4, atol=1e-6)
+
+
+def test_unit_scales_reduce_to_plain_matmul():
+    a, b, a_s, b_s = _inputs(16, 256, 384, 13)
+    one_a, one_b = torch.ones_like(a_s), torch.ones_like(b_s)
+    want = a.float() @ b.float().T  # exact: products of e4m3 values, small sums in fp32
+    for fn in (O.block_fp8_matmul_dequant_ref, O.block_fp8_matmul_tiled_ref):
+        got = fn(a, b, one_a, one_b, [128, 128], torch.float32)
+        torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-4)
+
+
+def test_one_hot_rows_pick_scaled_weight_entries():
+    # A row with a single 1.0 at column c: C[m, n] = B[n, c] * As[m, c//128] * Bs[n//128, c//128]
+    _, b, a_s, b_s = _inputs(4, 300, 512, 14)
+    cols = [0, 127, 128, 511]
+    a = torch.zeros(4, 512)
+    for r, c in enumerate(cols):
+        a[r, c] = 1.0
+    a = a.to(FP8)
+    for fn in (O.block_fp8_matmul_dequant_ref, O.block_fp8_matmul_tiled_ref):
+        got = fn(a, b, a_s, b_s, [128, 128], torch.float32)
+        for r, c in enumerate(cols):
+            want = b[:, c].float() * a_s[r, c // 128] * b_s[:, c // 128].repeat_interleave(128)[:300]
+            torch.testing.assert_close(got[r], want, rtol=1e-6, atol=0)
+
+
+def test_power_of_two_scales_are_exact_and_k_block_specific():
+    a, b, _, _ = _inputs(8, 128, 256, 15)
+    a_s = torch.tensor([[2.0, 0.5]]).repeat(8, 1)
+    b_s = torch.tensor([[0.25, 4.0]])
+    af, bf = a.float(), b.float()
+    want = (af[:, :128] @ bf[:, :128].T) * 0.5 + (af[:, 128:] @ bf[:, 128:].T) * 2.0
+    for fn in (O.block_fp8_matmul_dequant_ref, O.block_fp8_matmul_tiled_ref):
+        got = fn(a, b, a_s, b_s, [128, 128], torch.float32)
+        torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-5)
+
+
+def test_leading_dims_are_kept():
+    a, b, a_s, b_s = _inputs(6, 130, 256, 16)
+    got = O.block_fp8_matmul_tiled_ref(a.view(2, 3, 256), b, a_s.view(2, 3, 2), b_s, [128, 128], torch.bfloat16)
+    assert got.shape == (2, 3, 130) and got.dtype == torch.bfloat16
+    flat = O.block_fp8_matmul_tiled_ref(a, b, a_s, b_s, [128, 128], torch.bfloat16)
+    assert torch.equal(got.view(6, 130), flat)
+
+
+# ---------------------------------------------------------------- scaled_mm
+def _smm_inputs(m, n, k, seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(m, k, generator=g).to(FP8)
+    b = torch.randn(k, n, generator=g).t().contiguous().t().to(FP8)  # column-major
+    sa = torch.randn(m, 1, generator=g)
+    sb = torch.randn(1, n, generator=g)
+    bias = torch.randn(n, generator=g).bfloat16()
+    return a, b, sa, sb, bias
+
+
+def test_scaled_mm_refs_vs_f64_loop_and_each_other():
+    a, b, sa, sb, bias = _smm_inputs(5, 9, 64, 21)
+    dec = e4m3.decode_table().astype(np.float64)
+    an = dec[a.view(torch.uint8).numpy()]
+    bn = dec[b.view(torch.uint8).numpy()]
+    want = np.zeros((5, 9))
+    for i in range(5):
+        for j in range(9):
+            want[i, j] = sum(an[i, kk] * bn[kk, j] for kk in range(64)) * float(sa[i, 0]) * float(sb[0, j])
+    got = O.scaled_mm_ref(a, b, sa, sb, torch.float32).double().numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+    got2 = O.scaled_mm_ref_postscale(a, b, sa, sb, None, torch.float32).double().numpy()
+    np.testing.assert_allclose(got2, want, rtol=1e-6, atol=1e-6)
+    # bias is added after the cast, in the output dtype
+    with_bias = O.scaled_mm_ref(a, b, sa, sb, torch.bfloat16, bias)
+    no_bias = O.scaled_mm_ref(a, b, sa, sb, torch.bfloat16)
+    assert torch.equal(with_bias, no_bias + bias)
+
+
+def test_scaled_mm_scalar_and_unit_scales():
+    a, b, _, _, _ = _smm_inputs(7, 33, 128, 22)
+    one = torch.ones(1)
+    plain = a.float() @ b.float()
+    torch.testing.assert_close(O.scaled_mm_ref(a, b, one, one, torch.float32), plain, rtol=0, atol=0)
+    s = torch.tensor([0.5])
+    torch.testing.assert_close(O.scaled_mm_ref(a, b, s, one, torch.float32), plain * 0.5, rtol=0, atol=0)
+    # per-row scale really scales rows (a transposed broadcast would fail here)
+    sa = torch.arange(1, 8).float().reshape(7, 1)
+    torch.testing.assert_close(O.scaled_mm_ref(a, b, sa, one, torch.float32), plain * sa, rtol=1e-6, atol=1e-5)
+    sb = torch.arange(1, 34).float().reshape(1, 33)
+    torch.testing.assert_close(O.scaled_mm_ref(a, b, one, sb, torch.float32), plain * sb, rtol=1e-6, atol=1e-5)
+
+
+def test_config1_pipeline_is_self_consistent():
+    r = O.run_config1(0)
+    assert r["xq"].shape == (64, 1024) and r["xs"].shape == (64, 8)
+    assert r["wq"].shape == (512, 1024) and r["ws"].shape == (4, 8)
+    assert r["c"].shape == (64, 512) and r["c"].dtype == torch.bfloat16
+    # quantized linear approximates the bf16 linear: relative Frobenius error of fp8 (3 mantissa bits)
+    want = r["x"].float() @ r["w"].float().T
+    rel = (r["c"].float() - want).norm() / want.norm()
+    assert rel < 0.05

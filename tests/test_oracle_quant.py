@@ -1,0 +1,213 @@
+"""Pins the quantizer functions of oracle/fp8_linear_oracle.py.
+
+Checks: a numpy brute-force quantizer built on the bit-level encoder of
+oracle/e4m3.py, hand-worked known answers, and invariants that hold for any
+seed.  Reference functions restated by the oracle are cited there."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import e4m3
+from oracle import fp8_linear_oracle as O
+
+F32 = np.float32
+
+
+def _brute_quant(x_f32: np.ndarray, group: int, floor: float, scale_rule: str, quot_rule: str, ue8m0: str = "none"):
+    """Scalar loops over groups; IEEE float32 arithmetic through numpy scalars."""
+    rows, cols = x_f32.shape
+    codes = np.zeros((rows, cols), dtype=np.uint8)
+    scales = np.zeros((rows, cols // group), dtype=np.float32)
+    inv448 = F32(1.0) / F32(448.0)
+    for r in range(rows):
+        for g in range(cols // group):
+            seg = x_f32[r, g * group : (g + 1) * group]
+            amax = F32(0.0)
+            for v in seg:
+                av = F32(abs(v))
+                if np.isnan(av) or av > amax:
+                    amax = av
+                    if np.isnan(av):
+                        break
+            if not np.isnan(amax) and amax < F32(floor):
+                amax = F32(floor)
+            s = amax * inv448 if scale_rule == "mul" else amax / F32(448.0)
+            if ue8m0 == "bits":
+                b = np.array([s], dtype=np.float32).view(np.uint32)[0]
+                e = ((b >> 23) & 0xFF) + (1 if b & 0x7FFFFF else 0)
+                s = np.array([e << 23], dtype=np.uint32).view(np.float32)[0]
+            elif ue8m0 == "log2":
+                s = F32(2.0) ** F32(np.ceil(np.log2(max(abs(s), F32(1e-10)))))
+            if quot_rule == "recip":
+                q = seg * (F32(1.0) / s)
+            else:
+                q = seg / s
+            q = np.minimum(np.maximum(q, F32(-448.0)), F32(448.0))  # propagates NaN
+            codes[r, g * group : (g + 1) * group] = e4m3.encode(q.astype(np.float32))
+            scales[r, g] = s
+    return codes, scales
+
+
+def _rand_bf16(rows, cols, seed, kind="randn"):
+    g = torch.Generator().manual_seed(seed)
+    if kind == "randn":
+        x = torch.randn(rows, cols, generator=g)
+    elif kind == "rand":
+        x = torch.rand(rows, cols, generator=g)
+    else:  # heavy tailed, spans many binades
+        x = torch.randn(rows, cols, generator=g) * torch.exp(3 * torch.randn(rows, cols, generator=g))
+    return x.bfloat16()
+
+
+@pytest.mark.parametrize("kind", ["randn", "rand", "wide"])
+@pytest.mark.parametrize("group", [64, 128])
+def test_act_quant_ref_vs_brute_force(kind, group):
+    x = _rand_bf16(6, 512, 3, kind)
+    y, s = O.act_quant_ref(x, group)
+    codes, scales = _brute_quant(x.float().numpy(), group, 1e-4, "mul", "recip")
+    assert np.array_equal(y.view(torch.uint8).numpy(), codes)
+    assert np.array_equal(s.numpy().view(np.uint32), scales.view(np.uint32))
+
+
+@pytest.mark.parametrize("kind", ["randn", "wide"])
+def test_act_quant_ref_ue8m0_vs_brute_force(kind):
+    x = _rand_bf16(5, 384, 4, kind)
+    y, s = O.act_quant_ref(x, 128, "ue8m0")
+    codes, scales = _brute_quant(x.float().numpy(), 128, 1e-4, "mul", "recip", "bits")
+    assert np.array_equal(y.view(torch.uint8).numpy(), codes)
+    assert np.array_equal(s.numpy().view(np.uint32), scales.view(np.uint32))
+    # a power of two in [raw, 2*raw)
+    raw = x.float().view(5, 3, 128).abs().amax(-1).clamp(min=1e-4) * (1.0 / 448.0)
+    assert torch.all(s >= raw) and torch.all(s < 2 * raw)
+    assert torch.all((s.view(torch.int32) & 0x7FFFFF) == 0)
+
+
+@pytest.mark.parametrize("kind", ["randn", "rand", "wide"])
+@pytest.mark.parametrize("group", [64, 128, 256])
+@pytest.mark.parametrize("ue8m0", [False, True])
+def test_group_quant_ref_vs_brute_force(kind, group, ue8m0):
+    x = _rand_bf16(4, 512, 5, kind)
+    y, s = O.per_token_group_quant_fp8_ref(x, group, scale_ue8m0=ue8m0)
+    # bf16 amax then widening equals fp32 amax of the widened values (max is exact);
+    # the eps floor is applied in bf16: bf16(1e-10)
+    floor = float(torch.tensor(1e-10, dtype=torch.bfloat16).float())
+    codes, scales = _brute_quant(x.float().numpy(), group, floor, "mul", "div", "log2" if ue8m0 else "none")
+    assert np.array_equal(y.view(torch.uint8).numpy(), codes)
+    assert np.array_equal(s.numpy().view(np.uint32), scales.view(np.uint32))
+
+
+def test_group_quant_div_ref_vs_brute_force():
+    x = _rand_bf16(4, 512, 6, "wide")
+    y, s = O.per_token_group_quant_fp8_div_ref(x, 128)
+    floor = float(torch.tensor(1e-10, dtype=torch.bfloat16).float())
+    codes, scales = _brute_quant(x.float().numpy(), 128, floor, "div", "div")
+    assert np.array_equal(y.view(torch.uint8).numpy(), codes)
+    assert np.array_equal(s.numpy().view(np.uint32), scales.view(np.uint32))
+
+
+def test_mul_and_div_scale_rules_really_differ():
+    # the two scale formulas disagree in the last bit for about half of all amax
+    # values, so a test that passes with the wrong rule would show here
+    amax = torch.arange(0x3C00, 0x4400, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    a = amax * torch.tensor(1.0 / 448.0)
+    b = amax / 448.0
+    frac = (a != b).float().mean().item()
+    assert 0.3 < frac < 0.8
+
+
+def test_known_answers_unit_scale_group():
+    # amax 448 -> scale = 448 * fp32(1/448) = 1.0 exactly, so codes are the plain cast
+    vals = [448.0, 224.0, 1.0, 0.30078125, -17.25, 0.0, -0.0, 2.0 ** -9]
+    x = torch.zeros(1, 128)
+    x[0, : len(vals)] = torch.tensor(vals)
+    x = x.bfloat16()
+    want = [0x7E, 0x76, 0x38, 0x2A, 0xD9, 0x00, 0x80, 0x01]
+    for fn in (lambda t: O.act_quant_ref(t, 128), lambda t: O.per_token_group_quant_fp8_ref(t, 128)):
+        y, s = fn(x)
+        assert s.item() == 1.0
+        assert list(y.view(torch.uint8)[0, : len(vals)].numpy()) == want
+
+
+def test_special_cases():
+    x = torch.zeros(2, 256).bfloat16()
+    y, s = O.act_quant_ref(x, 128)
+    assert torch.all(y.view(torch.uint8) == 0)
+    assert torch.all(s == torch.tensor(1e-4) * torch.tensor(1.0 / 448.0))
+    y, s = O.per_token_group_quant_fp8_ref(x, 128)
+    assert torch.all(y.view(torch.uint8) == 0)
+    assert torch.all(s == torch.tensor(1e-10, dtype=torch.bfloat16).float() * torch.tensor(1.0 / 448.0))
+    # NaN poisons its own group only
+    x = torch.ones(1, 256).bfloat16()
+    x[0, 5] = float("nan")
+    y, s = O.act_quant_ref(x, 128)
+    assert torch.isnan(s[0, 0]) and not torch.isnan(s[0, 1])
+    assert torch.all((y.view(torch.uint8)[0, :128] & 0x7F) == 0x7F)
+    assert torch.all(y.view(torch.uint8)[0, 128:] == 0x7E)
+    # Inf: scale inf, finite elements -> 0, the Inf itself -> NaN (inf * 0)
+    x = torch.ones(1, 128).bfloat16()
+    x[0, 7] = float("inf")
+    y, s = O.act_quant_ref(x, 128)
+    assert torch.isinf(s[0, 0])
+    c = y.view(torch.uint8)[0]
+    assert c[7] & 0x7F == 0x7F and c[0] == 0
+    # lone huge element: everything else flushes to zero, the element itself is 448
+    x = torch.full((1, 128), 1e-3).bfloat16()
+    x[0, 100] = -3e38
+    y, s = O.act_quant_ref(x, 128)
+    c = y.view(torch.uint8)[0]
+    assert c[100] == 0xFE and torch.all(c[:100] == 0)
+
+
+@pytest.mark.parametrize("fn", ["act", "group", "div"])
+def test_invariants(fn):
+    x = _rand_bf16(64, 1024, 7, "wide")
+    f = {
+        "act": lambda t: O.act_quant_ref(t, 128),
+        "group": lambda t: O.per_token_group_quant_fp8_ref(t, 128),
+        "div": lambda t: O.per_token_group_quant_fp8_div_ref(t, 128),
+    }[fn]
+    y, s = f(x)
+    yn, sn = f(-x)
+    assert torch.equal(s, sn)
+    assert torch.equal(y.view(torch.uint8) ^ 0x80, yn.view(torch.uint8))
+    # the max-magnitude element of every group encodes to +-448
+    xg = x.float().view(64, 8, 128)
+    idx = xg.abs().argmax(-1, keepdim=True)
+    top = y.view(torch.uint8).view(64, 8, 128).gather(-1, idx)
+    assert torch.all((top & 0x7F) == 0x7E)
+    # dequantised value within half an fp8 step of x/s (step <= 2**-4 relative, 2**-10 absolute)
+    q = xg / s.unsqueeze(-1)
+    d = y.float().view(64, 8, 128)
+    err = (d - q).abs()
+    assert torch.all(err <= torch.maximum(q.abs() * 2.0 ** -4, torch.tensor(2.0 ** -10)) * 1.0001)
+    # row order does not matter
+    perm = torch.randperm(64, generator=torch.Generator().manual_seed(0))
+    yp, sp = f(x[perm].contiguous())
+    assert torch.equal(sp, s[perm]) and torch.equal(yp.view(torch.uint8), y.view(torch.uint8)[perm])
+
+
+def test_per_block_cast_vs_brute_force():
+    g = torch.Generator().manual_seed(8)
+    w = (0.02 * torch.randn(200, 300, generator=g)).bfloat16()
+    wq, ws = O.per_block_cast_to_fp8_ref(w)
+    assert wq.shape == (200, 300) and ws.shape == (2, 3)
+    wn = w.float().numpy()
+    for bi in range(2):
+        for bj in range(3):
+            blk = wn[bi * 128 : (bi + 1) * 128, bj * 128 : (bj + 1) * 128]
+            amax = max(F32(np.abs(blk).max()), F32(1e-4))
+            sf = F32(amax) / F32(448.0)
+            assert ws[bi, bj].item() == sf
+            codes = e4m3.encode((blk * (F32(1.0) / sf)).astype(np.float32))
+            got = wq.view(torch.uint8).numpy()[bi * 128 : (bi + 1) * 128, bj * 128 : (bj + 1) * 128]
+            assert np.array_equal(codes, got)
+
+
+def test_per_token_cast_matches_group_quant_shape_and_scale():
+    x = _rand_bf16(5, 300, 9)
+    xq, sf = O.per_token_cast_to_fp8_ref(x, use_ue8m0=False)
+    assert xq.shape == (5, 300) and sf.shape == (5, 3)
+    amax = torch.zeros(5, 384)
+    amax[:, :300] = x.float()
+    want = amax.view(5, 3, 128).abs().amax(-1).clamp(1e-4) / 448.0
+    assert torch.equal(sf, want)
