@@ -1,0 +1,47 @@
+"""flaggems_amd: MI355X (gfx950) implementation of FlagGems' FP8 quantized-linear operators.
+
+The public names, signatures and registration entry points follow the reference package
+``flag_gems`` for this path (see each module's docstring for file:line citations); the compute is
+hand-written HIP reached through the C ABI in include/flaggems_amd.h.  Importing the package does
+not touch a GPU and does not load the shared library; the first operator call does, and fails
+loudly if the library has not been built (``python -m flaggems_amd.build``).
+"""
+from .act_quant import (  # noqa: F401
+    SUPPORTED_FP8_DTYPE,
+    act_quant_triton,
+    per_token_group_quant_fp8,
+)
+from .cutlass_scaled_mm import SM_VERSION_NUM, cutlass_scaled_mm, get_sm_version_num  # noqa: F401
+from .registration import (  # noqa: F401
+    all_registered_keys,
+    all_registered_ops,
+    apply_gems_patches_to_vllm,
+    enable,
+    only_enable,
+    patch_empty_vllm,
+    use_gems,
+)
+from .scaled_mm import scaled_mm, scaled_mm_out  # noqa: F401
+from .w8a8_block_fp8_matmul import fp8_matmul, w8a8_block_fp8_matmul  # noqa: F401
+
+__version__ = "0.1.0"
+device = "cuda"  # PyTorch-ROCm device type of an MI355X
+vendor_name = "amd"
+
+__all__ = [
+    "SUPPORTED_FP8_DTYPE",
+    "act_quant_triton",
+    "all_registered_keys",
+    "all_registered_ops",
+    "apply_gems_patches_to_vllm",
+    "cutlass_scaled_mm",
+    "enable",
+    "fp8_matmul",
+    "only_enable",
+    "patch_empty_vllm",
+    "per_token_group_quant_fp8",
+    "scaled_mm",
+    "scaled_mm_out",
+    "use_gems",
+    "w8a8_block_fp8_matmul",
+]

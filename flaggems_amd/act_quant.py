@@ -1,0 +1,207 @@
+"""Per-token-group activation quantizers (host side).
+
+Mirrors the reference entry points
+  act_quant_triton          src/flag_gems/fused/act_quant.py:111-174
+  per_token_group_quant_fp8 src/flag_gems/ops/per_token_group_quant_fp8.py:227-336
+and the vLLM op adapter     src/flag_gems/patches/patch_vllm_all.py:425-448
+with the same parameters, defaults, return conventions and assertion behaviour.  The work is done
+by the HIP kernel behind fg_group_quant_fp8.
+
+Rounding contract.  Codes and scales are bit-identical to the reference's torch implementations
+(tests/test_act_quant.py:48-98 for act_quant_triton, tests/test_per_token_group_quant_fp8.py:23-48
+for per_token_group_quant_fp8): scale = amax * fp32(1/448); act_quant multiplies by the rounded
+reciprocal of the scale, per_token_group_quant_fp8 divides; the eps floor of
+per_token_group_quant_fp8 is applied in the input's dtype.  ``scale_rule="div"`` selects the
+true-quotient scale amax / 448 that the reference's device kernel and MoE fallback use
+(src/flag_gems/fused/fused_moe.py:664-668).
+"""
+from __future__ import annotations
+
+import functools
+import logging
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+logger = logging.getLogger("flag_gems." + __name__.split(".")[-1])
+
+# gfx950 converts to and from OCP e4m3fn natively
+SUPPORTED_FP8_DTYPE = torch.float8_e4m3fn
+
+_IN_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
+_FP8_DTYPES = (torch.float8_e4m3fn, torch.float8_e5m2)
+
+
+@functools.lru_cache(maxsize=64)
+def _round_to_dtype(value: float, dtype: torch.dtype) -> float:
+    return float(torch.tensor(value, dtype=dtype).float())
+
+
+def _scale_rule_code(rule: Optional[str]) -> int:
+    if rule is None or rule == "mul":
+        return _lib.FG_SCALE_MUL_INV
+    if rule == "div":
+        return _lib.FG_SCALE_DIV
+    raise ValueError(f"scale_rule must be 'mul' or 'div', got {rule!r}")
+
+
+def _launch_group_quant(
+    x2d: torch.Tensor,
+    q2d: torch.Tensor,
+    s2d: torch.Tensor,
+    group_size: int,
+    floor: float,
+    fp8_min: float,
+    fp8_max: float,
+    scale_rule: int,
+    quotient_rule: int,
+    pow2_rule: int,
+) -> None:
+    """x2d [R, C] unit column stride; q2d same shape; s2d [R, C/g] any strides."""
+    _lib.require_gpu(x2d, "group quantizer")
+    lib = _lib.load()
+    rows, cols = x2d.shape
+    with torch.cuda.device(x2d.device):
+        status = lib.fg_group_quant_fp8(
+            x2d.data_ptr(), _lib.DTYPE_CODE[x2d.dtype], rows, cols, x2d.stride(0) if rows > 1 else max(cols, x2d.stride(0)),
+            q2d.data_ptr(), _lib.DTYPE_CODE[q2d.dtype], q2d.stride(0) if rows > 1 else max(cols, q2d.stride(0)),
+            s2d.data_ptr(), s2d.stride(0), s2d.stride(1),
+            group_size, floor, fp8_min, fp8_max, 1.0 / fp8_max,
+            scale_rule, quotient_rule, pow2_rule,
+            _lib.current_stream_ptr(x2d.device),
+        )
+    _lib.check(status, "fg_group_quant_fp8")
+
+
+def act_quant_triton(
+    x: torch.Tensor, block_size: int = 128, scale_fmt: Optional[str] = None
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Block-wise FP8 quantization of the last dimension.
+
+    Returns (y, s): y has x's shape and dtype float8_e4m3fn, s has shape
+    ``x.shape[:-1] + (x.shape[-1] // block_size,)`` and dtype float32.  With ``scale_fmt`` set the
+    scale is rounded up to a power of two.  The name is kept for drop-in compatibility; nothing
+    here uses Triton.
+    """
+    logger.debug("GEMS ACT_QUANT")
+    assert x.is_contiguous(), "Input tensor must be contiguous"
+    assert (
+        x.size(-1) % block_size == 0
+    ), f"Last dimension size must be divisible by block_size (block_size={block_size})"
+    if x.dtype not in _IN_DTYPES:
+        raise NotImplementedError(f"act_quant: unsupported input dtype {x.dtype}")
+    n = x.size(-1)
+    n_blocks = n // block_size
+    y = torch.empty_like(x, dtype=torch.float8_e4m3fn)
+    s = x.new_empty(*x.size()[:-1], n_blocks, dtype=torch.float32)
+    if x.numel() == 0:
+        return y, s
+    _launch_group_quant(
+        x.view(-1, n), y.view(-1, n), s.view(-1, n_blocks), block_size,
+        floor=1e-4, fp8_min=-448.0, fp8_max=448.0,
+        scale_rule=_lib.FG_SCALE_MUL_INV, quotient_rule=_lib.FG_QUOT_RECIP_MUL,
+        pow2_rule=_lib.FG_POW2_BITS if scale_fmt is not None else _lib.FG_POW2_NONE,
+    )
+    return y, s
+
+
+def _as_rows(x: torch.Tensor) -> torch.Tensor:
+    """View x as [rows, last] with unit column stride (copies only if the layout forces it)."""
+    if x.dim() == 2:
+        return x
+    if x.dim() == 1:
+        return x.view(1, -1)
+    if not x.is_contiguous():
+        x = x.contiguous()
+    return x.view(-1, x.shape[-1])
+
+
+def per_token_group_quant_fp8(
+    x: torch.Tensor,
+    group_size: int,
+    eps: float = 1e-10,
+    dtype: Optional[torch.dtype] = None,
+    column_major_scales: bool = False,
+    scale_ue8m0: bool = False,
+    *,
+    scale_rule: Optional[str] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-token-group quantization of ``x`` along its last dimension.
+
+    Returns (x_q, x_s).  ``x_s`` is float32 of shape ``x.shape[:-1] + (x.shape[-1] // group_size,)``,
+    row-major, or with strides (1, M) when ``column_major_scales`` is set.
+    """
+    logger.debug("GEMS PER TOKEN GROUP QUANT FP8")
+    fp8_dtype = SUPPORTED_FP8_DTYPE if dtype is None else dtype
+    assert x.shape[-1] % group_size == 0, (
+        f"the last dimension of `x` {x.shape[-1]} must be divisible "
+        f"by `group_size` {group_size}"
+    )
+    assert x.stride(-1) == 1, "`x` groups must be contiguous"
+    if fp8_dtype not in _FP8_DTYPES:
+        raise NotImplementedError(f"per_token_group_quant_fp8: unsupported output dtype {fp8_dtype}")
+    if x.dtype not in _IN_DTYPES:
+        raise NotImplementedError(f"per_token_group_quant_fp8: unsupported input dtype {x.dtype}")
+    finfo = torch.finfo(fp8_dtype)
+
+    # the reference kernel addresses x_q as a dense row-major image of x; allocate it that way
+    x_q = torch.empty(x.shape, device=x.device, dtype=fp8_dtype)
+    if column_major_scales:
+        shape = (x.shape[-1] // group_size,) + x.shape[:-1]
+        x_s = torch.empty(shape, device=x.device, dtype=torch.float32).permute(-1, -2)
+    else:
+        shape = x.shape[:-1] + (x.shape[-1] // group_size,)
+        x_s = torch.empty(shape, device=x.device, dtype=torch.float32)
+    if x.numel() == 0:
+        return x_q, x_s
+
+    x2d = _as_rows(x)
+    q2d = x_q.view(-1, x.shape[-1])
+    if x_s.dim() == 2:
+        s2d = x_s
+    elif not column_major_scales:
+        s2d = x_s.view(-1, x_s.shape[-1])
+    else:
+        raise NotImplementedError("column_major_scales needs a 2-D input")
+    _launch_group_quant(
+        x2d, q2d, s2d, group_size,
+        floor=_round_to_dtype(float(eps), x.dtype), fp8_min=finfo.min, fp8_max=finfo.max,
+        scale_rule=_scale_rule_code(scale_rule), quotient_rule=_lib.FG_QUOT_DIV,
+        pow2_rule=_lib.FG_POW2_LOG2 if scale_ue8m0 else _lib.FG_POW2_NONE,
+    )
+    return x_q, x_s
+
+
+def per_token_group_fp8_quant_into(
+    input: torch.Tensor,
+    output_q: torch.Tensor,
+    output_s: torch.Tensor,
+    group_size: int,
+    eps: float,
+    fp8_min: float,
+    fp8_max: float,
+    scale_ue8m0: bool = False,
+) -> None:
+    """vLLM ``_C::per_token_group_fp8_quant``: quantize into caller-owned buffers, honouring the
+    strides of ``output_s`` (row- or column-major).  The reference adapter computes into fresh
+    tensors and copies (src/flag_gems/patches/patch_vllm_all.py:425-448); here the kernel writes
+    the caller's buffers directly."""
+    logger.debug("GEMS PER TOKEN GROUP QUANT FP8")
+    assert input.shape[-1] % group_size == 0
+    assert input.stride(-1) == 1, "`x` groups must be contiguous"
+    assert output_q.shape == input.shape and output_s.dtype == torch.float32
+    if input.numel() == 0:
+        return
+    x2d = _as_rows(input)
+    if output_q.stride(-1) != 1 or (output_q.dim() > 2 and not output_q.is_contiguous()):
+        raise NotImplementedError("output_q must have unit stride in its last dimension")
+    q2d = output_q if output_q.dim() == 2 else output_q.view(-1, input.shape[-1])
+    s2d = output_s if output_s.dim() == 2 else output_s.view(-1, output_s.shape[-1])
+    _launch_group_quant(
+        x2d, q2d, s2d, group_size,
+        floor=_round_to_dtype(float(eps), input.dtype), fp8_min=float(fp8_min), fp8_max=float(fp8_max),
+        scale_rule=_lib.FG_SCALE_MUL_INV, quotient_rule=_lib.FG_QUOT_DIV,
+        pow2_rule=_lib.FG_POW2_LOG2 if scale_ue8m0 else _lib.FG_POW2_NONE,
+    )

@@ -1,0 +1,455 @@
+// FP8 (OCP e4m3fn) GEMM kernels for gfx950: block-scaled (1x128 activation scales, 128x128 weight
+// scales) and per-row x per-column scaled with optional bias.
+//
+// Operand roles.  The problem is C[m, n] = sum_k X[m, k] * W[n, k] with both operands K-contiguous
+// ("NT").  The weight tile takes the MFMA A slot and the activation tile the B slot
+// (v_mfma_f32_16x16x128_f8f6f4 computes D[i][j] += sum_k A[i][k] B[j][k] with i = weight row n,
+// j = activation row m).  A lane then holds four consecutive n for a single m, so one fp32 scale
+// value As[m, kb] * Bs[n / 128, kb] covers all four of its results and the four results form one
+// 8-byte bf16 store.
+//
+// Data path.  Tiles of BN x 128 weight bytes and BM x 128 activation bytes per K-block are staged in
+// LDS, double buffered.  When rows are 16-byte aligned and K % 128 == 0 the tiles go from global
+// memory straight into LDS (global_load_lds_dwordx4, 1 KB per wavefront instruction); otherwise a
+// guarded register-staged loader zero-fills the K tail.  The 16-byte chunk index of every row is
+// XOR-swizzled with (row >> 1) & 7 so that the 16 rows read by one ds_read_b128 fall into 16
+// different bank groups.  In block-scaled mode every K-block's MFMA result is multiplied by its fp32
+// scale and added to the running fp32 accumulator (4 VALU FMAs per MFMA); in row/column mode the
+// MFMA accumulates directly and the scales are applied once in the epilogue.
+
+#include "fg_common.h"
+
+namespace fg {
+namespace {
+
+enum { kModeBlock = 0, kModeRowCol = 1 };
+
+struct GemmArgs {
+  const uint8_t* X;  // activations [M, K]
+  const uint8_t* W;  // weights [N, K]
+  void* C;
+  const float* xs;   // block: As [M, KB]; rowcol: a_scale
+  const float* ws;   // block: Bs [NB, KB]; rowcol: b_scale
+  const void* bias;
+  int64_t ldx, ldw, ldc;
+  int64_t xs_rs, xs_cs, ws_rs, ws_cs;
+  int M, N, K, KB;
+  int tiles_m, tiles_n;
+  int c_dtype, bias_dtype;
+  int xs_per_row, ws_per_col;
+};
+
+__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
+
+// s_waitcnt vmcnt(0) with expcnt/lgkmcnt left at their maxima (gfx9 encoding)
+__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return bits_to_float((uint32_t)b << 16); }
+
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = float_to_bits(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);  // quiet NaN
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float load_as_float(const void* p, int64_t i, int dtype) {
+  if (dtype == FG_F32) return reinterpret_cast<const float*>(p)[i];
+  if (dtype == FG_F16) return (float)reinterpret_cast<const _Float16*>(p)[i];
+  return bf16_bits_to_float(reinterpret_cast<const uint16_t*>(p)[i]);
+}
+
+// Map the hardware block id to a tile so that (a) the blocks one XCD receives (ids congruent mod 8)
+// form a contiguous run of tiles and (b) a run walks GROUP_M tile rows before moving along N, which
+// keeps the 32 tiles resident on an XCD inside a compact patch that shares operand panels in its L2.
+__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  const int xcd = bid & 7, local = bid >> 3;
+  const int base = total >> 3, rem = total & 7;
+  const int sid = xcd * base + (xcd < rem ? xcd : rem) + local;
+  constexpr int GROUP_M = 4;
+  const int per_group = GROUP_M * tiles_n;
+  const int g = sid / per_group;
+  const int first_m = g * GROUP_M;
+  const int gm = (tiles_m - first_m < GROUP_M) ? tiles_m - first_m : GROUP_M;
+  const int r = sid - g * per_group;
+  tm = first_m + r % gm;
+  tn = r / gm;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Tile loaders.  A tile is ROWS rows of 128 bytes; chunk i (16 bytes) of the LDS image holds logical
+// chunk (i & 7) ^ swz(i >> 3) of row i >> 3.
+// ---------------------------------------------------------------------------------------------
+template <int ROWS, int NTHREADS>
+__device__ __forceinline__ void load_tile_direct(const uint8_t* __restrict__ g, int64_t ld, int row0, int row_max,
+                                                 int k0, uint8_t* lds_tile, int wave, int lane) {
+  constexpr int kWaves = NTHREADS / 64;
+  constexpr int kSlabs = ROWS / 8;  // 1 KB slabs
+  static_assert(kSlabs % kWaves == 0, "tile rows must split evenly over the wavefronts");
+#pragma unroll
+  for (int j = 0; j < kSlabs / kWaves; ++j) {
+    const int slab = wave + j * kWaves;
+    const int r = slab * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ swz(r);
+    int gr = row0 + r;
+    gr = gr < row_max ? gr : row_max;  // rows past the edge re-read the last valid row
+    const uint8_t* src = g + (int64_t)gr * ld + k0 + c * 16;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                     (__attribute__((address_space(3))) void*)(lds_tile + slab * 1024), 16, 0, 0);
+  }
+}
+
+template <int ROWS, int NTHREADS>
+struct StagedTile {
+  static constexpr int kChunks = ROWS * 8 / NTHREADS;
+  static_assert(ROWS * 8 % NTHREADS == 0, "tile chunks must split evenly over the threads");
+  u32x4 v[kChunks];
+
+  // Loads with row and K guards; bytes past K are zero.  `aligned16` selects 16-byte loads.
+  __device__ __forceinline__ void load(const uint8_t* __restrict__ g, int64_t ld, int row0, int row_max, int k0,
+                                       int K, bool aligned16, int tid) {
+#pragma unroll
+    for (int j = 0; j < kChunks; ++j) {
+      const int i = tid + j * NTHREADS;
+      const int r = i >> 3;
+      const int c = (i & 7) ^ swz(r);
+      int gr = row0 + r;
+      gr = gr < row_max ? gr : row_max;
+      const int k = k0 + c * 16;
+      const uint8_t* src = g + (int64_t)gr * ld + k;
+      u32x4 t = {0u, 0u, 0u, 0u};
+      if (aligned16 && k + 16 <= K) {
+        t = *reinterpret_cast<const u32x4*>(src);
+      } else if (k < K) {
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+        const int nb = (K - k < 16) ? K - k : 16;
+        for (int b = 0; b < nb; ++b) w[b >> 2] |= (uint32_t)src[b] << (8 * (b & 3));
+        t = u32x4{w[0], w[1], w[2], w[3]};
+      }
+      v[j] = t;
+    }
+  }
+  __device__ __forceinline__ void store(uint8_t* lds_tile, int tid) const {
+#pragma unroll
+    for (int j = 0; j < kChunks; ++j) {
+      const int i = tid + j * NTHREADS;
+      *reinterpret_cast<u32x4*>(lds_tile + i * 16) = v[j];
+    }
+  }
+};
+
+// 32 K-contiguous bytes of row `r` starting at logical chunk 2*g: one MFMA operand fragment.
+__device__ __forceinline__ v8i read_fragment(const uint8_t* lds_tile, int r, int g) {
+  const int s = swz(r);
+  const u32x4 lo = *reinterpret_cast<const u32x4*>(lds_tile + r * 128 + (((2 * g) ^ s) << 4));
+  const u32x4 hi = *reinterpret_cast<const u32x4*>(lds_tile + r * 128 + (((2 * g + 1) ^ s) << 4));
+  v8i f;
+  f[0] = (int)lo.x; f[1] = (int)lo.y; f[2] = (int)lo.z; f[3] = (int)lo.w;
+  f[4] = (int)hi.x; f[5] = (int)hi.y; f[6] = (int)hi.z; f[7] = (int)hi.w;
+  return f;
+}
+
+__device__ __forceinline__ v4f mfma_fp8_16x16x128(v8i a, v8i b, v4f c) {
+  // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled instruction
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+template <int BM, int BN, int WM, int WN>
+struct TileCfg {
+  static constexpr int kThreads = WM * WN * 64;
+  static constexpr int kWaveM = BM / WM, kWaveN = BN / WN;
+  static constexpr int TM = kWaveM / 16, TN = kWaveN / 16;
+  static constexpr int kStageBytes = (BM + BN) * 128;
+  static constexpr int kScaleBytes = 2 * BM * 4;
+  static constexpr int kLdsBytes = 2 * kStageBytes + kScaleBytes;
+  static_assert(BM <= kThreads, "one thread per activation row stages the row scales");
+  static_assert(kWaveN <= 128 && 128 % kWaveN == 0, "a wavefront's N extent must stay inside one 128-wide scale block");
+};
+
+// ---------------------------------------------------------------------------------------------
+// Main kernel
+// ---------------------------------------------------------------------------------------------
+template <int BM, int BN, int WM, int WN, int MODE, bool DIRECT>
+__global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
+  using Cfg = TileCfg<BM, BN, WM, WN>;
+  constexpr int NT = Cfg::kThreads;
+  constexpr int TM = Cfg::TM, TN = Cfg::TN;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  auto lds_w = [&](int stage) -> uint8_t* { return lds + stage * Cfg::kStageBytes; };
+  auto lds_x = [&](int stage) -> uint8_t* { return lds + stage * Cfg::kStageBytes + BN * 128; };
+  float* const lds_xs = reinterpret_cast<float*>(lds + 2 * Cfg::kStageBytes);  // [2][BM]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave % WM, wave_n = wave / WM;
+
+  int tile_m, tile_n;
+  tile_of_block(blockIdx.x, a.tiles_m, a.tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int wm0 = wave_m * Cfg::kWaveM, wn0 = wave_n * Cfg::kWaveN;
+  const int l16 = lane & 15, lg = lane >> 4;
+
+  v4f acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  const bool aligned16 = ((a.ldx | a.ldw) % 16 == 0) && (((uintptr_t)a.X | (uintptr_t)a.W) % 16 == 0);
+  StagedTile<BN, NT> st_w;
+  StagedTile<BM, NT> st_x;
+  (void)st_w; (void)st_x; (void)aligned16;
+
+  // activation-scale staging: thread t < BM owns row m0 + t
+  const int xs_row = (m0 + tid < a.M) ? m0 + tid : a.M - 1;
+  const float* xs_ptr = a.xs + (int64_t)xs_row * a.xs_rs;
+  // weight-scale row of this wavefront's N range (one 128-wide block)
+  const int nb_last = (a.N - 1) >> 7;
+  const int wn_blk = ((n0 + wn0) >> 7) < nb_last ? ((n0 + wn0) >> 7) : nb_last;
+  const float* ws_ptr = a.ws + (int64_t)wn_blk * a.ws_rs;
+
+  // ---- prologue: stage 0
+  if (a.KB == 0) {
+    // K == 0: nothing to stage, the accumulators stay zero
+  } else if (DIRECT) {
+    load_tile_direct<BN, NT>(a.W, a.ldw, n0, a.N - 1, 0, lds_w(0), wave, lane);
+    load_tile_direct<BM, NT>(a.X, a.ldx, m0, a.M - 1, 0, lds_x(0), wave, lane);
+  } else {
+    st_w.load(a.W, a.ldw, n0, a.N - 1, 0, a.K, aligned16, tid);
+    st_x.load(a.X, a.ldx, m0, a.M - 1, 0, a.K, aligned16, tid);
+    st_w.store(lds_w(0), tid);
+    st_x.store(lds_x(0), tid);
+  }
+  if (MODE == kModeBlock && a.KB > 0 && tid < BM) lds_xs[tid] = xs_ptr[0];
+
+  for (int kb = 0; kb < a.KB; ++kb) {
+    const int cur = kb & 1, nxt = cur ^ 1;
+    if (DIRECT) wait_vmem_all();
+    __syncthreads();
+
+    const bool more = kb + 1 < a.KB;
+    float xs_next = 0.f;
+    if (more) {
+      const int k1 = (kb + 1) * 128;
+      if (DIRECT) {
+        load_tile_direct<BN, NT>(a.W, a.ldw, n0, a.N - 1, k1, lds_w(nxt), wave, lane);
+        load_tile_direct<BM, NT>(a.X, a.ldx, m0, a.M - 1, k1, lds_x(nxt), wave, lane);
+      } else {
+        st_w.load(a.W, a.ldw, n0, a.N - 1, k1, a.K, aligned16, tid);
+        st_x.load(a.X, a.ldx, m0, a.M - 1, k1, a.K, aligned16, tid);
+      }
+      if (MODE == kModeBlock && tid < BM) xs_next = xs_ptr[(int64_t)(kb + 1) * a.xs_cs];
+    }
+
+    // ---- compute on stage `cur`
+    float sc[TM];
+    if (MODE == kModeBlock) {
+      const float wsv = ws_ptr[(int64_t)kb * a.ws_cs];
+#pragma unroll
+      for (int j = 0; j < TM; ++j) sc[j] = lds_xs[cur * BM + wm0 + j * 16 + l16] * wsv;
+    }
+    v8i xf[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) xf[j] = read_fragment(lds_x(cur), wm0 + j * 16 + l16, lg);
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+      const v8i wf = read_fragment(lds_w(cur), wn0 + i * 16 + l16, lg);
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        if (MODE == kModeBlock) {
+          const v4f p = mfma_fp8_16x16x128(wf, xf[j], v4f{0.f, 0.f, 0.f, 0.f});
+          acc[i][j][0] = __builtin_fmaf(p[0], sc[j], acc[i][j][0]);
+          acc[i][j][1] = __builtin_fmaf(p[1], sc[j], acc[i][j][1]);
+          acc[i][j][2] = __builtin_fmaf(p[2], sc[j], acc[i][j][2]);
+          acc[i][j][3] = __builtin_fmaf(p[3], sc[j], acc[i][j][3]);
+        } else {
+          acc[i][j] = mfma_fp8_16x16x128(wf, xf[j], acc[i][j]);
+        }
+      }
+    }
+
+    if (more) {
+      if (!DIRECT) {
+        st_w.store(lds_w(nxt), tid);
+        st_x.store(lds_x(nxt), tid);
+      }
+      if (MODE == kModeBlock && tid < BM) lds_xs[nxt * BM + tid] = xs_next;
+    }
+  }
+
+  // ---- epilogue
+#pragma unroll
+  for (int j = 0; j < TM; ++j) {
+    const int m = m0 + wm0 + j * 16 + l16;
+    if (m >= a.M) continue;
+    float sa = 1.f;
+    if (MODE == kModeRowCol) sa = a.xs[a.xs_per_row ? m : 0];
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+      const int n = n0 + wn0 + i * 16 + lg * 4;
+      if (n >= a.N) continue;
+      float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+      const int nv = (a.N - n < 4) ? a.N - n : 4;
+      if (MODE == kModeRowCol) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int ne = (e < nv) ? n + e : n;
+          const float sb = a.ws[a.ws_per_col ? ne : 0];
+          v[e] = (v[e] * sa) * sb;
+        }
+      }
+      const int64_t off = (int64_t)m * a.ldc + n;
+      if (a.c_dtype == FG_BF16) {
+        uint16_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          h[e] = float_to_bf16_bits(v[e]);
+          if (MODE == kModeRowCol && a.bias) {
+            const int ne = (e < nv) ? n + e : n;
+            h[e] = float_to_bf16_bits(bf16_bits_to_float(h[e]) + load_as_float(a.bias, ne, a.bias_dtype));
+          }
+        }
+        uint16_t* cp = reinterpret_cast<uint16_t*>(a.C) + off;
+        if (nv == 4 && ((uintptr_t)cp % 8 == 0)) {
+          u32x2 o = {(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+          *reinterpret_cast<u32x2*>(cp) = o;
+        } else {
+          for (int e = 0; e < nv; ++e) cp[e] = h[e];
+        }
+      } else if (a.c_dtype == FG_F16) {
+        _Float16* cp = reinterpret_cast<_Float16*>(a.C) + off;
+        for (int e = 0; e < nv; ++e) {
+          _Float16 h = (_Float16)v[e];
+          if (MODE == kModeRowCol && a.bias) h = (_Float16)((float)h + load_as_float(a.bias, n + e, a.bias_dtype));
+          cp[e] = h;
+        }
+      } else if (a.c_dtype == FG_F32) {
+        float* cp = reinterpret_cast<float*>(a.C) + off;
+        for (int e = 0; e < nv; ++e) {
+          float h = v[e];
+          if (MODE == kModeRowCol && a.bias) h = h + load_as_float(a.bias, n + e, a.bias_dtype);
+          cp[e] = h;
+        }
+      } else {  // FG_FP8_E4M3FN
+        uint8_t* cp = reinterpret_cast<uint8_t*>(a.C) + off;
+        for (int e = 0; e < nv; ++e) {
+          float h = v[e];
+          uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(h, 0.f, 0, false) & 0xFFu;
+          if (MODE == kModeRowCol && a.bias) {
+            // the reference adds the bias to the already rounded output, in the output type
+            const float back = __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
+            h = back + load_as_float(a.bias, n + e, a.bias_dtype);
+            code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(h, 0.f, 0, false) & 0xFFu;
+          }
+          cp[e] = (uint8_t)code;
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WM, int WN, int MODE, bool DIRECT>
+int launch_cfg(GemmArgs a, hipStream_t stream) {
+  using Cfg = TileCfg<BM, BN, WM, WN>;
+  a.tiles_m = (int)ceil_div(a.M, BM);
+  a.tiles_n = (int)ceil_div(a.N, BN);
+  auto kern = fp8_gemm_kernel<BM, BN, WM, WN, MODE, DIRECT>;
+  static bool attr_set = false;  // per instantiation; benign if raced
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
+    if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
+    attr_set = true;
+  }
+  const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
+  if (blocks > 0x7FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: too many tiles");
+  hipLaunchKernelGGL(kern, dim3((uint32_t)blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, a);
+  FG_CHECK_LAUNCH("fp8_gemm_kernel");
+  return FG_OK;
+}
+
+template <int MODE>
+int launch_gemm(const GemmArgs& a, hipStream_t stream) {
+  const bool direct = (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) &&
+                      ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
+  const bool big = a.M > 128;
+  if (big) {
+    return direct ? launch_cfg<256, 256, 4, 2, MODE, true>(a, stream)
+                  : launch_cfg<256, 256, 4, 2, MODE, false>(a, stream);
+  }
+  return direct ? launch_cfg<128, 128, 2, 2, MODE, true>(a, stream)
+                : launch_cfg<128, 128, 2, 2, MODE, false>(a, stream);
+}
+
+int check_common(const void* A, const void* B, const void* C, int64_t lda, int64_t ldb, int64_t ldc,
+                 int64_t M, int64_t N, int64_t K, const char* who) {
+  if (M < 0 || N < 0 || K < 0) FG_FAIL(FG_ERR_INVALID_ARG, "%s: negative size", who);
+  if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFF00) FG_FAIL(FG_ERR_UNSUPPORTED, "%s: size exceeds 2^31", who);
+  if (M == 0 || N == 0) return 1;
+  if (!C) FG_FAIL(FG_ERR_INVALID_ARG, "%s: null output", who);
+  if (K > 0 && (!A || !B)) FG_FAIL(FG_ERR_INVALID_ARG, "%s: null operand", who);
+  if (lda < K || ldb < K || ldc < N) FG_FAIL(FG_ERR_INVALID_ARG, "%s: leading dimension smaller than row length", who);
+  return 0;
+}
+
+}  // namespace
+}  // namespace fg
+
+extern "C" size_t fg_block_fp8_gemm_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
+extern "C" size_t fg_scaled_fp8_gemm_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
+
+extern "C" int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
+                                 const float* As, int64_t as_row_stride, int64_t as_col_stride,
+                                 const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride,
+                                 void* C, int64_t ldc, int c_dtype,
+                                 int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace fg;
+  (void)workspace; (void)workspace_bytes;
+  if (block_n != 128 || block_k != 128)
+    FG_FAIL(FG_ERR_UNSUPPORTED, "fg_block_fp8_gemm: only 128x128 scale blocks are implemented (got %lld x %lld)",
+            (long long)block_n, (long long)block_k);
+  if (c_dtype != FG_BF16 && c_dtype != FG_F16 && c_dtype != FG_F32)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_block_fp8_gemm: c_dtype %d", c_dtype);
+  int rc = check_common(A, B, C, lda, ldb, ldc, M, N, K, "fg_block_fp8_gemm");
+  if (rc < 0) return rc;
+  if (rc == 1) return FG_OK;
+  if (K > 0 && (!As || !Bs)) FG_FAIL(FG_ERR_INVALID_ARG, "fg_block_fp8_gemm: null scale pointer");
+  GemmArgs a = {};
+  a.X = (const uint8_t*)A; a.W = (const uint8_t*)B; a.C = C;
+  a.xs = As; a.ws = Bs; a.bias = nullptr;
+  a.ldx = lda; a.ldw = ldb; a.ldc = ldc;
+  a.xs_rs = as_row_stride; a.xs_cs = as_col_stride; a.ws_rs = bs_row_stride; a.ws_cs = bs_col_stride;
+  a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)ceil_div(K, 128);
+  a.c_dtype = c_dtype;
+  return launch_gemm<kModeBlock>(a, (hipStream_t)stream);
+}
+
+extern "C" int fg_scaled_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
+                                  const float* a_scale, int a_scale_per_row,
+                                  const float* b_scale, int b_scale_per_col,
+                                  const void* bias, int bias_dtype,
+                                  void* C, int64_t ldc, int c_dtype,
+                                  int64_t M, int64_t N, int64_t K,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace fg;
+  (void)workspace; (void)workspace_bytes;
+  if (c_dtype != FG_BF16 && c_dtype != FG_F16 && c_dtype != FG_F32 && c_dtype != FG_FP8_E4M3FN)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_scaled_fp8_gemm: c_dtype %d", c_dtype);
+  if (bias && bias_dtype != FG_BF16 && bias_dtype != FG_F16 && bias_dtype != FG_F32)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_scaled_fp8_gemm: bias_dtype %d", bias_dtype);
+  int rc = check_common(A, B, C, lda, ldb, ldc, M, N, K, "fg_scaled_fp8_gemm");
+  if (rc < 0) return rc;
+  if (rc == 1) return FG_OK;
+  if (!a_scale || !b_scale) FG_FAIL(FG_ERR_INVALID_ARG, "fg_scaled_fp8_gemm: null scale pointer");
+  GemmArgs a = {};
+  a.X = (const uint8_t*)A; a.W = (const uint8_t*)B; a.C = C;
+  a.xs = a_scale; a.ws = b_scale; a.bias = bias;
+  a.ldx = lda; a.ldw = ldb; a.ldc = ldc;
+  a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)ceil_div(K, 128);
+  a.c_dtype = c_dtype; a.bias_dtype = bias_dtype;
+  a.xs_per_row = a_scale_per_row; a.ws_per_col = b_scale_per_col;
+  return launch_gemm<kModeRowCol>(a, (hipStream_t)stream);
+}

@@ -1,0 +1,338 @@
+// Per-token-group FP8 quantizer for gfx950.
+//
+// One group of G consecutive elements is owned by G/8 adjacent lanes of a wavefront; every lane
+// loads 8 elements with one (bf16/f16) or two (f32) 16-byte loads, the group's absolute maximum is
+// reduced across those lanes with DPP / cross-lane moves, the scale is derived redundantly in every
+// lane, and each lane writes its 8 codes with one 8-byte store.  The kernel is pure streaming:
+// 2 (or 4) bytes read and 1 byte written per element plus 4 bytes of scale per group.
+//
+// Arithmetic is IEEE fp32 throughout (correctly rounded multiply, reciprocal and division) so the
+// codes and scales are bit-identical to the torch reference implementations:
+//   tests/test_act_quant.py:48-98 and tests/test_per_token_group_quant_fp8.py:23-48 of the reference.
+
+#include "fg_common.h"
+
+namespace fg {
+namespace {
+
+struct QuantArgs {
+  const void* x;
+  uint8_t* q;
+  float* s;
+  int64_t x_row_stride, q_row_stride, s_row_stride, s_col_stride;
+  uint32_t groups_per_row;
+  uint32_t total_groups;
+  uint32_t group_size;
+  float floor, lo, hi, inv_max;
+  int scale_rule, quotient_rule, pow2_rule, e5m2;
+};
+
+template <int XDT> struct Elem;
+template <> struct Elem<FG_BF16> {
+  using raw = uint16_t;
+  static constexpr uint32_t kAbs = 0x7FFFu, kInf = 0x7F80u;
+  __device__ static float widen(uint32_t b) { return bits_to_float(b << 16); }
+};
+template <> struct Elem<FG_F16> {
+  using raw = uint16_t;
+  static constexpr uint32_t kAbs = 0x7FFFu, kInf = 0x7C00u;
+  __device__ static float widen(uint32_t b) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+  }
+};
+template <> struct Elem<FG_F32> {
+  using raw = uint32_t;
+  static constexpr uint32_t kAbs = 0x7FFFFFFFu, kInf = 0x7F800000u;
+  __device__ static float widen(uint32_t b) { return bits_to_float(b); }
+};
+
+// scale from the group's absolute maximum (already floored), following the requested rules
+__device__ __forceinline__ float derive_scale(float amax, const QuantArgs& a) {
+  float s = (a.scale_rule == FG_SCALE_MUL_INV) ? amax * a.inv_max : amax / a.hi;
+  if (a.pow2_rule == FG_POW2_BITS) {
+    // exponent + (mantissa != 0) re-assembled with 32-bit wrap-around
+    // (reference src/flag_gems/fused/act_quant.py:22-41)
+    uint32_t b = float_to_bits(s);
+    uint32_t e = (b >> 23) & 0xFFu;
+    uint32_t m = b & 0x7FFFFFu;
+    uint32_t l = e - 127u + (m != 0u ? 1u : 0u);
+    s = bits_to_float((l + 127u) << 23);
+  } else if (a.pow2_rule == FG_POW2_LOG2) {
+    // exp2(ceil(log2(max(|s|, 1e-10)))) with log2 rounded to fp32 the way a correctly rounded
+    // libm does it (reference src/flag_gems/ops/per_token_group_quant_fp8.py:65-66)
+    float t = fmaxf(fabsf(s), 1e-10f);
+    if (s != s) {
+      // NaN stays NaN
+    } else if (t < __builtin_huge_valf()) {
+      float l = (float)log2((double)t);
+      int k = (int)ceilf(l);
+      s = (k >= -126) ? bits_to_float((uint32_t)(k + 127) << 23) : ldexpf(1.0f, k);
+    } else {
+      s = t;
+    }
+  }
+  return s;
+}
+
+__device__ __forceinline__ float quantize_value(float x, float s, float r, const QuantArgs& a) {
+  float y = (a.quotient_rule == FG_QUOT_RECIP_MUL) ? x * r : x / s;
+  // clamp that lets NaN through, as torch.clamp does
+  float c = fminf(fmaxf(y, a.lo), a.hi);
+  return (y != y) ? y : c;
+}
+
+template <bool HI>
+__device__ __forceinline__ uint32_t pack2(float v0, float v1, uint32_t old, int e5m2) {
+  if (e5m2) return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(v0, v1, (int)old, HI);
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, (int)old, HI);
+}
+
+// NaN keeps its sign and takes the all-ones magnitude, whatever the converter does with it
+__device__ __forceinline__ uint32_t fix_nan_byte(uint32_t word, int byte, float v, int e5m2) {
+  if (v != v) {
+    uint32_t code = ((float_to_bits(v) >> 24) & 0x80u) | (e5m2 ? 0x7Fu : 0x7Fu);
+    word = (word & ~(0xFFu << (8 * byte))) | (code << (8 * byte));
+  }
+  return word;
+}
+
+template <int LPG>
+__device__ __forceinline__ uint32_t group_max_u32(uint32_t v) {
+  // max over LPG adjacent lanes; every lane ends with the group's value
+  if (LPG >= 2) v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+  if (LPG >= 4) v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+  if (LPG >= 8) v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x141, 0xF, 0xF, true));  // row_half_mirror
+  if (LPG >= 16) v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x140, 0xF, 0xF, true)); // row_mirror
+  if (LPG >= 32) v = max(v, (uint32_t)__shfl_xor((int)v, 16, 64));
+  if (LPG >= 64) v = max(v, (uint32_t)__shfl_xor((int)v, 32, 64));
+  return v;
+}
+
+constexpr int kQuantThreads = 256;
+constexpr int kQuantUnroll = 4;
+
+// Vector kernel: group_size == 8 * LPG, rows 16-byte aligned.
+template <int XDT, int LPG>
+__global__ __launch_bounds__(kQuantThreads) void group_quant_vec_kernel(QuantArgs a) {
+  using E = Elem<XDT>;
+  constexpr int kWords = sizeof(typename E::raw) * 8 / 4;  // 32-bit words per lane: 4 or 8
+  const uint32_t total_chunks = a.total_groups * (uint32_t)LPG;  // host guarantees no overflow
+  const uint32_t stride = gridDim.x * kQuantThreads;
+  const uint32_t first = blockIdx.x * kQuantThreads + threadIdx.x;
+
+  uint32_t w[kQuantUnroll][kWords];
+  uint32_t gid[kQuantUnroll], row[kQuantUnroll], gcol[kQuantUnroll];
+  bool live[kQuantUnroll];
+
+#pragma unroll
+  for (int u = 0; u < kQuantUnroll; ++u) {
+    uint32_t c = first + (uint32_t)u * stride;
+    live[u] = c < total_chunks && c >= first;  // second test: wrap-around guard
+    uint32_t cc = live[u] ? c : 0u;
+    gid[u] = cc / LPG;
+    uint32_t lig = cc % LPG;
+    row[u] = gid[u] / a.groups_per_row;
+    gcol[u] = gid[u] - row[u] * a.groups_per_row;
+    const typename E::raw* p = reinterpret_cast<const typename E::raw*>(a.x) +
+                               (int64_t)row[u] * a.x_row_stride + (int64_t)gcol[u] * (LPG * 8) + lig * 8;
+    const u32x4* p4 = reinterpret_cast<const u32x4*>(p);
+    if (live[u]) {
+      u32x4 v = p4[0];
+      w[u][0] = v.x; w[u][1] = v.y; w[u][2] = v.z; w[u][3] = v.w;
+      if constexpr (kWords == 8) {
+        u32x4 v2 = p4[1];
+        w[u][4] = v2.x; w[u][5] = v2.y; w[u][6] = v2.z; w[u][7] = v2.w;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kWords; ++i) w[u][i] = 0u;
+    }
+  }
+
+#pragma unroll
+  for (int u = 0; u < kQuantUnroll; ++u) {
+    // absolute maximum on the raw bit patterns: NaN patterns compare above everything
+    uint32_t m = 0u;
+    float xv[8];
+    if constexpr (kWords == 4) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint32_t lo = w[u][i] & 0xFFFFu, hi = w[u][i] >> 16;
+        m = max(m, max(lo & E::kAbs, hi & E::kAbs));
+        xv[2 * i] = E::widen(lo);
+        xv[2 * i + 1] = E::widen(hi);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        m = max(m, w[u][i] & E::kAbs);
+        xv[i] = E::widen(w[u][i]);
+      }
+    }
+    m = group_max_u32<LPG>(m);
+    float amax = E::widen(m);
+    const bool special = m >= E::kInf;  // Inf or NaN somewhere in the group
+    if (!(amax != amax)) amax = fmaxf(amax, a.floor);
+    const float s = derive_scale(amax, a);
+    const float r = 1.0f / s;
+
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = quantize_value(xv[i], s, r, a);
+    uint32_t w0 = pack2<false>(y[0], y[1], 0u, a.e5m2);
+    w0 = pack2<true>(y[2], y[3], w0, a.e5m2);
+    uint32_t w1 = pack2<false>(y[4], y[5], 0u, a.e5m2);
+    w1 = pack2<true>(y[6], y[7], w1, a.e5m2);
+    if (special || !(s == s)) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        w0 = fix_nan_byte(w0, i, y[i], a.e5m2);
+        w1 = fix_nan_byte(w1, i, y[4 + i], a.e5m2);
+      }
+    }
+    if (live[u]) {
+      uint32_t c = first + (uint32_t)u * stride;
+      uint32_t lig = c % LPG;
+      uint8_t* qp = a.q + (int64_t)row[u] * a.q_row_stride + (int64_t)gcol[u] * (LPG * 8) + lig * 8;
+      u32x2 out = {w0, w1};
+      *reinterpret_cast<u32x2*>(qp) = out;
+      if (lig == 0) a.s[(int64_t)row[u] * a.s_row_stride + (int64_t)gcol[u] * a.s_col_stride] = s;
+    }
+  }
+}
+
+// Generic kernel: any group size and alignment; one wavefront per group, two passes.
+template <int XDT>
+__global__ __launch_bounds__(kQuantThreads) void group_quant_generic_kernel(QuantArgs a) {
+  using E = Elem<XDT>;
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t gid = blockIdx.x * (kQuantThreads / 64) + (threadIdx.x >> 6);
+  if (gid >= a.total_groups) return;  // whole wavefront leaves together
+  const uint32_t row = gid / a.groups_per_row;
+  const uint32_t gcol = gid - row * a.groups_per_row;
+  const typename E::raw* xp = reinterpret_cast<const typename E::raw*>(a.x) +
+                              (int64_t)row * a.x_row_stride + (int64_t)gcol * a.group_size;
+  uint8_t* qp = a.q + (int64_t)row * a.q_row_stride + (int64_t)gcol * a.group_size;
+
+  uint32_t m = 0u;
+  for (uint32_t i = lane; i < a.group_size; i += 64) m = max(m, (uint32_t)xp[i] & E::kAbs);
+  m = group_max_u32<64>(m);
+  float amax = E::widen(m);
+  if (!(amax != amax)) amax = fmaxf(amax, a.floor);
+  const float s = derive_scale(amax, a);
+  const float r = 1.0f / s;
+  for (uint32_t i = lane; i < a.group_size; i += 64) {
+    float y = quantize_value(E::widen((uint32_t)xp[i]), s, r, a);
+    uint32_t wd = pack2<false>(y, 0.0f, 0u, a.e5m2);
+    wd = fix_nan_byte(wd, 0, y, a.e5m2);
+    qp[i] = (uint8_t)(wd & 0xFFu);
+  }
+  if (lane == 0) a.s[(int64_t)row * a.s_row_stride + (int64_t)gcol * a.s_col_stride] = s;
+}
+
+template <int XDT>
+int launch_quant(const QuantArgs& a, bool vec_ok, hipStream_t stream) {
+  const uint32_t g = a.group_size;
+  int lpg = 0;
+  if (vec_ok && g % 8 == 0) {
+    uint32_t l = g / 8;
+    if (l == 1 || l == 2 || l == 4 || l == 8 || l == 16 || l == 32 || l == 64) lpg = (int)l;
+  }
+  if (lpg == 0) {
+    dim3 grid((uint32_t)ceil_div(a.total_groups, kQuantThreads / 64));
+    hipLaunchKernelGGL(group_quant_generic_kernel<XDT>, grid, dim3(kQuantThreads), 0, stream, a);
+    FG_CHECK_LAUNCH("group_quant_generic_kernel");
+    return FG_OK;
+  }
+  const uint64_t chunks = (uint64_t)a.total_groups * (uint64_t)lpg;
+  dim3 grid((uint32_t)ceil_div((int64_t)chunks, (int64_t)kQuantThreads * kQuantUnroll));
+  switch (lpg) {
+#define FG_CASE(L)                                                                                  \
+  case L:                                                                                           \
+    hipLaunchKernelGGL((group_quant_vec_kernel<XDT, L>), grid, dim3(kQuantThreads), 0, stream, a); \
+    break;
+    FG_CASE(1) FG_CASE(2) FG_CASE(4) FG_CASE(8) FG_CASE(16) FG_CASE(32) FG_CASE(64)
+#undef FG_CASE
+  }
+  FG_CHECK_LAUNCH("group_quant_vec_kernel");
+  return FG_OK;
+}
+
+}  // namespace
+}  // namespace fg
+
+extern "C" int fg_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride,
+                                  void* q, int q_dtype, int64_t q_row_stride,
+                                  float* s, int64_t s_row_stride, int64_t s_col_stride,
+                                  int64_t group_size, float amax_floor, float fp8_min, float fp8_max,
+                                  float inv_fp8_max, int scale_rule, int quotient_rule, int pow2_rule,
+                                  void* stream) {
+  using namespace fg;
+  if (rows < 0 || cols < 0) FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: negative size");
+  if (rows == 0 || cols == 0) return FG_OK;
+  if (!x || !q || !s) FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: null pointer");
+  if (group_size <= 0 || cols % group_size != 0)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: cols %lld not divisible by group_size %lld",
+            (long long)cols, (long long)group_size);
+  if (x_dtype != FG_BF16 && x_dtype != FG_F16 && x_dtype != FG_F32)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: x_dtype %d", x_dtype);
+  if (q_dtype != FG_FP8_E4M3FN && q_dtype != FG_FP8_E5M2)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: q_dtype %d", q_dtype);
+  if (scale_rule < 0 || scale_rule > 1 || quotient_rule < 0 || quotient_rule > 1 || pow2_rule < 0 || pow2_rule > 2)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: bad rule selector");
+  if (x_row_stride < cols || q_row_stride < cols)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: row stride smaller than cols");
+  if (group_size > (int64_t)1 << 24) FG_FAIL(FG_ERR_UNSUPPORTED, "fg_group_quant_fp8: group_size too large");
+
+  const int64_t groups_per_row = cols / group_size;
+  if (groups_per_row > 0x7FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fg_group_quant_fp8: too many groups per row");
+  const size_t esz = (x_dtype == FG_F32) ? 4 : 2;
+  const bool vec_ok = ((uintptr_t)x % 16 == 0) && ((x_row_stride * esz) % 16 == 0) &&
+                      ((uintptr_t)q % 8 == 0) && (q_row_stride % 8 == 0);
+
+  // Launch in row slabs so that 32-bit chunk indices cannot overflow.
+  const int64_t max_groups = (int64_t)1 << 24;
+  int64_t rows_per_launch = max_groups / groups_per_row;
+  if (rows_per_launch < 1) rows_per_launch = 1;
+  for (int64_t r0 = 0; r0 < rows; r0 += rows_per_launch) {
+    const int64_t nr = (rows - r0 < rows_per_launch) ? rows - r0 : rows_per_launch;
+    QuantArgs a;
+    a.x = (const char*)x + r0 * x_row_stride * (int64_t)esz;
+    a.q = (uint8_t*)q + r0 * q_row_stride;
+    a.s = s + r0 * s_row_stride;
+    a.x_row_stride = x_row_stride;
+    a.q_row_stride = q_row_stride;
+    a.s_row_stride = s_row_stride;
+    a.s_col_stride = s_col_stride;
+    a.groups_per_row = (uint32_t)groups_per_row;
+    a.total_groups = (uint32_t)(nr * groups_per_row);
+    a.group_size = (uint32_t)group_size;
+    a.floor = amax_floor;
+    a.lo = fp8_min;
+    a.hi = fp8_max;
+    a.inv_max = inv_fp8_max;
+    a.scale_rule = scale_rule;
+    a.quotient_rule = quotient_rule;
+    a.pow2_rule = pow2_rule;
+    a.e5m2 = (q_dtype == FG_FP8_E5M2);
+    int rc;
+    if (x_dtype == FG_BF16) rc = launch_quant<FG_BF16>(a, vec_ok, (hipStream_t)stream);
+    else if (x_dtype == FG_F16) rc = launch_quant<FG_F16>(a, vec_ok, (hipStream_t)stream);
+    else rc = launch_quant<FG_F32>(a, vec_ok, (hipStream_t)stream);
+    if (rc != FG_OK) return rc;
+  }
+  return FG_OK;
+}
+
+extern "C" int fg_act_quant_bf16(const void* x, void* y, float* s, int64_t rows, int64_t cols,
+                                 int64_t block_size, int round_scale, void* stream) {
+  if (block_size <= 0 || cols % (block_size > 0 ? block_size : 1) != 0) {
+    snprintf(fg::error_buffer(), fg::kErrorBufferBytes,
+             "fg_act_quant_bf16: last dimension %lld must be divisible by block_size %lld",
+             (long long)cols, (long long)block_size);
+    return FG_ERR_INVALID_ARG;
+  }
+  return fg_group_quant_fp8(x, FG_BF16, rows, cols, cols, y, FG_FP8_E4M3FN, cols, s, cols / block_size, 1,
+                            block_size, 1e-4f, -448.0f, 448.0f, 1.0f / 448.0f, FG_SCALE_MUL_INV,
+                            FG_QUOT_RECIP_MUL, round_scale ? FG_POW2_BITS : FG_POW2_NONE, stream);
+}

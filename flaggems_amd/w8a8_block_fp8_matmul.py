@@ -1,0 +1,124 @@
+"""Block-scaled FP8 GEMM (host side).
+
+Mirrors the reference entry points
+  w8a8_block_fp8_matmul  src/flag_gems/ops/w8a8_block_fp8_matmul.py:173-232
+  fp8_matmul             src/flag_gems/ops/fp8_matmul.py:137-205
+with the same parameters, defaults and assertions.  The reference picks a Triton tile from a
+per-device YAML table; here the C library picks the HIP kernel variant from (M, N, K).
+"""
+from __future__ import annotations
+
+import logging
+import math
+from typing import List
+
+import torch
+
+from . import _lib
+
+logger = logging.getLogger("flag_gems." + __name__.split(".")[-1])
+
+GROUP_SIZE = 128  # scale granularity of fp8_matmul (reference src/flag_gems/ops/fp8_matmul.py:42)
+_OUT_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
+
+
+def _cdiv(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+def _launch_block_gemm(a2d, b, as2d, bs, c2d, block_n: int, block_k: int) -> None:
+    _lib.require_gpu(a2d, "block fp8 gemm")
+    lib = _lib.load()
+    m, k = a2d.shape
+    n = b.shape[0]
+    dev = a2d.device
+    with torch.cuda.device(dev):
+        ws_bytes = lib.fg_block_fp8_gemm_workspace_bytes(m, n, k)
+        ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
+        status = lib.fg_block_fp8_gemm(
+            a2d.data_ptr(), a2d.stride(0) if m > 1 else max(k, a2d.stride(0)),
+            b.data_ptr(), b.stride(0) if n > 1 else max(k, b.stride(0)),
+            as2d.data_ptr(), as2d.stride(0), as2d.stride(1),
+            bs.data_ptr(), bs.stride(0), bs.stride(1),
+            c2d.data_ptr(), c2d.stride(0) if m > 1 else max(n, c2d.stride(0)), _lib.DTYPE_CODE[c2d.dtype],
+            m, n, k, block_n, block_k,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+            _lib.current_stream_ptr(dev),
+        )
+    _lib.check(status, "fg_block_fp8_gemm")
+
+
+def w8a8_block_fp8_matmul(
+    A: torch.Tensor,
+    B: torch.Tensor,
+    As: torch.Tensor,
+    Bs: torch.Tensor,
+    block_size: List[int],
+    output_dtype: torch.dtype = torch.bfloat16,
+) -> torch.Tensor:
+    """C = (A dequantised by As per 1 x block_k group) @ (B dequantised by Bs per block_n x block_k block)^T.
+
+    A [..., K] contiguous e4m3fn, As [..., ceil(K/block_k)] fp32, B [N, K] e4m3fn,
+    Bs [ceil(N/block_n), ceil(K/block_k)] fp32; returns [..., N] in ``output_dtype``.
+    """
+    logger.debug("GEMS W8A8_BLOCK_FP8_MATMUL")
+    assert len(block_size) == 2
+    block_n, block_k = block_size[0], block_size[1]
+
+    assert A.shape[-1] == B.shape[-1]
+    assert A.shape[:-1] == As.shape[:-1] and A.is_contiguous()
+    assert _cdiv(A.shape[-1], block_k) == As.shape[-1]
+    M = math.prod(A.shape[:-1])
+
+    assert B.ndim == 2 and Bs.ndim == 2
+    N, K = B.shape
+    assert _cdiv(N, block_n) == Bs.shape[0]
+    assert _cdiv(K, block_k) == Bs.shape[1]
+    if A.dtype != torch.float8_e4m3fn or B.dtype != torch.float8_e4m3fn:
+        raise NotImplementedError(f"w8a8_block_fp8_matmul: operands must be float8_e4m3fn, got {A.dtype}, {B.dtype}")
+    if output_dtype not in _OUT_DTYPES:
+        raise NotImplementedError(f"w8a8_block_fp8_matmul: unsupported output dtype {output_dtype}")
+    if As.dtype != torch.float32 or Bs.dtype != torch.float32:
+        As, Bs = As.to(torch.float32), Bs.to(torch.float32)
+
+    C_shape = A.shape[:-1] + (N,)
+    C = A.new_empty(C_shape, dtype=output_dtype)
+    if M == 0 or N == 0:
+        return C
+    if B.stride(1) != 1:
+        B = B.contiguous()
+    a2d = A.view(M, K)
+    as2d = As if As.dim() == 2 else As.reshape(M, As.shape[-1])
+    _launch_block_gemm(a2d, B, as2d, Bs, C.view(M, N), block_n, block_k)
+    return C
+
+
+def fp8_matmul(
+    a: torch.Tensor,
+    a_s: torch.Tensor,
+    b: torch.Tensor,
+    b_s: torch.Tensor,
+    scale_dtype: torch.dtype = torch.float32,
+) -> torch.Tensor:
+    """Block-wise scaled FP8 matmul with 128-wide groups and bf16 output.
+
+    a [..., K] e4m3fn contiguous, a_s [..., K/128], b [N, K] e4m3fn contiguous, b_s [N/128, K/128];
+    scales given as float8_e8m0fnu are widened to fp32 first.
+    """
+    logger.debug("GEMS FP8_MATMUL")
+    assert b.ndim == 2
+    assert a.is_contiguous() and b.is_contiguous()
+    assert a_s.is_contiguous() and b_s.is_contiguous()
+    K = a.size(-1)
+    M = a.numel() // K
+    N, K2 = b.shape
+    assert K == K2
+    if scale_dtype == torch.float8_e8m0fnu:
+        a_s = a_s.to(torch.float32)
+        b_s = b_s.to(torch.float32)
+    out_shape = (*a.size()[:-1], N)
+    C = torch.empty((M, N), device=a.device, dtype=torch.bfloat16)
+    if M == 0 or N == 0:
+        return C.view(out_shape)
+    _launch_block_gemm(a.view(M, K), b, a_s.view(M, -1), b_s, C, GROUP_SIZE, GROUP_SIZE)
+    return C.view(out_shape)

@@ -1,0 +1,155 @@
+/*
+ * flaggems_amd -- C ABI of the MI355X (gfx950) FP8 quantized-linear kernels.
+ *
+ * Every entry point takes raw device pointers, element counts, element strides and a
+ * HIP stream.  None of them allocates, frees, synchronises or throws: the work is
+ * enqueued on `stream` and the call returns 0 (FG_OK) or a negative fg_status; the
+ * text of the last error on the calling thread is available from
+ * fg_last_error_string().  The caller owns every buffer, selects the device
+ * (hipSetDevice / torch device guard) and validates tensor-level preconditions.
+ *
+ * The reference library (FlagGems) has no C ABI: its native layer is C++ functions
+ * taking at::Tensor, exposed through pybind11.  Each declaration below names the
+ * reference interface it stands in for (paths relative to the reference checkout).
+ */
+#ifndef FLAGGEMS_AMD_H_
+#define FLAGGEMS_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum fg_status {
+  FG_OK = 0,
+  FG_ERR_INVALID_ARG = -1, /* null pointer, negative size, bad enum, bad alignment */
+  FG_ERR_UNSUPPORTED = -2, /* valid request the kernels do not implement */
+  FG_ERR_WORKSPACE = -3,   /* workspace missing or smaller than fg_*_workspace_bytes */
+  FG_ERR_LAUNCH = -4       /* hipLaunchKernel reported an error */
+} fg_status;
+
+typedef enum fg_dtype {
+  FG_BF16 = 0,
+  FG_F16 = 1,
+  FG_F32 = 2,
+  FG_FP8_E4M3FN = 3, /* OCP e4m3fn: max 448, no inf */
+  FG_FP8_E5M2 = 4    /* OCP e5m2 */
+} fg_dtype;
+
+/* How the per-group scale is derived from the group's absolute maximum. */
+typedef enum fg_scale_rule {
+  FG_SCALE_MUL_INV = 0, /* scale = amax * inv_fp8_max   (torch references: amax * fp32(1/448)) */
+  FG_SCALE_DIV = 1      /* scale = amax / fp8_max       (reference device kernels, MoE fallback) */
+} fg_scale_rule;
+
+/* How an element is divided by its scale. */
+typedef enum fg_quotient_rule {
+  FG_QUOT_RECIP_MUL = 0, /* x * (1.0f / scale), both IEEE-rounded (torch_act_quant) */
+  FG_QUOT_DIV = 1        /* x / scale, IEEE-rounded division   (per_token_group_quant_fp8) */
+} fg_quotient_rule;
+
+/* Optional rounding of the scale up to a power of two (UE8M0-representable). */
+typedef enum fg_pow2_rule {
+  FG_POW2_NONE = 0,
+  FG_POW2_BITS = 1, /* exponent + (mantissa != 0), 32-bit wrap-around as in fast_round_scale */
+  FG_POW2_LOG2 = 2  /* exp2(ceil(log2(max(|s|, 1e-10)))) */
+} fg_pow2_rule;
+
+/* Library version (major*10000 + minor*100 + patch) and last error text (thread-local). */
+int fg_version(void);
+const char* fg_last_error_string(void);
+
+/*
+ * Per-token-group FP8 quantization: for every row r and every group g of `group_size`
+ * consecutive columns,
+ *     amax  = max |x[r, g*G : (g+1)*G]|          (NaN propagates)
+ *     amax  = max(amax, amax_floor)
+ *     scale = scale_rule(amax)  then  pow2_rule(scale)
+ *     q     = cast_fp8(clamp(quotient_rule(x, scale), fp8_min, fp8_max))   round-to-nearest-even
+ * writes q[r*q_row_stride + c] (1 byte each) and s[r*s_row_stride + g*s_col_stride].
+ *
+ * x_dtype in {FG_BF16, FG_F16, FG_F32}; q_dtype in {FG_FP8_E4M3FN, FG_FP8_E5M2};
+ * cols % group_size == 0; strides are in elements.  rows*cols == 0 is a no-op.
+ *
+ * Stands in for: per_token_group_quant_fp8 (src/flag_gems/ops/per_token_group_quant_fp8.py:227-336,
+ * kernels :34-216), act_quant_triton (src/flag_gems/fused/act_quant.py:111-174, kernel :45-108),
+ * the native wrapper flag_gems::act_quant_triton (cpp/lib/act_quant.cpp:26-129) and the vLLM op
+ * _C::per_token_group_fp8_quant (src/flag_gems/patches/patch_vllm_all.py:425-448), which can pass
+ * the caller's output buffers straight through.
+ */
+int fg_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride,
+                       void* q, int q_dtype, int64_t q_row_stride,
+                       float* s, int64_t s_row_stride, int64_t s_col_stride,
+                       int64_t group_size, float amax_floor, float fp8_min, float fp8_max,
+                       float inv_fp8_max, int scale_rule, int quotient_rule, int pow2_rule,
+                       void* stream);
+
+/*
+ * act_quant with the reference's fixed rules (bf16 in, e4m3fn out, floor 1e-4,
+ * scale = amax * fp32(1/448), reciprocal-multiply quotient, power-of-two scale when
+ * round_scale != 0), contiguous [rows, cols] input and outputs.
+ * Stands in for flag_gems::act_quant_triton (cpp/lib/act_quant.cpp:26-129,
+ * cpp/include/flag_gems/operators.h:59-61).
+ */
+int fg_act_quant_bf16(const void* x, void* y, float* s, int64_t rows, int64_t cols,
+                      int64_t block_size, int round_scale, void* stream);
+
+/*
+ * Block-scaled FP8 GEMM:
+ *     C[m, n] = sum_kb ( sum_{k in kb} A[m,k] * B[n,k] ) * As[m, kb] * Bs[n / block_n, kb]
+ * A: e4m3fn [M, K], row stride lda, unit column stride.  B: e4m3fn [N, K], row stride ldb, unit
+ * column stride.  As: fp32 [M, ceil(K/block_k)] with both strides given.  Bs: fp32
+ * [ceil(N/block_n), ceil(K/block_k)] with both strides given.  C: [M, N] row stride ldc,
+ * c_dtype in {FG_BF16, FG_F16, FG_F32}.  Products are accumulated in fp32 per K-block, scaled,
+ * and accumulated in fp32 across K-blocks; the result is rounded once to c_dtype.
+ * Only block_n == block_k == 128 is implemented (FG_ERR_UNSUPPORTED otherwise).
+ * `workspace` must hold at least fg_block_fp8_gemm_workspace_bytes(M, N, K) bytes (may be null
+ * when that is 0); it carries split-K partial sums and needs no initialisation by the caller
+ * beyond a one-time zero fill of its first FG_WORKSPACE_COUNTER_BYTES bytes.
+ *
+ * Stands in for: w8a8_block_fp8_matmul (src/flag_gems/ops/w8a8_block_fp8_matmul.py:173-232,
+ * kernel :51-122), fp8_matmul (src/flag_gems/ops/fp8_matmul.py:137-205, kernel :58-134), the native
+ * wrappers fp8_matmul / fp8_matmul_direct (cpp/lib/fp8_matmul.cpp:25-102,
+ * cpp/lib/fp8_matmul_direct.cpp:25-180) and the block-wise branch of cutlass_scaled_mm
+ * (src/flag_gems/fused/cutlass_scaled_mm.py:87-194).
+ */
+int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
+                      const float* As, int64_t as_row_stride, int64_t as_col_stride,
+                      const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride,
+                      void* C, int64_t ldc, int c_dtype,
+                      int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+#define FG_WORKSPACE_COUNTER_BYTES 16384
+size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Per-tensor / per-token x per-channel scaled FP8 GEMM with optional bias:
+ *     C[m, n] = cast( (sum_k A[m,k] * B[n,k]) * a_scale[m or 0] * b_scale[n or 0] ) (+ bias[n])
+ * The bias is added after the cast, in c_dtype, as the reference does.  A: e4m3fn [M, K] row stride
+ * lda; B: e4m3fn given as N rows of K contiguous bytes with row stride ldb (that is the reference's
+ * column-major [K, N] operand: ldb = b.stride(1)).  a_scale has M entries when a_scale_per_row != 0,
+ * else 1; b_scale has N entries when b_scale_per_col != 0, else 1.  bias may be null; bias_dtype in
+ * {FG_BF16, FG_F16, FG_F32}.  c_dtype in {FG_BF16, FG_F16, FG_F32, FG_FP8_E4M3FN}.
+ *
+ * Stands in for: cutlass_scaled_mm per-tensor/per-token path
+ * (src/flag_gems/fused/cutlass_scaled_mm.py:198-344, 475-526), reached from aten::_scaled_mm
+ * (src/flag_gems/ops/scaled_mm.py:333-452) and the vLLM op _C::cutlass_scaled_mm
+ * (src/flag_gems/patches/patch_vllm_all.py:451-459).
+ */
+int fg_scaled_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
+                       const float* a_scale, int a_scale_per_row,
+                       const float* b_scale, int b_scale_per_col,
+                       const void* bias, int bias_dtype,
+                       void* C, int64_t ldc, int c_dtype,
+                       int64_t M, int64_t N, int64_t K,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+size_t fg_scaled_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLAGGEMS_AMD_H_ */

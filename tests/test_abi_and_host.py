@@ -1,0 +1,121 @@
+"""CPU-only checks: the shared library loads and exports every symbol the header declares, the
+Python host mirrors the reference's argument checking before any launch, and importing the
+package needs neither a GPU nor the library."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import flag_gems
+import flaggems_amd
+from flaggems_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "flaggems_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_all_bound_and_exported():
+    declared = _declared_symbols()
+    assert declared == sorted(_lib.SIGNATURES), "ctypes table and header disagree"
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("shared library not built on this host")
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert _lib.load().fg_version() >= 100
+    assert _lib.load().fg_last_error_string() is not None
+
+
+def test_c_abi_argument_validation_needs_no_gpu():
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("shared library not built on this host")
+    lib = _lib.load()
+    # cols not divisible by the group size -> FG_ERR_INVALID_ARG before any launch
+    rc = lib.fg_group_quant_fp8(1, _lib.FG_BF16, 4, 100, 100, 1, _lib.FG_FP8_E4M3FN, 100, 1, 1, 1,
+                                128, 1e-4, -448.0, 448.0, 1.0 / 448.0, 0, 0, 0, None)
+    assert rc == _lib.FG_ERR_INVALID_ARG
+    assert b"divisible" in lib.fg_last_error_string()
+    rc = lib.fg_block_fp8_gemm(1, 128, 1, 128, 1, 1, 1, 1, 1, 1, 1, 128, _lib.FG_BF16, 4, 4, 128, 64, 64, None, 0, None)
+    assert rc == _lib.FG_ERR_UNSUPPORTED
+    rc = lib.fg_block_fp8_gemm(None, 128, None, 128, None, 1, 1, None, 1, 1, None, 128, _lib.FG_BF16, 4, 4, 128, 128, 128, None, 0, None)
+    assert rc == _lib.FG_ERR_INVALID_ARG
+    # empty problems are accepted without touching the device
+    assert lib.fg_group_quant_fp8(None, _lib.FG_BF16, 0, 128, 128, None, _lib.FG_FP8_E4M3FN, 128, None, 1, 1,
+                                  128, 1e-4, -448.0, 448.0, 1.0 / 448.0, 0, 0, 0, None) == 0
+    assert lib.fg_scaled_fp8_gemm(None, 0, None, 0, None, 0, None, 0, None, 0, None, 0, _lib.FG_BF16, 0, 8, 8, None, 0, None) == 0
+
+
+def test_public_surface_matches_the_reference_names():
+    for name in ["act_quant_triton", "per_token_group_quant_fp8", "SUPPORTED_FP8_DTYPE", "w8a8_block_fp8_matmul",
+                 "fp8_matmul", "cutlass_scaled_mm", "scaled_mm", "scaled_mm_out", "enable", "only_enable", "use_gems",
+                 "all_registered_ops", "all_registered_keys", "patch_empty_vllm"]:
+        assert hasattr(flag_gems, name), name
+    assert flag_gems.SUPPORTED_FP8_DTYPE == torch.float8_e4m3fn
+    assert flag_gems.act_quant_triton is flaggems_amd.act_quant_triton
+
+
+def test_no_cpu_fallback():
+    x = torch.zeros(2, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        flag_gems.act_quant_triton(x)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        flag_gems.per_token_group_quant_fp8(x, 128)
+    a = torch.zeros(2, 128, dtype=torch.float8_e4m3fn)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        flag_gems.w8a8_block_fp8_matmul(a, a, torch.ones(2, 1), torch.ones(1, 1), [128, 128])
+
+
+def test_assertions_fire_before_any_launch():
+    x = torch.zeros(4, 100, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="divisible by block_size"):
+        flag_gems.act_quant_triton(x, 128)
+    with pytest.raises(AssertionError, match="contiguous"):
+        flag_gems.act_quant_triton(torch.zeros(128, 4, dtype=torch.bfloat16).t(), 128)
+    with pytest.raises(AssertionError, match="must be divisible"):
+        flag_gems.per_token_group_quant_fp8(x, 128)
+    with pytest.raises(AssertionError, match="groups must be contiguous"):
+        flag_gems.per_token_group_quant_fp8(torch.zeros(128, 4, dtype=torch.bfloat16).t(), 128)
+    a = torch.zeros(4, 256, dtype=torch.float8_e4m3fn)
+    with pytest.raises(AssertionError):
+        flag_gems.w8a8_block_fp8_matmul(a, a[:, :128], torch.ones(4, 2), torch.ones(1, 1), [128, 128])
+    with pytest.raises(AssertionError):
+        flag_gems.w8a8_block_fp8_matmul(a, a, torch.ones(4, 3), torch.ones(1, 2), [128, 128])
+    c = torch.zeros(4, 4, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="column-major"):
+        flag_gems.cutlass_scaled_mm(c, a, torch.zeros(256, 4, dtype=torch.float8_e4m3fn), torch.ones(1), torch.ones(1))
+    with pytest.raises(AssertionError, match="2D"):
+        flag_gems.cutlass_scaled_mm(c, a[0], a, torch.ones(1), torch.ones(1))
+    with pytest.raises(RuntimeError, match="cannot be multiplied"):
+        flag_gems.scaled_mm(a, a, torch.ones(1), torch.ones(1))
+    with pytest.raises(RuntimeError, match="scale_a must be"):
+        flag_gems.scaled_mm(a, a.t(), torch.ones(3), torch.ones(1))
+
+
+def test_registration_roundtrip_on_cpu_host():
+    with flag_gems.use_gems():
+        assert flag_gems.all_registered_keys() == ["_scaled_mm", "_scaled_mm.out"]
+        assert flag_gems.all_registered_ops() == ["scaled_mm", "scaled_mm_out"]
+    assert flag_gems.all_registered_keys() == []
+    with flag_gems.use_gems(include=["scaled_mm"]):
+        assert flag_gems.all_registered_keys() == ["_scaled_mm"]
+    with flag_gems.use_gems(exclude=["scaled_mm_out"]):
+        assert flag_gems.all_registered_keys() == ["_scaled_mm"]
+    flag_gems.patch_empty_vllm()
+    flag_gems.patch_empty_vllm()
+    assert hasattr(torch.ops._C, "cutlass_scaled_mm") and hasattr(torch.ops._C, "per_token_group_fp8_quant")
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "flaggems_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, os.path.join(dirpath, f)

@@ -1,0 +1,160 @@
+"""GPU parity of the block-scaled FP8 GEMM against the CPU oracle.
+
+Tolerance: BASELINE bar rtol 1e-2 / atol 1e-2 against the fp32-dequantised matmul for bf16 output;
+the reference's own tolerance (fp16 output, atol 1e-4*K, rtol 1e-3,
+tests/test_w8a8_block_fp8_matmul.py:107) is applied to its own shape list as well."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import flag_gems
+from oracle import fp8_linear_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+FP8 = torch.float8_e4m3fn
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _ref_inputs(M, N, K, seed=0):
+    """Inputs as the reference test builds them (tests/test_w8a8_block_fp8_matmul.py:65-74)."""
+    g = torch.Generator().manual_seed(seed)
+    A = torch.randn(M, K, generator=g).to(FP8)
+    B = torch.randn(N, K, generator=g).to(FP8)
+    kb, nb = (K + 127) // 128, (N + 127) // 128
+    As = 0.01 * torch.rand(M, kb, generator=g) + 0.005
+    Bs = 0.01 * torch.rand(nb, kb, generator=g) + 0.005
+    return A, B, As, Bs
+
+
+def _quantized_inputs(M, N, K, seed=0):
+    """Inputs as the benchmark configurations build them: X ~ N(0,1) act-quantized 1x128,
+    W ~ N(0, 0.02) quantized 128x128."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (0.02 * torch.randn(N, K, generator=g)).bfloat16()
+    xq, xs = O.act_quant_ref(x, 128)
+    wq, ws = O.per_block_cast_to_fp8_ref(w)
+    return xq, wq, xs, ws
+
+
+REF_SHAPES = [(128, 256, 512), (64, 128, 128), (256, 256, 256), (83, 7748, 3884), (84, 7168, 3884)]
+
+
+@pytest.mark.parametrize("M,N,K", REF_SHAPES)
+def test_reference_shapes_fp16_reference_tolerance(M, N, K):
+    A, B, As, Bs = _ref_inputs(M, N, K)
+    want = O.block_fp8_matmul_dequant_ref(A, B, As, Bs, [128, 128], torch.float32, torch.float64)
+    got = flag_gems.w8a8_block_fp8_matmul(A.to(DEV), B.to(DEV), As.to(DEV), Bs.to(DEV), [128, 128], output_dtype=torch.float16)
+    assert got.dtype == torch.float16 and got.shape == (M, N)
+    torch.testing.assert_close(got.cpu(), want.to(torch.float16), atol=1e-4 * K, rtol=1e-3)
+    # and much tighter than the reference asks: fp32 accumulation error only
+    torch.testing.assert_close(got.cpu().float(), want.float(), atol=2e-3, rtol=2e-3)
+
+
+@pytest.mark.parametrize("M", [1, 8, 64, 200, 512])
+@pytest.mark.parametrize("N,K", [(2112, 7168), (4096, 512), (1536, 1536), (7168, 2304)])
+def test_quantized_linear_shapes_bf16(M, N, K):
+    xq, wq, xs, ws = _quantized_inputs(M, N, K)
+    want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32)
+    got = flag_gems.w8a8_block_fp8_matmul(xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    assert got.dtype == torch.bfloat16 and got.shape == (M, N)
+    torch.testing.assert_close(got.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    got32 = flag_gems.w8a8_block_fp8_matmul(xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128], output_dtype=torch.float32)
+    torch.testing.assert_close(got32.cpu(), want, rtol=1e-4, atol=1e-5)
+
+
+def test_closed_forms():
+    A, B, As, Bs = _ref_inputs(48, 384, 512, seed=3)
+    # unit scales -> plain matmul, exact in fp32 for these magnitudes up to summation order
+    got = flag_gems.w8a8_block_fp8_matmul(A.to(DEV), B.to(DEV), torch.ones_like(As).to(DEV), torch.ones_like(Bs).to(DEV), [128, 128], output_dtype=torch.float32)
+    torch.testing.assert_close(got.cpu(), A.float() @ B.float().T, rtol=1e-6, atol=1e-3)
+    # one-hot rows pick single scaled weight entries exactly
+    cols = [0, 127, 128, 511]
+    a = torch.zeros(48, 512)
+    for r in range(48):
+        a[r, cols[r % 4]] = 1.0
+    got = flag_gems.w8a8_block_fp8_matmul(a.to(FP8).to(DEV), B.to(DEV), As.to(DEV), Bs.to(DEV), [128, 128], output_dtype=torch.float32).cpu()
+    for r in range(48):
+        c = cols[r % 4]
+        want = B[:, c].float() * As[r, c // 128] * Bs[:, c // 128].repeat_interleave(128)[:384]
+        torch.testing.assert_close(got[r], want, rtol=1e-6, atol=0)
+    # K-block-specific power-of-two scales are applied to the right block, exactly
+    as2 = torch.tensor([[2.0, 0.5, 4.0, 0.25]]).repeat(48, 1)
+    bs2 = torch.tensor([[0.25, 4.0, 1.0, 8.0]]).repeat(3, 1)
+    got = flag_gems.w8a8_block_fp8_matmul(A.to(DEV), B.to(DEV), as2.to(DEV), bs2.to(DEV), [128, 128], output_dtype=torch.float32).cpu()
+    af, bf = A.float(), B.float()
+    want = sum((af[:, i * 128:(i + 1) * 128] @ bf[:, i * 128:(i + 1) * 128].T) * float(as2[0, i] * bs2[0, i]) for i in range(4))
+    torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-4)
+
+
+def test_leading_dims_strided_scales_and_fp8_matmul_alias():
+    xq, wq, xs, ws = _quantized_inputs(24, 640, 1024, seed=5)
+    want = O.block_fp8_matmul_tiled_ref(xq, wq, xs, ws, [128, 128], torch.float32)
+    a = xq.view(2, 3, 4, 1024).to(DEV)
+    s = xs.view(2, 3, 4, 8).to(DEV)
+    got = flag_gems.w8a8_block_fp8_matmul(a, wq.to(DEV), s, ws.to(DEV), [128, 128])
+    assert got.shape == (2, 3, 4, 640)
+    torch.testing.assert_close(got.view(24, 640).cpu().float(), want, rtol=1e-2, atol=1e-2)
+    # column-major activation scales (strides (1, M)) and a weight that is a row-slice of a bigger one
+    s_cm = xs.t().contiguous().t().to(DEV)
+    big = torch.zeros(700, 1024, dtype=FP8)
+    big[30:670] = wq
+    got2 = flag_gems.w8a8_block_fp8_matmul(xq.to(DEV), big.to(DEV)[30:670], s_cm, ws.to(DEV), [128, 128])
+    assert torch.equal(got2.view(torch.int16), got.view(24, 640).view(torch.int16))
+    got3 = flag_gems.fp8_matmul(a, s, wq.to(DEV), ws.to(DEV))
+    assert got3.shape == (2, 3, 4, 640) and got3.dtype == torch.bfloat16
+    assert torch.equal(got3.view(torch.int16), got.view(torch.int16))
+
+
+def test_config1_golden():
+    z = np.load(os.path.join(GOLD, "config1.npz"))
+    x, w = O.make_config1(0)
+    xq, xs = flag_gems.act_quant_triton(x.to(DEV), 128)
+    wq, ws = O.per_block_cast_to_fp8_ref(w)
+    c = flag_gems.w8a8_block_fp8_matmul(xq, wq.to(DEV), xs, ws.to(DEV), [128, 128])
+    want = torch.from_numpy(z["c_bits"]).view(torch.bfloat16)
+    assert c.shape == (64, 512)
+    torch.testing.assert_close(c.cpu().float(), want.float(), rtol=1e-2, atol=1e-2)
+    # in practice within one bf16 step of the CPU result
+    assert ((c.cpu().float() - want.float()).abs() <= want.float().abs() * 2 ** -7 + 1e-6).all()
+
+
+@pytest.mark.parametrize("N,K", [(2112, 7168), (24576, 1536), (32768, 512), (7168, 16384), (4608, 7168), (7168, 2304)])
+def test_full_size_linearity_and_row_consistency(N, K):
+    """M = 4096 DeepSeek-V3 shapes: properties that need no CPU matmul.
+    (1) rows are independent: the first 8 rows equal an M=8 call (compared with the oracle);
+    (2) doubling one K-block's activation scale adds exactly that block's contribution."""
+    M = 4096
+    g = torch.Generator(device=DEV).manual_seed(0)
+    A = torch.randn(M, K, device=DEV, generator=g).to(FP8)
+    B = (torch.randn(N, K, device=DEV, generator=g)).to(FP8)
+    As = 0.01 * torch.rand(M, K // 128, device=DEV, generator=g) + 0.005
+    Bs = 0.01 * torch.rand((N + 127) // 128, K // 128, device=DEV, generator=g) + 0.005
+    C = flag_gems.w8a8_block_fp8_matmul(A, B, As, Bs, [128, 128], output_dtype=torch.float32)
+    rows = torch.tensor([0, 1, 255, 256, 2047, 4095], device=DEV)
+    want = O.block_fp8_matmul_dequant_ref(A[rows].cpu(), B.cpu(), As[rows].cpu(), Bs.cpu(), [128, 128], torch.float32)
+    torch.testing.assert_close(C[rows].cpu(), want, rtol=1e-4, atol=1e-5)
+    As2 = As.clone()
+    As2[:, 1] *= 2
+    C2 = flag_gems.w8a8_block_fp8_matmul(A, B, As2, Bs, [128, 128], output_dtype=torch.float32)
+    only1 = torch.zeros_like(As)
+    only1[:, 1] = As[:, 1]
+    C1 = flag_gems.w8a8_block_fp8_matmul(A, B, only1, Bs, [128, 128], output_dtype=torch.float32)
+    torch.testing.assert_close(C2 - C, C1, rtol=1e-3, atol=1e-5)
+
+
+def test_host_side_assertions():
+    A, B, As, Bs = (t.to(DEV) for t in _ref_inputs(16, 256, 256))
+    with pytest.raises(AssertionError):
+        flag_gems.w8a8_block_fp8_matmul(A, B[:, :128], As, Bs, [128, 128])
+    with pytest.raises(AssertionError):
+        flag_gems.w8a8_block_fp8_matmul(A, B, As[:, :1], Bs, [128, 128])
+    with pytest.raises(AssertionError):
+        flag_gems.w8a8_block_fp8_matmul(A.t(), B, As, Bs, [128, 128])
+    with pytest.raises(NotImplementedError):
+        flag_gems.w8a8_block_fp8_matmul(A, B, As.repeat(1, 2), Bs.repeat(2, 2), [64, 64])
+    out = flag_gems.w8a8_block_fp8_matmul(A[:0], B, As[:0], Bs, [128, 128])
+    assert out.shape == (0, 256)

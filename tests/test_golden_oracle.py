@@ -25,7 +25,9 @@ def test_config1_golden():
     assert _sha(r["wq"]) == str(z["wq_sha"])
     assert np.array_equal(r["wq"].view(torch.uint8).numpy()[:8], z["wq_head"])
     assert np.array_equal(r["ws"].numpy().view(np.uint32), z["ws"].view(np.uint32))
-    assert np.array_equal(r["c"].view(torch.int16).numpy(), z["c_bits"])
+    # fp32 matmul summation order may differ between hosts: within one bf16 step
+    want = torch.from_numpy(z["c_bits"]).view(torch.bfloat16)
+    torch.testing.assert_close(r["c"].float(), want.float(), rtol=2 ** -7, atol=2 ** -7)
 
 
 def test_quant_variants_golden():
