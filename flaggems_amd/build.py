@@ -25,7 +25,9 @@ HIPCC_FLAGS = [
     "-fPIC",
     # keep the compiler from forming packed-fp32 VALU instructions out of scalar float code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-command-line-argument",
+    # MFMA results land in architectural VGPRs, where the scale FMAs can read them directly
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
+    "-w",
 ]
 
 

@@ -11,9 +11,8 @@
 // Data path.  Tiles of BN x 128 weight bytes and BM x 128 activation bytes per K-block are staged in
 // LDS, double buffered.  When rows are 16-byte aligned and K % 128 == 0 the tiles go from global
 // memory straight into LDS (global_load_lds_dwordx4, 1 KB per wavefront instruction); otherwise a
-// guarded register-staged loader zero-fills the K tail.  The 16-byte chunk index of every row is
-// XOR-swizzled with (row >> 1) & 7 so that the 16 rows read by one ds_read_b128 fall into 16
-// different bank groups.  In block-scaled mode every K-block's MFMA result is multiplied by its fp32
+// guarded register-staged loader zero-fills the K tail.  Tiles sit in LDS in fragment order (see
+// the loaders below) so that every MFMA operand read is a lane-linear ds_read_b128.  In block-scaled mode every K-block's MFMA result is multiplied by its fp32
 // scale and added to the running fp32 accumulator (4 VALU FMAs per MFMA); in row/column mode the
 // MFMA accumulates directly and the scales are applied once in the epilogue.
 
@@ -38,8 +37,6 @@ struct GemmArgs {
   int c_dtype, bias_dtype;
   int xs_per_row, ws_per_col;
 };
-
-__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 
 // s_waitcnt vmcnt(0) with expcnt/lgkmcnt left at their maxima (gfx9 encoding)
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
@@ -78,27 +75,44 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 }
 
 // ---------------------------------------------------------------------------------------------
-// Tile loaders.  A tile is ROWS rows of 128 bytes; chunk i (16 bytes) of the LDS image holds logical
-// chunk (i & 7) ^ swz(i >> 3) of row i >> 3.
+// LDS image of a tile.  A tile is ROWS rows of one 128-byte K-block, row-major, with the eight
+// 16-byte chunks of row R permuted: physical chunk p holds logical chunk p ^ (R & 7).  One
+// global_load_lds_dwordx4 wavefront instruction fills 8 consecutive rows (1 KB, lane l writes byte
+// l*16) and fetches 8 whole 128-byte lines.  Lane l of an MFMA operand fragment owns row (l & 15) and
+// the logical chunks g and g+4 (g = l >> 4), i.e. K bytes [16g, 16g+16) and [64+16g, 64+16g+16); the K
+// order inside a fragment therefore differs from memory order, identically for both operands, which
+// leaves the dot product unchanged.  Both 16-byte reads of a fragment are bank-conflict free with this
+// permutation (measured 218 B/clk/CU; 117 B/clk/CU when a lane reads the adjacent chunks 2g and 2g+1).
 // ---------------------------------------------------------------------------------------------
 template <int ROWS, int NTHREADS>
-__device__ __forceinline__ void load_tile_direct(const uint8_t* __restrict__ g, int64_t ld, int row0, int row_max,
-                                                 int k0, uint8_t* lds_tile, int wave, int lane) {
-  constexpr int kWaves = NTHREADS / 64;
-  constexpr int kSlabs = ROWS / 8;  // 1 KB slabs
-  static_assert(kSlabs % kWaves == 0, "tile rows must split evenly over the wavefronts");
+struct DirectTile {
+  static constexpr int kWaves = NTHREADS / 64;
+  static constexpr int kSlabs = ROWS / 8;  // 1 KB each
+  static constexpr int kPerWave = kSlabs / kWaves;
+  static_assert(kSlabs % kWaves == 0, "tile slabs must split evenly over the wavefronts");
+  uint32_t off[kPerWave];  // byte offset of this lane's 16 bytes from the tile's first row, K-block 0
+
+  // rows past the edge re-read the last valid row (their results are never stored)
+  __device__ __forceinline__ void init(int64_t ld, int rows_valid, int wave, int lane) {
 #pragma unroll
-  for (int j = 0; j < kSlabs / kWaves; ++j) {
+    for (int j = 0; j < kPerWave; ++j) {
+      const int slab = wave + j * kWaves;
+      const int r = slab * 8 + (lane >> 3);
+      const int rc = r < rows_valid ? r : rows_valid - 1;
+      off[j] = (uint32_t)rc * (uint32_t)ld + (uint32_t)(((lane & 7) ^ (r & 7)) << 4);
+    }
+  }
+  // `base` is wave-uniform: first row of the tile, first byte of the K-block
+  __device__ __forceinline__ void issue_one(const uint8_t* __restrict__ base, uint8_t* lds_tile, int wave, int j) const {
     const int slab = wave + j * kWaves;
-    const int r = slab * 8 + (lane >> 3);
-    const int c = (lane & 7) ^ swz(r);
-    int gr = row0 + r;
-    gr = gr < row_max ? gr : row_max;  // rows past the edge re-read the last valid row
-    const uint8_t* src = g + (int64_t)gr * ld + k0 + c * 16;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + off[j]),
                                      (__attribute__((address_space(3))) void*)(lds_tile + slab * 1024), 16, 0, 0);
   }
-}
+  __device__ __forceinline__ void issue(const uint8_t* __restrict__ base, uint8_t* lds_tile, int wave) const {
+#pragma unroll
+    for (int j = 0; j < kPerWave; ++j) issue_one(base, lds_tile, wave, j);
+  }
+};
 
 template <int ROWS, int NTHREADS>
 struct StagedTile {
@@ -111,12 +125,11 @@ struct StagedTile {
                                        int K, bool aligned16, int tid) {
 #pragma unroll
     for (int j = 0; j < kChunks; ++j) {
-      const int i = tid + j * NTHREADS;
+      const int i = tid + j * NTHREADS;  // 16-byte chunk of the LDS image
       const int r = i >> 3;
-      const int c = (i & 7) ^ swz(r);
       int gr = row0 + r;
       gr = gr < row_max ? gr : row_max;
-      const int k = k0 + c * 16;
+      const int k = k0 + (((i & 7) ^ (r & 7)) << 4);
       const uint8_t* src = g + (int64_t)gr * ld + k;
       u32x4 t = {0u, 0u, 0u, 0u};
       if (aligned16 && k + 16 <= K) {
@@ -139,11 +152,15 @@ struct StagedTile {
   }
 };
 
-// 32 K-contiguous bytes of row `r` starting at logical chunk 2*g: one MFMA operand fragment.
-__device__ __forceinline__ v8i read_fragment(const uint8_t* lds_tile, int r, int g) {
-  const int s = swz(r);
-  const u32x4 lo = *reinterpret_cast<const u32x4*>(lds_tile + r * 128 + (((2 * g) ^ s) << 4));
-  const u32x4 hi = *reinterpret_cast<const u32x4*>(lds_tile + r * 128 + (((2 * g + 1) ^ s) << 4));
+// MFMA operand fragment of the 16-row group `rg` for this lane; `lane_off` = fragment_lane_offset(lane)
+__device__ __forceinline__ int fragment_lane_offset(int lane) {
+  const int r = lane & 15, g = lane >> 4;
+  return r * 128 + ((g ^ (r & 7)) << 4);
+}
+__device__ __forceinline__ v8i read_fragment(const uint8_t* lds_tile, int rg, int lane_off) {
+  // row group rg starts at rg*2048 and (16*rg) & 7 == 0, so the permutation depends on the lane only
+  const u32x4 lo = *reinterpret_cast<const u32x4*>(lds_tile + rg * 2048 + lane_off);
+  const u32x4 hi = *reinterpret_cast<const u32x4*>(lds_tile + rg * 2048 + (lane_off ^ 64));
   v8i f;
   f[0] = (int)lo.x; f[1] = (int)lo.y; f[2] = (int)lo.z; f[3] = (int)lo.w;
   f[4] = (int)hi.x; f[5] = (int)hi.y; f[6] = (int)hi.z; f[7] = (int)hi.w;
@@ -153,6 +170,33 @@ __device__ __forceinline__ v8i read_fragment(const uint8_t* lds_tile, int r, int
 __device__ __forceinline__ v4f mfma_fp8_16x16x128(v8i a, v8i b, v4f c) {
   // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled instruction
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+// One K-block partial product with a zero accumulator input, result in architectural VGPRs.
+__device__ __forceinline__ v4f mfma_fp8_block_partial(v8i a, v8i b) {
+  v4f p;
+  asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=&v"(p) : "v"(a), "v"(b));
+  return p;
+}
+
+// acc += p * s.  `p` was written by the MFMA issued one step earlier (an 8-pass instruction): between
+// that MFMA and these reads lie the previous step's four FMAs, one more MFMA and the s_nop below, which
+// covers the 11 wait states gfx950 requires between an 8-pass matrix write and a VALU read of it.
+#ifndef FG_MFMA_READ_NOPS
+#define FG_MFMA_READ_NOPS 5
+#endif
+#define FG_STR2(x) #x
+#define FG_STR(x) FG_STR2(x)
+__device__ __forceinline__ void scale_accumulate(v4f& acc, const v4f& p, float s) {
+  float a0 = acc[0], a1 = acc[1], a2 = acc[2], a3 = acc[3];
+  asm volatile("s_nop " FG_STR(FG_MFMA_READ_NOPS) "\n\t"
+               "v_fmac_f32 %0, %4, %8\n\t"
+               "v_fmac_f32 %1, %5, %8\n\t"
+               "v_fmac_f32 %2, %6, %8\n\t"
+               "v_fmac_f32 %3, %7, %8"
+               : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3)
+               : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(s));
+  acc[0] = a0; acc[1] = a1; acc[2] = a2; acc[3] = a3;
 }
 
 template <int BM, int BN, int WM, int WN>
@@ -190,6 +234,7 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int wm0 = wave_m * Cfg::kWaveM, wn0 = wave_n * Cfg::kWaveN;
   const int l16 = lane & 15, lg = lane >> 4;
+  const int frag_off = fragment_lane_offset(lane);
 
   v4f acc[TN][TM];
 #pragma unroll
@@ -200,7 +245,16 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
   const bool aligned16 = ((a.ldx | a.ldw) % 16 == 0) && (((uintptr_t)a.X | (uintptr_t)a.W) % 16 == 0);
   StagedTile<BN, NT> st_w;
   StagedTile<BM, NT> st_x;
+  DirectTile<BN, NT> dt_w;
+  DirectTile<BM, NT> dt_x;
   (void)st_w; (void)st_x; (void)aligned16;
+  // wave-uniform tile origins; a tile spans at most 256 rows, so lane offsets fit 32 bits (host checks ld)
+  const uint8_t* const w_base = a.W + (int64_t)n0 * a.ldw;
+  const uint8_t* const x_base = a.X + (int64_t)m0 * a.ldx;
+  if (DIRECT) {
+    dt_w.init(a.ldw, a.N - n0, wave, lane);
+    dt_x.init(a.ldx, a.M - m0, wave, lane);
+  }
 
   // activation-scale staging: thread t < BM owns row m0 + t
   const int xs_row = (m0 + tid < a.M) ? m0 + tid : a.M - 1;
@@ -214,8 +268,8 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
   if (a.KB == 0) {
     // K == 0: nothing to stage, the accumulators stay zero
   } else if (DIRECT) {
-    load_tile_direct<BN, NT>(a.W, a.ldw, n0, a.N - 1, 0, lds_w(0), wave, lane);
-    load_tile_direct<BM, NT>(a.X, a.ldx, m0, a.M - 1, 0, lds_x(0), wave, lane);
+    dt_w.issue(w_base, lds_w(0), wave);
+    dt_x.issue(x_base, lds_x(0), wave);
   } else {
     st_w.load(a.W, a.ldw, n0, a.N - 1, 0, a.K, aligned16, tid);
     st_x.load(a.X, a.ldx, m0, a.M - 1, 0, a.K, aligned16, tid);
@@ -223,6 +277,7 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
     st_x.store(lds_x(0), tid);
   }
   if (MODE == kModeBlock && a.KB > 0 && tid < BM) lds_xs[tid] = xs_ptr[0];
+  float ws_cur = (MODE == kModeBlock && a.KB > 0) ? ws_ptr[0] : 1.f;
 
   for (int kb = 0; kb < a.KB; ++kb) {
     const int cur = kb & 1, nxt = cur ^ 1;
@@ -230,43 +285,80 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
     __syncthreads();
 
     const bool more = kb + 1 < a.KB;
-    float xs_next = 0.f;
+    float xs_next = 0.f, ws_next = 1.f;
     if (more) {
       const int k1 = (kb + 1) * 128;
+      // the scale loads go first: their consumers then wait for them alone, not for the tile loads
+      if (MODE == kModeBlock) {
+        if (tid < BM) xs_next = xs_ptr[(int64_t)(kb + 1) * a.xs_cs];
+        ws_next = ws_ptr[(int64_t)(kb + 1) * a.ws_cs];
+      }
       if (DIRECT) {
-        load_tile_direct<BN, NT>(a.W, a.ldw, n0, a.N - 1, k1, lds_w(nxt), wave, lane);
-        load_tile_direct<BM, NT>(a.X, a.ldx, m0, a.M - 1, k1, lds_x(nxt), wave, lane);
+        // block-scaled mode spreads the tile loads over the MFMA steps below: issued as one burst
+        // they fill the CU's address queue and every wavefront stalls in the issue for ~1-2k cycles
+        if (MODE != kModeBlock) {
+          dt_w.issue(w_base + k1, lds_w(nxt), wave);
+          dt_x.issue(x_base + k1, lds_x(nxt), wave);
+        }
       } else {
         st_w.load(a.W, a.ldw, n0, a.N - 1, k1, a.K, aligned16, tid);
         st_x.load(a.X, a.ldx, m0, a.M - 1, k1, a.K, aligned16, tid);
       }
-      if (MODE == kModeBlock && tid < BM) xs_next = xs_ptr[(int64_t)(kb + 1) * a.xs_cs];
     }
 
     // ---- compute on stage `cur`
+    const uint8_t* const tw = lds_w(cur) + (wn0 >> 4) * 2048;
+    const uint8_t* const tx = lds_x(cur) + (wm0 >> 4) * 2048;
     float sc[TM];
     if (MODE == kModeBlock) {
-      const float wsv = ws_ptr[(int64_t)kb * a.ws_cs];
 #pragma unroll
-      for (int j = 0; j < TM; ++j) sc[j] = lds_xs[cur * BM + wm0 + j * 16 + l16] * wsv;
+      for (int j = 0; j < TM; ++j) sc[j] = lds_xs[cur * BM + wm0 + j * 16 + l16] * ws_cur;
     }
     v8i xf[TM];
 #pragma unroll
-    for (int j = 0; j < TM; ++j) xf[j] = read_fragment(lds_x(cur), wm0 + j * 16 + l16, lg);
+    for (int j = 0; j < TM; ++j) xf[j] = read_fragment(tx, j, frag_off);
+    if (MODE == kModeBlock) {
+      // Software pipeline with a pinned issue order: MFMA t, then the four scale-FMAs of MFMA t-1,
+      // which execute while the matrix core works on t.  The steps are volatile asm statements
+      // because the compiler otherwise clusters all MFMAs of the K-block, keeps every partial result
+      // live and spills the accumulators.
+      v8i wf = read_fragment(tw, 0, frag_off);
+      constexpr int kLoadsW = DirectTile<BN, NT>::kPerWave, kLoadsX = DirectTile<BM, NT>::kPerWave;
+      constexpr int kLoadEvery = (TN * TM) / (kLoadsW + kLoadsX);
+      static_assert(kLoadEvery >= 1, "more tile loads than MFMA steps");
+      const uint8_t* const w_next = w_base + (kb + 1) * 128;
+      const uint8_t* const x_next = x_base + (kb + 1) * 128;
+      v4f p_prev = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < TN; ++i) {
-      const v8i wf = read_fragment(lds_w(cur), wn0 + i * 16 + l16, lg);
+      for (int i = 0; i < TN; ++i) {
+        v8i wf_next = wf;
+        if (i + 1 < TN) wf_next = read_fragment(tw, i + 1, frag_off);
 #pragma unroll
-      for (int j = 0; j < TM; ++j) {
-        if (MODE == kModeBlock) {
-          const v4f p = mfma_fp8_16x16x128(wf, xf[j], v4f{0.f, 0.f, 0.f, 0.f});
-          acc[i][j][0] = __builtin_fmaf(p[0], sc[j], acc[i][j][0]);
-          acc[i][j][1] = __builtin_fmaf(p[1], sc[j], acc[i][j][1]);
-          acc[i][j][2] = __builtin_fmaf(p[2], sc[j], acc[i][j][2]);
-          acc[i][j][3] = __builtin_fmaf(p[3], sc[j], acc[i][j][3]);
-        } else {
-          acc[i][j] = mfma_fp8_16x16x128(wf, xf[j], acc[i][j]);
+        for (int j = 0; j < TM; ++j) {
+          const v4f p = mfma_fp8_block_partial(wf, xf[j]);
+          if (i > 0 || j > 0) {
+            const int pi = (j == 0) ? i - 1 : i, pj = (j == 0) ? TM - 1 : j - 1;
+            scale_accumulate(acc[pi][pj], p_prev, sc[pj]);
+          }
+          p_prev = p;
+          if (DIRECT) {
+            const int t = i * TM + j;
+            if (t % kLoadEvery == 0 && t / kLoadEvery < kLoadsW + kLoadsX && more) {
+              const int q = t / kLoadEvery;
+              if (q < kLoadsW) dt_w.issue_one(w_next, lds_w(nxt), wave, q);
+              else dt_x.issue_one(x_next, lds_x(nxt), wave, q - kLoadsW);
+            }
+          }
         }
+        wf = wf_next;
+      }
+      scale_accumulate(acc[TN - 1][TM - 1], p_prev, sc[TM - 1]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < TN; ++i) {
+        const v8i wf = read_fragment(tw, i, frag_off);
+#pragma unroll
+        for (int j = 0; j < TM; ++j) acc[i][j] = mfma_fp8_16x16x128(wf, xf[j], acc[i][j]);
       }
     }
 
@@ -277,6 +369,7 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
       }
       if (MODE == kModeBlock && tid < BM) lds_xs[nxt * BM + tid] = xs_next;
     }
+    ws_cur = ws_next;
   }
 
   // ---- epilogue
@@ -373,6 +466,7 @@ int launch_cfg(GemmArgs a, hipStream_t stream) {
 template <int MODE>
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   const bool direct = (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) &&
+                      (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
                       ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
   const bool big = a.M > 128;
   if (big) {
