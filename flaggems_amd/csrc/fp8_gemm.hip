@@ -276,8 +276,17 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
     st_w.store(lds_w(0), tid);
     st_x.store(lds_x(0), tid);
   }
-  if (MODE == kModeBlock && a.KB > 0 && tid < BM) lds_xs[tid] = xs_ptr[0];
-  float ws_cur = (MODE == kModeBlock && a.KB > 0) ? ws_ptr[0] : 1.f;
+  // Scales travel one K-block ahead of the tiles: every wait for them then falls right after the
+  // tile-load wait at the top of an iteration, where they have been in flight for a whole iteration.
+  // (A wait at the end of the iteration would also wait for the tile loads issued moments before.)
+  float xs_pend = 0.f, ws_pend = 1.f, ws_cur = 1.f;
+  if (MODE == kModeBlock && a.KB > 0) {
+    if (tid < BM) {
+      lds_xs[tid] = xs_ptr[0];
+      if (a.KB > 1) xs_pend = xs_ptr[a.xs_cs];
+    }
+    ws_pend = ws_ptr[0];
+  }
 
   for (int kb = 0; kb < a.KB; ++kb) {
     const int cur = kb & 1, nxt = cur ^ 1;
@@ -285,14 +294,18 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
     __syncthreads();
 
     const bool more = kb + 1 < a.KB;
-    float xs_next = 0.f, ws_next = 1.f;
+    if (MODE == kModeBlock) {
+      ws_cur = ws_pend;
+      if (more) {
+        if (tid < BM) {
+          lds_xs[nxt * BM + tid] = xs_pend;  // scales of K-block kb+1, read after the next barrier
+          if (kb + 2 < a.KB) xs_pend = xs_ptr[(int64_t)(kb + 2) * a.xs_cs];
+        }
+        ws_pend = ws_ptr[(int64_t)(kb + 1) * a.ws_cs];
+      }
+    }
     if (more) {
       const int k1 = (kb + 1) * 128;
-      // the scale loads go first: their consumers then wait for them alone, not for the tile loads
-      if (MODE == kModeBlock) {
-        if (tid < BM) xs_next = xs_ptr[(int64_t)(kb + 1) * a.xs_cs];
-        ws_next = ws_ptr[(int64_t)(kb + 1) * a.ws_cs];
-      }
       if (DIRECT) {
         // block-scaled mode spreads the tile loads over the MFMA steps below: issued as one burst
         // they fill the CU's address queue and every wavefront stalls in the issue for ~1-2k cycles
@@ -309,20 +322,24 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
     // ---- compute on stage `cur`
     const uint8_t* const tw = lds_w(cur) + (wn0 >> 4) * 2048;
     const uint8_t* const tx = lds_x(cur) + (wm0 >> 4) * 2048;
+    // LDS reads in the order the first MFMAs need them: all wavefronts leave the barrier together
+    // and the reads of this phase queue up in the LDS, so the first operands should be at the front
+    v8i xf[TM];
+    xf[0] = read_fragment(tx, 0, frag_off);
+    v8i wf_first = read_fragment(tw, 0, frag_off);
+#pragma unroll
+    for (int j = 1; j < TM; ++j) xf[j] = read_fragment(tx, j, frag_off);
     float sc[TM];
     if (MODE == kModeBlock) {
 #pragma unroll
       for (int j = 0; j < TM; ++j) sc[j] = lds_xs[cur * BM + wm0 + j * 16 + l16] * ws_cur;
     }
-    v8i xf[TM];
-#pragma unroll
-    for (int j = 0; j < TM; ++j) xf[j] = read_fragment(tx, j, frag_off);
     if (MODE == kModeBlock) {
       // Software pipeline with a pinned issue order: MFMA t, then the four scale-FMAs of MFMA t-1,
       // which execute while the matrix core works on t.  The steps are volatile asm statements
       // because the compiler otherwise clusters all MFMAs of the K-block, keeps every partial result
       // live and spills the accumulators.
-      v8i wf = read_fragment(tw, 0, frag_off);
+      v8i wf = wf_first;
       constexpr int kLoadsW = DirectTile<BN, NT>::kPerWave, kLoadsX = DirectTile<BM, NT>::kPerWave;
       constexpr int kLoadEvery = (TN * TM) / (kLoadsW + kLoadsX);
       static_assert(kLoadEvery >= 1, "more tile loads than MFMA steps");
@@ -356,7 +373,7 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
     } else {
 #pragma unroll
       for (int i = 0; i < TN; ++i) {
-        const v8i wf = read_fragment(tw, i, frag_off);
+        const v8i wf = (i == 0) ? wf_first : read_fragment(tw, i, frag_off);
 #pragma unroll
         for (int j = 0; j < TM; ++j) acc[i][j] = mfma_fp8_16x16x128(wf, xf[j], acc[i][j]);
       }
@@ -367,9 +384,7 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
         st_w.store(lds_w(nxt), tid);
         st_x.store(lds_x(nxt), tid);
       }
-      if (MODE == kModeBlock && tid < BM) lds_xs[nxt * BM + tid] = xs_next;
     }
-    ws_cur = ws_next;
   }
 
   // ---- epilogue
