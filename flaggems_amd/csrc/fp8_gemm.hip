@@ -16,45 +16,10 @@
 // scale and added to the running fp32 accumulator (4 VALU FMAs per MFMA); in row/column mode the
 // MFMA accumulates directly and the scales are applied once in the epilogue.
 
-#include "fg_common.h"
+#include "fp8_gemm_common.h"
 
 namespace fg {
 namespace {
-
-enum { kModeBlock = 0, kModeRowCol = 1 };
-
-struct GemmArgs {
-  const uint8_t* X;  // activations [M, K]
-  const uint8_t* W;  // weights [N, K]
-  void* C;
-  const float* xs;   // block: As [M, KB]; rowcol: a_scale
-  const float* ws;   // block: Bs [NB, KB]; rowcol: b_scale
-  const void* bias;
-  int64_t ldx, ldw, ldc;
-  int64_t xs_rs, xs_cs, ws_rs, ws_cs;
-  int M, N, K, KB;
-  int tiles_m, tiles_n;
-  int c_dtype, bias_dtype;
-  int xs_per_row, ws_per_col;
-};
-
-// s_waitcnt vmcnt(0) with expcnt/lgkmcnt left at their maxima (gfx9 encoding)
-__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
-
-__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return bits_to_float((uint32_t)b << 16); }
-
-__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
-  uint32_t u = float_to_bits(f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);  // quiet NaN
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
-}
-
-__device__ __forceinline__ float load_as_float(const void* p, int64_t i, int dtype) {
-  if (dtype == FG_F32) return reinterpret_cast<const float*>(p)[i];
-  if (dtype == FG_F16) return (float)reinterpret_cast<const _Float16*>(p)[i];
-  return bf16_bits_to_float(reinterpret_cast<const uint16_t*>(p)[i]);
-}
 
 // Map the hardware block id to a tile so that (a) the blocks one XCD receives (ids congruent mod 8)
 // form a contiguous run of tiles and (b) a run walks GROUP_M tile rows before moving along N, which
@@ -167,10 +132,6 @@ __device__ __forceinline__ v8i read_fragment(const uint8_t* lds_tile, int rg, in
   return f;
 }
 
-__device__ __forceinline__ v4f mfma_fp8_16x16x128(v8i a, v8i b, v4f c) {
-  // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled instruction
-  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
-}
 
 // One K-block partial product with a zero accumulator input, result in architectural VGPRs.
 __device__ __forceinline__ v4f mfma_fp8_block_partial(v8i a, v8i b) {
@@ -479,10 +440,14 @@ int launch_cfg(GemmArgs a, hipStream_t stream) {
 }
 
 template <int MODE>
-int launch_gemm(const GemmArgs& a, hipStream_t stream) {
+int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   const bool direct = (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) &&
                       (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
                       ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
+  if (direct) {
+    const SmallMPlan plan = plan_small_m(a.M, a.N, a.K);
+    if (plan.use) return launch_small_m(a, MODE, plan, workspace, workspace_bytes, stream);
+  }
   const bool big = a.M > 128;
   if (big) {
     return direct ? launch_cfg<256, 256, 4, 2, MODE, true>(a, stream)
@@ -506,8 +471,13 @@ int check_common(const void* A, const void* B, const void* C, int64_t lda, int64
 }  // namespace
 }  // namespace fg
 
-extern "C" size_t fg_block_fp8_gemm_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
-extern "C" size_t fg_scaled_fp8_gemm_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
+extern "C" size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  const fg::SmallMPlan plan = fg::plan_small_m(M, N, K);
+  return plan.use ? plan.workspace_bytes : 0;
+}
+extern "C" size_t fg_scaled_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  return fg_block_fp8_gemm_workspace_bytes(M, N, K);
+}
 
 extern "C" int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
                                  const float* As, int64_t as_row_stride, int64_t as_col_stride,
@@ -516,7 +486,6 @@ extern "C" int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int6
                                  int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
                                  void* workspace, size_t workspace_bytes, void* stream) {
   using namespace fg;
-  (void)workspace; (void)workspace_bytes;
   if (block_n != 128 || block_k != 128)
     FG_FAIL(FG_ERR_UNSUPPORTED, "fg_block_fp8_gemm: only 128x128 scale blocks are implemented (got %lld x %lld)",
             (long long)block_n, (long long)block_k);
@@ -533,7 +502,7 @@ extern "C" int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int6
   a.xs_rs = as_row_stride; a.xs_cs = as_col_stride; a.ws_rs = bs_row_stride; a.ws_cs = bs_col_stride;
   a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)ceil_div(K, 128);
   a.c_dtype = c_dtype;
-  return launch_gemm<kModeBlock>(a, (hipStream_t)stream);
+  return launch_gemm<kModeBlock>(a, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int fg_scaled_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
@@ -544,7 +513,6 @@ extern "C" int fg_scaled_fp8_gemm(const void* A, int64_t lda, const void* B, int
                                   int64_t M, int64_t N, int64_t K,
                                   void* workspace, size_t workspace_bytes, void* stream) {
   using namespace fg;
-  (void)workspace; (void)workspace_bytes;
   if (c_dtype != FG_BF16 && c_dtype != FG_F16 && c_dtype != FG_F32 && c_dtype != FG_FP8_E4M3FN)
     FG_FAIL(FG_ERR_INVALID_ARG, "fg_scaled_fp8_gemm: c_dtype %d", c_dtype);
   if (bias && bias_dtype != FG_BF16 && bias_dtype != FG_F16 && bias_dtype != FG_F32)
@@ -560,5 +528,5 @@ extern "C" int fg_scaled_fp8_gemm(const void* A, int64_t lda, const void* B, int
   a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)ceil_div(K, 128);
   a.c_dtype = c_dtype; a.bias_dtype = bias_dtype;
   a.xs_per_row = a_scale_per_row; a.ws_per_col = b_scale_per_col;
-  return launch_gemm<kModeRowCol>(a, (hipStream_t)stream);
+  return launch_gemm<kModeRowCol>(a, workspace, workspace_bytes, (hipStream_t)stream);
 }

@@ -1,0 +1,92 @@
+// Pieces shared by the FP8 GEMM kernels: argument block, conversions, per-element epilogue.
+#pragma once
+
+#include "fg_common.h"
+
+namespace fg {
+
+enum { kModeBlock = 0, kModeRowCol = 1 };
+
+struct GemmArgs {
+  const uint8_t* X;  // activations [M, K]
+  const uint8_t* W;  // weights [N, K]
+  void* C;
+  const float* xs;   // block: As [M, KB]; rowcol: a_scale
+  const float* ws;   // block: Bs [NB, KB]; rowcol: b_scale
+  const void* bias;
+  int64_t ldx, ldw, ldc;
+  int64_t xs_rs, xs_cs, ws_rs, ws_cs;
+  int M, N, K, KB;
+  int tiles_m, tiles_n;
+  int c_dtype, bias_dtype;
+  int xs_per_row, ws_per_col;
+};
+
+// s_waitcnt vmcnt(0) with expcnt/lgkmcnt left at their maxima (gfx9 encoding)
+__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return bits_to_float((uint32_t)b << 16); }
+
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = float_to_bits(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);  // quiet NaN
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float load_as_float(const void* p, int64_t i, int dtype) {
+  if (dtype == FG_F32) return reinterpret_cast<const float*>(p)[i];
+  if (dtype == FG_F16) return (float)reinterpret_cast<const _Float16*>(p)[i];
+  return bf16_bits_to_float(reinterpret_cast<const uint16_t*>(p)[i]);
+}
+
+
+// Final value of one output element: row/column scaling (row/column mode only), rounding to the
+// output type and the bias added after that rounding, in the output type, as the reference's epilogue
+// does (src/flag_gems/fused/cutlass_scaled_mm.py:288-305).
+template <int MODE>
+__device__ __forceinline__ void store_output(const GemmArgs& a, int m, int n, float v) {
+  if (MODE == kModeRowCol) v = (v * a.xs[a.xs_per_row ? m : 0]) * a.ws[a.ws_per_col ? n : 0];
+  const bool has_bias = (MODE == kModeRowCol) && a.bias != nullptr;
+  const int64_t off = (int64_t)m * a.ldc + n;
+  if (a.c_dtype == FG_BF16) {
+    uint16_t h = float_to_bf16_bits(v);
+    if (has_bias) h = float_to_bf16_bits(bf16_bits_to_float(h) + load_as_float(a.bias, n, a.bias_dtype));
+    reinterpret_cast<uint16_t*>(a.C)[off] = h;
+  } else if (a.c_dtype == FG_F16) {
+    _Float16 h = (_Float16)v;
+    if (has_bias) h = (_Float16)((float)h + load_as_float(a.bias, n, a.bias_dtype));
+    reinterpret_cast<_Float16*>(a.C)[off] = h;
+  } else if (a.c_dtype == FG_F32) {
+    if (has_bias) v = v + load_as_float(a.bias, n, a.bias_dtype);
+    reinterpret_cast<float*>(a.C)[off] = v;
+  } else {  // FG_FP8_E4M3FN
+    uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(v, 0.f, 0, false) & 0xFFu;
+    if (has_bias) {
+      const float back = __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
+      code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(back + load_as_float(a.bias, n, a.bias_dtype), 0.f, 0, false) & 0xFFu;
+    }
+    reinterpret_cast<uint8_t*>(a.C)[off] = (uint8_t)code;
+  }
+}
+
+__device__ __forceinline__ v4f mfma_fp8_16x16x128(v8i a, v8i b, v4f c) {
+  // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled instruction
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+// Small-M (decode) path, fp8_gemm_smallm.hip.  `use` reports whether the kernel takes the problem.
+struct SmallMPlan {
+  bool use;
+  int tmx;        // 16-row activation fragments: 1, 2 or 4
+  int waves;      // wavefronts per block: 4 or 8
+  int kpw;        // K-blocks per wavefront
+  int splits;     // blocks along K that share one 64-row output chunk
+  int n_chunks;   // ceil(N / 64)
+  size_t workspace_bytes;
+};
+SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K);
+int launch_small_m(const GemmArgs& a, int mode, const SmallMPlan& plan, void* workspace, size_t workspace_bytes,
+                   hipStream_t stream);
+
+}  // namespace fg
