@@ -78,11 +78,13 @@ __device__ __forceinline__ v4f mfma_fp8_16x16x128(v8i a, v8i b, v4f c) {
 // Small-M (decode) path, fp8_gemm_smallm.hip.  `use` reports whether the kernel takes the problem.
 struct SmallMPlan {
   bool use;
+  bool staged;    // weight bytes fetched in 256-byte runs (K-block pairs) and transposed through LDS
   int tmx;        // 16-row activation fragments: 1, 2 or 4
+  int rg;         // 16-row weight groups per output chunk: 1, 2 or 4
   int waves;      // wavefronts per block: 4 or 8
-  int kpw;        // K-blocks per wavefront
+  int kpw;        // K-blocks (K-block pairs when staged) per wavefront
   int splits;     // blocks along K that share one 64-row output chunk
-  int n_chunks;   // ceil(N / 64)
+  int n_chunks;   // ceil(N / (16 * rg))
   size_t workspace_bytes;
 };
 SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K);

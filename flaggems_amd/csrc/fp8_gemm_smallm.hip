@@ -90,6 +90,70 @@ __device__ __forceinline__ void compute_unit(const Unit<TMX>& u, v4f (&acc)[kRow
   }
 }
 
+// Adds the wavefronts' accumulators in LDS and writes the chunk (or publishes a split-K partial tile and,
+// in the block that arrives last, adds the partial tiles in split order).  `red` is [WAVES][16*TMX][64].
+template <int TMX, int RG, int WAVES, int MODE>
+__device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int* last_flag,
+                                             const v4f (&acc)[RG][TMX], int chunk, int split) {
+  constexpr int NT = WAVES * 64;
+  constexpr int MROWS = 16 * TMX;
+  constexpr int kChunkRows = 16 * RG;
+  constexpr int kRowGroups = RG;
+  constexpr int kOut = MROWS * kChunkRows;
+  const GemmArgs& g = a.g;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, lg = lane >> 4;
+  const int n0 = chunk * kChunkRows;
+  // lane holds m = t*16 + l16, n = r*16 + 4*lg + [0,4)
+#pragma unroll
+  for (int r = 0; r < kRowGroups; ++r)
+#pragma unroll
+    for (int t = 0; t < TMX; ++t)
+      *reinterpret_cast<v4f*>(red + ((wave * MROWS + t * 16 + l16) * kChunkRows + r * 16 + lg * 4)) = acc[r][t];
+  __syncthreads();
+
+  if (a.splits == 1) {
+    for (int i = tid; i < kOut; i += NT) {
+      const int m = i / kChunkRows, nn = i % kChunkRows;
+      float v = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) v += red[w * kOut + i];
+      if (m < g.M && n0 + nn < g.N) store_output<MODE>(g, m, n0 + nn, v);
+    }
+    return;
+  }
+
+  float* const mine = a.partials + ((int64_t)chunk * a.splits + split) * kOut;
+  for (int i = tid; i < kOut; i += NT) {
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) v += red[w * kOut + i];
+    // device-scope store: written through to memory, where blocks on other XCDs (own L2 each) read it
+    __hip_atomic_store(mine + i, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // A device-scope fence here would write back and invalidate the whole L2 (measured ~50 us per
+  // launch).  The partial tiles bypass the L2 on both sides instead, so it is enough that every
+  // store of this block has been acknowledged before the counter moves.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (tid == 0) {
+    const unsigned int prev = __hip_atomic_fetch_add(&a.counters[chunk], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *last_flag = (prev == (unsigned int)(a.splits - 1)) ? 1 : 0;
+  }
+  __syncthreads();
+  if (!*last_flag) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  const float* const all = a.partials + (int64_t)chunk * a.splits * kOut;
+  for (int i = tid; i < kOut; i += NT) {
+    const int m = i / kChunkRows, nn = i % kChunkRows;
+    float v = 0.f;
+    for (int s = 0; s < a.splits; ++s)
+      v += __hip_atomic_load(all + (int64_t)s * kOut + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (m < g.M && n0 + nn < g.N) store_output<MODE>(g, m, n0 + nn, v);
+  }
+  if (tid == 0) __hip_atomic_store(&a.counters[chunk], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+}
+
 template <int TMX, int WAVES, int MODE>
 __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_smallm_kernel(SmallArgs a) {
   constexpr int NT = WAVES * 64;
@@ -146,57 +210,156 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_smallm_kernel(SmallArgs a
     compute_unit<TMX, MODE>(cur, acc);
   }
 
-  // ---- add the wavefronts' results in LDS: lane holds m = t*16 + l16, n = r*16 + 4*lg + [0,4)
-#pragma unroll
-  for (int r = 0; r < kRowGroups; ++r)
-#pragma unroll
-    for (int t = 0; t < TMX; ++t)
-      *reinterpret_cast<v4f*>(&red[wave][t * 16 + l16][r * 16 + lg * 4]) = acc[r][t];
-  __syncthreads();
+  finish_chunk<TMX, kRowGroups, WAVES, MODE>(a, &red[0][0][0], &last_flag, acc, chunk, split);
+}
 
-  constexpr int kOut = MROWS * kChunkRows;
-  if (a.splits == 1) {
-    for (int i = tid; i < kOut; i += NT) {
-      const int m = i / kChunkRows, nn = i % kChunkRows;
-      float v = 0.f;
+// ---------------------------------------------------------------------------------------------
+// Transposing variant (M <= 32, K >= 1024).  Same decomposition, but the weight bytes are fetched in
+// runs of 256 contiguous bytes per row (two K-blocks; 4 rows per wavefront load instruction) instead
+// of the 64-byte pieces the MFMA operand layout dictates: measured on MI355X a pure load of a
+// [7168, 16384] matrix reaches 5.8 TB/s with 256-byte runs against 5.0 TB/s with 64-byte pieces.  The
+// loads land in registers (the register file holds far more bytes in flight than LDS could); when a
+// pair of K-blocks has arrived the wavefront writes it to its private 16 KB LDS slab and reads it back
+// in operand layout.  No barrier is involved before the final reduction: a wavefront's LDS operations
+// execute in order.  Within a row the sixteen 16-byte chunks are permuted (physical chunk p holds
+// logical chunk p ^ (row & 15)) so that both the writes (4 rows x 256 B) and the operand reads (16 rows
+// 256 bytes apart) spread over all LDS banks.
+// ---------------------------------------------------------------------------------------------
+template <int TMX, int RG>
+struct PairRegs {
+  u32x4 w[4 * RG];             // load j: rows 4j..4j+3, lane -> row 4j + (l >> 4), bytes 16*(l & 15) of the pair
+  u32x4 xlo[2][TMX], xhi[2][TMX];
+  float xs[2][TMX];
+  float ws[2];
+};
+
+// RG = 16-row groups per chunk (1, 2 or 4), DEPTH = K-block pairs in flight per wavefront.
+template <int TMX, int RG, int DEPTH, int WAVES, int MODE>
+__global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArgs a) {
+  constexpr int kRows = 16 * RG;
+  constexpr int kSlab = kRows * 256;  // one K-block pair of the chunk
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // WAVES slabs; later the reduction buffer
+  __shared__ int last_flag;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int chunk = blockIdx.x % a.n_chunks;
+  const int split = blockIdx.x / a.n_chunks;
+  const int n0 = chunk * kRows;
+  const int l16 = lane & 15, lg = lane >> 4;
+  const GemmArgs& g = a.g;
+  uint8_t* const slab = lds + wave * kSlab;
+
+  const uint8_t* const w_base = g.W + (int64_t)n0 * g.ldw + l16 * 16;
+  const int rows_valid = g.N - n0;
+  uint32_t w_off[4 * RG];
 #pragma unroll
-      for (int w = 0; w < WAVES; ++w) v += red[w][m][nn];
-      if (m < g.M && n0 + nn < g.N) store_output<MODE>(g, m, n0 + nn, v);
+  for (int j = 0; j < 4 * RG; ++j) {
+    int r = 4 * j + lg;
+    r = r < rows_valid ? r : rows_valid - 1;  // rows past the edge alias the last valid row; never stored
+    w_off[j] = (uint32_t)r * (uint32_t)g.ldw;
+  }
+  const uint8_t* xrow[TMX];
+  const float* xsrow[TMX];
+#pragma unroll
+  for (int t = 0; t < TMX; ++t) {
+    int m = t * 16 + l16;
+    m = m < g.M ? m : g.M - 1;
+    xrow[t] = g.X + (int64_t)m * g.ldx + lg * 16;
+    xsrow[t] = (MODE == kModeBlock) ? g.xs + (int64_t)m * g.xs_rs : nullptr;
+  }
+  const float* wsrow = (MODE == kModeBlock) ? g.ws + (int64_t)(n0 >> 7) * g.ws_rs : nullptr;
+
+  v4f acc[RG][TMX];
+#pragma unroll
+  for (int r = 0; r < RG; ++r)
+#pragma unroll
+    for (int t = 0; t < TMX; ++t) acc[r][t] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  const int pairs_total = (g.KB + 1) >> 1;
+  const int per_split = a.kpw * WAVES;
+  const int pair_end = min(pairs_total, (split + 1) * per_split);
+
+  auto load_pair = [&](PairRegs<TMX, RG>& u, int pair) __attribute__((always_inline)) {
+    const int kb = pair * 2;
+    const bool two = kb + 1 < g.KB;  // an odd K-block count leaves a single block at the end
+    const int64_t k = (int64_t)kb * 128;
+    // lanes 8..15 of a row own the second K-block; when it does not exist they re-read the first
+    const int64_t kw = k - ((!two && l16 >= 8) ? 128 : 0);
+#pragma unroll
+    for (int j = 0; j < 4 * RG; ++j)
+      u.w[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w_base + kw + w_off[j]));
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int kbb = kb + ((b == 1 && two) ? 1 : 0);
+#pragma unroll
+      for (int t = 0; t < TMX; ++t) {
+        u.xlo[b][t] = *reinterpret_cast<const u32x4*>(xrow[t] + (int64_t)kbb * 128);
+        u.xhi[b][t] = *reinterpret_cast<const u32x4*>(xrow[t] + (int64_t)kbb * 128 + 64);
+        if (MODE == kModeBlock) u.xs[b][t] = xsrow[t][(int64_t)kbb * g.xs_cs];
+      }
+      if (MODE == kModeBlock) u.ws[b] = wsrow[(int64_t)kbb * g.ws_cs];
     }
-    return;
-  }
+  };
 
-  // ---- split K: publish this block's partial tile, last arriver reduces in split order
-  float* const mine = a.partials + ((int64_t)chunk * a.splits + split) * kOut;
-  for (int i = tid; i < kOut; i += NT) {
-    const int m = i / kChunkRows, nn = i % kChunkRows;
-    float v = 0.f;
+  auto multiply = [&](const PairRegs<TMX, RG>& u, int pair) __attribute__((always_inline)) {
+    const bool two = pair * 2 + 1 < g.KB;
+    // registers -> slab: row R = 4j + lg, logical chunk l16 goes to physical chunk l16 ^ (R & 15)
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) v += red[w][m][nn];
-    // device-scope store: written through to memory, where blocks on other XCDs (own L2 each) read it
-    __hip_atomic_store(mine + i, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int j = 0; j < 4 * RG; ++j) {
+      const int R = 4 * j + lg;
+      *reinterpret_cast<u32x4*>(slab + R * 256 + ((l16 ^ (R & 15)) << 4)) = u.w[j];
+    }
+    // slab -> operand fragments: lane owns row rg*16 + l16 and logical chunks b*8 + lg, b*8 + lg + 4
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      if (b == 1 && !two) break;
+#pragma unroll
+      for (int r = 0; r < RG; ++r) {
+        const uint8_t* row = slab + (r * 16 + l16) * 256;
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(row + (((b * 8 + lg) ^ l16) << 4));
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(row + (((b * 8 + lg + 4) ^ l16) << 4));
+        const v8i wf = join(lo, hi);
+#pragma unroll
+        for (int t = 0; t < TMX; ++t) {
+          const v8i xf = join(u.xlo[b][t], u.xhi[b][t]);
+          if (MODE == kModeBlock) {
+            const float sc = u.xs[b][t] * u.ws[b];
+            const v4f p = mfma_fp8_16x16x128(wf, xf, v4f{0.f, 0.f, 0.f, 0.f});
+            acc[r][t][0] = __builtin_fmaf(p[0], sc, acc[r][t][0]);
+            acc[r][t][1] = __builtin_fmaf(p[1], sc, acc[r][t][1]);
+            acc[r][t][2] = __builtin_fmaf(p[2], sc, acc[r][t][2]);
+            acc[r][t][3] = __builtin_fmaf(p[3], sc, acc[r][t][3]);
+          } else {
+            acc[r][t] = mfma_fp8_16x16x128(wf, xf, acc[r][t]);
+          }
+        }
+      }
+    }
+  };
+
+  // DEPTH register sets form a ring; the loop body is written out once per set so that the ring index
+  // is static and nothing is copied between sets
+  int pair = split * per_split + wave;
+  PairRegs<TMX, RG> ring[DEPTH];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (pair + d * WAVES < pair_end) load_pair(ring[d], pair + d * WAVES);
+  bool done = pair >= pair_end;
+  while (!done) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (!done) {
+        multiply(ring[d], pair);
+        const int refill = pair + DEPTH * WAVES;
+        if (refill < pair_end) load_pair(ring[d], refill);
+        pair += WAVES;
+        done = pair >= pair_end;
+      }
+    }
   }
-  // A device-scope fence here would write back and invalidate the whole L2 (measured ~50 us per
-  // launch).  The partial tiles bypass the L2 on both sides instead, so it is enough that every
-  // store of this block has been acknowledged before the counter moves.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-  __syncthreads();
-  if (tid == 0) {
-    const unsigned int prev = __hip_atomic_fetch_add(&a.counters[chunk], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    last_flag = (prev == (unsigned int)(a.splits - 1)) ? 1 : 0;
-  }
-  __syncthreads();
-  if (!last_flag) return;
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-  const float* const all = a.partials + (int64_t)chunk * a.splits * kOut;
-  for (int i = tid; i < kOut; i += NT) {
-    const int m = i / kChunkRows, nn = i % kChunkRows;
-    float v = 0.f;
-    for (int s = 0; s < a.splits; ++s)
-      v += __hip_atomic_load(all + (int64_t)s * kOut + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (m < g.M && n0 + nn < g.N) store_output<MODE>(g, m, n0 + nn, v);
-  }
-  if (tid == 0) __hip_atomic_store(&a.counters[chunk], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+  __syncthreads();  // the slabs are dead; their memory now holds the reduction buffer
+  finish_chunk<TMX, RG, WAVES, MODE>(a, reinterpret_cast<float*>(lds), &last_flag, acc, chunk, split);
 }
 
 template <int TMX, int WAVES>
@@ -208,6 +371,28 @@ int launch_t(const SmallArgs& sa, int mode, hipStream_t stream) {
   return FG_OK;
 }
 
+template <int TMX, int RG, int DEPTH, int WAVES>
+int launch_transpose(const SmallArgs& sa, int mode, hipStream_t stream) {
+  // WAVES slabs of RG * 4 KB; the reduction buffer (WAVES * 16*TMX * 16*RG floats) reuses the same memory
+  constexpr int kSlabs = WAVES * 16 * RG * 256;
+  constexpr int kRed = WAVES * 16 * TMX * 16 * RG * 4;
+  constexpr int kLds = kSlabs > kRed ? kSlabs : kRed;
+  const dim3 grid((uint32_t)(sa.n_chunks * sa.splits)), block(WAVES * 64);
+  auto kb = fp8_gemm_transpose_kernel<TMX, RG, DEPTH, WAVES, kModeBlock>;
+  auto kr = fp8_gemm_transpose_kernel<TMX, RG, DEPTH, WAVES, kModeRowCol>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(kb), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(kr), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e1 != hipSuccess || e2 != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS) failed", kLds);
+    attr_set = true;
+  }
+  if (mode == kModeBlock) hipLaunchKernelGGL(kb, grid, block, kLds, stream, sa);
+  else hipLaunchKernelGGL(kr, grid, block, kLds, stream, sa);
+  FG_CHECK_LAUNCH("fp8_gemm_transpose_kernel");
+  return FG_OK;
+}
+
 }  // namespace
 
 SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K) {
@@ -215,27 +400,46 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K) {
   p.use = false;
   if (M < 1 || M > 64 || N < 1 || K < 128 || K % 128 != 0) return p;
   p.tmx = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  p.waves = p.tmx == 4 ? 4 : 8;  // LDS reduction buffer is 4 KB * tmx per wavefront
-  p.n_chunks = (int)ceil_div(N, kChunkRows);
-  if (p.n_chunks > FG_WORKSPACE_COUNTER_BYTES / 4) return p;
   const int64_t KB = K / 128;
-  // aim for ~8 wavefronts per CU on 256 CUs, each with at least one K-block
-  const int64_t units = (int64_t)p.n_chunks * KB;
-  int64_t kpw = units / 2048;
-  if (kpw < 1) kpw = 1;
-  int64_t splits = ceil_div(KB, kpw * p.waves);
-  if (splits < 1) splits = 1;
-  // partial tiles cost 2 * splits * 16*tmx * 64 * 4 bytes per chunk against 64 * K weight bytes: keep
+  int64_t kpw, splits;
+  p.rg = kRowGroups;
+  p.staged = p.tmx <= 2 && KB >= 8;
+  if (p.staged) {
+    // Rows per chunk: the largest of 64 / 32 / 16 that still yields at least ~140 blocks, so that K is
+    // split across blocks only for very narrow weights (a split costs a round trip of partial tiles
+    // through memory: measured 6.1 us unsplit against 8.6 us split in two for N = 2112, K = 7168).
+    p.rg = 4;
+    while (p.rg > 1 && ceil_div(N, 16 * p.rg) < 140) p.rg >>= 1;
+    p.waves = (p.tmx == 2 && p.rg == 4) ? 4 : 8;
+  } else {
+    p.waves = p.tmx == 4 ? 4 : 8;  // LDS reduction buffer is 4 KB * tmx per wavefront
+  }
+  p.n_chunks = (int)ceil_div(N, 16 * p.rg);
+  if (p.n_chunks > FG_WORKSPACE_COUNTER_BYTES / 4) return p;
+  // partial tiles cost 2 * splits * 16*tmx * rows * 4 bytes per chunk against rows * K weight bytes: keep
   // them under a quarter of the weight traffic
   const int64_t max_splits = K / (32 * 16 * p.tmx) > 1 ? K / (32 * 16 * p.tmx) : 1;
-  if (splits > max_splits) splits = max_splits;
-  kpw = ceil_div(KB, splits * p.waves);  // even out
-  // a block with idle wavefronts wastes launch slots: fewer wavefronts when K is short
-  if (splits == 1 && KB <= 4) { p.waves = 4; kpw = ceil_div(KB, 4); }
+  if (p.staged) {
+    const int64_t pairs = (KB + 1) / 2;
+    splits = 1;
+    while (p.n_chunks * splits < 100 && splits * 2 <= max_splits && splits * 2 * p.waves <= pairs) splits *= 2;
+    kpw = ceil_div(pairs, splits * p.waves);
+  } else {
+    // aim for ~8 wavefronts per CU on 256 CUs, each with at least one K-block
+    const int64_t units = (int64_t)p.n_chunks * KB;
+    kpw = units / 2048;
+    if (kpw < 1) kpw = 1;
+    splits = ceil_div(KB, kpw * p.waves);
+    if (splits < 1) splits = 1;
+    if (splits > max_splits) splits = max_splits;
+    kpw = ceil_div(KB, splits * p.waves);  // even out
+    // a block with idle wavefronts wastes launch slots: fewer wavefronts when K is short
+    if (splits == 1 && KB <= 4) { p.waves = 4; kpw = ceil_div(KB, 4); }
+  }
   p.kpw = (int)kpw;
   p.splits = (int)splits;
   p.workspace_bytes = splits > 1
-      ? (size_t)FG_WORKSPACE_COUNTER_BYTES + (size_t)p.n_chunks * splits * 16 * p.tmx * kChunkRows * sizeof(float)
+      ? (size_t)FG_WORKSPACE_COUNTER_BYTES + (size_t)p.n_chunks * splits * 16 * p.tmx * 16 * p.rg * sizeof(float)
       : 0;
   p.use = true;
   return p;
@@ -257,6 +461,16 @@ int launch_small_m(const GemmArgs& g, int mode, const SmallMPlan& plan, void* wo
     if ((uintptr_t)workspace % 16 != 0) FG_FAIL(FG_ERR_INVALID_ARG, "fp8 gemm (small M): workspace must be 16-byte aligned");
     sa.counters = reinterpret_cast<unsigned int*>(workspace);
     sa.partials = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
+  }
+  if (plan.staged) {
+    if (plan.tmx == 1) {
+      if (plan.rg == 1) return launch_transpose<1, 1, 4, 8>(sa, mode, stream);
+      if (plan.rg == 2) return launch_transpose<1, 2, 3, 8>(sa, mode, stream);
+      return launch_transpose<1, 4, 2, 8>(sa, mode, stream);
+    }
+    if (plan.rg == 1) return launch_transpose<2, 1, 3, 8>(sa, mode, stream);
+    if (plan.rg == 2) return launch_transpose<2, 2, 2, 8>(sa, mode, stream);
+    return launch_transpose<2, 4, 2, 4>(sa, mode, stream);
   }
   if (plan.tmx == 1) return plan.waves == 8 ? launch_t<1, 8>(sa, mode, stream) : launch_t<1, 4>(sa, mode, stream);
   if (plan.tmx == 2) return plan.waves == 8 ? launch_t<2, 8>(sa, mode, stream) : launch_t<2, 4>(sa, mode, stream);
