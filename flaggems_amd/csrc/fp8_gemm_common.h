@@ -91,4 +91,10 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K);
 int launch_small_m(const GemmArgs& a, int mode, const SmallMPlan& plan, void* workspace, size_t workspace_bytes,
                    hipStream_t stream);
 
+
+// Persistent 256x256 kernel, fp8_gemm_pingpong.hip: block-scaled, bf16 output with 16-byte aligned rows, M > 128;
+// the caller has checked that the operands qualify for direct global->LDS loads.
+bool pingpong_takes(const GemmArgs& a, int mode);
+int launch_pingpong(const GemmArgs& a, int mode, hipStream_t stream);
+
 }  // namespace fg

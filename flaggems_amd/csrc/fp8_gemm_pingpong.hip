@@ -1,0 +1,509 @@
+// Persistent "ping-pong" FP8 GEMM for gfx950: 256 x 256 output tiles, 8 wavefronts per block, one block
+// per compute unit, block-scaled (1x128 activation scales, 128x128 weight scales) or row/column scaled.
+//
+// Why.  A compute unit has four SIMDs with one matrix pipe each, and a block of eight wavefronts puts two
+// wavefronts on every SIMD.  If both run the same program they leave a barrier together, queue their LDS
+// reads together and reach their MFMAs together, so the matrix pipe idles while operands are fetched and
+// is fought over afterwards.  Here the two wavefronts of a SIMD run the same program half a K-block
+// apart: while one executes its 32 MFMAs (operands already in registers, nothing else to wait for), the
+// other reads its operand fragments for the next K-block out of LDS, issues global->LDS loads and, at a
+// tile boundary, converts and stores its finished results.  Two block barriers per K-block hand the
+// roles over.  The matrix pipe sees an unbroken MFMA stream, and the epilogue of a tile costs nothing
+// because it runs under the partner's MFMAs.
+//
+// Slots.  Group A = wavefronts 0-3, group B = wavefronts 4-7 (one of each per SIMD).  With step T counting
+// K-blocks over all tiles a block processes:
+//     slot 2T   : A  fetch(T)     B  multiply(T-1)
+//     slot 2T+1 : A  multiply(T)  B  fetch(T)
+// A issues its share of the loads of stage T+1 at the start of fetch(T) and waits for them at the end of
+// multiply(T); B spreads its share of stage T+2 over multiply(T) and waits at the end of fetch(T+1).
+// Every load therefore has more than a whole slot to land, and every wait sits right before a barrier.
+//
+// LDS.  A stage is 256 x 128 weight bytes plus 256 x 128 activation bytes.  Activation fragments are all
+// read in the fetch phase (stage T: slots 2T and 2T+1), so two activation stages suffice for loads issued
+// from slot 2T+2 on.  Weight fragments are also read during the multiply phase (stage T: until the end of
+// slot 2T+2), so the weights get three stages.  3 x 32 KB + 2 x 32 KB = 160 KB.
+//
+// Operand roles and layouts are those of the tile kernel in fp8_gemm.hip (weights in the MFMA A slot,
+// XOR-permuted row-major LDS image filled by global_load_lds_dwordx4), with one change: the 128 weight
+// rows of a wavefront are dealt to the MFMA tiles so that a lane ends up with 32 *consecutive* output
+// columns (tile t, A-row i  <->  column (i >> 2) * 32 + 4 t + (i & 3)).  A lane then stores 64 contiguous
+// bytes of bf16 per output row and four lanes cover 256 contiguous bytes, instead of 8-byte pieces.
+//
+// Registers.  Two wavefronts per SIMD leave 256 registers each: 128 fp32 accumulators, the four activation
+// fragments of the K-block (32) and a ring of three weight fragments (24) that the multiply phase refills two
+// MFMA rows ahead of use.
+
+#include "fp8_gemm_common.h"
+
+#ifdef FG_PP_TRACE
+// development aid: per-slot timestamps of block 0, wavefronts 0 and 4
+__device__ unsigned long long fg_pp_trace_buf[2][64][8];
+#define FG_PP_STAMP(id)                                                                             \
+  do {                                                                                              \
+    if (blockIdx.x == 0 && (wave & 3) == 0 && lane == 0 && T < 64)                                  \
+      fg_pp_trace_buf[grp][T][id] = __builtin_readcyclecounter();                                   \
+  } while (0)
+extern "C" void fg_pp_trace_dump() {
+  static unsigned long long h[2][64][8];
+  hipMemcpyFromSymbol(h, HIP_SYMBOL(fg_pp_trace_buf), sizeof(h));
+  unsigned long long t0 = h[0][0][0];
+  for (int T = 0; T < 24; ++T)
+    for (int g = 0; g < 2; ++g) {
+      printf("T=%2d %c:", T, g ? 'B' : 'A');
+      for (int i = 0; i < 8; ++i) printf(" %8lld", (long long)(h[g][T][i] - t0));
+      printf("\n");
+    }
+}
+#else
+#define FG_PP_STAMP(id) do {} while (0)
+#endif
+
+namespace fg {
+namespace {
+
+constexpr int kBM = 256, kBN = 256;
+constexpr int kThreads = 512;
+constexpr int kWStageBytes = kBN * 128, kXStageBytes = kBM * 128;
+constexpr int kWStages = 3, kXStages = 2;  // see "LDS" in the header comment
+constexpr int kXRegion = kWStages * kWStageBytes;
+constexpr int kLdsBytes = kXRegion + kXStages * kXStageBytes;  // 160 KB, all of a compute unit's LDS
+constexpr int kTN = 8, kTM = 4;         // MFMA tiles per wavefront: 128 weight rows x 64 activation rows
+constexpr int kSlabsPerWave = 4;        // 1 KB global->LDS loads per wavefront, per operand, per stage
+
+struct PpArgs {
+  GemmArgs g;
+  int n_tiles;
+};
+
+// Same XCD-aware order as the tile kernel: ids congruent mod 8 (one XCD) walk a contiguous run of tiles,
+// four tile rows at a time.
+__device__ __forceinline__ void tile_of_index(int vid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  const int xcd = vid & 7, local = vid >> 3;
+  const int base = total >> 3, rem = total & 7;
+  const int sid = xcd * base + (xcd < rem ? xcd : rem) + local;
+  constexpr int GROUP_M = 4;
+  const int per_group = GROUP_M * tiles_n;
+  const int g = sid / per_group;
+  const int first_m = g * GROUP_M;
+  const int gm = (tiles_m - first_m < GROUP_M) ? tiles_m - first_m : GROUP_M;
+  const int r = sid - g * per_group;
+  tm = first_m + r % gm;
+  tn = r / gm;
+}
+
+// A block visits the virtual ids blockIdx.x, blockIdx.x + gridDim.x, ...  The grid is either the tile count
+// (one round) or the number of compute units, a multiple of 8, so a block stays on its XCD's run of tiles.
+// tile_of_index maps [0, n_tiles) onto the tiles one-to-one.
+__device__ __forceinline__ bool valid_vid(int vid, int n_tiles) { return vid < n_tiles; }
+
+// weight row (within the wavefront's 128) held by LDS row rho of the wavefront's region
+__device__ __forceinline__ int weight_row_of_lds_row(int rho) {
+  const int t = rho >> 4, i = rho & 15;
+  return (i >> 2) * 32 + t * 4 + (i & 3);
+}
+
+// Uniform (scalar) walk over the (tile, K-block) steps of this block, in processing order.  Three of these
+// run at different distances: the step being multiplied, the step whose scales are being fetched (one
+// ahead) and the stage being loaded (one or two ahead).  A tile change costs two integer divisions and
+// happens once per K / 128 steps; everything else per step is an add.
+struct Walk {
+  int vid, kb, m0, n0;
+  __device__ __forceinline__ void locate(const PpArgs& a) {
+    int tm = 0, tn = 0;
+    if (vid < a.n_tiles) tile_of_index(vid, a.g.tiles_m, a.g.tiles_n, tm, tn);
+    m0 = tm * kBM; n0 = tn * kBN;
+  }
+  __device__ __forceinline__ void start(const PpArgs& a) { vid = blockIdx.x; kb = 0; locate(a); }
+  // true when the walk entered a new tile
+  __device__ __forceinline__ bool next(const PpArgs& a) {
+    if (++kb < a.g.KB) return false;
+    kb = 0; vid += gridDim.x;
+    locate(a);
+    return true;
+  }
+};
+
+// This wavefront's share of the global->LDS loads of one stage: 4 slabs (1 KB, 8 LDS rows each) of the
+// weight tile and 4 of the activation tile.  Per-lane byte offsets are relative to the tile's first row.
+struct LoadShare {
+  uint32_t w_off[kSlabsPerWave], x_off[kSlabsPerWave];
+  const uint8_t* w_ptr;  // uniform: first row of the tile, K-block being loaded
+  const uint8_t* x_ptr;
+
+  __device__ __forceinline__ void set_tile(const GemmArgs& a, int m0, int n0, int wave, int lane) {
+    w_ptr = a.W + (int64_t)n0 * a.ldw;
+    x_ptr = a.X + (int64_t)m0 * a.ldx;
+    const int w_valid = a.N - n0, x_valid = a.M - m0;
+#pragma unroll
+    for (int j = 0; j < kSlabsPerWave; ++j) {
+      const int slab = wave + j * 8;
+      const int r = slab * 8 + (lane >> 3);  // LDS row
+      const uint32_t chunk = (uint32_t)(((lane & 7) ^ (r & 7)) << 4);
+      int wr = (r & 128) + weight_row_of_lds_row(r & 127);
+      wr = wr < w_valid ? wr : w_valid - 1;  // rows past the edge re-read the last row; never stored
+      const int xr = r < x_valid ? r : x_valid - 1;
+      w_off[j] = (uint32_t)wr * (uint32_t)a.ldw + chunk;
+      x_off[j] = (uint32_t)xr * (uint32_t)a.ldx + chunk;
+    }
+  }
+  // q in [0, 8): 0-3 weight slabs, 4-7 activation slabs
+  __device__ __forceinline__ void issue_one(uint8_t* w_stage, uint8_t* x_stage, int wave, int q) const {
+    const int j = q & 3;
+    const int slab = wave + j * 8;
+    if (q < 4) {
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(w_ptr + w_off[j]),
+                                       (__attribute__((address_space(3))) void*)(w_stage + slab * 1024), 16, 0, 0);
+    } else {
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(x_ptr + x_off[j]),
+                                       (__attribute__((address_space(3))) void*)(x_stage + slab * 1024), 16, 0, 0);
+    }
+  }
+};
+
+__device__ __forceinline__ int fragment_offset(int lane) {
+  const int r = lane & 15, g = lane >> 4;
+  return r * 128 + ((g ^ (r & 7)) << 4);
+}
+
+__device__ __forceinline__ v8i read_frag(const uint8_t* region, int rg, int lane_off) {
+  const u32x4 lo = *reinterpret_cast<const u32x4*>(region + rg * 2048 + lane_off);
+  const u32x4 hi = *reinterpret_cast<const u32x4*>(region + rg * 2048 + (lane_off ^ 64));
+  v8i f;
+  f[0] = (int)lo.x; f[1] = (int)lo.y; f[2] = (int)lo.z; f[3] = (int)lo.w;
+  f[4] = (int)hi.x; f[5] = (int)hi.y; f[6] = (int)hi.z; f[7] = (int)hi.w;
+  return f;
+}
+
+// MFMA with a zero accumulator input, result in architectural VGPRs
+__device__ __forceinline__ v4f mfma_partial(const v8i& w, const v8i& x) {
+  v4f p;
+  asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=&v"(p) : "v"(w), "v"(x));
+  return p;
+}
+
+// acc += p * s.  A wavefront issues one instruction every four cycles and the matrix pipe takes an MFMA of
+// this shape every 32, so a multiply step has eight issue slots: the MFMA, these four FMAs and three spare
+// (LDS reads, tile loads).  p is the result of the MFMA issued TWO steps earlier: at least 64 cycles have
+// passed since its issue, more than the 11 wait states (44 cycles) gfx950 requires between an 8-pass MFMA
+// write and a VALU read, so no s_nop is spent in the steady state.  NOPS > 0 pads the tail of the phase.
+template <int NOPS>
+__device__ __forceinline__ void scale_into(v4f& acc, const v4f& p, float s) {
+  float a0 = acc[0], a1 = acc[1], a2 = acc[2], a3 = acc[3];
+  if (NOPS > 0) {
+    asm volatile("s_nop %9\n\t"
+                 "v_fmac_f32 %0, %4, %8\n\t"
+                 "v_fmac_f32 %1, %5, %8\n\t"
+                 "v_fmac_f32 %2, %6, %8\n\t"
+                 "v_fmac_f32 %3, %7, %8"
+                 : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3)
+                 : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(s), "n"(NOPS - 1));
+  } else {
+    asm volatile("v_fmac_f32 %0, %4, %8\n\t"
+                 "v_fmac_f32 %1, %5, %8\n\t"
+                 "v_fmac_f32 %2, %6, %8\n\t"
+                 "v_fmac_f32 %3, %7, %8"
+                 : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3)
+                 : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(s));
+  }
+  acc[0] = a0; acc[1] = a1; acc[2] = a2; acc[3] = a3;
+}
+
+// Activation scales are fetched one step ahead with loads the compiler does not track, and picked up after an
+// explicit count.  Left to the compiler, the wait for these four values becomes vmcnt(0) in the middle of a
+// slot, which also waits for the tile loads issued after them.  The destination is an in/out operand so that
+// the value keeps one register across loop iterations.
+__device__ __forceinline__ void load_f32_untracked(float& v, uint32_t byte_off, const float* base) {
+  asm volatile("global_load_dword %0, %1, %2" : "+v"(v) : "v"(byte_off), "s"(base) : "memory");
+}
+// cur = nxt once at most PENDING younger vector-memory operations are outstanding
+template <int PENDING>
+__device__ __forceinline__ void wait_and_take(float (&cur)[kTM], const float (&nxt)[kTM]) {
+  static_assert(kTM == 4, "four activation fragments per wavefront");
+  asm volatile("s_waitcnt vmcnt(%8)\n\t"
+               "v_mov_b32 %0, %4\n\t"
+               "v_mov_b32 %1, %5\n\t"
+               "v_mov_b32 %2, %6\n\t"
+               "v_mov_b32 %3, %7"
+               : "=&v"(cur[0]), "=&v"(cur[1]), "=&v"(cur[2]), "=&v"(cur[3])
+               : "v"(nxt[0]), "v"(nxt[1]), "v"(nxt[2]), "v"(nxt[3]), "n"(PENDING)
+               : "memory");
+}
+template <int PENDING>
+__device__ __forceinline__ void wait_vmem() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PENDING) : "memory");
+}
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  const bf16x2_t h = __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, h);
+}
+
+// Stores the wavefront's 64 x 128 results as bf16.  Lane (l16, lg) holds, for every activation tile j, the
+// 32 consecutive columns n_base + lg * 32 + 4 t + v of row m_base + 16 j + l16.  The host guarantees
+// ldc % 8 == 0 and a 16-byte aligned C, so full runs leave as four 16-byte stores.
+__device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[kTN][kTM], int m_base, int n_base,
+                                           int l16, int lg) {
+  const int n = n_base + lg * 32;
+  const bool full = n + 32 <= a.N;
+#pragma unroll
+  for (int j = 0; j < kTM; ++j) {
+    const int m = m_base + j * 16 + l16;
+    if (m >= a.M) continue;
+    uint16_t* const cp = reinterpret_cast<uint16_t*>(a.C) + (int64_t)m * a.ldc + n;
+    uint32_t w[16];
+#pragma unroll
+    for (int t = 0; t < kTN; ++t) {
+      w[2 * t] = pack_bf16(acc[t][j][0], acc[t][j][1]);
+      w[2 * t + 1] = pack_bf16(acc[t][j][2], acc[t][j][3]);
+    }
+    if (full) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<u32x4*>(cp + q * 8) = u32x4{w[4 * q], w[4 * q + 1], w[4 * q + 2], w[4 * q + 3]};
+    } else {
+#pragma unroll
+      for (int e = 0; e < 32; ++e)
+        if (n + e < a.N) cp[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const GemmArgs& g = a.g;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = wave >> 2;       // 0: group A, 1: group B
+  const int wave_m = wave & 3;     // 64-row quarter of the activation tile
+  const int wm0 = wave_m * 64, wn0 = grp * 128;
+  const int l16 = lane & 15, lg = lane >> 4;
+  const int frag_off = fragment_offset(lane);
+
+  // steps of this block
+  const int my_tiles = (a.n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;  // grid <= n_tiles
+  const int total = my_tiles * g.KB;
+  if (total <= 0) return;  // uniform over the block
+
+  // ---- the stage being loaded
+  Walk lw;
+  lw.start(a);
+  LoadShare share;
+  share.set_tile(g, lw.m0, lw.n0, wave, lane);
+  int loaded = 0, w_slot = 0, x_slot = 0;  // stages issued by this wavefront; LDS slots of the next stage
+  auto issue_stage_part = [&](int q) {
+    share.issue_one(lds + w_slot * kWStageBytes, lds + kXRegion + x_slot * kXStageBytes, wave, q);
+  };
+  auto finish_stage = [&]() {
+    ++loaded;
+    w_slot = (w_slot + 1 == kWStages) ? 0 : w_slot + 1;
+    x_slot ^= 1;
+    if (lw.next(a)) {
+      if (lw.vid < a.n_tiles) share.set_tile(g, lw.m0, lw.n0, wave, lane);
+    } else {
+      share.w_ptr += 128;
+      share.x_ptr += 128;
+    }
+  };
+  auto issue_stage_all = [&]() {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) issue_stage_part(q);
+    finish_stage();
+  };
+
+  // ---- the step whose activation scales are being fetched: four rows per lane, 32-bit byte offsets from
+  // a uniform pointer that moves along K (the host checks that M * row stride fits)
+  Walk sw;
+  sw.start(a);
+  uint32_t xs_off[kTM];
+  const float* xs_ptr = g.xs;
+  auto set_scale_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < kTM; ++j) {
+      int m = sw.m0 + wm0 + j * 16 + l16;
+      m = m < g.M ? m : g.M - 1;
+      xs_off[j] = (uint32_t)m * (uint32_t)g.xs_rs * 4u;
+    }
+    xs_ptr = g.xs;
+  };
+  set_scale_tile();
+  float xs_nxt[kTM] = {0.f, 0.f, 0.f, 0.f};
+  auto request_scales = [&]() {
+#pragma unroll
+    for (int j = 0; j < kTM; ++j) load_f32_untracked(xs_nxt[j], xs_off[j], xs_ptr);
+  };
+
+  // ---- the step being multiplied; its weight-block scale is one scalar load per step
+  Walk cw;
+  cw.start(a);
+  const int nb_last = (g.N - 1) >> 7;
+  auto ws_row = [&]() -> const float* {
+    int nb = (cw.n0 + wn0) >> 7;
+    nb = nb < nb_last ? nb : nb_last;
+    return g.ws + (int64_t)nb * g.ws_rs;
+  };
+  const float* ws_ptr = ws_row();
+
+  // ---- prologue: A has stage 0 in flight, B stages 0 and 1; scales of step 0
+  issue_stage_all();
+  if (grp == 1 && total > 1) issue_stage_all();
+  request_scales();
+  wait_vmem_all();
+  __builtin_amdgcn_s_barrier();
+  if (grp == 1) __builtin_amdgcn_s_barrier();  // B runs one slot behind A
+  bool b_loaded_prev = false;  // B issued tile loads during its previous multiply
+
+  v4f acc[kTN][kTM];
+#pragma unroll
+  for (int t = 0; t < kTN; ++t)
+#pragma unroll
+    for (int j = 0; j < kTM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  // A finished tile is stored at the end of its wavefront's next fetch slot, under the partner's MFMAs.
+  bool pending = false;
+  int pend_m = 0, pend_n = 0;
+  auto flush_tile = [&]() {
+    store_tile(g, acc, pend_m, pend_n, l16, lg);
+    // (a second copy of the multiply phase that overwrites instead of accumulating makes the register
+    // allocator shuffle the accumulators through scratch at the join; zeroing costs 128 moves per tile)
+#pragma unroll
+    for (int t = 0; t < kTN; ++t)
+#pragma unroll
+      for (int j = 0; j < kTM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    pending = false;
+  };
+
+  int rw_slot = 0, rx_slot = 0;  // LDS slots of the stage being read
+  for (int T = 0; T < total; ++T) {
+    // ================= fetch(T)
+    // Scales of this step were requested a step ago.  Younger than them: for A nothing (it waited for
+    // everything at the end of its multiply), for B the eight tile loads of its previous multiply.
+    FG_PP_STAMP(0);
+    float xs[kTM], sc[kTM];
+    if (b_loaded_prev) wait_and_take<8>(xs, xs_nxt); else wait_and_take<0>(xs, xs_nxt);
+    const bool more = T + 1 < total;
+    if (more) {
+      if (sw.next(a)) set_scale_tile(); else xs_ptr += g.xs_cs;
+      request_scales();
+    }
+    FG_PP_STAMP(1);
+    const float ws = *(const __attribute__((address_space(4))) float*)ws_ptr;
+    const uint8_t* const tw = lds + rw_slot * kWStageBytes + (wn0 >> 4) * 2048;
+    const uint8_t* const tx = lds + kXRegion + rx_slot * kXStageBytes + (wm0 >> 4) * 2048;
+    // all activation fragments and the first two weight fragments; the other six follow during the
+    // multiply, each two MFMA rows before its use
+    v8i xf[kTM], wr[3];
+#pragma unroll
+    for (int j = 0; j < kTM; ++j) xf[j] = read_frag(tx, j, frag_off);
+    wr[0] = read_frag(tw, 0, frag_off);
+    wr[1] = read_frag(tw, 1, frag_off);
+    FG_PP_STAMP(2);
+    // after the LDS reads: the four wavefronts of A issue 32 KB of loads at once and stall in the issue
+    // while the address unit works through them
+    if (grp == 0 && loaded < total) issue_stage_all();  // stage T+1
+    FG_PP_STAMP(3);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): fragments are in registers
+    // B's share of stage T+1 (issued during multiply(T-1)) must have landed before the barrier; only the
+    // scale requests of this slot are younger.
+    if (grp == 1) {
+      if (more) wait_vmem<4>(); else wait_vmem<0>();
+    }
+#pragma unroll
+    for (int j = 0; j < kTM; ++j) sc[j] = xs[j] * ws;
+    FG_PP_STAMP(4);
+    if (pending) flush_tile();  // after the waits, so that no wait of this slot covers the stores
+    __builtin_amdgcn_s_barrier();
+    FG_PP_STAMP(5);
+
+    // ================= multiply(T)
+    const bool b_loads = grp == 1 && loaded < total;  // B: stage T+2, spread over the MFMA steps
+    __builtin_amdgcn_s_setprio(1);
+    {
+      v4f p[3];
+#pragma unroll
+      for (int st = 0; st < kTN * kTM; ++st) {
+        const int t = st / kTM, j = st % kTM;
+        p[st % 3] = mfma_partial(wr[t % 3], xf[j]);
+        // refill the ring after the row's first MFMA: the wait the compiler puts before that MFMA then
+        // covers only reads issued a whole row earlier
+        if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
+        if (st >= 2) scale_into<0>(acc[(st - 2) / kTM][(st - 2) % kTM], p[(st - 2) % 3], sc[(st - 2) % kTM]);
+        // B's tile loads go out in the first half of the phase so that they have landed by the end of its
+        // next fetch slot
+        if (st % 2 == 1 && st < 16 && b_loads) issue_stage_part(st / 2);
+      }
+      constexpr int L = kTN * kTM;
+      scale_into<0>(acc[(L - 2) / kTM][(L - 2) % kTM], p[(L - 2) % 3], sc[(L - 2) % kTM]);
+      scale_into<4>(acc[(L - 1) / kTM][(L - 1) % kTM], p[(L - 1) % 3], sc[(L - 1) % kTM]);
+    }
+    __builtin_amdgcn_s_setprio(0);
+    FG_PP_STAMP(6);
+    if (b_loads) finish_stage();
+    b_loaded_prev = b_loads;
+    if (grp == 0) wait_vmem_all();  // A's share of stage T+1 has landed
+    FG_PP_STAMP(7);
+    __builtin_amdgcn_s_barrier();
+
+    // ================= next step; a finished tile is stored in this wavefront's next fetch slot
+    rw_slot = (rw_slot + 1 == kWStages) ? 0 : rw_slot + 1;
+    rx_slot ^= 1;
+    pend_m = cw.m0 + wm0; pend_n = cw.n0 + wn0;
+    pending = cw.next(a);
+    if (pending) ws_ptr = ws_row(); else ws_ptr += g.ws_cs;
+  }
+  if (pending) flush_tile();
+  if (grp == 0) __builtin_amdgcn_s_barrier();  // pairs with B's extra barrier at the start
+}
+
+int cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+int launch_block(const GemmArgs& g, hipStream_t stream) {
+  PpArgs a;
+  a.g = g;
+  a.g.tiles_m = (int)ceil_div(g.M, kBM);
+  a.g.tiles_n = (int)ceil_div(g.N, kBN);
+  const int64_t tiles = (int64_t)a.g.tiles_m * a.g.tiles_n;
+  if (tiles > 0x3FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: too many tiles");
+  a.n_tiles = (int)tiles;
+  auto kern = fp8_gemm_pingpong_kernel;
+  static bool attr_set = false;  // benign if raced
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
+    attr_set = true;
+  }
+  int grid = cu_count();
+  if (tiles < grid) grid = (int)tiles;
+  hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
+  FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel");
+  return FG_OK;
+}
+
+}  // namespace
+
+bool pingpong_takes(const GemmArgs& g, int mode) {
+  // bf16 rows that take 16-byte stores; activation-scale offsets (bytes from the first row) that fit 32 bits
+  return mode == kModeBlock && g.M > 128 && g.c_dtype == FG_BF16 && g.ldc % 8 == 0 && (uintptr_t)g.C % 16 == 0 &&
+         g.xs_rs >= 0 && g.xs_cs >= 0 && g.ws_rs >= 0 && g.ws_cs >= 0 && (int64_t)g.M * g.xs_rs < (1ll << 29);
+}
+
+int launch_pingpong(const GemmArgs& g, int mode, hipStream_t stream) {
+  if (!pingpong_takes(g, mode)) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: persistent kernel does not take this problem");
+  return launch_block(g, stream);
+}
+
+}  // namespace fg

@@ -67,6 +67,28 @@ def test_quantized_linear_shapes_bf16(M, N, K):
     torch.testing.assert_close(got32.cpu(), want, rtol=1e-4, atol=2e-4)
 
 
+def test_persistent_kernel_several_rounds_ragged_edges_and_strides():
+    """M > 128 with 16-byte aligned rows takes the persistent 256x256 kernel: more tiles than compute units
+    (a block walks several tiles), M and N that end inside a tile (N not a multiple of 32 either),
+    column-major activation scales, a weight that is a row slice, and an output written through a view."""
+    M, N, K = 1100, 13400, 384  # 5 x 53 = 265 tiles
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=3)
+    want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
+    got = flag_gems.w8a8_block_fp8_matmul(xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    torch.testing.assert_close(got.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    # accumulate-level check against the float64 oracle: at most one bf16 rounding plus fp32 accumulation noise
+    err = (got.cpu().double() - want.double()).abs()
+    assert float((err / (want.double().abs() / 128 + 2e-3)).max()) < 1.0
+    s_cm = xs.t().contiguous().t().to(DEV)
+    big = torch.zeros(N + 77, K, dtype=FP8)
+    big[40:40 + N] = wq
+    got2 = flag_gems.w8a8_block_fp8_matmul(xq.to(DEV), big.to(DEV)[40:40 + N], s_cm, ws.to(DEV), [128, 128])
+    assert torch.equal(got2.view(torch.int16), got.view(torch.int16))
+    # the same problem twice gives the same bits
+    got3 = flag_gems.w8a8_block_fp8_matmul(xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    assert torch.equal(got3.view(torch.int16), got.view(torch.int16))
+
+
 def test_closed_forms():
     A, B, As, Bs = _ref_inputs(48, 384, 512, seed=3)
     # unit scales -> plain matmul, exact in fp32 for these magnitudes up to summation order
