@@ -449,7 +449,7 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
     if (plan.use) return launch_small_m(a, MODE, plan, workspace, workspace_bytes, stream);
   }
   const bool big = a.M > 128;
-  if (direct && pingpong_takes(a, MODE)) return launch_pingpong(a, MODE, stream);
+  if (direct && pingpong_takes(a, MODE)) return launch_pingpong(a, MODE, workspace, workspace_bytes, stream);
   if (big) {
     return direct ? launch_cfg<256, 256, 4, 2, MODE, true>(a, stream)
                   : launch_cfg<256, 256, 4, 2, MODE, false>(a, stream);
@@ -474,7 +474,8 @@ int check_common(const void* A, const void* B, const void* C, int64_t lda, int64
 
 extern "C" size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   const fg::SmallMPlan plan = fg::plan_small_m(M, N, K);
-  return plan.use ? plan.workspace_bytes : 0;
+  if (plan.use) return plan.workspace_bytes;
+  return fg::pingpong_workspace_bytes(M, N, K);
 }
 extern "C" size_t fg_scaled_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return fg_block_fp8_gemm_workspace_bytes(M, N, K);

@@ -74,7 +74,17 @@ constexpr int kSlabsPerWave = 4;        // 1 KB global->LDS loads per wavefront,
 struct PpArgs {
   GemmArgs g;
   int n_tiles;
+  // Stream-K (sk != 0): the n_tiles * KB steps, tile after tile, are cut into gridDim.x contiguous ranges of
+  // sk_q or sk_q + 1 steps (the first sk_r ranges get the extra step).  A tile that straddles ranges is
+  // finished through the workspace: fp32 partial tiles and one arrival counter per (range, wavefront).
+  int sk, sk_q, sk_r;
+  float* partials;
+  unsigned int* counters;
 };
+
+constexpr int kPartialFloatsPerWave = 64 * 128;                      // one wavefront's 64 x 128 results
+constexpr int kPartialFloatsPerSlot = 8 * kPartialFloatsPerWave;     // a whole 256 x 256 tile
+constexpr size_t kPartialSlotBytes = (size_t)kPartialFloatsPerSlot * 4;  // 256 KB
 
 // Same XCD-aware order as the tile kernel: ids congruent mod 8 (one XCD) walk a contiguous run of tiles,
 // four tile rows at a time.
@@ -83,6 +93,19 @@ __device__ __forceinline__ void tile_of_index(int vid, int tiles_m, int tiles_n,
   const int xcd = vid & 7, local = vid >> 3;
   const int base = total >> 3, rem = total & 7;
   const int sid = xcd * base + (xcd < rem ? xcd : rem) + local;
+  constexpr int GROUP_M = 4;
+  const int per_group = GROUP_M * tiles_n;
+  const int g = sid / per_group;
+  const int first_m = g * GROUP_M;
+  const int gm = (tiles_m - first_m < GROUP_M) ? tiles_m - first_m : GROUP_M;
+  const int r = sid - g * per_group;
+  tm = first_m + r % gm;
+  tn = r / gm;
+}
+
+// Stream-K order: consecutive tile numbers walk four tile rows before moving along N, so the ranges of
+// neighbouring blocks (which the launch places on one XCD) share operand panels.
+__device__ __forceinline__ void tile_of_sid(int sid, int tiles_m, int tiles_n, int& tm, int& tn) {
   constexpr int GROUP_M = 4;
   const int per_group = GROUP_M * tiles_n;
   const int g = sid / per_group;
@@ -109,17 +132,23 @@ __device__ __forceinline__ int weight_row_of_lds_row(int rho) {
 // ahead) and the stage being loaded (one or two ahead).  A tile change costs two integer divisions and
 // happens once per K / 128 steps; everything else per step is an add.
 struct Walk {
-  int vid, kb, m0, n0;
+  int idx, kb, m0, n0;  // idx: virtual id (data-parallel rounds) or tile number (stream-K)
   __device__ __forceinline__ void locate(const PpArgs& a) {
     int tm = 0, tn = 0;
-    if (vid < a.n_tiles) tile_of_index(vid, a.g.tiles_m, a.g.tiles_n, tm, tn);
+    if (idx < a.n_tiles) {
+      if (a.sk) tile_of_sid(idx, a.g.tiles_m, a.g.tiles_n, tm, tn);
+      else tile_of_index(idx, a.g.tiles_m, a.g.tiles_n, tm, tn);
+    }
     m0 = tm * kBM; n0 = tn * kBN;
   }
-  __device__ __forceinline__ void start(const PpArgs& a) { vid = blockIdx.x; kb = 0; locate(a); }
+  __device__ __forceinline__ void start(const PpArgs& a, int first_idx, int first_kb) {
+    idx = first_idx; kb = first_kb;
+    locate(a);
+  }
   // true when the walk entered a new tile
   __device__ __forceinline__ bool next(const PpArgs& a) {
     if (++kb < a.g.KB) return false;
-    kb = 0; vid += gridDim.x;
+    kb = 0; idx += a.sk ? 1 : (int)gridDim.x;
     locate(a);
     return true;
   }
@@ -214,6 +243,14 @@ __device__ __forceinline__ void scale_into(v4f& acc, const v4f& p, float s) {
 // explicit count.  Left to the compiler, the wait for these four values becomes vmcnt(0) in the middle of a
 // slot, which also waits for the tile loads issued after them.  The destination is an in/out operand so that
 // the value keeps one register across loop iterations.
+// The "s" operands below must be in scalar registers; the value is uniform, this makes the compiler see it.
+template <typename T>
+__device__ __forceinline__ T* uniform_ptr(T* p) {
+  const uint64_t v = (uint64_t)p;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return (T*)(((uint64_t)hi << 32) | lo);
+}
 __device__ __forceinline__ void load_f32_untracked(float& v, uint32_t byte_off, const float* base) {
   asm volatile("global_load_dword %0, %1, %2" : "+v"(v) : "v"(byte_off), "s"(base) : "memory");
 }
@@ -272,6 +309,106 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
   }
 }
 
+// 16-byte accesses that other XCDs can see: written through to memory / read past this XCD's L2 (the same
+// cache-control bit the compiler sets for agent-scope atomic loads and stores).  Not tracked by the
+// compiler's wait-count insertion: callers wait explicitly.
+__device__ __forceinline__ void store_x4_agent(float* base, uint32_t byte_off, const v4f& v) {
+  asm volatile("global_store_dwordx4 %0, %1, %2 sc1" : : "v"(byte_off), "v"(v), "s"(base) : "memory");
+}
+__device__ __forceinline__ void load_x4_agent(v4f& v, const float* base, uint32_t byte_off) {
+  asm volatile("global_load_dwordx4 %0, %1, %2 sc1" : "=v"(v) : "v"(byte_off), "s"(base) : "memory");
+}
+
+// Range arithmetic of the stream-K split (all uniform).
+__device__ __forceinline__ int sk_range_begin(const PpArgs& a, int pos) {
+  return pos * a.sk_q + (pos < a.sk_r ? pos : a.sk_r);
+}
+__device__ __forceinline__ int sk_range_of_step(const PpArgs& a, int step) {
+  const int big = a.sk_r * (a.sk_q + 1);
+  return step < big ? step / (a.sk_q + 1) : a.sk_r + (step - big) / a.sk_q;
+}
+
+// Finishes a tile that this block computed only part of.  Each wavefront handles its own 64 x 128 piece:
+// it publishes its partial sums, then counts itself in; the wavefront that arrives last (of the ranges that
+// share the tile) adds all partial sums in range order -- the same order whoever comes last, so the
+// result does not depend on timing -- stores the piece, and resets the counter for the next launch.
+// Nobody waits for anybody.  On entry and exit no vector-memory operation of this wavefront is pending.
+__device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (&acc)[kTN][kTM], int tile, int pos,
+                                                    int m_base, int n_base, int wave, int lane, int l16, int lg) {
+  const int s_lo = tile * a.g.KB;
+  const int first = sk_range_of_step(a, s_lo), last = sk_range_of_step(a, s_lo + a.g.KB - 1);
+  const int nseg = last - first + 1;
+  // a range owns two slots: [0] for the tile its range starts in, [1] for the tile it ends in when that is
+  // another one
+  auto slot_of = [&](int q) __attribute__((always_inline)) -> float* {
+    const int which = (sk_range_begin(a, q) >= s_lo) ? 0 : 1;
+    return a.partials + ((size_t)(q * 2 + which) * 8 + wave) * kPartialFloatsPerWave;
+  };
+  const uint32_t lane_off = (uint32_t)lane * 16u;
+  float* const mine = uniform_ptr(slot_of(pos));
+#pragma unroll
+  for (int t = 0; t < kTN; ++t)
+#pragma unroll
+    for (int j = 0; j < kTM; ++j) store_x4_agent(mine + (t * kTM + j) * 256, lane_off, acc[t][j]);
+  wait_vmem<0>();
+  unsigned int* const cnt = a.counters + first * 8 + wave;
+  unsigned int prev = 0;
+  if (lane == 0) prev = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  prev = (unsigned int)__builtin_amdgcn_readfirstlane((int)prev);
+  if (prev != (unsigned int)(nseg - 1)) return;
+  // Last to arrive.  Its own sums are in the workspace like everybody's, so the accumulators are free:
+  // half of the piece (16 columns per lane and row) is summed at a time, every range's loads in flight together
+  // with the running sum.
+  const int n = n_base + lg * 32;
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    v4f r[kTN / 2][kTM];
+    for (int q = first; q <= last; ++q) {
+      const float* const src = uniform_ptr(slot_of(q));
+      v4f tmp[kTN / 2][kTM];
+#pragma unroll
+      for (int t = 0; t < kTN / 2; ++t)
+#pragma unroll
+        for (int j = 0; j < kTM; ++j) load_x4_agent(tmp[t][j], src + ((half * (kTN / 2) + t) * kTM + j) * 256, lane_off);
+#pragma unroll
+      for (int t = 0; t < kTN / 2; ++t)  // the values are operands of the wait, so no use can move above it
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[t][0]), "+v"(tmp[t][1]), "+v"(tmp[t][2]), "+v"(tmp[t][3]) : : "memory");
+#pragma unroll
+      for (int t = 0; t < kTN / 2; ++t)
+#pragma unroll
+        for (int j = 0; j < kTM; ++j) {
+          // plain assignment for the first range keeps "0 + x" out of the sum
+          if (q == first) r[t][j] = tmp[t][j]; else r[t][j] += tmp[t][j];
+        }
+    }
+    // 16 consecutive columns per lane and row: two 16-byte stores, or single elements at the ragged edge
+    const int nh = n + half * 16;
+#pragma unroll
+    for (int j = 0; j < kTM; ++j) {
+      const int m = m_base + j * 16 + l16;
+      if (m >= a.g.M) continue;
+      uint16_t* const cp = reinterpret_cast<uint16_t*>(a.g.C) + (int64_t)m * a.g.ldc + nh;
+      uint32_t w[8];
+#pragma unroll
+      for (int t = 0; t < kTN / 2; ++t) {
+        w[2 * t] = pack_bf16(r[t][j][0], r[t][j][1]);
+        w[2 * t + 1] = pack_bf16(r[t][j][2], r[t][j][3]);
+      }
+      if (nh + 16 <= a.g.N) {
+        *reinterpret_cast<u32x4*>(cp) = u32x4{w[0], w[1], w[2], w[3]};
+        *reinterpret_cast<u32x4*>(cp + 8) = u32x4{w[4], w[5], w[6], w[7]};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          if (nh + e < a.g.N) cp[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+      }
+    }
+  }
+  if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the counted waits of the main loop start from zero
+}
+
+template <bool SK>
 __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const GemmArgs& g = a.g;
@@ -284,32 +421,44 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   const int l16 = lane & 15, lg = lane >> 4;
   const int frag_off = fragment_offset(lane);
 
-  // steps of this block
-  const int my_tiles = (a.n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;  // grid <= n_tiles
-  const int total = my_tiles * g.KB;
+  // steps of this block: whole tiles blockIdx.x, blockIdx.x + gridDim.x, ... or one contiguous range
+  int pos = (int)blockIdx.x, first_idx = (int)blockIdx.x, first_kb = 0, total;
+  if (SK) {
+    // ranges that are neighbours in the step order go to one XCD (block ids congruent mod 8)
+    if ((gridDim.x & 7) == 0) pos = (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3);
+    const int s0 = sk_range_begin(a, pos);
+    total = a.sk_q + (pos < a.sk_r ? 1 : 0);
+    first_idx = s0 / g.KB;
+    first_kb = s0 - first_idx * g.KB;
+  } else {
+    const int my_tiles = (a.n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;  // grid <= n_tiles
+    total = my_tiles * g.KB;
+  }
   if (total <= 0) return;  // uniform over the block
 
   // ---- the stage being loaded
   Walk lw;
-  lw.start(a);
+  lw.start(a, first_idx, first_kb);
   LoadShare share;
   share.set_tile(g, lw.m0, lw.n0, wave, lane);
+  share.w_ptr += (int64_t)first_kb * 128;
+  share.x_ptr += (int64_t)first_kb * 128;
   int loaded = 0, w_slot = 0, x_slot = 0;  // stages issued by this wavefront; LDS slots of the next stage
-  auto issue_stage_part = [&](int q) {
+  auto issue_stage_part = [&](int q) __attribute__((always_inline)) {
     share.issue_one(lds + w_slot * kWStageBytes, lds + kXRegion + x_slot * kXStageBytes, wave, q);
   };
-  auto finish_stage = [&]() {
+  auto finish_stage = [&]() __attribute__((always_inline)) {
     ++loaded;
     w_slot = (w_slot + 1 == kWStages) ? 0 : w_slot + 1;
     x_slot ^= 1;
     if (lw.next(a)) {
-      if (lw.vid < a.n_tiles) share.set_tile(g, lw.m0, lw.n0, wave, lane);
+      if (lw.idx < a.n_tiles) share.set_tile(g, lw.m0, lw.n0, wave, lane);
     } else {
       share.w_ptr += 128;
       share.x_ptr += 128;
     }
   };
-  auto issue_stage_all = [&]() {
+  auto issue_stage_all = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int q = 0; q < 8; ++q) issue_stage_part(q);
     finish_stage();
@@ -318,10 +467,10 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   // ---- the step whose activation scales are being fetched: four rows per lane, 32-bit byte offsets from
   // a uniform pointer that moves along K (the host checks that M * row stride fits)
   Walk sw;
-  sw.start(a);
+  sw.start(a, first_idx, first_kb);
   uint32_t xs_off[kTM];
   const float* xs_ptr = g.xs;
-  auto set_scale_tile = [&]() {
+  auto set_scale_tile = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < kTM; ++j) {
       int m = sw.m0 + wm0 + j * 16 + l16;
@@ -331,22 +480,24 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     xs_ptr = g.xs;
   };
   set_scale_tile();
+  xs_ptr += (int64_t)first_kb * g.xs_cs;
   float xs_nxt[kTM] = {0.f, 0.f, 0.f, 0.f};
-  auto request_scales = [&]() {
+  auto request_scales = [&]() __attribute__((always_inline)) {
+    const float* const base = uniform_ptr(xs_ptr);
 #pragma unroll
-    for (int j = 0; j < kTM; ++j) load_f32_untracked(xs_nxt[j], xs_off[j], xs_ptr);
+    for (int j = 0; j < kTM; ++j) load_f32_untracked(xs_nxt[j], xs_off[j], base);
   };
 
   // ---- the step being multiplied; its weight-block scale is one scalar load per step
   Walk cw;
-  cw.start(a);
+  cw.start(a, first_idx, first_kb);
   const int nb_last = (g.N - 1) >> 7;
-  auto ws_row = [&]() -> const float* {
+  auto ws_row = [&]() __attribute__((always_inline)) -> const float* {
     int nb = (cw.n0 + wn0) >> 7;
     nb = nb < nb_last ? nb : nb_last;
     return g.ws + (int64_t)nb * g.ws_rs;
   };
-  const float* ws_ptr = ws_row();
+  const float* ws_ptr = ws_row() + (int64_t)first_kb * g.ws_cs;
 
   // ---- prologue: A has stage 0 in flight, B stages 0 and 1; scales of step 0
   issue_stage_all();
@@ -364,10 +515,11 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     for (int j = 0; j < kTM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
   // A finished tile is stored at the end of its wavefront's next fetch slot, under the partner's MFMAs.
+  // A tile of which this block computed only some K-blocks (stream-K) goes through finish_partial_tile at
+  // the start of that slot instead: its waits may stall the pair for a few microseconds, twice per block.
   bool pending = false;
-  int pend_m = 0, pend_n = 0;
-  auto flush_tile = [&]() {
-    store_tile(g, acc, pend_m, pend_n, l16, lg);
+  int pend_m = 0, pend_n = 0, pend_idx = 0;
+  auto clear_acc = [&]() __attribute__((always_inline)) {
     // (a second copy of the multiply phase that overwrites instead of accumulating makes the register
     // allocator shuffle the accumulators through scratch at the join; zeroing costs 128 moves per tile)
 #pragma unroll
@@ -376,9 +528,19 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
       for (int j = 0; j < kTM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
     pending = false;
   };
+  auto flush_whole_tile = [&]() __attribute__((always_inline)) {
+    store_tile(g, acc, pend_m, pend_n, l16, lg);
+    clear_acc();
+  };
+  auto flush_partial_tile = [&]() __attribute__((always_inline)) {
+    wait_vmem<0>();
+    finish_partial_tile(a, acc, pend_idx, pos, pend_m, pend_n, wave, lane, l16, lg);
+    clear_acc();
+  };
 
   int rw_slot = 0, rx_slot = 0;  // LDS slots of the stage being read
-  for (int T = 0; T < total; ++T) {
+  auto run_steps = [&](int t_begin, int t_end) __attribute__((always_inline)) {
+  for (int T = t_begin; T < t_end; ++T) {
     // ================= fetch(T)
     // Scales of this step were requested a step ago.  Younger than them: for A nothing (it waited for
     // everything at the end of its multiply), for B the eight tile loads of its previous multiply.
@@ -415,7 +577,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
 #pragma unroll
     for (int j = 0; j < kTM; ++j) sc[j] = xs[j] * ws;
     FG_PP_STAMP(4);
-    if (pending) flush_tile();  // after the waits, so that no wait of this slot covers the stores
+    if (pending) flush_whole_tile();  // after the waits, so that no wait of this slot covers the stores
     __builtin_amdgcn_s_barrier();
     FG_PP_STAMP(5);
 
@@ -451,11 +613,33 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     // ================= next step; a finished tile is stored in this wavefront's next fetch slot
     rw_slot = (rw_slot + 1 == kWStages) ? 0 : rw_slot + 1;
     rx_slot ^= 1;
-    pend_m = cw.m0 + wm0; pend_n = cw.n0 + wn0;
+    pend_m = cw.m0 + wm0; pend_n = cw.n0 + wn0; pend_idx = cw.idx;
     pending = cw.next(a);
     if (pending) ws_ptr = ws_row(); else ws_ptr += g.ws_cs;
   }
-  if (pending) flush_tile();
+  };
+
+  if (SK) {
+    // A range is [part of a tile] [whole tiles] [part of a tile]; the hot loop runs once for each piece and
+    // the partial pieces are finished between the runs, outside any loop.
+    const int n_head = first_kb != 0 ? (total < g.KB - first_kb ? total : g.KB - first_kb) : 0;
+    const int n_whole = (total - n_head) / g.KB * g.KB;
+    if (n_head > 0) {
+      run_steps(0, n_head);
+      flush_partial_tile();
+      b_loaded_prev = false;  // everything this wavefront had in flight has been waited for
+    }
+    run_steps(n_head, n_head + n_whole);
+    if (n_head + n_whole < total) {
+      run_steps(n_head + n_whole, total);  // (stores the last whole tile in its first fetch slot)
+      flush_partial_tile();
+    } else if (pending) {
+      flush_whole_tile();
+    }
+  } else {
+    run_steps(0, total);
+    if (pending) flush_whole_tile();
+  }
   if (grp == 0) __builtin_amdgcn_s_barrier();  // pairs with B's extra barrier at the start
 }
 
@@ -471,24 +655,62 @@ int cu_count() {
   return cached[dev];
 }
 
-int launch_block(const GemmArgs& g, hipStream_t stream) {
-  PpArgs a;
+// Stream-K pays when whole-tile rounds leave compute units idle: `steps` K-blocks per block either way.
+struct SkPlan {
+  bool use;
+  int grid, q, r;
+};
+SkPlan plan_stream_k(int64_t tiles, int KB, int cus) {
+  SkPlan p = {false, 0, 0, 0};
+  const int64_t total = tiles * KB;
+  if (cus < 8 || total < cus || total > 0x7FFFFFFF) return p;
+  const int64_t dp_grid = tiles < cus ? tiles : cus;
+  const int64_t dp_steps = ceil_div(tiles, dp_grid) * KB;
+  const int64_t q = total / cus;
+  // Measured on DeepSeek-V3 shapes: finishing the shared tiles (publish, count, read back past the L2) adds
+  // about as much time as 25 K-blocks to a launch, and ranges that start at different K offsets stop sharing
+  // operand panels in their XCD's L2.  Stream-K is chosen when it saves more steps than that.  A tile shared by
+  // more than 8 ranges would make its last wavefront read too many partial tiles.
+  const int64_t sk_steps = ceil_div(total, cus) + 25;
+  if (sk_steps >= dp_steps || q * 8 < KB) return p;
+  p.use = true;
+  p.grid = cus;
+  p.q = (int)q;
+  p.r = (int)(total % cus);
+  return p;
+}
+
+int launch_block(const GemmArgs& g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  PpArgs a = {};
   a.g = g;
   a.g.tiles_m = (int)ceil_div(g.M, kBM);
   a.g.tiles_n = (int)ceil_div(g.N, kBN);
   const int64_t tiles = (int64_t)a.g.tiles_m * a.g.tiles_n;
   if (tiles > 0x3FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: too many tiles");
   a.n_tiles = (int)tiles;
-  auto kern = fp8_gemm_pingpong_kernel;
   static bool attr_set = false;  // benign if raced
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-    if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
+    for (const void* k : {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false>),
+                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true>)}) {
+      hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+      if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
+    }
     attr_set = true;
   }
-  int grid = cu_count();
-  if (tiles < grid) grid = (int)tiles;
-  hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
+  const int cus = cu_count();
+  int grid = tiles < cus ? (int)tiles : cus;
+  // Stream-K is an optimisation the workspace enables: without one (or with a small one) whole tiles go round-robin.
+  const SkPlan sk = plan_stream_k(tiles, g.KB, cus);
+  const size_t need = FG_WORKSPACE_COUNTER_BYTES + (size_t)sk.grid * 2 * kPartialSlotBytes;
+  if (sk.use && workspace != nullptr && workspace_bytes >= need && (size_t)sk.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
+      (uintptr_t)workspace % 16 == 0) {
+    a.sk = 1; a.sk_q = sk.q; a.sk_r = sk.r;
+    a.counters = reinterpret_cast<unsigned int*>(workspace);
+    a.partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
+    grid = sk.grid;
+  }
+  if (a.sk) hipLaunchKernelGGL(fp8_gemm_pingpong_kernel<true>, dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
+  else hipLaunchKernelGGL(fp8_gemm_pingpong_kernel<false>, dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
   FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel");
   return FG_OK;
 }
@@ -501,9 +723,15 @@ bool pingpong_takes(const GemmArgs& g, int mode) {
          g.xs_rs >= 0 && g.xs_cs >= 0 && g.ws_rs >= 0 && g.ws_cs >= 0 && (int64_t)g.M * g.xs_rs < (1ll << 29);
 }
 
-int launch_pingpong(const GemmArgs& g, int mode, hipStream_t stream) {
+size_t pingpong_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 128 || K <= 0 || K % 128 != 0) return 0;
+  const SkPlan sk = plan_stream_k(ceil_div(M, kBM) * ceil_div(N, kBN), (int)(K / 128), cu_count());
+  return sk.use ? FG_WORKSPACE_COUNTER_BYTES + (size_t)sk.grid * 2 * kPartialSlotBytes : 0;
+}
+
+int launch_pingpong(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   if (!pingpong_takes(g, mode)) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: persistent kernel does not take this problem");
-  return launch_block(g, stream);
+  return launch_block(g, workspace, workspace_bytes, stream);
 }
 
 }  // namespace fg

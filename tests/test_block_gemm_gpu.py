@@ -89,6 +89,27 @@ def test_persistent_kernel_several_rounds_ragged_edges_and_strides():
     assert torch.equal(got3.view(torch.int16), got.view(torch.int16))
 
 
+def test_tiles_split_along_k_between_blocks():
+    """40 tiles of 32 K-blocks on a 256-unit GPU: the persistent kernel cuts the 1280 steps into contiguous
+    ranges, so every tile is computed by several blocks and finished through the workspace.  Ragged M and N,
+    results against the oracle, and bit-identical on a second run (partial sums are added in a fixed order)."""
+    M, N, K = 1200, 2000, 4096
+    from flaggems_amd import _lib
+    lib = _lib.load()
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=11)
+    want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
+    args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    got = flag_gems.w8a8_block_fp8_matmul(*args)
+    torch.testing.assert_close(got.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    err = (got.cpu().double() - want.double()).abs()
+    assert float((err / (want.double().abs() / 128 + 2e-3)).max()) < 1.0
+    for _ in range(3):
+        again = flag_gems.w8a8_block_fp8_matmul(*args)
+        assert torch.equal(again.view(torch.int16), got.view(torch.int16))
+    # the shape is one the library wants a workspace for
+    assert lib.fg_block_fp8_gemm_workspace_bytes(M, N, K) > 16384
+
+
 def test_closed_forms():
     A, B, As, Bs = _ref_inputs(48, 384, 512, seed=3)
     # unit scales -> plain matmul, exact in fp32 for these magnitudes up to summation order
