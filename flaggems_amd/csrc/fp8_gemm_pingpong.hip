@@ -667,11 +667,11 @@ SkPlan plan_stream_k(int64_t tiles, int KB, int cus) {
   const int64_t dp_grid = tiles < cus ? tiles : cus;
   const int64_t dp_steps = ceil_div(tiles, dp_grid) * KB;
   const int64_t q = total / cus;
-  // Measured on DeepSeek-V3 shapes: finishing the shared tiles (publish, count, read back past the L2) adds
-  // about as much time as 25 K-blocks to a launch, and ranges that start at different K offsets stop sharing
-  // operand panels in their XCD's L2.  Stream-K is chosen when it saves more steps than that.  A tile shared by
-  // more than 8 ranges would make its last wavefront read too many partial tiles.
-  const int64_t sk_steps = ceil_div(total, cus) + 25;
+  // Measured on DeepSeek-V3 shapes: ranges that start at different K offsets stop sharing operand panels in
+  // their XCD's L2, which makes a K-block about 1.3 times as expensive, and finishing the shared tiles adds
+  // about as much as 14 K-blocks to a launch.  Stream-K is chosen when it still comes out ahead.  A tile
+  // shared by more than 8 ranges would make its last wavefront read too many partial tiles.
+  const int64_t sk_steps = ceil_div(total, cus) * 13 / 10 + 14;
   if (sk_steps >= dp_steps || q * 8 < KB) return p;
   p.use = true;
   p.grid = cus;
