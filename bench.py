@@ -201,7 +201,7 @@ def main():
                 "flops_per_launch": big_flops / len(big), "algorithmic_bytes_per_launch":
                     sum(gemm_bytes(d["M"], d["N"], d["K"]) for d in big) / len(big),
                 "avg_launch_us": round(big_time * 1e6 / len(big), 2),
-                "kernel": "fp8_gemm_kernel<256,256,4,2,block,direct>, the six M=4096 launches of the sweep"}
+                "kernel": "fp8_gemm_pingpong_kernel, the six M=4096 launches of the sweep"}
     small = [d for d in detail if d["M"] <= 8]
     small_bytes = sum(gemm_bytes(d["M"], d["N"], d["K"]) for d in small)
     small_time = sum(d["us"] for d in small) * 1e-6

@@ -106,8 +106,17 @@ def test_tiles_split_along_k_between_blocks():
     for _ in range(3):
         again = flag_gems.w8a8_block_fp8_matmul(*args)
         assert torch.equal(again.view(torch.int16), got.view(torch.int16))
-    # the shape is one the library wants a workspace for
+    # the shape is one the library wants a workspace for; without one (C ABI called directly) whole tiles
+    # go to the blocks and the result differs at most by fp32 summation order
     assert lib.fg_block_fp8_gemm_workspace_bytes(M, N, K) > 16384
+    a, b, s_a, s_b = args[:4]
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    rc = lib.fg_block_fp8_gemm(a.data_ptr(), K, b.data_ptr(), K, s_a.data_ptr(), s_a.stride(0), s_a.stride(1),
+                               s_b.data_ptr(), s_b.stride(0), s_b.stride(1), c.data_ptr(), N, _lib.DTYPE_CODE[torch.bfloat16],
+                               M, N, K, 128, 128, None, 0, _lib.current_stream_ptr(torch.device(DEV)))
+    assert rc == 0
+    torch.testing.assert_close(c.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(c.float(), got.float(), rtol=8e-3, atol=1e-3)
 
 
 def test_closed_forms():
