@@ -212,6 +212,10 @@ __device__ __forceinline__ v4f mfma_partial(const v8i& w, const v8i& x) {
   return p;
 }
 
+__device__ __forceinline__ void mfma_accumulate(v4f& c, const v8i& w, const v8i& x) {
+  asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(c) : "v"(w), "v"(x));
+}
+
 // acc += p * s.  A wavefront issues one instruction every four cycles and the matrix pipe takes an MFMA of
 // this shape every 32, so a multiply step has eight issue slots: the MFMA, these four FMAs and three spare
 // (LDS reads, tile loads).  p is the result of the MFMA issued TWO steps earlier: at least 64 cycles have
@@ -282,10 +286,52 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 // Stores the wavefront's 64 x 128 results as bf16.  Lane (l16, lg) holds, for every activation tile j, the
 // 32 consecutive columns n_base + lg * 32 + 4 t + v of row m_base + 16 j + l16.  The host guarantees
 // ldc % 8 == 0 and a 16-byte aligned C, so full runs leave as four 16-byte stores.
+// Row/column mode: the sums are scaled by a_scale[m] * b_scale[n] first, and the bias is added to the rounded
+// value, in bf16, as the reference's epilogue does (src/flag_gems/fused/cutlass_scaled_mm.py:288-305).
+template <int MODE>
 __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[kTN][kTM], int m_base, int n_base,
                                            int l16, int lg) {
   const int n = n_base + lg * 32;
   const bool full = n + 32 <= a.N;
+  if (MODE == kModeRowCol) {
+    // eight columns at a time, so that only eight column scales and bias values are live
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      float sb[8], bias[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int ne = n + q * 8 + e < a.N ? n + q * 8 + e : a.N - 1;
+        sb[e] = a.ws[a.ws_per_col ? ne : 0];
+        bias[e] = a.bias ? load_as_float(a.bias, ne, a.bias_dtype) : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < kTM; ++j) {
+        const int m = m_base + j * 16 + l16;
+        if (m >= a.M) continue;
+        const float sa = a.xs[a.xs_per_row ? m : 0];
+        uint32_t w[4];
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {  // two columns per word
+          const int t = 2 * q + (h >> 1), e0 = (h & 1) * 2;
+          const float v0 = (acc[t][j][e0] * sa) * sb[4 * (h >> 1) + e0];
+          const float v1 = (acc[t][j][e0 + 1] * sa) * sb[4 * (h >> 1) + e0 + 1];
+          w[h] = pack_bf16(v0, v1);
+          if (a.bias)
+            w[h] = pack_bf16(bits_to_float(w[h] << 16) + bias[4 * (h >> 1) + e0],
+                             bits_to_float(w[h] & 0xFFFF0000u) + bias[4 * (h >> 1) + e0 + 1]);
+        }
+        uint16_t* const cp = reinterpret_cast<uint16_t*>(a.C) + (int64_t)m * a.ldc + n + q * 8;
+        if (full) {
+          *reinterpret_cast<u32x4*>(cp) = u32x4{w[0], w[1], w[2], w[3]};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n + q * 8 + e < a.N) cp[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < kTM; ++j) {
     const int m = m_base + j * 16 + l16;
@@ -408,7 +454,7 @@ __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the counted waits of the main loop start from zero
 }
 
-template <bool SK>
+template <bool SK, int MODE>
 __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const GemmArgs& g = a.g;
@@ -479,10 +525,13 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     }
     xs_ptr = g.xs;
   };
-  set_scale_tile();
-  xs_ptr += (int64_t)first_kb * g.xs_cs;
+  if (MODE == kModeBlock) {
+    set_scale_tile();
+    xs_ptr += (int64_t)first_kb * g.xs_cs;
+  }
   float xs_nxt[kTM] = {0.f, 0.f, 0.f, 0.f};
   auto request_scales = [&]() __attribute__((always_inline)) {
+    if (MODE != kModeBlock) return;
     const float* const base = uniform_ptr(xs_ptr);
 #pragma unroll
     for (int j = 0; j < kTM; ++j) load_f32_untracked(xs_nxt[j], xs_off[j], base);
@@ -497,7 +546,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     nb = nb < nb_last ? nb : nb_last;
     return g.ws + (int64_t)nb * g.ws_rs;
   };
-  const float* ws_ptr = ws_row() + (int64_t)first_kb * g.ws_cs;
+  const float* ws_ptr = MODE == kModeBlock ? ws_row() + (int64_t)first_kb * g.ws_cs : nullptr;
 
   // ---- prologue: A has stage 0 in flight, B stages 0 and 1; scales of step 0
   issue_stage_all();
@@ -529,7 +578,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     pending = false;
   };
   auto flush_whole_tile = [&]() __attribute__((always_inline)) {
-    store_tile(g, acc, pend_m, pend_n, l16, lg);
+    store_tile<MODE>(g, acc, pend_m, pend_n, l16, lg);
     clear_acc();
   };
   auto flush_partial_tile = [&]() __attribute__((always_inline)) {
@@ -546,14 +595,17 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     // everything at the end of its multiply), for B the eight tile loads of its previous multiply.
     FG_PP_STAMP(0);
     float xs[kTM], sc[kTM];
-    if (b_loaded_prev) wait_and_take<8>(xs, xs_nxt); else wait_and_take<0>(xs, xs_nxt);
     const bool more = T + 1 < total;
-    if (more) {
-      if (sw.next(a)) set_scale_tile(); else xs_ptr += g.xs_cs;
-      request_scales();
+    float ws = 1.f;
+    if (MODE == kModeBlock) {
+      if (b_loaded_prev) wait_and_take<8>(xs, xs_nxt); else wait_and_take<0>(xs, xs_nxt);
+      if (more) {
+        if (sw.next(a)) set_scale_tile(); else xs_ptr += g.xs_cs;
+        request_scales();
+      }
+      ws = *(const __attribute__((address_space(4))) float*)ws_ptr;
     }
     FG_PP_STAMP(1);
-    const float ws = *(const __attribute__((address_space(4))) float*)ws_ptr;
     const uint8_t* const tw = lds + rw_slot * kWStageBytes + (wn0 >> 4) * 2048;
     const uint8_t* const tx = lds + kXRegion + rx_slot * kXStageBytes + (wm0 >> 4) * 2048;
     // all activation fragments and the first two weight fragments; the other six follow during the
@@ -572,10 +624,12 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     // B's share of stage T+1 (issued during multiply(T-1)) must have landed before the barrier; only the
     // scale requests of this slot are younger.
     if (grp == 1) {
-      if (more) wait_vmem<4>(); else wait_vmem<0>();
+      if (more && MODE == kModeBlock) wait_vmem<4>(); else wait_vmem<0>();
     }
+    if (MODE == kModeBlock) {
 #pragma unroll
-    for (int j = 0; j < kTM; ++j) sc[j] = xs[j] * ws;
+      for (int j = 0; j < kTM; ++j) sc[j] = xs[j] * ws;
+    }
     FG_PP_STAMP(4);
     if (pending) flush_whole_tile();  // after the waits, so that no wait of this slot covers the stores
     __builtin_amdgcn_s_barrier();
@@ -584,7 +638,16 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     // ================= multiply(T)
     const bool b_loads = grp == 1 && loaded < total;  // B: stage T+2, spread over the MFMA steps
     __builtin_amdgcn_s_setprio(1);
-    {
+    if (MODE != kModeBlock) {
+      // row/column mode: the matrix pipe accumulates; scales and bias wait for the epilogue
+#pragma unroll
+      for (int st = 0; st < kTN * kTM; ++st) {
+        const int t = st / kTM, j = st % kTM;
+        mfma_accumulate(acc[t][j], wr[t % 3], xf[j]);
+        if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
+        if (st % 2 == 1 && st < 16 && b_loads) issue_stage_part(st / 2);
+      }
+    } else {
       v4f p[3];
 #pragma unroll
       for (int st = 0; st < kTN * kTM; ++st) {
@@ -615,7 +678,9 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     rx_slot ^= 1;
     pend_m = cw.m0 + wm0; pend_n = cw.n0 + wn0; pend_idx = cw.idx;
     pending = cw.next(a);
-    if (pending) ws_ptr = ws_row(); else ws_ptr += g.ws_cs;
+    if (MODE == kModeBlock) {
+      if (pending) ws_ptr = ws_row(); else ws_ptr += g.ws_cs;
+    }
   }
   };
 
@@ -680,7 +745,7 @@ SkPlan plan_stream_k(int64_t tiles, int KB, int cus) {
   return p;
 }
 
-int launch_block(const GemmArgs& g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   PpArgs a = {};
   a.g = g;
   a.g.tiles_m = (int)ceil_div(g.M, kBM);
@@ -690,8 +755,9 @@ int launch_block(const GemmArgs& g, void* workspace, size_t workspace_bytes, hip
   a.n_tiles = (int)tiles;
   static bool attr_set = false;  // benign if raced
   if (!attr_set) {
-    for (const void* k : {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false>),
-                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true>)}) {
+    for (const void* k : {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock>),
+                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock>),
+                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol>)}) {
       hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
       if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
     }
@@ -702,15 +768,19 @@ int launch_block(const GemmArgs& g, void* workspace, size_t workspace_bytes, hip
   // Stream-K is an optimisation the workspace enables: without one (or with a small one) whole tiles go round-robin.
   const SkPlan sk = plan_stream_k(tiles, g.KB, cus);
   const size_t need = FG_WORKSPACE_COUNTER_BYTES + (size_t)sk.grid * 2 * kPartialSlotBytes;
-  if (sk.use && workspace != nullptr && workspace_bytes >= need && (size_t)sk.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
+  if (mode == kModeBlock && sk.use && workspace != nullptr && workspace_bytes >= need && (size_t)sk.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
       (uintptr_t)workspace % 16 == 0) {
     a.sk = 1; a.sk_q = sk.q; a.sk_r = sk.r;
     a.counters = reinterpret_cast<unsigned int*>(workspace);
     a.partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
     grid = sk.grid;
   }
-  if (a.sk) hipLaunchKernelGGL(fp8_gemm_pingpong_kernel<true>, dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
-  else hipLaunchKernelGGL(fp8_gemm_pingpong_kernel<false>, dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
+  if (mode != kModeBlock)
+    hipLaunchKernelGGL((fp8_gemm_pingpong_kernel<false, kModeRowCol>), dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
+  else if (a.sk)
+    hipLaunchKernelGGL((fp8_gemm_pingpong_kernel<true, kModeBlock>), dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
+  else
+    hipLaunchKernelGGL((fp8_gemm_pingpong_kernel<false, kModeBlock>), dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
   FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel");
   return FG_OK;
 }
@@ -719,8 +789,9 @@ int launch_block(const GemmArgs& g, void* workspace, size_t workspace_bytes, hip
 
 bool pingpong_takes(const GemmArgs& g, int mode) {
   // bf16 rows that take 16-byte stores; activation-scale offsets (bytes from the first row) that fit 32 bits
-  return mode == kModeBlock && g.M > 128 && g.c_dtype == FG_BF16 && g.ldc % 8 == 0 && (uintptr_t)g.C % 16 == 0 &&
-         g.xs_rs >= 0 && g.xs_cs >= 0 && g.ws_rs >= 0 && g.ws_cs >= 0 && (int64_t)g.M * g.xs_rs < (1ll << 29);
+  if (!(g.M > 128 && g.c_dtype == FG_BF16 && g.ldc % 8 == 0 && (uintptr_t)g.C % 16 == 0)) return false;
+  if (mode != kModeBlock) return true;
+  return g.xs_rs >= 0 && g.xs_cs >= 0 && g.ws_rs >= 0 && g.ws_cs >= 0 && (int64_t)g.M * g.xs_rs < (1ll << 29);
 }
 
 size_t pingpong_workspace_bytes(int64_t M, int64_t N, int64_t K) {
@@ -731,7 +802,7 @@ size_t pingpong_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 
 int launch_pingpong(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   if (!pingpong_takes(g, mode)) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: persistent kernel does not take this problem");
-  return launch_block(g, workspace, workspace_bytes, stream);
+  return launch_block(g, mode, workspace, workspace_bytes, stream);
 }
 
 }  // namespace fg
