@@ -16,6 +16,10 @@ Prints ONE JSON line with the driver's fields plus
   cpu_baseline  the CPU oracle (torch restatement of the reference's torch implementation) timed on
                 the host cores on a bounded sample of the same sweep
   detail        per-(M, N, K) time, TFLOP/s, GB/s and roofline fractions (MFMA for M >= 512, HBM below)
+  cutlass_scaled_mm_n8192_k8192_bias, llama3_8b_linears
+                the other configurations of the path (per-token x per-channel scaled GEMM with bias; Llama-3-8B
+                linears as GEMM alone and as act_quant + GEMM), graph replays of one shape at a time with ONE copy
+                of the weights (small-M figures there may be served by the 256 MB Infinity Cache), not part of `value`
 """
 from __future__ import annotations
 
@@ -224,6 +228,65 @@ def main():
     q_gbs = 3.03125 * 4096 * 7168 / (q_us * 1e-6) / 1e9
     quant = {"shape": [4096, 7168], "us": round(q_us, 2), "gbps": round(q_gbs, 1), "frac_hbm": round(q_gbs / PEAK_HBM_GBPS, 4)}
 
+    # ---- the other configurations of the path, each shape timed alone: HIP events around the replay of a graph
+    # of `reps` launches (as above: decode-sized launches are shorter than a Python call)
+    def time_eager(fn, reps):
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                fn()
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr, stream=side):
+                for _ in range(reps):
+                    fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(3):
+            s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s_.record()
+            gr.replay()
+            e_.record()
+            e_.synchronize()
+            ts.append(s_.elapsed_time(e_) * 1e3 / reps)
+        del gr
+        return sorted(ts)[1]
+
+    # cutlass_scaled_mm semantics (BASELINE configs[3]): per-token x per-channel scales, bf16 bias, N = K = 8192
+    scaled = []
+    nk = 8192
+    b_src = torch.randn(nk, nk, device=dev, generator=gen)
+    b_s = (b_src.abs().amax(dim=1) / 448.0).contiguous()
+    b_q = (b_src / b_s[:, None]).to(torch.float8_e4m3fn)
+    del b_src
+    bias = torch.randn(nk, device=dev, generator=gen).bfloat16()
+    for m in (1, 32, 256, 2048, 8192):
+        a_src = torch.randn(m, nk, device=dev, generator=gen)
+        a_s = (a_src.abs().amax(dim=1, keepdim=True) / 448.0).contiguous()
+        a_q = (a_src / a_s).to(torch.float8_e4m3fn)
+        c = torch.empty(m, nk, dtype=torch.bfloat16, device=dev)
+        us = time_eager(lambda: flag_gems.cutlass_scaled_mm(c, a_q, b_q.t(), a_s, b_s.view(1, nk), bias), 10 if m >= 2048 else 30)
+        nbytes = m * nk + nk * nk + 4 * m + 4 * nk + 2 * m * nk + 2 * nk
+        scaled.append({"M": m, "N": nk, "K": nk, "us": round(us, 2), "tflops": round(gemm_flops(m, nk, nk) / us / 1e6, 1),
+                       "gbps": round(nbytes / us / 1e3, 1)})
+    del b_q, a_q, c
+
+    # Llama-3-8B linears (BASELINE configs[1]): GEMM alone and act_quant + GEMM from bf16 activations
+    llama = []
+    for (n, k) in [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]:
+        wq, ws = make_weight(n, k, gen, dev)
+        for m in (1, 16, 128, 1024, 4096):
+            x = torch.randn(m, k, device=dev, generator=gen).bfloat16()
+            xq, xs = flag_gems.act_quant_triton(x, 128)
+            reps = 10 if m >= 1024 else 30
+            us_g = time_eager(lambda: flag_gems.w8a8_block_fp8_matmul(xq, wq, xs, ws, [128, 128]), reps)
+            def e2e():
+                q, s2 = flag_gems.act_quant_triton(x, 128)
+                return flag_gems.w8a8_block_fp8_matmul(q, wq, s2, ws, [128, 128])
+            us_e = time_eager(e2e, reps)
+            llama.append({"M": m, "N": n, "K": k, "gemm_us": round(us_g, 2), "quant_gemm_us": round(us_e, 2),
+                          "tflops": round(gemm_flops(m, n, k) / us_g / 1e6, 1), "gbps": round(gemm_bytes(m, n, k) / us_g / 1e3, 1)})
+        del wq, ws
+
     # ---- CPU baseline: the oracle on the host cores, bounded sample
     cpu = None
     if not args.no_cpu:
@@ -267,6 +330,8 @@ def main():
         "roofline": roofline,
         "roofline_small_m": roofline_small,
         "quantizer": quant,
+        "cutlass_scaled_mm_n8192_k8192_bias": scaled,
+        "llama3_8b_linears": llama,
         "cpu_baseline": cpu,
         "detail": detail,
     }

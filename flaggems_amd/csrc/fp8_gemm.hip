@@ -449,7 +449,7 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
     if (plan.use) return launch_small_m(a, MODE, plan, workspace, workspace_bytes, stream);
   }
   const bool big = a.M > 128;
-  if (direct && pingpong_takes(a, MODE)) return launch_pingpong(a, MODE, workspace, workspace_bytes, stream);
+  if (direct && pingpong_takes(a, MODE, workspace, workspace_bytes)) return launch_pingpong(a, MODE, workspace, workspace_bytes, stream);
   if (big) {
     return direct ? launch_cfg<256, 256, 4, 2, MODE, true>(a, stream)
                   : launch_cfg<256, 256, 4, 2, MODE, false>(a, stream);

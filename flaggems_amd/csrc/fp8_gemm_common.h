@@ -92,9 +92,10 @@ int launch_small_m(const GemmArgs& a, int mode, const SmallMPlan& plan, void* wo
                    hipStream_t stream);
 
 
-// Persistent 256x256 kernel, fp8_gemm_pingpong.hip: block-scaled, bf16 output with 16-byte aligned rows, M > 128;
+// Persistent 256x256 kernel, fp8_gemm_pingpong.hip: bf16 output with 16-byte aligned rows, M > 128 (or M > 64 when
+// the workspace lets it share tiles along K);
 // the caller has checked that the operands qualify for direct global->LDS loads.
-bool pingpong_takes(const GemmArgs& a, int mode);
+bool pingpong_takes(const GemmArgs& a, int mode, const void* workspace, size_t workspace_bytes);
 int launch_pingpong(const GemmArgs& a, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream);
 // workspace that lets the persistent kernel split tiles along K between blocks (0: never useful for this shape)
 size_t pingpong_workspace_bytes(int64_t M, int64_t N, int64_t K);

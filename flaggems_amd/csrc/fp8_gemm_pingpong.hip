@@ -732,12 +732,13 @@ SkPlan plan_stream_k(int64_t tiles, int KB, int cus) {
   const int64_t dp_grid = tiles < cus ? tiles : cus;
   const int64_t dp_steps = ceil_div(tiles, dp_grid) * KB;
   const int64_t q = total / cus;
-  // Measured on DeepSeek-V3 shapes: ranges that start at different K offsets stop sharing operand panels in
-  // their XCD's L2, which makes a K-block about 1.3 times as expensive, and finishing the shared tiles adds
-  // about as much as 14 K-blocks to a launch.  Stream-K is chosen when it still comes out ahead.  A tile
-  // shared by more than 8 ranges would make its last wavefront read too many partial tiles.
-  const int64_t sk_steps = ceil_div(total, cus) * 13 / 10 + 14;
-  if (sk_steps >= dp_steps || q * 8 < KB) return p;
+  // Measured on DeepSeek-V3 and Llama shapes: ranges that start at different K offsets stop sharing operand
+  // panels in their XCD's L2, which makes a K-block about 1.3 times as expensive, and finishing the shared tiles
+  // adds about as much as 8 K-blocks plus 2.5 per range that shares a tile (its last wavefront reads that many
+  // partial tiles).  Stream-K is chosen when it still comes out ahead, and never with more than 16 ranges a tile.
+  if (q * 16 < KB) return p;
+  const int64_t sk_steps_x10 = ceil_div(total, cus) * 13 + 80 + 25 * (KB + q) / q;
+  if (sk_steps_x10 >= dp_steps * 10) return p;
   p.use = true;
   p.grid = cus;
   p.q = (int)q;
@@ -787,21 +788,28 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
 
 }  // namespace
 
-bool pingpong_takes(const GemmArgs& g, int mode) {
+bool pingpong_takes(const GemmArgs& g, int mode, const void* workspace, size_t workspace_bytes) {
   // bf16 rows that take 16-byte stores; activation-scale offsets (bytes from the first row) that fit 32 bits
-  if (!(g.M > 128 && g.c_dtype == FG_BF16 && g.ldc % 8 == 0 && (uintptr_t)g.C % 16 == 0)) return false;
+  if (!(g.M > 64 && g.c_dtype == FG_BF16 && g.ldc % 8 == 0 && (uintptr_t)g.C % 16 == 0)) return false;
+  // 64 < M <= 128 wastes half of every 256-row tile: worth it only where tiles get shared along K (few, deep tiles)
+  if (g.M <= 128) {
+    const SkPlan sk = plan_stream_k(ceil_div(g.N, kBN), g.KB, cu_count());
+    if (!(mode == kModeBlock && sk.use && workspace != nullptr && (uintptr_t)workspace % 16 == 0 &&
+          workspace_bytes >= FG_WORKSPACE_COUNTER_BYTES + (size_t)sk.grid * 2 * kPartialSlotBytes))
+      return false;
+  }
   if (mode != kModeBlock) return true;
   return g.xs_rs >= 0 && g.xs_cs >= 0 && g.ws_rs >= 0 && g.ws_cs >= 0 && (int64_t)g.M * g.xs_rs < (1ll << 29);
 }
 
 size_t pingpong_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-  if (M <= 128 || K <= 0 || K % 128 != 0) return 0;
+  if (M <= 64 || K <= 0 || K % 128 != 0) return 0;
   const SkPlan sk = plan_stream_k(ceil_div(M, kBM) * ceil_div(N, kBN), (int)(K / 128), cu_count());
   return sk.use ? FG_WORKSPACE_COUNTER_BYTES + (size_t)sk.grid * 2 * kPartialSlotBytes : 0;
 }
 
 int launch_pingpong(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-  if (!pingpong_takes(g, mode)) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: persistent kernel does not take this problem");
+  if (!pingpong_takes(g, mode, workspace, workspace_bytes)) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: persistent kernel does not take this problem");
   return launch_block(g, mode, workspace, workspace_bytes, stream);
 }
 
