@@ -15,14 +15,19 @@
 // K-blocks over all tiles a block processes:
 //     slot 2T   : A  fetch(T)     B  multiply(T-1)
 //     slot 2T+1 : A  multiply(T)  B  fetch(T)
-// A issues its share of the loads of stage T+1 at the start of fetch(T) and waits for them at the end of
-// multiply(T); B spreads its share of stage T+2 over multiply(T) and waits at the end of fetch(T+1).
-// Every load therefore has more than a whole slot to land, and every wait sits right before a barrier.
+// All global->LDS loads are issued in the fetch phases: a wavefront issues one instruction in about six
+// cycles, an MFMA of this shape with its four FMAs fills the 32 cycles the matrix pipe takes, and anything
+// else in the multiply phase (a load that waits for the address unit, a branch, scalar bookkeeping) delays
+// the MFMAs by that much.  A's wavefronts load the activation tile, B's the weight tile:
+//     A, in fetch(T) (slot 2T): activations of stage T+1; waits for them at the end of multiply(T);
+//     B, in fetch(T) (slot 2T+1): weights of stage T+2; waits for them at the end of fetch(T+1).
+// Every load has more than a whole slot to land, and every wait sits right before a barrier.
 //
 // LDS.  A stage is 256 x 128 weight bytes plus 256 x 128 activation bytes.  Activation fragments are all
-// read in the fetch phase (stage T: slots 2T and 2T+1), so two activation stages suffice for loads issued
-// from slot 2T+2 on.  Weight fragments are also read during the multiply phase (stage T: until the end of
-// slot 2T+2), so the weights get three stages.  3 x 32 KB + 2 x 32 KB = 160 KB.
+// read in the fetch phases (stage T: slots 2T and 2T+1), so its slot is free for stage T+2 from slot 2T+2 on
+// and for A, which loads only one stage ahead, two activation stages suffice.  Weight fragments are also
+// read during the multiply phases (stage T: until the end of slot 2T+2); B writes stage T+2 from slot 2T+1
+// on, into the slot stage T-1 left at the end of slot 2T: three weight stages.  3 x 32 KB + 2 x 32 KB = 160 KB.
 //
 // Operand roles and layouts are those of the tile kernel in fp8_gemm.hip (weights in the MFMA A slot,
 // XOR-permuted row-major LDS image filled by global_load_lds_dwordx4), with one change: the 128 weight
@@ -38,25 +43,33 @@
 
 #ifdef FG_PP_TRACE
 // development aid: per-slot timestamps of block 0, wavefronts 0 and 4
-__device__ unsigned long long fg_pp_trace_buf[2][64][8];
-#define FG_PP_STAMP(id)                                                                             \
+__device__ unsigned long long fg_pp_trace_buf[2][64][20];
+// the clock reads stay in scalar registers until the end of the step, so that a stamp costs one issue slot
+#define FG_PP_STAMP(id) fg_ts[id] = __builtin_amdgcn_s_memtime()
+#define FG_PP_STAMPS_DECLARE unsigned long long fg_ts[18] = {}
+#define FG_PP_STAMPS_STORE                                                                          \
   do {                                                                                              \
-    if (blockIdx.x == 0 && (wave & 3) == 0 && lane == 0 && T < 64)                                  \
-      fg_pp_trace_buf[grp][T][id] = __builtin_readcyclecounter();                                   \
+    if (blockIdx.x == 0 && wave == 0 && lane == 0 && T > 0 && T <= 64)                              \
+      for (int i = 0; i < 18; ++i) if (i < 8 || i >= 10) fg_pp_trace_buf[grp][T - 1][i] = fg_ts[i];  \
+    fg_ts[0] = fg_ts[8]; fg_ts[1] = fg_ts[9];                                                       \
   } while (0)
 extern "C" void fg_pp_trace_dump() {
-  static unsigned long long h[2][64][8];
+  static unsigned long long h[2][64][20];
   hipMemcpyFromSymbol(h, HIP_SYMBOL(fg_pp_trace_buf), sizeof(h));
   unsigned long long t0 = h[0][0][0];
   for (int T = 0; T < 24; ++T)
     for (int g = 0; g < 2; ++g) {
       printf("T=%2d %c:", T, g ? 'B' : 'A');
       for (int i = 0; i < 8; ++i) printf(" %8lld", (long long)(h[g][T][i] - t0));
+      printf("  issue:");
+      for (int i = 10; i < 18; ++i) printf(" %5lld", (long long)(h[g][T][i] - h[g][T][1]));
       printf("\n");
     }
 }
 #else
 #define FG_PP_STAMP(id) do {} while (0)
+#define FG_PP_STAMPS_DECLARE do {} while (0)
+#define FG_PP_STAMPS_STORE do {} while (0)
 #endif
 
 namespace fg {
@@ -69,7 +82,10 @@ constexpr int kWStages = 3, kXStages = 2;  // see "LDS" in the header comment
 constexpr int kXRegion = kWStages * kWStageBytes;
 constexpr int kLdsBytes = kXRegion + kXStages * kXStageBytes;  // 160 KB, all of a compute unit's LDS
 constexpr int kTN = 8, kTM = 4;         // MFMA tiles per wavefront: 128 weight rows x 64 activation rows
-constexpr int kSlabsPerWave = 4;        // 1 KB global->LDS loads per wavefront, per operand, per stage
+// Wave priorities of the phases: the fetch phase is the longer one and every instruction of it sits on the
+// path to the barrier that releases the partner's next MFMAs.
+constexpr int kFetchPrio = 1, kMultiplyPrio = 0;
+constexpr int kSlabsPerWave = 8;        // 1 KB global->LDS loads per wavefront and stage
 
 struct PpArgs {
   GemmArgs g;
@@ -154,40 +170,47 @@ struct Walk {
   }
 };
 
-// This wavefront's share of the global->LDS loads of one stage: 4 slabs (1 KB, 8 LDS rows each) of the
-// weight tile and 4 of the activation tile.  Per-lane byte offsets are relative to the tile's first row.
+// This wavefront's share of the global->LDS loads of one stage: 8 slabs (1 KB, 8 LDS rows each) of one
+// operand tile.  The four wavefronts of group A load the activation tile, those of group B the weight
+// tile: the groups run half a step apart and each operand has a moment of its own when an LDS slot is
+// free for it (see the main loop).  Per-lane byte offsets are relative to the tile's first row.
 struct LoadShare {
-  uint32_t w_off[kSlabsPerWave], x_off[kSlabsPerWave];
-  const uint8_t* w_ptr;  // uniform: first row of the tile, K-block being loaded
-  const uint8_t* x_ptr;
+  uint32_t off[kSlabsPerWave];
+  const uint8_t* ptr;  // uniform: first row of the tile, K-block being loaded
 
-  __device__ __forceinline__ void set_tile(const GemmArgs& a, int m0, int n0, int wave, int lane) {
-    w_ptr = a.W + (int64_t)n0 * a.ldw;
-    x_ptr = a.X + (int64_t)m0 * a.ldx;
-    const int w_valid = a.N - n0, x_valid = a.M - m0;
+  // valid: rows of the tile inside the matrix; rows past the edge re-read the last row and are never stored
+  __device__ __forceinline__ void set_offsets(const GemmArgs& a, int valid, int wave, int lane) {
+    const bool weights = wave >= 4;
+    const uint32_t ld = (uint32_t)(weights ? a.ldw : a.ldx);
 #pragma unroll
     for (int j = 0; j < kSlabsPerWave; ++j) {
-      const int slab = wave + j * 8;
+      const int slab = (wave & 3) + j * 4;
       const int r = slab * 8 + (lane >> 3);  // LDS row
       const uint32_t chunk = (uint32_t)(((lane & 7) ^ (r & 7)) << 4);
-      int wr = (r & 128) + weight_row_of_lds_row(r & 127);
-      wr = wr < w_valid ? wr : w_valid - 1;  // rows past the edge re-read the last row; never stored
-      const int xr = r < x_valid ? r : x_valid - 1;
-      w_off[j] = (uint32_t)wr * (uint32_t)a.ldw + chunk;
-      x_off[j] = (uint32_t)xr * (uint32_t)a.ldx + chunk;
+      int row = weights ? (r & 128) + weight_row_of_lds_row(r & 127) : r;
+      row = row < valid ? row : valid - 1;
+      off[j] = __umul24((uint32_t)row, ld) + chunk;  // row < 256, ld < 2^23 (checked by the host)
     }
   }
-  // q in [0, 8): 0-3 weight slabs, 4-7 activation slabs
-  __device__ __forceinline__ void issue_one(uint8_t* w_stage, uint8_t* x_stage, int wave, int q) const {
-    const int j = q & 3;
-    const int slab = wave + j * 8;
-    if (q < 4) {
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(w_ptr + w_off[j]),
-                                       (__attribute__((address_space(3))) void*)(w_stage + slab * 1024), 16, 0, 0);
-    } else {
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(x_ptr + x_off[j]),
-                                       (__attribute__((address_space(3))) void*)(x_stage + slab * 1024), 16, 0, 0);
-    }
+  __device__ __forceinline__ void set_ptr(const GemmArgs& a, int m0, int n0, int wave) {
+    ptr = wave >= 4 ? a.W + (int64_t)n0 * a.ldw : a.X + (int64_t)m0 * a.ldx;
+  }
+  __device__ __forceinline__ void set_tile(const GemmArgs& a, int m0, int n0, int wave, int lane) {
+    set_ptr(a, m0, n0, wave);
+    const int valid = wave >= 4 ? a.N - n0 : a.M - m0;
+    set_offsets(a, valid < 256 ? valid : 256, wave, lane);
+  }
+  // The load is written out instead of using the compiler's builtin: the compiler books a global->LDS
+  // load as an access that may return through either counter, and from then on turns every wait for an LDS
+  // read into lgkmcnt(0), which makes the multiply phase wait for fragments it needs two rows later.
+  // stage_lds: LDS byte address of this wavefront's first slab in the stage (uniform).
+  __device__ __forceinline__ void issue_one(uint32_t stage_lds, int q) const {
+    asm volatile("s_add_u32 m0, %2, %3\n\t"
+                 "s_nop 0\n\t"
+                 "global_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(off[q]), "s"(ptr), "s"(stage_lds), "n"(q * 4 * 1024)
+                 : "memory", "m0", "scc");
   }
 };
 
@@ -454,7 +477,9 @@ __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the counted waits of the main loop start from zero
 }
 
-template <bool SK, int MODE>
+// ALIGNED: M and N are multiples of the tile; no tile has an edge, and the per-lane offsets of the tile loads
+// and of the scale loads never change (a tile change then touches scalar registers only).
+template <bool SK, int MODE, bool ALIGNED>
 __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const GemmArgs& g = a.g;
@@ -485,28 +510,30 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   // ---- the stage being loaded
   Walk lw;
   lw.start(a, first_idx, first_kb);
-  LoadShare share;
+  LoadShare share = {};
   share.set_tile(g, lw.m0, lw.n0, wave, lane);
-  share.w_ptr += (int64_t)first_kb * 128;
-  share.x_ptr += (int64_t)first_kb * 128;
+  share.ptr += (int64_t)first_kb * 128;
   int loaded = 0, w_slot = 0, x_slot = 0;  // stages issued by this wavefront; LDS slots of the next stage
   auto issue_stage_part = [&](int q) __attribute__((always_inline)) {
-    share.issue_one(lds + w_slot * kWStageBytes, lds + kXRegion + x_slot * kXStageBytes, wave, q);
+    const uint32_t region = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+    const uint32_t stage = grp ? (uint32_t)(w_slot * kWStageBytes) : (uint32_t)(kXRegion + x_slot * kXStageBytes);
+    share.issue_one(region + stage + (uint32_t)(wave & 3) * 1024u, q);
   };
   auto finish_stage = [&]() __attribute__((always_inline)) {
     ++loaded;
     w_slot = (w_slot + 1 == kWStages) ? 0 : w_slot + 1;
     x_slot ^= 1;
-    if (lw.next(a)) {
-      if (lw.idx < a.n_tiles) share.set_tile(g, lw.m0, lw.n0, wave, lane);
+    if (__builtin_expect(lw.next(a), 0)) {
+      if (lw.idx < a.n_tiles) {
+        if (ALIGNED) share.set_ptr(g, lw.m0, lw.n0, wave); else share.set_tile(g, lw.m0, lw.n0, wave, lane);
+      }
     } else {
-      share.w_ptr += 128;
-      share.x_ptr += 128;
+      share.ptr += 128;
     }
   };
   auto issue_stage_all = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int q = 0; q < 8; ++q) issue_stage_part(q);
+    for (int q = 0; q < kSlabsPerWave; ++q) issue_stage_part(q);
     finish_stage();
   };
 
@@ -514,21 +541,30 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   // a uniform pointer that moves along K (the host checks that M * row stride fits)
   Walk sw;
   sw.start(a, first_idx, first_kb);
-  uint32_t xs_off[kTM];
+  uint32_t xs_off[kTM] = {0u, 0u, 0u, 0u};
   const float* xs_ptr = g.xs;
-  auto set_scale_tile = [&]() __attribute__((always_inline)) {
+  // offsets are relative to the tile's first row; rows past the edge read the last row's scale
+  auto set_scale_offsets = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < kTM; ++j) {
-      int m = sw.m0 + wm0 + j * 16 + l16;
-      m = m < g.M ? m : g.M - 1;
-      xs_off[j] = (uint32_t)m * (uint32_t)g.xs_rs * 4u;
+      int r = wm0 + j * 16 + l16;
+      const int last = g.M - 1 - sw.m0;
+      r = r < last ? r : last;
+      xs_off[j] = (uint32_t)r * (uint32_t)g.xs_rs * 4u;
     }
-    xs_ptr = g.xs;
+  };
+  auto set_scale_tile = [&]() __attribute__((always_inline)) {
+    if (!ALIGNED) set_scale_offsets();
+    xs_ptr = g.xs + (int64_t)sw.m0 * g.xs_rs;
   };
   if (MODE == kModeBlock) {
+    set_scale_offsets();
     set_scale_tile();
     xs_ptr += (int64_t)first_kb * g.xs_cs;
   }
+  auto advance_scales = [&]() __attribute__((always_inline)) {
+    if (__builtin_expect(sw.next(a), 0)) set_scale_tile(); else xs_ptr += g.xs_cs;
+  };
   float xs_nxt[kTM] = {0.f, 0.f, 0.f, 0.f};
   auto request_scales = [&]() __attribute__((always_inline)) {
     if (MODE != kModeBlock) return;
@@ -552,10 +588,11 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   issue_stage_all();
   if (grp == 1 && total > 1) issue_stage_all();
   request_scales();
+  if (MODE == kModeBlock && total > 1) advance_scales();  // fetch(T) asks for the scales of step T+1
   wait_vmem_all();
   __builtin_amdgcn_s_barrier();
   if (grp == 1) __builtin_amdgcn_s_barrier();  // B runs one slot behind A
-  bool b_loaded_prev = false;  // B issued tile loads during its previous multiply
+  __builtin_amdgcn_s_setprio(kFetchPrio);
 
   v4f acc[kTN][kTM];
 #pragma unroll
@@ -588,43 +625,68 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   };
 
   int rw_slot = 0, rx_slot = 0;  // LDS slots of the stage being read
+  FG_PP_STAMPS_DECLARE;
   auto run_steps = [&](int t_begin, int t_end) __attribute__((always_inline)) {
   for (int T = t_begin; T < t_end; ++T) {
     // ================= fetch(T)
-    // Scales of this step were requested a step ago.  Younger than them: for A nothing (it waited for
-    // everything at the end of its multiply), for B the eight tile loads of its previous multiply.
-    FG_PP_STAMP(0);
+    // Scales of this step were requested a step ago; the only younger vector-memory operations are the eight
+    // tile loads that followed them (for A those have landed as well: it waited at the end of its multiply).
+    FG_PP_STAMP(8);
     float xs[kTM], sc[kTM];
     const bool more = T + 1 < total;
     float ws = 1.f;
     if (MODE == kModeBlock) {
-      if (b_loaded_prev) wait_and_take<8>(xs, xs_nxt); else wait_and_take<0>(xs, xs_nxt);
-      if (more) {
-        if (sw.next(a)) set_scale_tile(); else xs_ptr += g.xs_cs;
-        request_scales();
-      }
+      wait_and_take<8>(xs, xs_nxt);
+      if (more) request_scales();  // of step T+1; the pointer was moved there a step ago
       ws = *(const __attribute__((address_space(4))) float*)ws_ptr;
     }
-    FG_PP_STAMP(1);
+    FG_PP_STAMP(9);
+    FG_PP_STAMPS_STORE;  // of the previous step, behind this step's first wait
     const uint8_t* const tw = lds + rw_slot * kWStageBytes + (wn0 >> 4) * 2048;
     const uint8_t* const tx = lds + kXRegion + rx_slot * kXStageBytes + (wm0 >> 4) * 2048;
-    // all activation fragments and the first two weight fragments; the other six follow during the
-    // multiply, each two MFMA rows before its use
+    // All activation fragments and the first two weight fragments (the other six follow during the multiply,
+    // each two MFMA rows before its use), interleaved with this wavefront's eight tile loads: the address
+    // unit takes ~45 cycles per 1 KB load and the LDS ~25 per fragment half, and a wavefront that issues
+    // either kind back to back waits for the unit each time.
+    //   A loads the activations of stage T+1 into the slot that fetch(T-1) read,
+    //   B the weights of stage T+2 into the slot that multiply(T-1) left a slot ago.
+    // Past the last stage the loads are repeated from the last address into a slot nobody reads any more:
+    // cheaper than a branch per load, and the wait counts below stay the same on every step.
     v8i xf[kTM], wr[3];
-#pragma unroll
-    for (int j = 0; j < kTM; ++j) xf[j] = read_frag(tx, j, frag_off);
+    issue_stage_part(0);
+    FG_PP_STAMP(10);
+    xf[0] = read_frag(tx, 0, frag_off);
+    issue_stage_part(1);
+    FG_PP_STAMP(11);
+    xf[1] = read_frag(tx, 1, frag_off);
+    issue_stage_part(2);
+    FG_PP_STAMP(12);
+    xf[2] = read_frag(tx, 2, frag_off);
+    issue_stage_part(3);
+    FG_PP_STAMP(13);
+    xf[3] = read_frag(tx, 3, frag_off);
+    issue_stage_part(4);
+    FG_PP_STAMP(14);
     wr[0] = read_frag(tw, 0, frag_off);
+    issue_stage_part(5);
+    FG_PP_STAMP(15);
     wr[1] = read_frag(tw, 1, frag_off);
+    issue_stage_part(6);
+    FG_PP_STAMP(16);
+    issue_stage_part(7);
+    FG_PP_STAMP(17);
     FG_PP_STAMP(2);
-    // after the LDS reads: the four wavefronts of A issue 32 KB of loads at once and stall in the issue
-    // while the address unit works through them
-    if (grp == 0 && loaded < total) issue_stage_all();  // stage T+1
+    // scalar bookkeeping of the next step, under the latency of the LDS reads (in the multiply phase every
+    // extra instruction delays the MFMAs: a wavefront issues one instruction in ~6 cycles, and the MFMA with
+    // its four FMAs fills the 32 cycles the matrix pipe takes)
+    if (loaded < total) finish_stage();
+    if (MODE == kModeBlock && T + 2 < total) advance_scales();
     FG_PP_STAMP(3);
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): fragments are in registers
-    // B's share of stage T+1 (issued during multiply(T-1)) must have landed before the barrier; only the
-    // scale requests of this slot are younger.
+    // B's weights of stage T+1, issued a step ago, must have landed before the barrier; the scale requests
+    // and the tile loads of this slot are younger.
     if (grp == 1) {
-      if (more && MODE == kModeBlock) wait_vmem<4>(); else wait_vmem<0>();
+      if (more && MODE == kModeBlock) wait_vmem<12>(); else wait_vmem<8>();
     }
     if (MODE == kModeBlock) {
 #pragma unroll
@@ -636,8 +698,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     FG_PP_STAMP(5);
 
     // ================= multiply(T)
-    const bool b_loads = grp == 1 && loaded < total;  // B: stage T+2, spread over the MFMA steps
-    __builtin_amdgcn_s_setprio(1);
+    __builtin_amdgcn_s_setprio(kMultiplyPrio);
     if (MODE != kModeBlock) {
       // row/column mode: the matrix pipe accumulates; scales and bias wait for the epilogue
 #pragma unroll
@@ -645,7 +706,6 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
         const int t = st / kTM, j = st % kTM;
         mfma_accumulate(acc[t][j], wr[t % 3], xf[j]);
         if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
-        if (st % 2 == 1 && st < 16 && b_loads) issue_stage_part(st / 2);
       }
     } else {
       v4f p[3];
@@ -657,18 +717,13 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
         // covers only reads issued a whole row earlier
         if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
         if (st >= 2) scale_into<0>(acc[(st - 2) / kTM][(st - 2) % kTM], p[(st - 2) % 3], sc[(st - 2) % kTM]);
-        // B's tile loads go out in the first half of the phase so that they have landed by the end of its
-        // next fetch slot
-        if (st % 2 == 1 && st < 16 && b_loads) issue_stage_part(st / 2);
       }
       constexpr int L = kTN * kTM;
       scale_into<0>(acc[(L - 2) / kTM][(L - 2) % kTM], p[(L - 2) % 3], sc[(L - 2) % kTM]);
       scale_into<4>(acc[(L - 1) / kTM][(L - 1) % kTM], p[(L - 1) % 3], sc[(L - 1) % kTM]);
     }
-    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_s_setprio(kFetchPrio);
     FG_PP_STAMP(6);
-    if (b_loads) finish_stage();
-    b_loaded_prev = b_loads;
     if (grp == 0) wait_vmem_all();  // A's share of stage T+1 has landed
     FG_PP_STAMP(7);
     __builtin_amdgcn_s_barrier();
@@ -677,7 +732,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     rw_slot = (rw_slot + 1 == kWStages) ? 0 : rw_slot + 1;
     rx_slot ^= 1;
     pend_m = cw.m0 + wm0; pend_n = cw.n0 + wn0; pend_idx = cw.idx;
-    pending = cw.next(a);
+    pending = __builtin_expect(cw.next(a), 0);
     if (MODE == kModeBlock) {
       if (pending) ws_ptr = ws_row(); else ws_ptr += g.ws_cs;
     }
@@ -692,7 +747,6 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     if (n_head > 0) {
       run_steps(0, n_head);
       flush_partial_tile();
-      b_loaded_prev = false;  // everything this wavefront had in flight has been waited for
     }
     run_steps(n_head, n_head + n_whole);
     if (n_head + n_whole < total) {
@@ -705,6 +759,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     run_steps(0, total);
     if (pending) flush_whole_tile();
   }
+  wait_vmem_all();  // the tile loads repeated past the last stage
   if (grp == 0) __builtin_amdgcn_s_barrier();  // pairs with B's extra barrier at the start
 }
 
@@ -756,9 +811,12 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   a.n_tiles = (int)tiles;
   static bool attr_set = false;  // benign if raced
   if (!attr_set) {
-    for (const void* k : {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock>),
-                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock>),
-                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol>)}) {
+    for (const void* k : {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false>),
+                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, true>),
+                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false>),
+                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true>),
+                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, false>),
+                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, true>)}) {
       hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
       if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
     }
@@ -776,12 +834,15 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     a.partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
     grid = sk.grid;
   }
+  const bool aligned = g.M % kBM == 0 && g.N % kBN == 0;
+  void (*kern)(PpArgs);
   if (mode != kModeBlock)
-    hipLaunchKernelGGL((fp8_gemm_pingpong_kernel<false, kModeRowCol>), dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
+    kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeRowCol, true> : fp8_gemm_pingpong_kernel<false, kModeRowCol, false>;
   else if (a.sk)
-    hipLaunchKernelGGL((fp8_gemm_pingpong_kernel<true, kModeBlock>), dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
+    kern = aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true> : fp8_gemm_pingpong_kernel<true, kModeBlock, false>;
   else
-    hipLaunchKernelGGL((fp8_gemm_pingpong_kernel<false, kModeBlock>), dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
+    kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeBlock, true> : fp8_gemm_pingpong_kernel<false, kModeBlock, false>;
+  hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
   FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel");
   return FG_OK;
 }
