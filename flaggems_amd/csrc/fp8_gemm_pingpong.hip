@@ -42,14 +42,15 @@
 #include "fp8_gemm_common.h"
 
 #ifdef FG_PP_TRACE
-// development aid: per-slot timestamps of block 0, wavefronts 0 and 4
+// development aid: per-slot timestamps of block 0, wavefronts 0 and 4; every fourth step is recorded and
+// written out a step later, so that the stores do not disturb the step they describe
 __device__ unsigned long long fg_pp_trace_buf[2][64][20];
 // the clock reads stay in scalar registers until the end of the step, so that a stamp costs one issue slot
 #define FG_PP_STAMP(id) fg_ts[id] = __builtin_amdgcn_s_memtime()
 #define FG_PP_STAMPS_DECLARE unsigned long long fg_ts[18] = {}
 #define FG_PP_STAMPS_STORE                                                                          \
   do {                                                                                              \
-    if (blockIdx.x == 0 && wave == 0 && lane == 0 && T > 0 && T <= 64)                              \
+    if (blockIdx.x == 0 && (wave & 3) == 0 && lane == 0 && (T & 3) == 2 && T <= 64)                 \
       for (int i = 0; i < 18; ++i) if (i < 8 || i >= 10) fg_pp_trace_buf[grp][T - 1][i] = fg_ts[i];  \
     fg_ts[0] = fg_ts[8]; fg_ts[1] = fg_ts[9];                                                       \
   } while (0)
@@ -57,7 +58,7 @@ extern "C" void fg_pp_trace_dump() {
   static unsigned long long h[2][64][20];
   hipMemcpyFromSymbol(h, HIP_SYMBOL(fg_pp_trace_buf), sizeof(h));
   unsigned long long t0 = h[0][0][0];
-  for (int T = 0; T < 24; ++T)
+  for (int T = 1; T < 64; T += 4)
     for (int g = 0; g < 2; ++g) {
       printf("T=%2d %c:", T, g ? 'B' : 'A');
       for (int i = 0; i < 8; ++i) printf(" %8lld", (long long)(h[g][T][i] - t0));
@@ -801,6 +802,33 @@ SkPlan plan_stream_k(int64_t tiles, int KB, int cus) {
   return p;
 }
 
+// Activation scales [M, K/128] -> [K/128, M].  The GEMM reads four scales per lane and K-block, for rows 16
+// apart; with K-major rows that is a separate 128-byte line from L2 for every row and K-block (the tile loads
+// keep sweeping the L1), as many line requests as the tiles themselves need, and the tile loads queue behind
+// them in the address unit: measured 20 % of the run time on K = 16384.  From the transposed copy a
+// wavefront's 64 scales of a K-block are 256 contiguous bytes.
+__global__ __launch_bounds__(256) void transpose_scales_kernel(const float* __restrict__ xs, int64_t rs, int64_t cs, int M,
+                                                               int KB, float* __restrict__ out) {
+  __shared__ float tile[32][33];
+  const int kb0 = (int)blockIdx.x * 32, m0 = (int)blockIdx.y * 32;
+  const int tx = (int)threadIdx.x & 31, ty = (int)threadIdx.x >> 5;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + ty + i * 8, kb = kb0 + tx;
+    if (m < M && kb < KB) tile[ty + i * 8][tx] = xs[(int64_t)m * rs + (int64_t)kb * cs];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int kb = kb0 + ty + i * 8, m = m0 + tx;
+    if (m < M && kb < KB) out[(int64_t)kb * M + m] = tile[tx][ty + i * 8];
+  }
+}
+
+// rows of scales at least this many floats apart are worth transposing (below, 16 rows share a few lines)
+constexpr int64_t kTransposeMinRowStride = 4;
+size_t transposed_scales_bytes(int64_t M, int64_t KB) { return (size_t)((M * KB * 4 + 255) / 256 * 256); }
+
 int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   PpArgs a = {};
   a.g = g;
@@ -826,7 +854,17 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   int grid = tiles < cus ? (int)tiles : cus;
   // Stream-K is an optimisation the workspace enables: without one (or with a small one) whole tiles go round-robin.
   const SkPlan sk = plan_stream_k(tiles, g.KB, cus);
-  const size_t need = FG_WORKSPACE_COUNTER_BYTES + (size_t)sk.grid * 2 * kPartialSlotBytes;
+  const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : 0;
+  const size_t need = FG_WORKSPACE_COUNTER_BYTES + sk_bytes;
+  // workspace: [counters][partial tiles, if the shape is one that shares tiles][transposed activation scales]
+  if (mode == kModeBlock && g.xs_rs >= kTransposeMinRowStride && workspace != nullptr && (uintptr_t)workspace % 16 == 0 &&
+      workspace_bytes >= need + transposed_scales_bytes(g.M, g.KB)) {
+    float* const xs_t = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + need);
+    hipLaunchKernelGGL(transpose_scales_kernel, dim3((uint32_t)ceil_div(g.KB, 32), (uint32_t)ceil_div(g.M, 32)), dim3(256), 0, stream,
+                       g.xs, g.xs_rs, g.xs_cs, g.M, g.KB, xs_t);
+    FG_CHECK_LAUNCH("transpose_scales_kernel");
+    a.g.xs = xs_t; a.g.xs_rs = 1; a.g.xs_cs = g.M;
+  }
   if (mode == kModeBlock && sk.use && workspace != nullptr && workspace_bytes >= need && (size_t)sk.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
       (uintptr_t)workspace % 16 == 0) {
     a.sk = 1; a.sk_q = sk.q; a.sk_r = sk.r;
@@ -866,7 +904,10 @@ bool pingpong_takes(const GemmArgs& g, int mode, const void* workspace, size_t w
 size_t pingpong_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 64 || K <= 0 || K % 128 != 0) return 0;
   const SkPlan sk = plan_stream_k(ceil_div(M, kBM) * ceil_div(N, kBN), (int)(K / 128), cu_count());
-  return sk.use ? FG_WORKSPACE_COUNTER_BYTES + (size_t)sk.grid * 2 * kPartialSlotBytes : 0;
+  const int64_t KB = K / 128;
+  const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : 0;
+  const size_t tr_bytes = KB >= kTransposeMinRowStride ? transposed_scales_bytes(M, KB) : 0;  // for row-major scales
+  return sk_bytes + tr_bytes != 0 ? FG_WORKSPACE_COUNTER_BYTES + sk_bytes + tr_bytes : 0;
 }
 
 int launch_pingpong(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream) {
