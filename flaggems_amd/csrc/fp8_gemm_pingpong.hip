@@ -738,6 +738,12 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
       if (pending) ws_ptr = ws_row(); else ws_ptr += g.ws_cs;
     }
   }
+  // The scales requested for the next step are on their way into registers the compiler knows nothing about,
+  // and it copies them where one instance of this loop hands over to the next (three with stream-K): they must
+  // have arrived before that.  The operands make the copies come after the wait.
+  if (MODE == kModeBlock) {
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(xs_nxt[0]), "+v"(xs_nxt[1]), "+v"(xs_nxt[2]), "+v"(xs_nxt[3]) : : "memory");
+  }
   };
 
   if (SK) {
