@@ -89,6 +89,33 @@ def test_persistent_kernel_several_rounds_ragged_edges_and_strides():
     assert torch.equal(got3.view(torch.int16), got.view(torch.int16))
 
 
+@pytest.mark.parametrize("M,N,K", [(768, 1024, 2048), (300, 520, 1024)])
+def test_activation_scales_in_either_layout_give_the_same_bits(M, N, K):
+    """The persistent kernel reads activation scales K-block by K-block for 64 rows at a time.  Row-major
+    scales ([M, K/128] contiguous, what the quantizer returns) are first transposed into the workspace;
+    scales that already have the rows contiguous (strides (1, M), the reference's column_major_scales
+    layout) are read in place; a call without workspace reads the row-major ones as they are.  All three
+    must give identical results."""
+    from flaggems_amd import _lib
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=5)
+    xq, wq, xs, ws = xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV)
+    want = O.block_fp8_matmul_dequant_ref(xq.cpu(), wq.cpu(), xs.cpu(), ws.cpu(), [128, 128], torch.float32, torch.float64)
+    got = flag_gems.w8a8_block_fp8_matmul(xq, wq, xs, ws, [128, 128])
+    torch.testing.assert_close(got.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    xs_cm = xs.t().contiguous().t()
+    assert xs_cm.stride() == (1, M)
+    got_cm = flag_gems.w8a8_block_fp8_matmul(xq, wq, xs_cm, ws, [128, 128])
+    assert torch.equal(got_cm.view(torch.int16), got.view(torch.int16))
+    lib = _lib.load()
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    status = lib.fg_block_fp8_gemm(xq.data_ptr(), K, wq.data_ptr(), K, xs.data_ptr(), xs.stride(0), xs.stride(1),
+                                   ws.data_ptr(), ws.stride(0), ws.stride(1), out.data_ptr(), N, _lib.DTYPE_CODE[torch.bfloat16],
+                                   M, N, K, 128, 128, None, 0, _lib.current_stream_ptr(torch.device(DEV)))
+    _lib.check(status, "fg_block_fp8_gemm")
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), got.view(torch.int16))
+
+
 def test_tiles_split_along_k_between_blocks():
     """18 tiles of 64 K-blocks on a 256-unit GPU: the persistent kernel cuts the 1152 steps into contiguous
     ranges, so every tile is computed by many blocks and finished through the workspace.  Ragged M and N,
