@@ -794,12 +794,13 @@ SkPlan plan_stream_k(int64_t tiles, int KB, int cus) {
   const int64_t dp_grid = tiles < cus ? tiles : cus;
   const int64_t dp_steps = ceil_div(tiles, dp_grid) * KB;
   const int64_t q = total / cus;
-  // Measured on DeepSeek-V3 and Llama shapes: ranges that start at different K offsets stop sharing operand
-  // panels in their XCD's L2, which makes a K-block about 1.3 times as expensive, and finishing the shared tiles
-  // adds about as much as 8 K-blocks plus 2.5 per range that shares a tile (its last wavefront reads that many
-  // partial tiles).  Stream-K is chosen when it still comes out ahead, and never with more than 16 ranges a tile.
+  // Measured on DeepSeek-V3 shapes, M = 128 ... 4096, in units of a whole-tile K-block: ranges that start at
+  // different K offsets stop sharing operand panels in their XCD's L2, which makes a K-block about 1.35 times as
+  // expensive, and the tiles are finished only after the slowest of their ranges, which adds about 14 K-blocks
+  // plus 0.3 of a tile's K loop.  Stream-K is chosen when it still comes out ahead, and never with more than 16
+  // ranges a tile.
   if (q * 16 < KB) return p;
-  const int64_t sk_steps_x10 = ceil_div(total, cus) * 13 + 80 + 25 * (KB + q) / q;
+  const int64_t sk_steps_x10 = (ceil_div(total, cus) * 27 + 1) / 2 + 3 * KB + 140;
   if (sk_steps_x10 >= dp_steps * 10) return p;
   p.use = true;
   p.grid = cus;
