@@ -31,9 +31,12 @@
 //
 // Operand roles and layouts are those of the tile kernel in fp8_gemm.hip (weights in the MFMA A slot,
 // XOR-permuted row-major LDS image filled by global_load_lds_dwordx4), with one change: the 128 weight
-// rows of a wavefront are dealt to the MFMA tiles so that a lane ends up with 32 *consecutive* output
-// columns (tile t, A-row i  <->  column (i >> 2) * 32 + 4 t + (i & 3)).  A lane then stores 64 contiguous
-// bytes of bf16 per output row and four lanes cover 256 contiguous bytes, instead of 8-byte pieces.
+// rows of a wavefront are dealt to the MFMA tiles so that a 16-byte store instruction writes whole 64-byte
+// segments: tile t, A-row i  <->  column (t >> 1) * 32 + (i >> 2) * 8 + (t & 1) * 4 + (i & 3).  Lane group
+// lg = i >> 2 then holds eight consecutive columns per pair of tiles, and the four lanes that share an output
+// row (16 lanes apart) cover 64 contiguous bytes per store.  The memory side combines the lanes of one store
+// instruction, not the instructions: with 32 consecutive columns per lane (four stores of 16 bytes at a
+// 64-byte stride) results left at 3.1 TB/s, this way at 6.5 TB/s, and all compute units store at once.
 //
 // Registers.  Two wavefronts per SIMD leave 256 registers each: 128 fp32 accumulators, the four activation
 // fragments of the K-block (32) and a ring of three weight fragments (24) that the multiply phase refills two
@@ -42,6 +45,9 @@
 #include "fp8_gemm_common.h"
 
 #ifdef FG_PP_TRACE
+#ifndef FG_PP_TRACE_PHASE
+#define FG_PP_TRACE_PHASE 1
+#endif
 // development aid: per-slot timestamps of block 0, wavefronts 0 and 4; every fourth step is recorded and
 // written out a step later, so that the stores do not disturb the step they describe
 __device__ unsigned long long fg_pp_trace_buf[2][64][20];
@@ -50,7 +56,7 @@ __device__ unsigned long long fg_pp_trace_buf[2][64][20];
 #define FG_PP_STAMPS_DECLARE unsigned long long fg_ts[18] = {}
 #define FG_PP_STAMPS_STORE                                                                          \
   do {                                                                                              \
-    if (blockIdx.x == 0 && (wave & 3) == 0 && lane == 0 && (T & 3) == 2 && T <= 64)                 \
+    if (blockIdx.x == 0 && (wave & 3) == 0 && lane == 0 && (T & 3) == ((FG_PP_TRACE_PHASE + 1) & 3) && T > 0 && T <= 64)                 \
       for (int i = 0; i < 18; ++i) if (i < 8 || i >= 10) fg_pp_trace_buf[grp][T - 1][i] = fg_ts[i];  \
     fg_ts[0] = fg_ts[8]; fg_ts[1] = fg_ts[9];                                                       \
   } while (0)
@@ -58,7 +64,7 @@ extern "C" void fg_pp_trace_dump() {
   static unsigned long long h[2][64][20];
   hipMemcpyFromSymbol(h, HIP_SYMBOL(fg_pp_trace_buf), sizeof(h));
   unsigned long long t0 = h[0][0][0];
-  for (int T = 1; T < 64; T += 4)
+  for (int T = FG_PP_TRACE_PHASE; T < 64; T += 4)
     for (int g = 0; g < 2; ++g) {
       printf("T=%2d %c:", T, g ? 'B' : 'A');
       for (int i = 0; i < 8; ++i) printf(" %8lld", (long long)(h[g][T][i] - t0));
@@ -97,6 +103,11 @@ struct PpArgs {
   int sk, sk_q, sk_r;
   float* partials;
   unsigned int* counters;
+  // Start-up delay of block b: (b mod 16) * stagger sleeps of about 1000 cycles.  With short K loops all compute
+  // units would finish their tiles together and push 32 MB of results at the memory at once, over and over,
+  // each time stalling on the stores for longer than a tile takes to compute; spread over the time the
+  // memory needs for one such batch, the stores of one unit overlap the MFMAs of the others.
+  int stagger;
 };
 
 constexpr int kPartialFloatsPerWave = 64 * 128;                      // one wavefront's 64 x 128 results
@@ -141,8 +152,10 @@ __device__ __forceinline__ bool valid_vid(int vid, int n_tiles) { return vid < n
 // weight row (within the wavefront's 128) held by LDS row rho of the wavefront's region
 __device__ __forceinline__ int weight_row_of_lds_row(int rho) {
   const int t = rho >> 4, i = rho & 15;
-  return (i >> 2) * 32 + t * 4 + (i & 3);
+  return (t >> 1) * 32 + (i >> 2) * 8 + (t & 1) * 4 + (i & 3);
 }
+// first of the eight consecutive output columns that lane group lg holds in MFMA tiles 2q and 2q+1
+__device__ __forceinline__ int piece_column(int n_base, int q, int lg) { return n_base + q * 32 + lg * 8; }
 
 // Uniform (scalar) walk over the (tile, K-block) steps of this block, in processing order.  Three of these
 // run at different distances: the step being multiplied, the step whose scales are being fetched (one
@@ -307,31 +320,35 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, h);
 }
 
-// Stores the wavefront's 64 x 128 results as bf16.  Lane (l16, lg) holds, for every activation tile j, the
-// 32 consecutive columns n_base + lg * 32 + 4 t + v of row m_base + 16 j + l16.  The host guarantees
-// ldc % 8 == 0 and a 16-byte aligned C, so full runs leave as four 16-byte stores.
+// Stores the wavefront's 64 x 128 results as bf16.  Lane (l16, lg) holds, for every activation tile j, four
+// pieces of eight consecutive columns of row m_base + 16 j + l16: piece q starts at column
+// n_base + 32 q + 8 lg and comes from MFMA tiles 2q and 2q+1.  The host guarantees ldc % 8 == 0 and a 16-byte
+// aligned C, so a piece leaves as one 16-byte store, and the four lanes of a row cover 64 contiguous bytes per
+// store instruction.
 // Row/column mode: the sums are scaled by a_scale[m] * b_scale[n] first, and the bias is added to the rounded
 // value, in bf16, as the reference's epilogue does (src/flag_gems/fused/cutlass_scaled_mm.py:288-305).
-template <int MODE>
+// ALIGNED: the tile lies inside the matrix; a wavefront then issues exactly kStoresPerTile store instructions.
+constexpr int kStoresPerTile = 16;
+template <int MODE, bool ALIGNED>
 __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[kTN][kTM], int m_base, int n_base,
                                            int l16, int lg) {
-  const int n = n_base + lg * 32;
-  const bool full = n + 32 <= a.N;
   if (MODE == kModeRowCol) {
     // eight columns at a time, so that only eight column scales and bias values are live
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
+      const int n = piece_column(n_base, q, lg);
+      const bool full = ALIGNED || n + 8 <= a.N;
       float sb[8], bias[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const int ne = n + q * 8 + e < a.N ? n + q * 8 + e : a.N - 1;
+        const int ne = n + e < a.N ? n + e : a.N - 1;
         sb[e] = a.ws[a.ws_per_col ? ne : 0];
         bias[e] = a.bias ? load_as_float(a.bias, ne, a.bias_dtype) : 0.f;
       }
 #pragma unroll
       for (int j = 0; j < kTM; ++j) {
         const int m = m_base + j * 16 + l16;
-        if (m >= a.M) continue;
+        if (!ALIGNED && m >= a.M) continue;
         const float sa = a.xs[a.xs_per_row ? m : 0];
         uint32_t w[4];
 #pragma unroll
@@ -344,13 +361,13 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
             w[h] = pack_bf16(bits_to_float(w[h] << 16) + bias[4 * (h >> 1) + e0],
                              bits_to_float(w[h] & 0xFFFF0000u) + bias[4 * (h >> 1) + e0 + 1]);
         }
-        uint16_t* const cp = reinterpret_cast<uint16_t*>(a.C) + (int64_t)m * a.ldc + n + q * 8;
+        uint16_t* const cp = reinterpret_cast<uint16_t*>(a.C) + (int64_t)m * a.ldc + n;
         if (full) {
           *reinterpret_cast<u32x4*>(cp) = u32x4{w[0], w[1], w[2], w[3]};
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (n + q * 8 + e < a.N) cp[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+            if (n + e < a.N) cp[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
         }
       }
     }
@@ -359,22 +376,24 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
 #pragma unroll
   for (int j = 0; j < kTM; ++j) {
     const int m = m_base + j * 16 + l16;
-    if (m >= a.M) continue;
-    uint16_t* const cp = reinterpret_cast<uint16_t*>(a.C) + (int64_t)m * a.ldc + n;
+    if (!ALIGNED && m >= a.M) continue;
+    uint16_t* const row = reinterpret_cast<uint16_t*>(a.C) + (int64_t)m * a.ldc;
     uint32_t w[16];
 #pragma unroll
     for (int t = 0; t < kTN; ++t) {
       w[2 * t] = pack_bf16(acc[t][j][0], acc[t][j][1]);
       w[2 * t + 1] = pack_bf16(acc[t][j][2], acc[t][j][3]);
     }
-    if (full) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        *reinterpret_cast<u32x4*>(cp + q * 8) = u32x4{w[4 * q], w[4 * q + 1], w[4 * q + 2], w[4 * q + 3]};
-    } else {
+    for (int q = 0; q < 4; ++q) {
+      const int n = piece_column(n_base, q, lg);
+      if (ALIGNED || n + 8 <= a.N) {
+        *reinterpret_cast<u32x4*>(row + n) = u32x4{w[4 * q], w[4 * q + 1], w[4 * q + 2], w[4 * q + 3]};
+      } else {
 #pragma unroll
-      for (int e = 0; e < 32; ++e)
-        if (n + e < a.N) cp[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+        for (int e = 0; e < 8; ++e)
+          if (n + e < a.N) row[n + e] = (uint16_t)(w[4 * q + (e >> 1)] >> (16 * (e & 1)));
+      }
     }
   }
 }
@@ -429,7 +448,6 @@ __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (
   // Last to arrive.  Its own sums are in the workspace like everybody's, so the accumulators are free:
   // half of the piece (16 columns per lane and row) is summed at a time, every range's loads in flight together
   // with the running sum.
-  const int n = n_base + lg * 32;
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     v4f r[kTN / 2][kTM];
@@ -451,26 +469,28 @@ __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (
           if (q == first) r[t][j] = tmp[t][j]; else r[t][j] += tmp[t][j];
         }
     }
-    // 16 consecutive columns per lane and row: two 16-byte stores, or single elements at the ragged edge
-    const int nh = n + half * 16;
+    // two pieces of eight columns per lane and row: 16-byte stores, or single elements at the ragged edge
 #pragma unroll
     for (int j = 0; j < kTM; ++j) {
       const int m = m_base + j * 16 + l16;
       if (m >= a.g.M) continue;
-      uint16_t* const cp = reinterpret_cast<uint16_t*>(a.g.C) + (int64_t)m * a.g.ldc + nh;
+      uint16_t* const row = reinterpret_cast<uint16_t*>(a.g.C) + (int64_t)m * a.g.ldc;
       uint32_t w[8];
 #pragma unroll
       for (int t = 0; t < kTN / 2; ++t) {
         w[2 * t] = pack_bf16(r[t][j][0], r[t][j][1]);
         w[2 * t + 1] = pack_bf16(r[t][j][2], r[t][j][3]);
       }
-      if (nh + 16 <= a.g.N) {
-        *reinterpret_cast<u32x4*>(cp) = u32x4{w[0], w[1], w[2], w[3]};
-        *reinterpret_cast<u32x4*>(cp + 8) = u32x4{w[4], w[5], w[6], w[7]};
-      } else {
 #pragma unroll
-        for (int e = 0; e < 16; ++e)
-          if (nh + e < a.g.N) cp[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+      for (int qq = 0; qq < 2; ++qq) {
+        const int n = piece_column(n_base, half * 2 + qq, lg);
+        if (n + 8 <= a.g.N) {
+          *reinterpret_cast<u32x4*>(row + n) = u32x4{w[4 * qq], w[4 * qq + 1], w[4 * qq + 2], w[4 * qq + 3]};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n + e < a.g.N) row[n + e] = (uint16_t)(w[4 * qq + (e >> 1)] >> (16 * (e & 1)));
+        }
       }
     }
   }
@@ -507,6 +527,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     total = my_tiles * g.KB;
   }
   if (total <= 0) return;  // uniform over the block
+  for (int i = (int)(blockIdx.x & 15) * a.stagger; i > 0; --i) __builtin_amdgcn_s_sleep(15);
 
   // ---- the stage being loaded
   Walk lw;
@@ -616,7 +637,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     pending = false;
   };
   auto flush_whole_tile = [&]() __attribute__((always_inline)) {
-    store_tile<MODE>(g, acc, pend_m, pend_n, l16, lg);
+    store_tile<MODE, ALIGNED>(g, acc, pend_m, pend_n, l16, lg);
     clear_acc();
   };
   auto flush_partial_tile = [&]() __attribute__((always_inline)) {
@@ -626,8 +647,16 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   };
 
   int rw_slot = 0, rx_slot = 0;  // LDS slots of the stage being read
+  // The stores of a finished tile are counted by vmcnt like the loads, in issue order.  Where their number is
+  // known (kStoresPerTile, aligned shapes in block mode) the waits of the following slots allow that many
+  // younger operations more, so that nobody waits for the stores to reach memory before the first load issued
+  // after them is needed: all compute units finish tiles at about the same time, and 32 MB of results take
+  // several microseconds to drain.
+  constexpr bool kRelaxedStoreWaits = ALIGNED && MODE == kModeBlock;
+  bool flushed_prev = false;  // this wavefront stored a tile in its previous fetch phase
   FG_PP_STAMPS_DECLARE;
   auto run_steps = [&](int t_begin, int t_end) __attribute__((always_inline)) {
+  flushed_prev = false;  // every instance of this loop ends with all vector-memory operations complete
   for (int T = t_begin; T < t_end; ++T) {
     // ================= fetch(T)
     // Scales of this step were requested a step ago; the only younger vector-memory operations are the eight
@@ -637,7 +666,8 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     const bool more = T + 1 < total;
     float ws = 1.f;
     if (MODE == kModeBlock) {
-      wait_and_take<8>(xs, xs_nxt);
+      if (kRelaxedStoreWaits && flushed_prev) wait_and_take<8 + kStoresPerTile>(xs, xs_nxt);
+      else wait_and_take<8>(xs, xs_nxt);
       if (more) request_scales();  // of step T+1; the pointer was moved there a step ago
       ws = *(const __attribute__((address_space(4))) float*)ws_ptr;
     }
@@ -687,13 +717,18 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     // B's weights of stage T+1, issued a step ago, must have landed before the barrier; the scale requests
     // and the tile loads of this slot are younger.
     if (grp == 1) {
-      if (more && MODE == kModeBlock) wait_vmem<12>(); else wait_vmem<8>();
+      if (kRelaxedStoreWaits && flushed_prev) {
+        if (more) wait_vmem<12 + kStoresPerTile>(); else wait_vmem<8 + kStoresPerTile>();
+      } else {
+        if (more && MODE == kModeBlock) wait_vmem<12>(); else wait_vmem<8>();
+      }
     }
     if (MODE == kModeBlock) {
 #pragma unroll
       for (int j = 0; j < kTM; ++j) sc[j] = xs[j] * ws;
     }
     FG_PP_STAMP(4);
+    const bool flushed_now = pending;
     if (pending) flush_whole_tile();  // after the waits, so that no wait of this slot covers the stores
     __builtin_amdgcn_s_barrier();
     FG_PP_STAMP(5);
@@ -725,7 +760,10 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     }
     __builtin_amdgcn_s_setprio(kFetchPrio);
     FG_PP_STAMP(6);
-    if (grp == 0) wait_vmem_all();  // A's share of stage T+1 has landed
+    if (grp == 0) {  // A's share of stage T+1 has landed
+      if (kRelaxedStoreWaits && flushed_now) wait_vmem<kStoresPerTile>(); else wait_vmem_all();
+    }
+    flushed_prev = flushed_now;
     FG_PP_STAMP(7);
     __builtin_amdgcn_s_barrier();
 
@@ -878,6 +916,14 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     a.counters = reinterpret_cast<unsigned int*>(workspace);
     a.partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
     grid = sk.grid;
+  }
+  // Many whole tiles per block, each computed faster than the memory takes a batch of result tiles
+  // (256 x 256 bf16 per unit at ~3.3 TB/s; a K-block takes ~1.66 us): the run is bound by the stores, and
+  // starting the blocks spread over one tile time lets the stores of some overlap the MFMAs of others
+  // (M = 4096, N = 32768, K = 512: 113 -> 98 us).  Everywhere else the delay only costs.
+  if (!a.sk && tiles >= 6 * (int64_t)grid) {
+    const double tile_us = 1.66 * g.KB, batch_us = grid * 131072.0 / 3.3e6;
+    if (tile_us < batch_us) a.stagger = (int)(tile_us * 1.6e3 / 1000.0 / 16 + 0.5);  // 1.6 GHz, ~1000 cycles a sleep, 16 start slots
   }
   const bool aligned = g.M % kBM == 0 && g.N % kBN == 0;
   void (*kern)(PpArgs);
