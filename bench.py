@@ -38,17 +38,18 @@ DSV3_NK = [(2112, 7168), (24576, 1536), (32768, 512), (7168, 16384), (4608, 7168
 DSV3_M = [1, 8, 64, 512, 2048, 4096]
 CACHE_BYTES = 512 << 20   # rotate small-M weights through at least this much memory
 
-# Bytes that crossed the L2 <-> memory-fabric boundary in one launch of the M = 4096 persistent kernel, from two
+# Bytes that crossed the L2 <-> memory-fabric boundary in one M = 4096 call (the persistent kernel and, where the
+# call makes one, the transposition of the activation scales before it), from two
 # hardware-counter runs of `bench.py --counter-pass` (FETCH_SIZE, then WRITE_SIZE, in KiB per dispatch), each
 # scaled by what the same counter read for the 256 MiB device copy issued first in that run (FETCH_SIZE read
 # half of the copied bytes, factor 2.0; WRITE_SIZE read all of them, factor 1.0).  (N, K) -> (fetch, write) KiB.
 TRAFFIC_M4096_KIB = {
-    (2112, 7168): (2.0 * 63233.8, 16896.0),
-    (24576, 1536): (2.0 * 110835.4, 196608.0),
-    (32768, 512): (2.0 * 47731.1, 262144.2),
-    (7168, 16384): (2.0 * 364853.2, 57351.3),
-    (4608, 7168): (2.0 * 574931.8, 158697.7),   # stream-K launch: operand panels no longer shared in L2
-    (7168, 2304): (2.0 * 51177.8, 57344.2),
+    (2112, 7168): (2.0 * 63337.8, 17792.0),
+    (24576, 1536): (2.0 * 111908.5, 196800.6),
+    (32768, 512): (2.0 * 45767.8, 262147.8),
+    (7168, 16384): (2.0 * 367050.9, 59392.0),
+    (4608, 7168): (2.0 * 124243.4, 37760.0),
+    (7168, 2304): (2.0 * 51552.4, 57632.0),
 }
 
 
@@ -205,7 +206,7 @@ def main():
                 "flops_per_launch": big_flops / len(big), "algorithmic_bytes_per_launch":
                     sum(gemm_bytes(d["M"], d["N"], d["K"]) for d in big) / len(big),
                 "avg_launch_us": round(big_time * 1e6 / len(big), 2),
-                "kernel": "fp8_gemm_pingpong_kernel, the six M=4096 launches of the sweep"}
+                "kernel": "fp8_gemm_pingpong_kernel (with the scale transposition that precedes it), the six M=4096 calls of the sweep"}
     small = [d for d in detail if d["M"] <= 8]
     small_bytes = sum(gemm_bytes(d["M"], d["N"], d["K"]) for d in small)
     small_time = sum(d["us"] for d in small) * 1e-6

@@ -852,26 +852,42 @@ SkPlan plan_stream_k(int64_t tiles, int KB, int cus) {
 // keep sweeping the L1), as many line requests as the tiles themselves need, and the tile loads queue behind
 // them in the address unit: measured 20 % of the run time on K = 16384.  From the transposed copy a
 // wavefront's 64 scales of a K-block are 256 contiguous bytes.
+// One thread per row and 16 K-blocks: reads run along a row (16-byte loads where the layout allows), writes
+// run along M and are contiguous over the threads of a block.
+constexpr int kTransposeKbPerBlock = 16;
 __global__ __launch_bounds__(256) void transpose_scales_kernel(const float* __restrict__ xs, int64_t rs, int64_t cs, int M,
                                                                int KB, float* __restrict__ out) {
-  __shared__ float tile[32][33];
-  const int kb0 = (int)blockIdx.x * 32, m0 = (int)blockIdx.y * 32;
-  const int tx = (int)threadIdx.x & 31, ty = (int)threadIdx.x >> 5;
+  const int m = (int)blockIdx.x * 256 + (int)threadIdx.x;
+  const int kb0 = (int)blockIdx.y * kTransposeKbPerBlock;
+  if (m >= M) return;
+  const float* const row = xs + (int64_t)m * rs;
+  const bool vec = cs == 1 && (rs & 3) == 0 && ((uintptr_t)xs & 15) == 0;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = m0 + ty + i * 8, kb = kb0 + tx;
-    if (m < M && kb < KB) tile[ty + i * 8][tx] = xs[(int64_t)m * rs + (int64_t)kb * cs];
-  }
-  __syncthreads();
+  for (int i = 0; i < kTransposeKbPerBlock; i += 4) {
+    const int kb = kb0 + i;
+    float v[4];
+    if (vec && kb + 4 <= KB) {
+      const v4f q = *reinterpret_cast<const v4f*>(row + kb);
+      v[0] = q[0]; v[1] = q[1]; v[2] = q[2]; v[3] = q[3];
+    } else {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int kb = kb0 + ty + i * 8, m = m0 + tx;
-    if (m < M && kb < KB) out[(int64_t)kb * M + m] = tile[tx][ty + i * 8];
+      for (int e = 0; e < 4; ++e) v[e] = kb + e < KB ? row[(int64_t)(kb + e) * cs] : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (kb + e < KB) out[(int64_t)(kb + e) * M + m] = v[e];
   }
 }
 
-// rows of scales at least this many floats apart are worth transposing (below, 16 rows share a few lines)
-constexpr int64_t kTransposeMinRowStride = 4;
+// The extra launch costs ~5 us (it is all latency) and saves ~10 % of the GEMM: worth it for rows of scales at
+// least this many floats apart and a GEMM of more than ~50 us (a K-block takes ~1.66 us per round of tiles).
+constexpr int64_t kTransposeMinRowStride = 8;
+bool transposition_pays(int64_t tiles, int64_t KB, int cus) {
+  if (KB < kTransposeMinRowStride) return false;
+  const SkPlan sk = plan_stream_k(tiles, (int)KB, cus);
+  const double steps = sk.use ? 1.35 * (sk.q + 1) + 0.3 * KB + 14 : (double)ceil_div(tiles, (int64_t)cus) * (double)KB;
+  return steps * 1.66 > 50.0;
+}
 size_t transposed_scales_bytes(int64_t M, int64_t KB) { return (size_t)((M * KB * 4 + 255) / 256 * 256); }
 
 int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream) {
@@ -902,11 +918,12 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : 0;
   const size_t need = FG_WORKSPACE_COUNTER_BYTES + sk_bytes;
   // workspace: [counters][partial tiles, if the shape is one that shares tiles][transposed activation scales]
-  if (mode == kModeBlock && g.xs_rs >= kTransposeMinRowStride && workspace != nullptr && (uintptr_t)workspace % 16 == 0 &&
+  if (mode == kModeBlock && g.xs_rs >= kTransposeMinRowStride && transposition_pays(tiles, g.KB, cus) && workspace != nullptr &&
+      (uintptr_t)workspace % 16 == 0 &&
       workspace_bytes >= need + transposed_scales_bytes(g.M, g.KB)) {
     float* const xs_t = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + need);
-    hipLaunchKernelGGL(transpose_scales_kernel, dim3((uint32_t)ceil_div(g.KB, 32), (uint32_t)ceil_div(g.M, 32)), dim3(256), 0, stream,
-                       g.xs, g.xs_rs, g.xs_cs, g.M, g.KB, xs_t);
+    hipLaunchKernelGGL(transpose_scales_kernel, dim3((uint32_t)ceil_div(g.M, 256), (uint32_t)ceil_div(g.KB, kTransposeKbPerBlock)),
+                       dim3(256), 0, stream, g.xs, g.xs_rs, g.xs_cs, g.M, g.KB, xs_t);
     FG_CHECK_LAUNCH("transpose_scales_kernel");
     a.g.xs = xs_t; a.g.xs_rs = 1; a.g.xs_cs = g.M;
   }
@@ -959,7 +976,8 @@ size_t pingpong_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   const SkPlan sk = plan_stream_k(ceil_div(M, kBM) * ceil_div(N, kBN), (int)(K / 128), cu_count());
   const int64_t KB = K / 128;
   const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : 0;
-  const size_t tr_bytes = KB >= kTransposeMinRowStride ? transposed_scales_bytes(M, KB) : 0;  // for row-major scales
+  const size_t tr_bytes = transposition_pays(ceil_div(M, kBM) * ceil_div(N, kBN), KB, cu_count())
+                              ? transposed_scales_bytes(M, KB) : 0;  // for row-major scales
   return sk_bytes + tr_bytes != 0 ? FG_WORKSPACE_COUNTER_BYTES + sk_bytes + tr_bytes : 0;
 }
 
