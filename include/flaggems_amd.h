@@ -105,11 +105,13 @@ int fg_act_quant_bf16(const void* x, void* y, float* s, int64_t rows, int64_t co
  * c_dtype in {FG_BF16, FG_F16, FG_F32}.  Products are accumulated in fp32 per K-block, scaled,
  * and accumulated in fp32 across K-blocks; the result is rounded once to c_dtype.
  * Only block_n == block_k == 128 is implemented (FG_ERR_UNSUPPORTED otherwise).
- * `workspace` holds split-K partial sums.  fg_block_fp8_gemm_workspace_bytes(M, N, K) says how much the
- * kernels can use for the shape (0: none).  For M <= 64 that much is required (FG_ERR_WORKSPACE
- * otherwise); for larger M it is optional: with less, or with a null pointer, tiles are never shared
- * between blocks, which is slower for shapes whose tile count leaves much of the GPU idle, and gives the
- * same results to within fp32 summation order.  The caller zero-fills the first
+ * `workspace` holds split-K partial sums and, for long GEMMs, a transposed copy of As.
+ * fg_block_fp8_gemm_workspace_bytes(M, N, K) says how much the kernels can use for the shape (0: none).
+ * For M <= 64 that much is required (FG_ERR_WORKSPACE otherwise); for larger M it is optional: with less,
+ * or with a null pointer, tiles are never shared between blocks (slower for shapes whose tile count leaves
+ * much of the GPU idle; same results to within fp32 summation order) and row-major As is read as it is
+ * (10-20 % slower for M in the thousands; identical results).  As with unit row stride (column-major,
+ * as_row_stride == 1) is read in place in any case.  The caller zero-fills the first
  * FG_WORKSPACE_COUNTER_BYTES bytes once; every launch leaves them zero.  16-byte aligned.  Launches that
  * may run concurrently must not share a workspace.
  *
