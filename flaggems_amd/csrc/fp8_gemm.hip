@@ -175,7 +175,12 @@ struct TileCfg {
 // ---------------------------------------------------------------------------------------------
 // Main kernel
 // ---------------------------------------------------------------------------------------------
-template <int BM, int BN, int WM, int WN, int MODE, bool DIRECT>
+// SPLIT: the grid is tiles x a.splits and a block computes a range of K-blocks of its tile.  Every wavefront
+// publishes its fp32 sums in the workspace and counts itself in (one counter per tile and wavefront position);
+// the one that arrives last adds the sums of all splits in split order -- the same order whoever comes last --
+// and runs the epilogue.  For 32 < M <= 128, where a handful of 128 x 128 tiles would leave most of the GPU
+// idle and every K-block of a tile costs a full load latency.
+template <int BM, int BN, int WM, int WN, int MODE, bool DIRECT, bool SPLIT = false>
 __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
   using Cfg = TileCfg<BM, BN, WM, WN>;
   constexpr int NT = Cfg::kThreads;
@@ -190,8 +195,16 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave % WM, wave_n = wave / WM;
 
+  int tile_id = (int)blockIdx.x, split = 0;
+  if (SPLIT) {
+    const int n_tiles = a.tiles_m * a.tiles_n;
+    split = (int)blockIdx.x / n_tiles;
+    tile_id = (int)blockIdx.x - split * n_tiles;
+  }
+  const int kb_begin = SPLIT ? split * a.kb_per_split : 0;
+  const int kb_end = SPLIT ? (kb_begin + a.kb_per_split < a.KB ? kb_begin + a.kb_per_split : a.KB) : a.KB;
   int tile_m, tile_n;
-  tile_of_block(blockIdx.x, a.tiles_m, a.tiles_n, tile_m, tile_n);
+  tile_of_block(tile_id, a.tiles_m, a.tiles_n, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int wm0 = wave_m * Cfg::kWaveM, wn0 = wave_n * Cfg::kWaveN;
   const int l16 = lane & 15, lg = lane >> 4;
@@ -226,14 +239,14 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
   const float* ws_ptr = a.ws + (int64_t)wn_blk * a.ws_rs;
 
   // ---- prologue: stage 0
-  if (a.KB == 0) {
-    // K == 0: nothing to stage, the accumulators stay zero
+  if (kb_begin >= kb_end) {
+    // K == 0 (or an empty range): nothing to stage, the accumulators stay zero
   } else if (DIRECT) {
-    dt_w.issue(w_base, lds_w(0), wave);
-    dt_x.issue(x_base, lds_x(0), wave);
+    dt_w.issue(w_base + kb_begin * 128, lds_w(0), wave);
+    dt_x.issue(x_base + kb_begin * 128, lds_x(0), wave);
   } else {
-    st_w.load(a.W, a.ldw, n0, a.N - 1, 0, a.K, aligned16, tid);
-    st_x.load(a.X, a.ldx, m0, a.M - 1, 0, a.K, aligned16, tid);
+    st_w.load(a.W, a.ldw, n0, a.N - 1, kb_begin * 128, a.K, aligned16, tid);
+    st_x.load(a.X, a.ldx, m0, a.M - 1, kb_begin * 128, a.K, aligned16, tid);
     st_w.store(lds_w(0), tid);
     st_x.store(lds_x(0), tid);
   }
@@ -241,26 +254,26 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
   // tile-load wait at the top of an iteration, where they have been in flight for a whole iteration.
   // (A wait at the end of the iteration would also wait for the tile loads issued moments before.)
   float xs_pend = 0.f, ws_pend = 1.f, ws_cur = 1.f;
-  if (MODE == kModeBlock && a.KB > 0) {
+  if (MODE == kModeBlock && kb_begin < kb_end) {
     if (tid < BM) {
-      lds_xs[tid] = xs_ptr[0];
-      if (a.KB > 1) xs_pend = xs_ptr[a.xs_cs];
+      lds_xs[tid] = xs_ptr[(int64_t)kb_begin * a.xs_cs];
+      if (kb_begin + 1 < kb_end) xs_pend = xs_ptr[(int64_t)(kb_begin + 1) * a.xs_cs];
     }
-    ws_pend = ws_ptr[0];
+    ws_pend = ws_ptr[(int64_t)kb_begin * a.ws_cs];
   }
 
-  for (int kb = 0; kb < a.KB; ++kb) {
-    const int cur = kb & 1, nxt = cur ^ 1;
+  for (int kb = kb_begin; kb < kb_end; ++kb) {
+    const int cur = (kb - kb_begin) & 1, nxt = cur ^ 1;
     if (DIRECT) wait_vmem_all();
     __syncthreads();
 
-    const bool more = kb + 1 < a.KB;
+    const bool more = kb + 1 < kb_end;
     if (MODE == kModeBlock) {
       ws_cur = ws_pend;
       if (more) {
         if (tid < BM) {
           lds_xs[nxt * BM + tid] = xs_pend;  // scales of K-block kb+1, read after the next barrier
-          if (kb + 2 < a.KB) xs_pend = xs_ptr[(int64_t)(kb + 2) * a.xs_cs];
+          if (kb + 2 < kb_end) xs_pend = xs_ptr[(int64_t)(kb + 2) * a.xs_cs];
         }
         ws_pend = ws_ptr[(int64_t)(kb + 1) * a.ws_cs];
       }
@@ -346,6 +359,43 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
         st_x.store(lds_x(nxt), tid);
       }
     }
+  }
+
+  if (SPLIT && a.splits > 1) {
+    // element (i, j) of thread tid lives at ((i * TM + j) * NT + tid) * 16 bytes of the (tile, split) slot
+    constexpr int kSlotFloats = TN * TM * NT * 4;
+    const uint32_t t_off = (uint32_t)tid * 16u;
+    float* const mine = uniform_ptr(a.split_partials + ((size_t)tile_id * a.splits + split) * kSlotFloats);
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TM; ++j) store_x4_agent(mine + (i * TM + j) * NT * 4, t_off, acc[i][j]);
+    wait_vmem_all();
+    unsigned int* const cnt = a.split_counters + tile_id * (NT / 64) + wave;
+    unsigned int prev = 0;
+    if (lane == 0) prev = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    prev = (unsigned int)__builtin_amdgcn_readfirstlane((int)prev);
+    if (prev != (unsigned int)(a.splits - 1)) return;
+    for (int s = 0; s < a.splits; ++s) {
+      const float* const src = uniform_ptr(a.split_partials + ((size_t)tile_id * a.splits + s) * kSlotFloats);
+      v4f tmp[TN][TM];
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j) load_x4_agent(tmp[i][j], src + (i * TM + j) * NT * 4, t_off);
+#pragma unroll
+      for (int i = 0; i < TN; ++i)  // the values are operands of the wait, so no use can move above it
+#pragma unroll
+        for (int j = 0; j < TM; ++j) asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[i][j]) : : "memory");
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+          // plain assignment for the first split keeps "0 + x" out of the sum
+          if (s == 0) acc[i][j] = tmp[i][j]; else acc[i][j] += tmp[i][j];
+        }
+    }
+    if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
   // ---- epilogue
@@ -439,12 +489,66 @@ int launch_cfg(GemmArgs a, hipStream_t stream) {
   return FG_OK;
 }
 
+// 32 < M <= 128 with few 128 x 128 tiles: K split over blocks so that about two blocks per compute unit are
+// resident (a K-block of one tile costs a full load latency, ~1.8 us; the loads of several blocks overlap).
+struct TileSplitPlan {
+  bool use;
+  int splits, kb_per_split;
+  size_t workspace_bytes;
+};
+constexpr int kSplitTile = 128, kSplitWaves = 4;
+TileSplitPlan plan_tile_split(int64_t M, int64_t N, int64_t K) {
+  TileSplitPlan p = {false, 1, 0, 0};
+  if (M <= 32 || M > 128 || K % 128 != 0) return p;
+  const int64_t KB = K / 128;
+  const int64_t tiles = ceil_div(M, kSplitTile) * ceil_div(N, kSplitTile);
+  if (tiles * kSplitWaves * 4 > FG_WORKSPACE_COUNTER_BYTES) return p;
+  if (tiles > 128) return p;  // enough tiles to go round
+  // up to 64 rows the decode kernels are the alternative: they win unless K is long (measured: K = 7168 and
+  // 16384 faster here, K = 1024 ... 2304 faster there)
+  if (M <= 64 && KB < 32) return p;
+  int64_t splits = (320 + tiles / 2) / tiles;  // ~1.25 blocks per compute unit
+  if (splits > KB / 4) splits = KB / 4;  // at least four K-blocks per block
+  if (splits > 8) splits = 8;            // the wavefront that finishes a tile reads the splits one after another
+  if (splits < 2) return p;
+  p.kb_per_split = (int)ceil_div(KB, splits);
+  p.splits = (int)ceil_div(KB, (int64_t)p.kb_per_split);
+  p.workspace_bytes = FG_WORKSPACE_COUNTER_BYTES + (size_t)tiles * p.splits * kSplitTile * kSplitTile * sizeof(float);
+  p.use = p.splits >= 2;
+  return p;
+}
+
+template <int MODE>
+int launch_tile_split(GemmArgs a, const TileSplitPlan& plan, void* workspace, hipStream_t stream) {
+  using Cfg = TileCfg<kSplitTile, kSplitTile, 2, 2>;
+  a.tiles_m = (int)ceil_div(a.M, kSplitTile);
+  a.tiles_n = (int)ceil_div(a.N, kSplitTile);
+  a.splits = plan.splits;
+  a.kb_per_split = plan.kb_per_split;
+  a.split_counters = reinterpret_cast<unsigned int*>(workspace);
+  a.split_partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
+  auto kern = fp8_gemm_kernel<kSplitTile, kSplitTile, 2, 2, MODE, true, true>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
+    if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
+    attr_set = true;
+  }
+  const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n * a.splits;
+  hipLaunchKernelGGL(kern, dim3((uint32_t)blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, a);
+  FG_CHECK_LAUNCH("fp8_gemm_kernel (K split)");
+  return FG_OK;
+}
+
 template <int MODE>
 int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   const bool direct = (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) &&
                       (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
                       ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
   if (direct) {
+    const TileSplitPlan ts = plan_tile_split(a.M, a.N, a.K);
+    if (ts.use && workspace != nullptr && workspace_bytes >= ts.workspace_bytes && (uintptr_t)workspace % 16 == 0)
+      return launch_tile_split<MODE>(a, ts, workspace, stream);
     const SmallMPlan plan = plan_small_m(a.M, a.N, a.K);
     if (plan.use) return launch_small_m(a, MODE, plan, workspace, workspace_bytes, stream);
   }
@@ -473,9 +577,12 @@ int check_common(const void* A, const void* B, const void* C, int64_t lda, int64
 }  // namespace fg
 
 extern "C" size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  // the largest any kernel that may take the shape can use
+  size_t need = fg::plan_tile_split(M, N, K).workspace_bytes;
   const fg::SmallMPlan plan = fg::plan_small_m(M, N, K);
-  if (plan.use) return plan.workspace_bytes;
-  return fg::pingpong_workspace_bytes(M, N, K);
+  if (plan.use && plan.workspace_bytes > need) need = plan.workspace_bytes;
+  const size_t pp = fg::pingpong_workspace_bytes(M, N, K);
+  return pp > need ? pp : need;
 }
 extern "C" size_t fg_scaled_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return fg_block_fp8_gemm_workspace_bytes(M, N, K);

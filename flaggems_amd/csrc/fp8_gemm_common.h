@@ -20,6 +20,11 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int c_dtype, bias_dtype;
   int xs_per_row, ws_per_col;
+  // tile kernel with K split over blocks (fp8_gemm.hip): block b computes K-blocks
+  // [split * kb_per_split, ...) of tile b % tiles, split = b / tiles
+  int splits, kb_per_split;
+  float* split_partials;
+  unsigned int* split_counters;
 };
 
 // s_waitcnt vmcnt(0) with expcnt/lgkmcnt left at their maxima (gfx9 encoding)
@@ -74,6 +79,27 @@ __device__ __forceinline__ v4f mfma_fp8_16x16x128(v8i a, v8i b, v4f c) {
   // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled instruction
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
 }
+
+// Operands of inline assembly with an "s" constraint must be in scalar registers; this makes the compiler see
+// that a (uniform) pointer is.
+template <typename T>
+__device__ __forceinline__ T* uniform_ptr(T* p) {
+  const uint64_t v = (uint64_t)p;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return (T*)(((uint64_t)hi << 32) | lo);
+}
+
+// 16-byte accesses that other XCDs can see: written through to memory / read past this XCD's L2 (the same
+// cache-control bit the compiler sets for agent-scope atomic loads and stores).  Not tracked by the
+// compiler's wait-count insertion: callers wait explicitly.
+__device__ __forceinline__ void store_x4_agent(float* base, uint32_t byte_off, const v4f& v) {
+  asm volatile("global_store_dwordx4 %0, %1, %2 sc1" : : "v"(byte_off), "v"(v), "s"(base) : "memory");
+}
+__device__ __forceinline__ void load_x4_agent(v4f& v, const float* base, uint32_t byte_off) {
+  asm volatile("global_load_dwordx4 %0, %1, %2 sc1" : "=v"(v) : "v"(byte_off), "s"(base) : "memory");
+}
+
 
 // Small-M (decode) path, fp8_gemm_smallm.hip.  `use` reports whether the kernel takes the problem.
 struct SmallMPlan {

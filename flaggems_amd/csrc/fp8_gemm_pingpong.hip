@@ -284,14 +284,6 @@ __device__ __forceinline__ void scale_into(v4f& acc, const v4f& p, float s) {
 // explicit count.  Left to the compiler, the wait for these four values becomes vmcnt(0) in the middle of a
 // slot, which also waits for the tile loads issued after them.  The destination is an in/out operand so that
 // the value keeps one register across loop iterations.
-// The "s" operands below must be in scalar registers; the value is uniform, this makes the compiler see it.
-template <typename T>
-__device__ __forceinline__ T* uniform_ptr(T* p) {
-  const uint64_t v = (uint64_t)p;
-  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
-  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
-  return (T*)(((uint64_t)hi << 32) | lo);
-}
 __device__ __forceinline__ void load_f32_untracked(float& v, uint32_t byte_off, const float* base) {
   asm volatile("global_load_dword %0, %1, %2" : "+v"(v) : "v"(byte_off), "s"(base) : "memory");
 }
@@ -396,16 +388,6 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
       }
     }
   }
-}
-
-// 16-byte accesses that other XCDs can see: written through to memory / read past this XCD's L2 (the same
-// cache-control bit the compiler sets for agent-scope atomic loads and stores).  Not tracked by the
-// compiler's wait-count insertion: callers wait explicitly.
-__device__ __forceinline__ void store_x4_agent(float* base, uint32_t byte_off, const v4f& v) {
-  asm volatile("global_store_dwordx4 %0, %1, %2 sc1" : : "v"(byte_off), "v"(v), "s"(base) : "memory");
-}
-__device__ __forceinline__ void load_x4_agent(v4f& v, const float* base, uint32_t byte_off) {
-  asm volatile("global_load_dwordx4 %0, %1, %2 sc1" : "=v"(v) : "v"(byte_off), "s"(base) : "memory");
 }
 
 // Range arithmetic of the stream-K split (all uniform).

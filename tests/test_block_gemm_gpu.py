@@ -89,6 +89,24 @@ def test_persistent_kernel_several_rounds_ragged_edges_and_strides():
     assert torch.equal(got3.view(torch.int16), got.view(torch.int16))
 
 
+@pytest.mark.parametrize("M,N,K", [(100, 520, 2048), (128, 1300, 4096), (48, 384, 8192)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_few_tiles_split_along_k(M, N, K, dtype):
+    """32 < M <= 128 with a handful of 128 x 128 tiles: the tile kernel splits K over blocks and the last
+    wavefront of a tile adds the partial sums in split order.  Against the oracle in every output type, and
+    bit-identical on reruns."""
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=9)
+    want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
+    args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    got = flag_gems.w8a8_block_fp8_matmul(*args, output_dtype=dtype)
+    assert got.dtype == dtype and got.shape == (M, N)
+    tol = dict(rtol=1e-4, atol=2e-4) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(got.cpu().float(), want, **tol)
+    for _ in range(3):
+        again = flag_gems.w8a8_block_fp8_matmul(*args, output_dtype=dtype)
+        assert torch.equal(again.view(torch.int8), got.view(torch.int8))
+
+
 @pytest.mark.parametrize("M,N,K", [(768, 1024, 2048), (300, 520, 1024)])
 def test_activation_scales_in_either_layout_give_the_same_bits(M, N, K):
     """The persistent kernel reads activation scales K-block by K-block for 64 rows at a time.  Row-major
