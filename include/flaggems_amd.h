@@ -107,9 +107,10 @@ int fg_act_quant_bf16(const void* x, void* y, float* s, int64_t rows, int64_t co
  * Only block_n == block_k == 128 is implemented (FG_ERR_UNSUPPORTED otherwise).
  * `workspace` holds split-K partial sums and, for long GEMMs, a transposed copy of As.
  * fg_block_fp8_gemm_workspace_bytes(M, N, K) says how much the kernels can use for the shape (0: none).
- * For M <= 64 that much is required (FG_ERR_WORKSPACE otherwise); for larger M it is optional: with less,
- * or with a null pointer, tiles are never shared between blocks (slower for shapes whose tile count leaves
- * much of the GPU idle; same results to within fp32 summation order) and row-major As is read as it is
+ * For M <= 32 that much is required when it is not 0 (FG_ERR_WORKSPACE otherwise); for larger M it is
+ * optional: with less, or with a null pointer, K is never split between blocks (slower for shapes whose tile
+ * count leaves much of the GPU idle; same results to within fp32 summation order; M in 33..64 then needs what
+ * the decode kernels ask for, which is less) and row-major As is read as it is
  * (10-20 % slower for M in the thousands; identical results).  As with unit row stride (column-major,
  * as_row_stride == 1) is read in place in any case.  The caller zero-fills the first
  * FG_WORKSPACE_COUNTER_BYTES bytes once; every launch leaves them zero.  16-byte aligned.  Launches that
