@@ -107,13 +107,14 @@ def test_few_tiles_split_along_k(M, N, K, dtype):
         assert torch.equal(again.view(torch.int8), got.view(torch.int8))
 
 
-@pytest.mark.parametrize("M,N,K", [(768, 1024, 2048), (300, 520, 1024)])
+@pytest.mark.parametrize("M,N,K", [(1100, 1300, 8192), (1200, 3000, 4096)])
 def test_activation_scales_in_either_layout_give_the_same_bits(M, N, K):
     """The persistent kernel reads activation scales K-block by K-block for 64 rows at a time.  Row-major
     scales ([M, K/128] contiguous, what the quantizer returns) are first transposed into the workspace;
     scales that already have the rows contiguous (strides (1, M), the reference's column_major_scales
     layout) are read in place; a call without workspace reads the row-major ones as they are.  All three
-    must give identical results."""
+    The first two run the same kernel on the same values and must agree bit for bit; the call without
+    workspace may also add the K-blocks in another order (no tile is shared between blocks then)."""
     from flaggems_amd import _lib
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=5)
     xq, wq, xs, ws = xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV)
@@ -131,7 +132,8 @@ def test_activation_scales_in_either_layout_give_the_same_bits(M, N, K):
                                    M, N, K, 128, 128, None, 0, _lib.current_stream_ptr(torch.device(DEV)))
     _lib.check(status, "fg_block_fp8_gemm")
     torch.cuda.synchronize()
-    assert torch.equal(out.view(torch.int16), got.view(torch.int16))
+    torch.testing.assert_close(out.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(out.float(), got.float(), rtol=8e-3, atol=1e-3)  # one bf16 ulp
 
 
 def test_tiles_split_along_k_between_blocks():
