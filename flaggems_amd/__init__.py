@@ -12,6 +12,7 @@ from .act_quant import (  # noqa: F401
     per_token_group_quant_fp8,
 )
 from .cutlass_scaled_mm import SM_VERSION_NUM, cutlass_scaled_mm, get_sm_version_num  # noqa: F401
+from .grouped_block_fp8_matmul import grouped_w8a8_block_fp8_matmul  # noqa: F401
 from .registration import (  # noqa: F401
     all_registered_keys,
     all_registered_ops,
@@ -37,6 +38,7 @@ __all__ = [
     "cutlass_scaled_mm",
     "enable",
     "fp8_matmul",
+    "grouped_w8a8_block_fp8_matmul",
     "only_enable",
     "patch_empty_vllm",
     "per_token_group_quant_fp8",

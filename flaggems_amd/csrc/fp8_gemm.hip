@@ -616,6 +616,47 @@ extern "C" int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int6
   return launch_gemm<kModeBlock>(a, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
+extern "C" size_t fg_grouped_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  (void)N;
+  return fg::grouped_workspace_bytes(M, K);
+}
+
+extern "C" int fg_grouped_block_fp8_gemm(const void* A, int64_t lda,
+                                         const void* B, int64_t ldb, int64_t b_group_stride,
+                                         const float* As, int64_t as_row_stride, int64_t as_col_stride,
+                                         const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride, int64_t bs_group_stride,
+                                         const int32_t* group_ends, int64_t n_groups,
+                                         void* C, int64_t ldc, int c_dtype,
+                                         int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
+                                         void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace fg;
+  const char* const who = "fg_grouped_block_fp8_gemm";
+  if (block_n != 128 || block_k != 128)
+    FG_FAIL(FG_ERR_UNSUPPORTED, "%s: only 128x128 scale blocks are implemented (got %lld x %lld)", who,
+            (long long)block_n, (long long)block_k);
+  if (c_dtype != FG_BF16) FG_FAIL(FG_ERR_UNSUPPORTED, "%s: the result must be bf16 (c_dtype %d)", who, c_dtype);
+  if (n_groups <= 0) FG_FAIL(FG_ERR_INVALID_ARG, "%s: %lld groups", who, (long long)n_groups);
+  int rc = check_common(A, B, C, lda, ldb, ldc, M, N, K, who);
+  if (rc < 0) return rc;
+  if (rc == 1) return FG_OK;
+  if (!group_ends) FG_FAIL(FG_ERR_INVALID_ARG, "%s: null group table", who);
+  if (K == 0 || K % 128 != 0) FG_FAIL(FG_ERR_UNSUPPORTED, "%s: K = %lld is not a positive multiple of 128", who, (long long)K);
+  if (!As || !Bs) FG_FAIL(FG_ERR_INVALID_ARG, "%s: null scale pointer", who);
+  if (b_group_stride < 0 || bs_group_stride < 0) FG_FAIL(FG_ERR_INVALID_ARG, "%s: negative group stride", who);
+  if (!(lda % 16 == 0 && ldb % 16 == 0 && lda < (1 << 23) && ldb < (1 << 23) && (uintptr_t)A % 16 == 0 &&
+        (uintptr_t)B % 16 == 0 && b_group_stride % 16 == 0))
+    FG_FAIL(FG_ERR_UNSUPPORTED, "%s: operands must be 16-byte aligned with row and group strides that are multiples of 16 below 2^23", who);
+  GemmArgs a = {};
+  a.X = (const uint8_t*)A; a.W = (const uint8_t*)B; a.C = C;
+  a.xs = As; a.ws = Bs; a.bias = nullptr;
+  a.ldx = lda; a.ldw = ldb; a.ldc = ldc;
+  a.xs_rs = as_row_stride; a.xs_cs = as_col_stride; a.ws_rs = bs_row_stride; a.ws_cs = bs_col_stride;
+  a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)(K / 128);
+  a.c_dtype = c_dtype;
+  GroupedGemm grouped = {group_ends, n_groups, b_group_stride, bs_group_stride};
+  return launch_grouped(a, grouped, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
 extern "C" int fg_scaled_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
                                   const float* a_scale, int a_scale_per_row,
                                   const float* b_scale, int b_scale_per_col,

@@ -126,4 +126,16 @@ int launch_pingpong(const GemmArgs& a, int mode, void* workspace, size_t workspa
 // workspace that lets the persistent kernel split tiles along K between blocks (0: never useful for this shape)
 size_t pingpong_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
+// Grouped problem for the persistent kernel: rows [ends[e-1], ends[e]) of X and C (ends[-1] = 0; a device table
+// of cumulative int32 ends) meet weight matrix e, w_group_stride bytes and ws_group_stride scale floats after
+// matrix 0.  Block scales, bf16 result; a.M is the total row count, a.W / a.ws point at matrix 0.
+struct GroupedGemm {
+  const int* ends;
+  int64_t n_groups;
+  int64_t w_group_stride, ws_group_stride;
+};
+int launch_grouped(const GemmArgs& a, const GroupedGemm& grouped, void* workspace, size_t workspace_bytes, hipStream_t stream);
+// workspace that lets launch_grouped read row-major activation scales from a transposed copy
+size_t grouped_workspace_bytes(int64_t M, int64_t K);
+
 }  // namespace fg

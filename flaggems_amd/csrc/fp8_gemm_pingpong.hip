@@ -108,6 +108,15 @@ struct PpArgs {
   // each time stalling on the stores for longer than a tile takes to compute; spread over the time the
   // memory needs for one such batch, the stores of one unit overlap the MFMAs of the others.
   int stagger;
+  // Grouped problem (groups != nullptr): the rows of X and C are cut into n_groups consecutive segments,
+  // segment e ends before row groups[e] (cumulative ends, the `offs` convention of the reference's grouped GEMM,
+  // src/flag_gems/ops/scaled_grouped_mm.py:111-114) and is multiplied by weight matrix e (w_group_stride bytes and
+  // ws_group_stride floats apart).  Tiles never straddle segments: segment e has ceil(rows_e / 256) tile rows.  The
+  // host cannot know the tile count without reading groups back, so it passes an upper bound in n_tiles and
+  // g.tiles_m and the kernel derives the real ones.
+  const int* groups;
+  int n_groups;
+  int64_t w_group_stride, ws_group_stride;
 };
 
 constexpr int kPartialFloatsPerWave = 64 * 128;                      // one wavefront's 64 x 128 results
@@ -161,18 +170,42 @@ __device__ __forceinline__ int piece_column(int n_base, int q, int lg) { return 
 // run at different distances: the step being multiplied, the step whose scales are being fetched (one
 // ahead) and the stage being loaded (one or two ahead).  A tile change costs two integer divisions and
 // happens once per K / 128 steps; everything else per step is an add.
-struct Walk {
+// End of segment e of a grouped problem (uniform, a scalar load), forced into [begin, M]: a table that is not
+// ascending or runs past the rows must not send loads or stores outside the operands.
+__device__ __forceinline__ int segment_end(const PpArgs& a, int e, int begin) {
+  int end = ((const __attribute__((address_space(4))) int*)a.groups)[e];
+  end = end < a.g.M ? end : a.g.M;
+  return end > begin ? end : begin;
+}
+
+template <bool GROUPED>
+struct WalkT {
   int idx, kb, m0, n0;  // idx: virtual id (data-parallel rounds) or tile number (stream-K)
+  int m_end, group;     // first row past the tile's segment (M when the problem is not grouped); its weight matrix
+  int n_tiles, tiles_m; // of the whole problem (a grouped problem's are counted by the kernel)
   __device__ __forceinline__ void locate(const PpArgs& a) {
     int tm = 0, tn = 0;
-    if (idx < a.n_tiles) {
-      if (a.sk) tile_of_sid(idx, a.g.tiles_m, a.g.tiles_n, tm, tn);
-      else tile_of_index(idx, a.g.tiles_m, a.g.tiles_n, tm, tn);
+    if (idx < n_tiles) {
+      if (a.sk) tile_of_sid(idx, tiles_m, a.g.tiles_n, tm, tn);
+      else tile_of_index(idx, tiles_m, a.g.tiles_n, tm, tn);
     }
     m0 = tm * kBM; n0 = tn * kBN;
+    m_end = a.g.M; group = 0;
+    if (GROUPED) {
+      // tile row tm of the whole problem -> segment and tile row inside it
+      int begin = 0, t = tm, e = 0, end = 0;
+      for (; e < a.n_groups; ++e) {
+        end = segment_end(a, e, begin);
+        const int nt = (end - begin + kBM - 1) / kBM;
+        if (t < nt) break;
+        t -= nt;
+        begin = end;
+      }
+      m0 = begin + t * kBM; m_end = end; group = e < a.n_groups ? e : 0;
+    }
   }
-  __device__ __forceinline__ void start(const PpArgs& a, int first_idx, int first_kb) {
-    idx = first_idx; kb = first_kb;
+  __device__ __forceinline__ void start(const PpArgs& a, int first_idx, int first_kb, int n_tiles_, int tiles_m_) {
+    idx = first_idx; kb = first_kb; n_tiles = n_tiles_; tiles_m = tiles_m_;
     locate(a);
   }
   // true when the walk entered a new tile
@@ -206,12 +239,13 @@ struct LoadShare {
       off[j] = __umul24((uint32_t)row, ld) + chunk;  // row < 256, ld < 2^23 (checked by the host)
     }
   }
-  __device__ __forceinline__ void set_ptr(const GemmArgs& a, int m0, int n0, int wave) {
-    ptr = wave >= 4 ? a.W + (int64_t)n0 * a.ldw : a.X + (int64_t)m0 * a.ldx;
+  __device__ __forceinline__ void set_ptr(const GemmArgs& a, int m0, int n0, int wave, int64_t w_group_off = 0) {
+    ptr = wave >= 4 ? a.W + w_group_off + (int64_t)n0 * a.ldw : a.X + (int64_t)m0 * a.ldx;
   }
-  __device__ __forceinline__ void set_tile(const GemmArgs& a, int m0, int n0, int wave, int lane) {
-    set_ptr(a, m0, n0, wave);
-    const int valid = wave >= 4 ? a.N - n0 : a.M - m0;
+  // m_end: first row past the segment the tile belongs to (M when the problem is not grouped)
+  __device__ __forceinline__ void set_tile(const GemmArgs& a, int m0, int n0, int wave, int lane, int m_end, int64_t w_group_off = 0) {
+    set_ptr(a, m0, n0, wave, w_group_off);
+    const int valid = wave >= 4 ? a.N - n0 : m_end - m0;
     set_offsets(a, valid < 256 ? valid : 256, wave, lane);
   }
   // The load is written out instead of using the compiler's builtin: the compiler books a global->LDS
@@ -323,7 +357,7 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 constexpr int kStoresPerTile = 16;
 template <int MODE, bool ALIGNED>
 __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[kTN][kTM], int m_base, int n_base,
-                                           int l16, int lg) {
+                                           int l16, int lg, int m_end) {
   if (MODE == kModeRowCol) {
     // eight columns at a time, so that only eight column scales and bias values are live
 #pragma unroll
@@ -340,7 +374,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
 #pragma unroll
       for (int j = 0; j < kTM; ++j) {
         const int m = m_base + j * 16 + l16;
-        if (!ALIGNED && m >= a.M) continue;
+        if (!ALIGNED && m >= m_end) continue;
         const float sa = a.xs[a.xs_per_row ? m : 0];
         uint32_t w[4];
 #pragma unroll
@@ -368,7 +402,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
 #pragma unroll
   for (int j = 0; j < kTM; ++j) {
     const int m = m_base + j * 16 + l16;
-    if (!ALIGNED && m >= a.M) continue;
+    if (!ALIGNED && m >= m_end) continue;
     uint16_t* const row = reinterpret_cast<uint16_t*>(a.C) + (int64_t)m * a.ldc;
     uint32_t w[16];
 #pragma unroll
@@ -482,8 +516,11 @@ __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (
 
 // ALIGNED: M and N are multiples of the tile; no tile has an edge, and the per-lane offsets of the tile loads
 // and of the scale loads never change (a tile change then touches scalar registers only).
-template <bool SK, int MODE, bool ALIGNED>
+// GROUPED: the rows are segments with a weight matrix each (see PpArgs::groups).
+template <bool SK, int MODE, bool ALIGNED, bool GROUPED = false>
 __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
+  static_assert(!GROUPED || (!SK && !ALIGNED && MODE == kModeBlock), "grouped problems: whole tiles with edges, block scales");
+  using Walk = WalkT<GROUPED>;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const GemmArgs& g = a.g;
   const int tid = threadIdx.x;
@@ -495,6 +532,16 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   const int l16 = lane & 15, lg = lane >> 4;
   const int frag_off = fragment_offset(lane);
 
+  int n_tiles = a.n_tiles, tiles_m = g.tiles_m;
+  if (GROUPED) {
+    tiles_m = 0;
+    for (int e = 0, begin = 0; e < a.n_groups; ++e) {
+      const int end = segment_end(a, e, begin);
+      tiles_m += (end - begin + kBM - 1) / kBM;
+      begin = end;
+    }
+    n_tiles = tiles_m * g.tiles_n;
+  }
   // steps of this block: whole tiles blockIdx.x, blockIdx.x + gridDim.x, ... or one contiguous range
   int pos = (int)blockIdx.x, first_idx = (int)blockIdx.x, first_kb = 0, total;
   if (SK) {
@@ -505,17 +552,18 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     first_idx = s0 / g.KB;
     first_kb = s0 - first_idx * g.KB;
   } else {
-    const int my_tiles = (a.n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;  // grid <= n_tiles
-    total = my_tiles * g.KB;
+    // (a grouped launch sizes its grid for an upper bound of the tile count: the blocks past the real one leave)
+    const int my_tiles = (n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    total = my_tiles > 0 ? my_tiles * g.KB : 0;
   }
   if (total <= 0) return;  // uniform over the block
   for (int i = (int)(blockIdx.x & 15) * a.stagger; i > 0; --i) __builtin_amdgcn_s_sleep(15);
 
   // ---- the stage being loaded
   Walk lw;
-  lw.start(a, first_idx, first_kb);
+  lw.start(a, first_idx, first_kb, n_tiles, tiles_m);
   LoadShare share = {};
-  share.set_tile(g, lw.m0, lw.n0, wave, lane);
+  share.set_tile(g, lw.m0, lw.n0, wave, lane, lw.m_end, (int64_t)lw.group * a.w_group_stride);
   share.ptr += (int64_t)first_kb * 128;
   int loaded = 0, w_slot = 0, x_slot = 0;  // stages issued by this wavefront; LDS slots of the next stage
   auto issue_stage_part = [&](int q) __attribute__((always_inline)) {
@@ -528,8 +576,9 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     w_slot = (w_slot + 1 == kWStages) ? 0 : w_slot + 1;
     x_slot ^= 1;
     if (__builtin_expect(lw.next(a), 0)) {
-      if (lw.idx < a.n_tiles) {
-        if (ALIGNED) share.set_ptr(g, lw.m0, lw.n0, wave); else share.set_tile(g, lw.m0, lw.n0, wave, lane);
+      if (lw.idx < n_tiles) {
+        if (ALIGNED) share.set_ptr(g, lw.m0, lw.n0, wave);
+        else share.set_tile(g, lw.m0, lw.n0, wave, lane, lw.m_end, GROUPED ? (int64_t)lw.group * a.w_group_stride : 0);
       }
     } else {
       share.ptr += 128;
@@ -544,7 +593,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   // ---- the step whose activation scales are being fetched: four rows per lane, 32-bit byte offsets from
   // a uniform pointer that moves along K (the host checks that M * row stride fits)
   Walk sw;
-  sw.start(a, first_idx, first_kb);
+  sw.start(a, first_idx, first_kb, n_tiles, tiles_m);
   uint32_t xs_off[kTM] = {0u, 0u, 0u, 0u};
   const float* xs_ptr = g.xs;
   // offsets are relative to the tile's first row; rows past the edge read the last row's scale
@@ -552,7 +601,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
 #pragma unroll
     for (int j = 0; j < kTM; ++j) {
       int r = wm0 + j * 16 + l16;
-      const int last = g.M - 1 - sw.m0;
+      const int last = sw.m_end - 1 - sw.m0;
       r = r < last ? r : last;
       xs_off[j] = (uint32_t)r * (uint32_t)g.xs_rs * 4u;
     }
@@ -579,12 +628,12 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
 
   // ---- the step being multiplied; its weight-block scale is one scalar load per step
   Walk cw;
-  cw.start(a, first_idx, first_kb);
+  cw.start(a, first_idx, first_kb, n_tiles, tiles_m);
   const int nb_last = (g.N - 1) >> 7;
   auto ws_row = [&]() __attribute__((always_inline)) -> const float* {
     int nb = (cw.n0 + wn0) >> 7;
     nb = nb < nb_last ? nb : nb_last;
-    return g.ws + (int64_t)nb * g.ws_rs;
+    return g.ws + (GROUPED ? (int64_t)cw.group * a.ws_group_stride : 0) + (int64_t)nb * g.ws_rs;
   };
   const float* ws_ptr = MODE == kModeBlock ? ws_row() + (int64_t)first_kb * g.ws_cs : nullptr;
 
@@ -608,7 +657,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   // A tile of which this block computed only some K-blocks (stream-K) goes through finish_partial_tile at
   // the start of that slot instead: its waits may stall the pair for a few microseconds, twice per block.
   bool pending = false;
-  int pend_m = 0, pend_n = 0, pend_idx = 0;
+  int pend_m = 0, pend_n = 0, pend_idx = 0, pend_m_end = 0;
   auto clear_acc = [&]() __attribute__((always_inline)) {
     // (a second copy of the multiply phase that overwrites instead of accumulating makes the register
     // allocator shuffle the accumulators through scratch at the join; zeroing costs 128 moves per tile)
@@ -619,7 +668,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     pending = false;
   };
   auto flush_whole_tile = [&]() __attribute__((always_inline)) {
-    store_tile<MODE, ALIGNED>(g, acc, pend_m, pend_n, l16, lg);
+    store_tile<MODE, ALIGNED>(g, acc, pend_m, pend_n, l16, lg, pend_m_end);
     clear_acc();
   };
   auto flush_partial_tile = [&]() __attribute__((always_inline)) {
@@ -752,7 +801,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     // ================= next step; a finished tile is stored in this wavefront's next fetch slot
     rw_slot = (rw_slot + 1 == kWStages) ? 0 : rw_slot + 1;
     rx_slot ^= 1;
-    pend_m = cw.m0 + wm0; pend_n = cw.n0 + wn0; pend_idx = cw.idx;
+    pend_m = cw.m0 + wm0; pend_n = cw.n0 + wn0; pend_idx = cw.idx; pend_m_end = cw.m_end;
     pending = __builtin_expect(cw.next(a), 0);
     if (MODE == kModeBlock) {
       if (pending) ws_ptr = ws_row(); else ws_ptr += g.ws_cs;
@@ -872,10 +921,18 @@ bool transposition_pays(int64_t tiles, int64_t KB, int cus) {
 }
 size_t transposed_scales_bytes(int64_t M, int64_t KB) { return (size_t)((M * KB * 4 + 255) / 256 * 256); }
 
-int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream,
+                 const GroupedGemm* grouped = nullptr) {
   PpArgs a = {};
   a.g = g;
   a.g.tiles_m = (int)ceil_div(g.M, kBM);
+  if (grouped != nullptr) {
+    // every segment ends with at most one tile that is not full; the kernel counts the real tiles
+    const int64_t bound = g.M / kBM + grouped->n_groups;
+    a.g.tiles_m = (int)(bound < g.M ? bound : g.M);
+    a.groups = grouped->ends; a.n_groups = (int)grouped->n_groups;
+    a.w_group_stride = grouped->w_group_stride; a.ws_group_stride = grouped->ws_group_stride;
+  }
   a.g.tiles_n = (int)ceil_div(g.N, kBN);
   const int64_t tiles = (int64_t)a.g.tiles_m * a.g.tiles_n;
   if (tiles > 0x3FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: too many tiles");
@@ -887,7 +944,8 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
                           reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false>),
                           reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true>),
                           reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, false>),
-                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, true>)}) {
+                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, true>),
+                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false, true>)}) {
       hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
       if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
     }
@@ -896,7 +954,8 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   const int cus = cu_count();
   int grid = tiles < cus ? (int)tiles : cus;
   // Stream-K is an optimisation the workspace enables: without one (or with a small one) whole tiles go round-robin.
-  const SkPlan sk = plan_stream_k(tiles, g.KB, cus);
+  SkPlan sk = plan_stream_k(tiles, g.KB, cus);
+  if (grouped != nullptr) sk.use = false;  // ranges of steps would need the tile count on the host
   const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : 0;
   const size_t need = FG_WORKSPACE_COUNTER_BYTES + sk_bytes;
   // workspace: [counters][partial tiles, if the shape is one that shares tiles][transposed activation scales]
@@ -920,13 +979,15 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   // (256 x 256 bf16 per unit at ~3.3 TB/s; a K-block takes ~1.66 us): the run is bound by the stores, and
   // starting the blocks spread over one tile time lets the stores of some overlap the MFMAs of others
   // (M = 4096, N = 32768, K = 512: 113 -> 98 us).  Everywhere else the delay only costs.
-  if (!a.sk && tiles >= 6 * (int64_t)grid) {
+  if (!a.sk && grouped == nullptr && tiles >= 6 * (int64_t)grid) {
     const double tile_us = 1.66 * g.KB, batch_us = grid * 131072.0 / 3.3e6;
     if (tile_us < batch_us) a.stagger = (int)(tile_us * 1.6e3 / 1000.0 / 16 + 0.5);  // 1.6 GHz, ~1000 cycles a sleep, 16 start slots
   }
   const bool aligned = g.M % kBM == 0 && g.N % kBN == 0;
   void (*kern)(PpArgs);
-  if (mode != kModeBlock)
+  if (grouped != nullptr)
+    kern = fp8_gemm_pingpong_kernel<false, kModeBlock, false, true>;
+  else if (mode != kModeBlock)
     kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeRowCol, true> : fp8_gemm_pingpong_kernel<false, kModeRowCol, false>;
   else if (a.sk)
     kern = aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true> : fp8_gemm_pingpong_kernel<true, kModeBlock, false>;
@@ -961,6 +1022,20 @@ size_t pingpong_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   const size_t tr_bytes = transposition_pays(ceil_div(M, kBM) * ceil_div(N, kBN), KB, cu_count())
                               ? transposed_scales_bytes(M, KB) : 0;  // for row-major scales
   return sk_bytes + tr_bytes != 0 ? FG_WORKSPACE_COUNTER_BYTES + sk_bytes + tr_bytes : 0;
+}
+
+size_t grouped_workspace_bytes(int64_t M, int64_t K) {
+  if (M <= 0 || K <= 0 || K % 128 != 0) return 0;
+  return FG_WORKSPACE_COUNTER_BYTES + transposed_scales_bytes(M, K / 128);
+}
+
+int launch_grouped(const GemmArgs& g, const GroupedGemm& grouped, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  if (!(g.c_dtype == FG_BF16 && g.ldc % 8 == 0 && (uintptr_t)g.C % 16 == 0))
+    FG_FAIL(FG_ERR_UNSUPPORTED, "grouped fp8 gemm: the result must be bf16 with rows that take 16-byte stores");
+  if (!(g.xs_rs >= 0 && g.xs_cs >= 0 && g.ws_rs >= 0 && g.ws_cs >= 0 && (int64_t)g.M * g.xs_rs < (1ll << 29)))
+    FG_FAIL(FG_ERR_UNSUPPORTED, "grouped fp8 gemm: scale strides must be non-negative and M * row stride below 2^29");
+  if (grouped.n_groups <= 0 || grouped.n_groups > 65536) FG_FAIL(FG_ERR_INVALID_ARG, "grouped fp8 gemm: 1..65536 groups");
+  return launch_block(g, kModeBlock, workspace, workspace_bytes, stream, &grouped);
 }
 
 int launch_pingpong(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream) {

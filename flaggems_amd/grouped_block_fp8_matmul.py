@@ -1,0 +1,85 @@
+"""Grouped block-scaled FP8 GEMM for mixture-of-experts layers (host side).
+
+The reference runs its block-fp8 experts through ``fused_moe_kernel``
+(src/flag_gems/fused/fused_moe.py:1378-1450), which gathers token rows through
+``sorted_token_ids``; its grouped GEMM operator ``aten::_scaled_grouped_mm``
+(src/flag_gems/ops/scaled_grouped_mm.py:240-583) takes rows already sorted by group with a table
+``offs`` of cumulative int32 row ends (:111-114, :275-287) but only row-wise scales.  This operator
+joins the two: the 2-D x 3-D case of ``_scaled_grouped_mm`` (rows of ``A`` cut by ``offs``, one weight
+matrix per group) with the 1 x 128 / 128 x 128 block scales of ``w8a8_block_fp8_matmul``.  ``offs``
+stays on the device; the kernel reads it, so the call never synchronises.
+"""
+from __future__ import annotations
+
+import logging
+from typing import List
+
+import torch
+
+from . import _lib
+
+logger = logging.getLogger("flag_gems." + __name__.split(".")[-1])
+
+
+def _cdiv(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+def grouped_w8a8_block_fp8_matmul(
+    A: torch.Tensor,
+    B: torch.Tensor,
+    As: torch.Tensor,
+    Bs: torch.Tensor,
+    offs: torch.Tensor,
+    block_size: List[int],
+    output_dtype: torch.dtype = torch.bfloat16,
+) -> torch.Tensor:
+    """C[offs[e-1]:offs[e]] = block_fp8_matmul(A[offs[e-1]:offs[e]], B[e]) for every group e.
+
+    A [M, K] contiguous e4m3fn (rows sorted by group), As [M, K/block_k] fp32, B [E, N, K] e4m3fn,
+    Bs [E, ceil(N/block_n), K/block_k] fp32, offs [E] int32 cumulative row ends on A's device.
+    Returns bf16 [M, N]; rows at or past offs[-1] are left unwritten (as ``torch.empty`` made them).
+    """
+    logger.debug("GEMS GROUPED_W8A8_BLOCK_FP8_MATMUL")
+    assert len(block_size) == 2
+    block_n, block_k = block_size[0], block_size[1]
+    assert A.ndim == 2 and B.ndim == 3 and As.ndim == 2 and Bs.ndim == 3
+    assert A.is_contiguous()
+    M, K = A.shape
+    E, N, K2 = B.shape
+    assert K == K2
+    assert As.shape[0] == M and As.shape[1] == _cdiv(K, block_k)
+    assert Bs.shape == (E, _cdiv(N, block_n), _cdiv(K, block_k))
+    assert offs.ndim == 1 and offs.numel() == E and offs.dtype == torch.int32
+    assert offs.device == A.device and offs.is_contiguous()
+    if A.dtype != torch.float8_e4m3fn or B.dtype != torch.float8_e4m3fn:
+        raise NotImplementedError(f"grouped_w8a8_block_fp8_matmul: operands must be float8_e4m3fn, got {A.dtype}, {B.dtype}")
+    if output_dtype != torch.bfloat16:
+        raise NotImplementedError(f"grouped_w8a8_block_fp8_matmul: output dtype {output_dtype} (only bfloat16)")
+    if As.dtype != torch.float32 or Bs.dtype != torch.float32:
+        As, Bs = As.to(torch.float32), Bs.to(torch.float32)
+    if B.stride(2) != 1:
+        B = B.contiguous()
+
+    C = A.new_empty((M, N), dtype=output_dtype)
+    if M == 0 or N == 0:
+        return C
+    _lib.require_gpu(A, "grouped block fp8 gemm")
+    lib = _lib.load()
+    dev = A.device
+    with torch.cuda.device(dev):
+        ws_bytes = lib.fg_grouped_block_fp8_gemm_workspace_bytes(M, N, K)
+        ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
+        status = lib.fg_grouped_block_fp8_gemm(
+            A.data_ptr(), A.stride(0) if M > 1 else max(K, A.stride(0)),
+            B.data_ptr(), B.stride(1) if N > 1 else max(K, B.stride(1)), B.stride(0) if E > 1 else N * K,
+            As.data_ptr(), As.stride(0), As.stride(1),
+            Bs.data_ptr(), Bs.stride(1), Bs.stride(2), Bs.stride(0),
+            offs.data_ptr(), E,
+            C.data_ptr(), C.stride(0), _lib.DTYPE_CODE[C.dtype],
+            M, N, K, block_n, block_k,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+            _lib.current_stream_ptr(dev),
+        )
+    _lib.check(status, "fg_grouped_block_fp8_gemm")
+    return C

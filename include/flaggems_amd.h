@@ -133,6 +133,38 @@ int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
 size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
+ * Grouped block-scaled FP8 GEMM (mixture-of-experts layers with the tokens sorted by expert):
+ *     C[m, n] = sum_kb ( sum_{k in kb} A[m,k] * B[e(m)][n,k] ) * As[m, kb] * Bs[e(m)][n / block_n, kb]
+ * where row m belongs to group e(m): group e owns rows [group_ends[e-1], group_ends[e]) with
+ * group_ends[-1] = 0.  group_ends is a DEVICE table of n_groups cumulative int32 row ends, read by the
+ * kernel (the host never waits for it); empty groups are allowed; rows at or past the last end are not
+ * written; ends are forced into ascending order and into [0, M] before use.
+ * A: e4m3fn [M, K] (all groups' rows), As: fp32 [M, K/block_k], C: bf16 [M, N], as in fg_block_fp8_gemm.
+ * B: e4m3fn [n_groups, N, K]: matrix e starts b_group_stride bytes after matrix e-1, rows ldb apart.
+ * Bs: fp32 [n_groups, ceil(N/block_n), K/block_k]: matrix e starts bs_group_stride floats after matrix e-1.
+ * K must be a positive multiple of 128; A, B 16-byte aligned with lda, ldb, b_group_stride multiples of 16;
+ * C 16-byte aligned with ldc a multiple of 8; c_dtype FG_BF16 (FG_ERR_UNSUPPORTED otherwise: there is no
+ * slower general path behind this entry point).
+ * `workspace` (optional, 16-byte aligned, fg_grouped_block_fp8_gemm_workspace_bytes(M, N, K) bytes, first
+ * FG_WORKSPACE_COUNTER_BYTES zero-filled once) lets row-major As be read from a transposed copy.
+ *
+ * Stands in for the block-wise fp8 branch of fused_moe_kernel (src/flag_gems/fused/fused_moe.py:1378-1450)
+ * applied to rows already gathered in expert order, with the group table of aten::_scaled_grouped_mm
+ * (`offs`: cumulative int32 ends, src/flag_gems/ops/scaled_grouped_mm.py:111-114,275-287).  Per group the
+ * arithmetic is that of w8a8_block_fp8_matmul (src/flag_gems/ops/w8a8_block_fp8_matmul.py:51-122), which is
+ * how the reference's own MoE test states it (tests/test_fused_experts_impl.py:604-662).
+ */
+int fg_grouped_block_fp8_gemm(const void* A, int64_t lda,
+                              const void* B, int64_t ldb, int64_t b_group_stride,
+                              const float* As, int64_t as_row_stride, int64_t as_col_stride,
+                              const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride, int64_t bs_group_stride,
+                              const int32_t* group_ends, int64_t n_groups,
+                              void* C, int64_t ldc, int c_dtype,
+                              int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
+                              void* workspace, size_t workspace_bytes, void* stream);
+size_t fg_grouped_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
  * Per-tensor / per-token x per-channel scaled FP8 GEMM with optional bias:
  *     C[m, n] = cast( (sum_k A[m,k] * B[n,k]) * a_scale[m or 0] * b_scale[n or 0] ) (+ bias[n])
  * The bias is added after the cast, in c_dtype, as the reference does.  A: e4m3fn [M, K] row stride

@@ -25,6 +25,10 @@ the checks live in tests/test_oracle_*.py):
   other (two different algorithms from two reference files), a float64 triple
   loop on tiny shapes, and closed forms (unit scales -> plain matmul, one-hot
   rows pick scaled weight rows exactly, power-of-two scales are exact).
+* grouped_block_fp8_matmul_ref -- a loop of block_fp8_matmul_tiled_ref over row
+  segments; pinned by the dequantise-then-matmul reference per segment, by "one
+  group = the plain GEMM", by "identical weights in every group = the plain GEMM
+  whatever the segment ends", and by a float64 loop on a tiny ragged case.
 * scaled_mm_ref, scaled_mm_ref_postscale -- pinned against each other, a float64
   loop, and the unit-scale/zero-bias closed form.
 
@@ -260,6 +264,51 @@ def block_fp8_matmul_tiled_ref(
             scale = a_scales[:, i : i + 1] * b_scales[j][i]
             c[:, j * block_n : min((j + 1) * block_n, n)] += torch.matmul(a_t, b_t.t()) * scale
     return c.reshape(origin_c_shape).to(output_dtype)
+
+
+def grouped_block_fp8_matmul_ref(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    a_scales: torch.Tensor,
+    b_scales: torch.Tensor,
+    offs: torch.Tensor,
+    block_size: List[int],
+    output_dtype: torch.dtype = torch.float32,
+) -> torch.Tensor:
+    """Rows ``offs[e-1]:offs[e]`` of ``a`` [M, K] times weight matrix ``b[e]`` [N, K] with
+    scales ``b_scales[e]``: the per-expert loop of the reference's block-fp8 MoE check
+    (tests/test_fused_experts_impl.py:636-646, each expert's rows through
+    ``torch_w8a8_block_matmul``) over rows already sorted by expert, the segments given as
+    the cumulative int32 ends of ``aten::_scaled_grouped_mm``
+    (src/flag_gems/ops/scaled_grouped_mm.py:111-114, 275-287).  Rows at or past the last end
+    come back as zeros (the device leaves them unwritten)."""
+    m = a.shape[0]
+    e_count, n, _ = b.shape
+    assert offs.numel() == e_count
+    c = torch.zeros((m, n), dtype=output_dtype)
+    begin = 0
+    for e in range(e_count):
+        end = int(offs[e])
+        if end > begin:
+            c[begin:end] = block_fp8_matmul_tiled_ref(
+                a[begin:end], b[e], a_scales[begin:end], b_scales[e], block_size, output_dtype
+            )
+        begin = max(begin, end)
+    return c
+
+
+def make_moe_rows(tokens: int, experts: int = 8, top_k: int = 2, seed: int = 0) -> torch.Tensor:
+    """Cumulative int32 row ends of ``tokens * top_k`` rows sorted by expert, with expert loads
+    proportional to a Zipf(1.1) law over a seeded permutation of the experts (the synthetic
+    routing of the Mixtral-shaped benchmark configuration; no counterpart in the reference)."""
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(experts, generator=g)
+    p = torch.zeros(experts, dtype=torch.float64)
+    p[perm] = 1.0 / torch.arange(1, experts + 1, dtype=torch.float64) ** 1.1
+    p /= p.sum()
+    ids = torch.multinomial(p, tokens * top_k, replacement=True, generator=g)
+    counts = torch.bincount(ids, minlength=experts)
+    return torch.cumsum(counts, 0).to(torch.int32)
 
 
 # --------------------------------------------------------------------------------------

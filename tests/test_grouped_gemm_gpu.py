@@ -1,0 +1,132 @@
+"""GPU parity of the grouped (mixture-of-experts) block-scaled FP8 GEMM against the CPU oracle.
+
+Tolerance: rtol 1e-2 / atol 1e-2 for the bf16 result against the per-group fp32 restatement of the
+reference's MoE check (tests/test_fused_experts_impl.py:636-646); where a plain GEMM computes the same
+tiles in the same order the results are compared bit for bit."""
+import ctypes
+
+import pytest
+import torch
+
+import flag_gems
+from flaggems_amd import _lib
+from oracle import fp8_linear_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+FP8 = torch.float8_e4m3fn
+
+
+def _inputs(M, N, K, E, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    xq, xs = O.act_quant_ref(x, 128)
+    wq, ws = [], []
+    for _ in range(E):
+        q, s = O.per_block_cast_to_fp8_ref((0.02 * torch.randn(N, K, generator=g)).bfloat16())
+        wq.append(q)
+        ws.append(s)
+    return xq, torch.stack(wq), xs, torch.stack(ws)
+
+
+def _run(xq, wq, xs, ws, ends):
+    return flag_gems.grouped_w8a8_block_fp8_matmul(
+        xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), ends.to(DEV), [128, 128])
+
+
+def _check(got, xq, wq, xs, ws, ends):
+    want = O.grouped_block_fp8_matmul_ref(xq, wq, xs, ws, ends, [128, 128])
+    rows = min(int(ends.max()), xq.shape[0])
+    assert got.dtype == torch.bfloat16 and got.shape == want.shape
+    torch.testing.assert_close(got.cpu().float()[:rows], want[:rows], rtol=1e-2, atol=1e-2)
+    # at most one bf16 rounding plus fp32 accumulation noise
+    err = (got.cpu().double()[:rows] - want.double()[:rows]).abs()
+    assert float((err / (want[:rows].double().abs() / 128 + 2e-3)).max()) < 1.0
+
+
+CASES = [
+    # M, N, K, ends
+    (1024, 640, 512, [300, 300, 301, 1000]),          # an empty group, a one-row group, rows nobody owns
+    (128, 1024, 1024, None),                           # 64 tokens, top-2, 8 experts: every tile is mostly edge
+    (2048, 2144, 1024, None),                          # N ends inside a scale block
+    (3000, 6144, 256, [1000, 1900, 3000]),             # more tiles than compute units: blocks walk several
+    (700, 384, 2048, [0, 0, 0, 0, 0, 0, 0, 700]),      # all rows in the last group
+    (513, 256, 128, [256, 512, 513]),                  # segments that end on tile boundaries, one K-block
+]
+
+
+@pytest.mark.parametrize("M,N,K,ends", CASES)
+def test_grouped_gemm_matches_the_oracle(M, N, K, ends):
+    ends = O.make_moe_rows(M // 2, 8, 2, seed=M) if ends is None else torch.tensor(ends, dtype=torch.int32)
+    xq, wq, xs, ws = _inputs(M, N, K, ends.numel(), seed=N)
+    got = _run(xq, wq, xs, ws, ends)
+    _check(got, xq, wq, xs, ws, ends)
+    # a second call gives the same bits (no order of arrival enters the sums)
+    assert torch.equal(got, _run(xq, wq, xs, ws, ends))
+
+
+def test_grouped_gemm_equals_plain_gemm_where_the_tiles_coincide():
+    """Segment ends on tile boundaries and the same weights in every group: the grouped kernel computes the tiles
+    of the plain GEMM (256 of them, which the plain path gives whole to the persistent kernel), bit for bit."""
+    M, N, K = 4096, 4096, 256
+    xq, wq, xs, ws = _inputs(M, N, K, 1, seed=5)
+    ends = torch.tensor([1024, 1024, 4096], dtype=torch.int32)
+    got = _run(xq, wq.expand(3, -1, -1).contiguous(), xs, ws.expand(3, -1, -1).contiguous(), ends)
+    plain = flag_gems.w8a8_block_fp8_matmul(xq.to(DEV), wq[0].to(DEV), xs.to(DEV), ws[0].to(DEV), [128, 128])
+    assert torch.equal(got, plain)
+    # ends inside tiles change which tile a row falls in, not its sums
+    ends = torch.tensor([1000, 1001, 4096], dtype=torch.int32)
+    got = _run(xq, wq.expand(3, -1, -1).contiguous(), xs, ws.expand(3, -1, -1).contiguous(), ends)
+    assert torch.equal(got, plain)
+
+
+def test_group_table_is_forced_into_range():
+    """Ends that go backwards or past the rows are forced into [previous end, M]: no row is read or written
+    outside the operands, and the result is that of the forced table."""
+    M, N, K = 1000, 512, 256
+    xq, wq, xs, ws = _inputs(M, N, K, 3, seed=8)
+    got = _run(xq, wq, xs, ws, torch.tensor([500, 200, 5000], dtype=torch.int32))
+    _check(got, xq, wq, xs, ws, torch.tensor([500, 500, 1000], dtype=torch.int32))
+
+
+def test_scale_layouts_and_missing_workspace_through_the_c_abi():
+    """Column-major activation scales are read in place; without a workspace row-major scales are read as they
+    lie.  Both give the bits of the default call."""
+    M, N, K, E = 1500, 768, 2048, 4
+    ends = torch.tensor([100, 900, 900, 1500], dtype=torch.int32)
+    xq, wq, xs, ws = _inputs(M, N, K, E, seed=9)
+    base = _run(xq, wq, xs, ws, ends)
+    _check(base, xq, wq, xs, ws, ends)
+    xs_cm = xs.to(DEV).t().contiguous().t()
+    assert xs_cm.stride() == (1, M)
+    got = flag_gems.grouped_w8a8_block_fp8_matmul(xq.to(DEV), wq.to(DEV), xs_cm, ws.to(DEV), ends.to(DEV), [128, 128])
+    assert torch.equal(got, base)
+    a, b, a_s, b_s, e = xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), ends.to(DEV)
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    st = _lib.load().fg_grouped_block_fp8_gemm(
+        a.data_ptr(), K, b.data_ptr(), K, N * K, a_s.data_ptr(), a_s.stride(0), 1,
+        b_s.data_ptr(), b_s.stride(1), 1, b_s.stride(0), e.data_ptr(), E,
+        c.data_ptr(), N, _lib.DTYPE_CODE[torch.bfloat16], M, N, K, 128, 128,
+        None, 0, _lib.current_stream_ptr(torch.device(DEV)))
+    _lib.check(st, "fg_grouped_block_fp8_gemm")
+    torch.cuda.synchronize()
+    assert torch.equal(c, base)
+
+
+def test_unsupported_requests_fail_loudly():
+    xq, wq, xs, ws = _inputs(64, 256, 256, 2, seed=1)
+    ends = torch.tensor([10, 64], dtype=torch.int32)
+    args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), ends.to(DEV))
+    with pytest.raises(NotImplementedError):
+        flag_gems.grouped_w8a8_block_fp8_matmul(*args, [128, 128], output_dtype=torch.float32)
+    with pytest.raises(NotImplementedError):  # scale blocks other than 128 x 128
+        flag_gems.grouped_w8a8_block_fp8_matmul(*args[:3], torch.ones(2, 4, 2, device=DEV), args[4], [64, 128])
+    with pytest.raises(AssertionError):
+        flag_gems.grouped_w8a8_block_fp8_matmul(*args[:4], ends.to(torch.int64).to(DEV), [128, 128])
+    # K that is not a multiple of 128
+    g = torch.Generator().manual_seed(2)
+    a = torch.randn(64, 192, generator=g).to(FP8).to(DEV)
+    b = torch.randn(2, 256, 192, generator=g).to(FP8).to(DEV)
+    with pytest.raises(NotImplementedError):
+        flag_gems.grouped_w8a8_block_fp8_matmul(a, b, torch.ones(64, 2, device=DEV), torch.ones(2, 2, 2, device=DEV),
+                                                ends.to(DEV), [128, 128])

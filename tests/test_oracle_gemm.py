@@ -154,3 +154,68 @@ def test_config1_pipeline_is_self_consistent():
     want = r["x"].float() @ r["w"].float().T
     rel = (r["c"].float() - want).norm() / want.norm()
     assert rel < 0.05
+
+
+# ---- grouped (mixture-of-experts) block GEMM
+
+
+def _grouped_inputs(m, n, k, experts, seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(m, k, generator=g).to(FP8)
+    b = torch.randn(experts, n, k, generator=g).to(FP8)
+    kb, nb = (k + 127) // 128, (n + 127) // 128
+    a_s = 0.01 * torch.rand(m, kb, generator=g) + 0.005
+    b_s = 0.01 * torch.rand(experts, nb, kb, generator=g) + 0.005
+    return a, b, a_s, b_s
+
+
+def test_grouped_ref_vs_f64_loop_on_ragged_segments():
+    ends = torch.tensor([2, 2, 5, 6], dtype=torch.int32)  # segment 1 is empty, row 6 belongs to nobody
+    a, b, a_s, b_s = _grouped_inputs(7, 130, 256, 4, 21)
+    got = O.grouped_block_fp8_matmul_ref(a, b, a_s, b_s, ends, [128, 128]).double().numpy()
+    begin = 0
+    for e, end in enumerate(ends.tolist()):
+        if end > begin:
+            want = _loop_f64(a[begin:end], b[e], a_s[begin:end], b_s[e])
+            np.testing.assert_allclose(got[begin:end], want, rtol=1e-5, atol=1e-7)
+        begin = end
+    assert not got[6].any()
+
+
+def test_grouped_ref_vs_dequantised_matmul_per_segment():
+    ends = torch.tensor([40, 41, 41, 100], dtype=torch.int32)
+    a, b, a_s, b_s = _grouped_inputs(100, 260, 384, 4, 22)
+    got = O.grouped_block_fp8_matmul_ref(a, b, a_s, b_s, ends, [128, 128])
+    begin = 0
+    for e, end in enumerate(ends.tolist()):
+        if end > begin:
+            want = O.block_fp8_matmul_dequant_ref(a[begin:end], b[e], a_s[begin:end], b_s[e], [128, 128])
+            torch.testing.assert_close(got[begin:end], want, rtol=1e-4, atol=1e-6)
+        begin = end
+
+
+def test_grouped_ref_closed_forms():
+    a, b, a_s, b_s = _grouped_inputs(50, 256, 256, 3, 23)
+    plain = O.block_fp8_matmul_tiled_ref(a, b[1], a_s, b_s[1], [128, 128])
+    # one group holding every row is the plain GEMM with that group's weights
+    ends = torch.tensor([0, 50, 50], dtype=torch.int32)
+    assert torch.equal(O.grouped_block_fp8_matmul_ref(a, b, a_s, b_s, ends, [128, 128]), plain)
+    # the same weights in every group: the segment ends stop mattering
+    same_b, same_s = b[1:2].expand(3, -1, -1), b_s[1:2].expand(3, -1, -1)
+    for ends in ([7, 7, 50], [13, 30, 50], [50, 50, 50]):
+        got = O.grouped_block_fp8_matmul_ref(a, same_b, a_s, same_s, torch.tensor(ends, dtype=torch.int32), [128, 128])
+        torch.testing.assert_close(got, plain, rtol=1e-6, atol=1e-7)
+    # swapping two groups' weights changes exactly those groups' rows
+    ends = torch.tensor([10, 30, 50], dtype=torch.int32)
+    base = O.grouped_block_fp8_matmul_ref(a, b, a_s, b_s, ends, [128, 128])
+    swapped = O.grouped_block_fp8_matmul_ref(a, b[[2, 1, 0]], a_s, b_s[[2, 1, 0]], ends, [128, 128])
+    assert torch.equal(base[10:30], swapped[10:30])
+    assert not torch.equal(base[:10], swapped[:10]) and not torch.equal(base[30:], swapped[30:])
+
+
+def test_moe_rows_are_cumulative_and_skewed():
+    ends = O.make_moe_rows(4096, 8, 2, seed=0)
+    assert ends.dtype == torch.int32 and ends.numel() == 8 and int(ends[-1]) == 8192
+    counts = torch.diff(ends, prepend=torch.zeros(1, dtype=torch.int32))
+    assert (counts >= 0).all() and counts.max() > 2 * counts.min()
+    assert torch.equal(ends, O.make_moe_rows(4096, 8, 2, seed=0))
