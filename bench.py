@@ -20,6 +20,9 @@ Prints ONE JSON line with the driver's fields plus
                 the other configurations of the path (per-token x per-channel scaled GEMM with bias; Llama-3-8B
                 linears as GEMM alone and as act_quant + GEMM), graph replays of one shape at a time with ONE copy
                 of the weights (small-M figures there may be served by the 256 MB Infinity Cache), not part of `value`
+  mixtral_moe_grouped_gemm
+                BASELINE.json configs[4]: 8 experts, top-2 over T tokens with Zipf(1.1) expert loads, rows sorted by
+                expert; the grouped block-fp8 GEMM with W1 [8,28672,4096] and W2 [8,4096,14336]; not part of `value`
 """
 from __future__ import annotations
 
@@ -60,6 +63,19 @@ def gemm_flops(m, n, k):
 def gemm_bytes(m, n, k):
     kb, nb = (k + 127) // 128, (n + 127) // 128
     return m * k + n * k + 4 * m * kb + 4 * nb * kb + 2 * m * n
+
+
+def moe_row_ends(tokens, experts, top_k, seed):
+    """Cumulative int32 row ends of tokens * top_k rows sorted by expert; expert loads follow a Zipf(1.1) law over a
+    seeded permutation of the experts."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(experts, generator=g)
+    p = torch.zeros(experts, dtype=torch.float64)
+    p[perm] = 1.0 / torch.arange(1, experts + 1, dtype=torch.float64) ** 1.1
+    ids = torch.multinomial(p / p.sum(), tokens * top_k, replacement=True, generator=g)
+    return torch.cumsum(torch.bincount(ids, minlength=experts), 0).to(torch.int32)
 
 
 def make_weight(n, k, gen, dev):
@@ -288,6 +304,26 @@ def main():
                           "tflops": round(gemm_flops(m, n, k) / us_g / 1e6, 1), "gbps": round(gemm_bytes(m, n, k) / us_g / 1e3, 1)})
         del wq, ws
 
+    # Mixtral-8x7B expert layers (BASELINE configs[4]): grouped block-fp8 GEMM over rows sorted by expert
+    moe = []
+    experts = 8
+    for (n, k) in [(28672, 4096), (4096, 14336)]:
+        parts = [make_weight(n, k, gen, dev) for _ in range(experts)]
+        wq = torch.stack([q for (q, _) in parts])
+        ws = torch.stack([s_ for (_, s_) in parts])
+        del parts
+        for tokens in (64, 1024, 4096):
+            rows = 2 * tokens
+            ends = moe_row_ends(tokens, experts, 2, 0).to(dev)
+            xq, xs = flag_gems.act_quant_triton(torch.randn(rows, k, device=dev, generator=gen).bfloat16(), 128)
+            us = time_eager(lambda: flag_gems.grouped_w8a8_block_fp8_matmul(xq, wq, xs, ws, ends, [128, 128]), 10)
+            nbytes = experts * (n * k + 4 * (n // 128) * (k // 128)) + rows * k + 4 * rows * (k // 128) + 2 * rows * n
+            tf = gemm_flops(rows, n, k) / us / 1e6
+            moe.append({"tokens": tokens, "rows": rows, "N": n, "K": k, "row_ends": ends.tolist(), "us": round(us, 2),
+                        "tflops": round(tf, 1), "gbps": round(nbytes / us / 1e3, 1),
+                        "frac_mfma": round(tf / PEAK_FP8_TFLOPS, 4), "frac_hbm": round(nbytes / us / 1e3 / PEAK_HBM_GBPS, 4)})
+        del wq, ws
+
     # ---- CPU baseline: the oracle on the host cores, bounded sample
     cpu = None
     if not args.no_cpu:
@@ -335,6 +371,7 @@ def main():
         "quantizer": quant,
         "cutlass_scaled_mm_n8192_k8192_bias": scaled,
         "llama3_8b_linears": llama,
+        "mixtral_moe_grouped_gemm": moe,
         "cpu_baseline": cpu,
         "detail": detail,
     }
