@@ -245,6 +245,22 @@ def main():
     q_gbs = 3.03125 * 4096 * 7168 / (q_us * 1e-6) / 1e9
     quant = {"shape": [4096, 7168], "us": round(q_us, 2), "gbps": round(q_gbs, 1), "frac_hbm": round(q_gbs / PEAK_HBM_GBPS, 4)}
 
+    # ---- 128 x 128 weight quantizer (HBM bound): bf16 [28672, 4096] -> e4m3fn + one scale per block
+    w_in = (0.02 * torch.randn(28672, 4096, device=dev, generator=gen)).bfloat16()
+    for _ in range(3):
+        flag_gems.per_block_cast_to_fp8(w_in, use_ue8m0=False)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(20):
+        flag_gems.per_block_cast_to_fp8(w_in, use_ue8m0=False)
+    end.record()
+    end.synchronize()
+    wq_us = start.elapsed_time(end) * 1e3 / 20
+    wq_gbs = (3.0 + 4.0 / 16384) * 28672 * 4096 / (wq_us * 1e-6) / 1e9
+    weight_quant = {"shape": [28672, 4096], "us": round(wq_us, 2), "gbps": round(wq_gbs, 1),
+                    "frac_hbm": round(wq_gbs / PEAK_HBM_GBPS, 4)}
+    del w_in
+
     # ---- the other configurations of the path, each shape timed alone: HIP events around the replay of a graph
     # of `reps` launches (as above: decode-sized launches are shorter than a Python call)
     def time_eager(fn, reps):
@@ -369,6 +385,7 @@ def main():
         "roofline": roofline,
         "roofline_small_m": roofline_small,
         "quantizer": quant,
+        "weight_quantizer_128x128": weight_quant,
         "cutlass_scaled_mm_n8192_k8192_bias": scaled,
         "llama3_8b_linears": llama,
         "mixtral_moe_grouped_gemm": moe,

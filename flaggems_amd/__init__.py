@@ -9,6 +9,7 @@ loudly if the library has not been built (``python -m flaggems_amd.build``).
 from .act_quant import (  # noqa: F401
     SUPPORTED_FP8_DTYPE,
     act_quant_triton,
+    per_block_cast_to_fp8,
     per_token_group_quant_fp8,
 )
 from .cutlass_scaled_mm import SM_VERSION_NUM, cutlass_scaled_mm, get_sm_version_num  # noqa: F401
@@ -41,6 +42,7 @@ __all__ = [
     "grouped_w8a8_block_fp8_matmul",
     "only_enable",
     "patch_empty_vllm",
+    "per_block_cast_to_fp8",
     "per_token_group_quant_fp8",
     "scaled_mm",
     "scaled_mm_out",

@@ -21,7 +21,7 @@ FG_ERR_INVALID_ARG, FG_ERR_UNSUPPORTED, FG_ERR_WORKSPACE, FG_ERR_LAUNCH = -1, -2
 FG_BF16, FG_F16, FG_F32, FG_FP8_E4M3FN, FG_FP8_E5M2 = 0, 1, 2, 3, 4
 FG_SCALE_MUL_INV, FG_SCALE_DIV = 0, 1
 FG_QUOT_RECIP_MUL, FG_QUOT_DIV = 0, 1
-FG_POW2_NONE, FG_POW2_BITS, FG_POW2_LOG2 = 0, 1, 2
+FG_POW2_NONE, FG_POW2_BITS, FG_POW2_LOG2, FG_POW2_BITS_CLAMPED = 0, 1, 2, 3
 FG_WORKSPACE_COUNTER_BYTES = 16384
 
 DTYPE_CODE = {
@@ -40,6 +40,11 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64,
          c_int64, c_float, c_float, c_float, c_float, c_int, c_int, c_int, c_void_p],
+    ),
+    "fg_block_quant_fp8": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64,
+         c_int64, c_int64, c_float, c_float, c_float, c_float, c_int, c_int, c_int, c_void_p],
     ),
     "fg_act_quant_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "fg_block_fp8_gemm": (

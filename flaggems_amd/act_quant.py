@@ -205,3 +205,40 @@ def per_token_group_fp8_quant_into(
         scale_rule=_lib.FG_SCALE_MUL_INV, quotient_rule=_lib.FG_QUOT_DIV,
         pow2_rule=_lib.FG_POW2_LOG2 if scale_ue8m0 else _lib.FG_POW2_NONE,
     )
+
+
+def per_block_cast_to_fp8(
+    x: torch.Tensor, use_ue8m0: bool = True, gran_k: int = 128
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Quantize a 2-D weight to e4m3fn with one fp32 scale per ``gran_k x gran_k`` block.
+
+    Same parameters, defaults and results (bit for bit) as the torch helper the reference builds its
+    block-quantized weights with (tests/test_fp8_einsum.py:89-103, benchmark/test_fp8_einsum.py:82-96):
+    blocks over the edge are padded with zeros, amax is floored at 1e-4, scale = amax / 448 (rounded up to
+    a power of two when ``use_ue8m0``), codes = x * (1 / scale).  Returns (codes [m, n] contiguous,
+    scales [ceil(m / gran_k), ceil(n / gran_k)] fp32).
+    """
+    logger.debug("GEMS PER_BLOCK_CAST_TO_FP8")
+    assert x.dim() == 2
+    if x.dtype not in _IN_DTYPES:
+        raise NotImplementedError(f"per_block_cast_to_fp8: unsupported input dtype {x.dtype}")
+    m, n = x.shape
+    q = torch.empty((m, n), dtype=torch.float8_e4m3fn, device=x.device)
+    sf = torch.empty((-(-m // gran_k), -(-n // gran_k)), dtype=torch.float32, device=x.device)
+    if x.numel() == 0:
+        return q, sf
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    _lib.require_gpu(x, "block quantizer")
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        status = lib.fg_block_quant_fp8(
+            x.data_ptr(), _lib.DTYPE_CODE[x.dtype], m, n, x.stride(0) if m > 1 else max(n, x.stride(0)),
+            q.data_ptr(), _lib.DTYPE_CODE[q.dtype], n,
+            sf.data_ptr(), sf.stride(0), sf.stride(1),
+            gran_k, gran_k, 1e-4, -448.0, 448.0, 1.0 / 448.0,
+            _lib.FG_SCALE_DIV, _lib.FG_QUOT_RECIP_MUL, _lib.FG_POW2_BITS_CLAMPED if use_ue8m0 else _lib.FG_POW2_NONE,
+            _lib.current_stream_ptr(x.device),
+        )
+    _lib.check(status, "fg_block_quant_fp8")
+    return q, sf

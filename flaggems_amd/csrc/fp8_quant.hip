@@ -57,6 +57,12 @@ __device__ __forceinline__ float derive_scale(float amax, const QuantArgs& a) {
     uint32_t m = b & 0x7FFFFFu;
     uint32_t l = e - 127u + (m != 0u ? 1u : 0u);
     s = bits_to_float((l + 127u) << 23);
+  } else if (a.pow2_rule == FG_POW2_BITS_CLAMPED) {
+    // the same on |s| with the exponent field held in [1, 254] (reference tests/test_fp8_einsum.py:63-67)
+    const uint32_t b = float_to_bits(s) & 0x7FFFFFFFu;
+    uint32_t e = (b >> 23) + ((b & 0x7FFFFFu) != 0u ? 1u : 0u);
+    e = e < 1u ? 1u : (e > 254u ? 254u : e);
+    s = bits_to_float(e << 23);
   } else if (a.pow2_rule == FG_POW2_LOG2) {
     // exp2(ceil(log2(max(|s|, 1e-10)))) with log2 rounded to fp32 the way a correctly rounded
     // libm does it (reference src/flag_gems/ops/per_token_group_quant_fp8.py:65-66)
@@ -258,8 +264,166 @@ int launch_quant(const QuantArgs& a, bool vec_ok, hipStream_t stream) {
   return FG_OK;
 }
 
+// ---- 128 x 128 block quantizer (weights)
+//
+// One workgroup per block: thread t owns the 8-element chunk (t & 15) of rows (t >> 4) + 16 i, i < 8, so a
+// wavefront reads four whole 256-byte (bf16) row pieces per load instruction.  The block's absolute maximum goes
+// through DPP within a wavefront and through LDS across the four; scale and codes follow the group
+// quantizer's rules.  Elements past the matrix edge count as zeros (the reference pads with zeros,
+// tests/test_fp8_einsum.py:89-103) and are not written.
+constexpr int kBlockQuantEdge = 128;
+
+struct BlockQuantArgs {
+  QuantArgs r;         // pointers, row strides, rules; group fields unused
+  uint32_t rows, cols;
+  int vec;             // rows of x are 16-byte aligned and rows of q 8-byte aligned
+};
+
+template <int XDT>
+__global__ __launch_bounds__(kQuantThreads) void block_quant_kernel(BlockQuantArgs b) {
+  using E = Elem<XDT>;
+  using Raw = typename E::raw;
+  constexpr int kWords = sizeof(Raw) * 8 / 4;
+  constexpr int kIters = kBlockQuantEdge * kBlockQuantEdge / 8 / kQuantThreads;  // 8
+  __shared__ uint32_t wave_max[kQuantThreads / 64];
+  const QuantArgs& a = b.r;
+  const uint32_t t = threadIdx.x;
+  const uint32_t col = blockIdx.x * kBlockQuantEdge + (t & 15u) * 8u;
+  const uint32_t row0 = blockIdx.y * kBlockQuantEdge + (t >> 4);
+  const bool whole = b.vec && col + 8u <= b.cols;  // the chunk lies inside the row and takes vector accesses
+
+  uint32_t w[kIters][kWords];
+#pragma unroll
+  for (int i = 0; i < kIters; ++i) {
+    const uint32_t row = row0 + 16u * (uint32_t)i;
+#pragma unroll
+    for (int k = 0; k < kWords; ++k) w[i][k] = 0u;
+    if (row < b.rows && col < b.cols) {
+      const Raw* p = reinterpret_cast<const Raw*>(a.x) + (int64_t)row * a.x_row_stride + col;
+      if (whole) {
+        const u32x4* p4 = reinterpret_cast<const u32x4*>(p);
+        u32x4 v = p4[0];
+        w[i][0] = v.x; w[i][1] = v.y; w[i][2] = v.z; w[i][3] = v.w;
+        if constexpr (kWords == 8) {
+          u32x4 v2 = p4[1];
+          w[i][4] = v2.x; w[i][5] = v2.y; w[i][6] = v2.z; w[i][7] = v2.w;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint32_t v = (col + (uint32_t)e < b.cols) ? (uint32_t)p[e] : 0u;
+          if constexpr (kWords == 4) w[i][e >> 1] |= v << (16 * (e & 1));
+          else w[i][e] = v;
+        }
+      }
+    }
+  }
+
+  // absolute maximum on the raw bit patterns: NaN patterns compare above everything
+  uint32_t m = 0u;
+#pragma unroll
+  for (int i = 0; i < kIters; ++i)
+#pragma unroll
+    for (int k = 0; k < kWords; ++k) {
+      if constexpr (kWords == 4) m = max(m, max(w[i][k] & E::kAbs, (w[i][k] >> 16) & E::kAbs));
+      else m = max(m, w[i][k] & E::kAbs);
+    }
+  m = group_max_u32<64>(m);
+  if ((t & 63u) == 0u) wave_max[t >> 6] = m;
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kQuantThreads / 64; ++k) m = max(m, wave_max[k]);
+
+  float amax = E::widen(m);
+  const bool special = m >= E::kInf;  // Inf or NaN somewhere in the block
+  if (!(amax != amax)) amax = fmaxf(amax, a.floor);
+  const float s = derive_scale(amax, a);
+  const float r = 1.0f / s;
+  if (t == 0) a.s[(int64_t)blockIdx.y * a.s_row_stride + (int64_t)blockIdx.x * a.s_col_stride] = s;
+
+#pragma unroll
+  for (int i = 0; i < kIters; ++i) {
+    const uint32_t row = row0 + 16u * (uint32_t)i;
+    if (!(row < b.rows && col < b.cols)) continue;
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float xv;
+      if constexpr (kWords == 4) xv = E::widen((w[i][e >> 1] >> (16 * (e & 1))) & 0xFFFFu);
+      else xv = E::widen(w[i][e]);
+      y[e] = quantize_value(xv, s, r, a);
+      // The reference casts the quotient without clamping it, and an e4m3fn cast has no infinity: what lies
+      // past the last finite code's rounding interval (|y| > 464) becomes NaN.  Only an infinite input gets there.
+      if (special && !a.e5m2) {
+        const float raw = (a.quotient_rule == FG_QUOT_RECIP_MUL) ? xv * r : xv / s;
+        if (fabsf(raw) > 464.0f) y[e] = bits_to_float(0x7FC00000u | (float_to_bits(raw) & 0x80000000u));
+      }
+    }
+    uint32_t w0 = pack2<false>(y[0], y[1], 0u, a.e5m2);
+    w0 = pack2<true>(y[2], y[3], w0, a.e5m2);
+    uint32_t w1 = pack2<false>(y[4], y[5], 0u, a.e5m2);
+    w1 = pack2<true>(y[6], y[7], w1, a.e5m2);
+    if (special || !(s == s)) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        w0 = fix_nan_byte(w0, e, y[e], a.e5m2);
+        w1 = fix_nan_byte(w1, e, y[4 + e], a.e5m2);
+      }
+    }
+    uint8_t* qp = a.q + (int64_t)row * a.q_row_stride + col;
+    if (whole) {
+      u32x2 out = {w0, w1};
+      *reinterpret_cast<u32x2*>(qp) = out;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (col + (uint32_t)e < b.cols) qp[e] = (uint8_t)(((e < 4 ? w0 : w1) >> (8 * (e & 3))) & 0xFFu);
+    }
+  }
+}
+
 }  // namespace
 }  // namespace fg
+
+extern "C" int fg_block_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride,
+                                  void* q, int q_dtype, int64_t q_row_stride,
+                                  float* s, int64_t s_row_stride, int64_t s_col_stride,
+                                  int64_t block_rows, int64_t block_cols, float amax_floor, float fp8_min, float fp8_max,
+                                  float inv_fp8_max, int scale_rule, int quotient_rule, int pow2_rule,
+                                  void* stream) {
+  using namespace fg;
+  const char* const who = "fg_block_quant_fp8";
+  if (rows < 0 || cols < 0) FG_FAIL(FG_ERR_INVALID_ARG, "%s: negative size", who);
+  if (rows == 0 || cols == 0) return FG_OK;
+  if (!x || !q || !s) FG_FAIL(FG_ERR_INVALID_ARG, "%s: null pointer", who);
+  if (block_rows != kBlockQuantEdge || block_cols != kBlockQuantEdge)
+    FG_FAIL(FG_ERR_UNSUPPORTED, "%s: only 128 x 128 blocks are implemented (got %lld x %lld)", who,
+            (long long)block_rows, (long long)block_cols);
+  if (x_dtype != FG_BF16 && x_dtype != FG_F16 && x_dtype != FG_F32) FG_FAIL(FG_ERR_INVALID_ARG, "%s: x_dtype %d", who, x_dtype);
+  if (q_dtype != FG_FP8_E4M3FN && q_dtype != FG_FP8_E5M2) FG_FAIL(FG_ERR_INVALID_ARG, "%s: q_dtype %d", who, q_dtype);
+  if (scale_rule < 0 || scale_rule > 1 || quotient_rule < 0 || quotient_rule > 1 || pow2_rule < 0 || pow2_rule > 3)
+    FG_FAIL(FG_ERR_INVALID_ARG, "%s: bad rule selector", who);
+  if (x_row_stride < cols || q_row_stride < cols) FG_FAIL(FG_ERR_INVALID_ARG, "%s: row stride smaller than cols", who);
+  const int64_t block_rows_n = ceil_div(rows, (int64_t)kBlockQuantEdge), block_cols_n = ceil_div(cols, (int64_t)kBlockQuantEdge);
+  if (block_rows_n > 65535 || block_cols_n > 0x7FFFFFFF || cols > 0x7FFFFF00ll)
+    FG_FAIL(FG_ERR_UNSUPPORTED, "%s: more than 65535 block rows or 2^31 columns", who);
+  const size_t esz = (x_dtype == FG_F32) ? 4 : 2;
+  BlockQuantArgs b = {};
+  b.r.x = x; b.r.q = (uint8_t*)q; b.r.s = s;
+  b.r.x_row_stride = x_row_stride; b.r.q_row_stride = q_row_stride;
+  b.r.s_row_stride = s_row_stride; b.r.s_col_stride = s_col_stride;
+  b.r.floor = amax_floor; b.r.lo = fp8_min; b.r.hi = fp8_max; b.r.inv_max = inv_fp8_max;
+  b.r.scale_rule = scale_rule; b.r.quotient_rule = quotient_rule; b.r.pow2_rule = pow2_rule;
+  b.r.e5m2 = (q_dtype == FG_FP8_E5M2);
+  b.rows = (uint32_t)rows; b.cols = (uint32_t)cols;
+  b.vec = ((uintptr_t)x % 16 == 0) && ((x_row_stride * esz) % 16 == 0) && ((uintptr_t)q % 8 == 0) && (q_row_stride % 8 == 0);
+  const dim3 grid((uint32_t)block_cols_n, (uint32_t)block_rows_n);
+  if (x_dtype == FG_BF16) hipLaunchKernelGGL(block_quant_kernel<FG_BF16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, b);
+  else if (x_dtype == FG_F16) hipLaunchKernelGGL(block_quant_kernel<FG_F16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, b);
+  else hipLaunchKernelGGL(block_quant_kernel<FG_F32>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, b);
+  FG_CHECK_LAUNCH("block_quant_kernel");
+  return FG_OK;
+}
 
 extern "C" int fg_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride,
                                   void* q, int q_dtype, int64_t q_row_stride,
@@ -278,7 +442,7 @@ extern "C" int fg_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int6
     FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: x_dtype %d", x_dtype);
   if (q_dtype != FG_FP8_E4M3FN && q_dtype != FG_FP8_E5M2)
     FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: q_dtype %d", q_dtype);
-  if (scale_rule < 0 || scale_rule > 1 || quotient_rule < 0 || quotient_rule > 1 || pow2_rule < 0 || pow2_rule > 2)
+  if (scale_rule < 0 || scale_rule > 1 || quotient_rule < 0 || quotient_rule > 1 || pow2_rule < 0 || pow2_rule > 3)
     FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: bad rule selector");
   if (x_row_stride < cols || q_row_stride < cols)
     FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: row stride smaller than cols");

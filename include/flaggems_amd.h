@@ -54,7 +54,9 @@ typedef enum fg_quotient_rule {
 typedef enum fg_pow2_rule {
   FG_POW2_NONE = 0,
   FG_POW2_BITS = 1, /* exponent + (mantissa != 0), 32-bit wrap-around as in fast_round_scale */
-  FG_POW2_LOG2 = 2  /* exp2(ceil(log2(max(|s|, 1e-10)))) */
+  FG_POW2_LOG2 = 2, /* exp2(ceil(log2(max(|s|, 1e-10)))) */
+  FG_POW2_BITS_CLAMPED = 3 /* |s|: exponent + (mantissa != 0) held in [1, 254], as in _ceil_to_ue8m0
+                              (tests/test_fp8_einsum.py:63-67): Inf and NaN become 2^127 */
 } fg_pow2_rule;
 
 /* Library version (major*10000 + minor*100 + patch) and last error text (thread-local). */
@@ -83,6 +85,23 @@ int fg_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, i
                        void* q, int q_dtype, int64_t q_row_stride,
                        float* s, int64_t s_row_stride, int64_t s_col_stride,
                        int64_t group_size, float amax_floor, float fp8_min, float fp8_max,
+                       float inv_fp8_max, int scale_rule, int quotient_rule, int pow2_rule,
+                       void* stream);
+
+/*
+ * Block quantizer for weights: one fp32 scale per block_rows x block_cols block of x [rows, cols] (unit column
+ * stride); blocks that hang over the matrix edge see zeros there (the reference pads with zeros) and only the
+ * rows x cols codes are written.  s: [ceil(rows/block_rows), ceil(cols/block_cols)] with both strides given.
+ * The rule selectors, the floor and the fp8 limits mean what they mean in fg_group_quant_fp8.  Only 128 x 128
+ * blocks are implemented (FG_ERR_UNSUPPORTED otherwise).
+ * The reference keeps this quantizer in torch, next to the tests and benchmarks that need block-quantized
+ * weights: per_block_cast_to_fp8 (tests/test_fp8_einsum.py:89-103, benchmark/test_fp8_einsum.py:82-96), which is
+ * floor 1e-4, FG_SCALE_DIV, FG_QUOT_RECIP_MUL, limits -/+448 and FG_POW2_BITS_CLAMPED when use_ue8m0 else FG_POW2_NONE.
+ */
+int fg_block_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride,
+                       void* q, int q_dtype, int64_t q_row_stride,
+                       float* s, int64_t s_row_stride, int64_t s_col_stride,
+                       int64_t block_rows, int64_t block_cols, float amax_floor, float fp8_min, float fp8_max,
                        float inv_fp8_max, int scale_rule, int quotient_rule, int pow2_rule,
                        void* stream);
 
