@@ -10,9 +10,11 @@ from .act_quant import (  # noqa: F401
     SUPPORTED_FP8_DTYPE,
     act_quant_triton,
     per_block_cast_to_fp8,
+    per_token_cast_to_fp8,
     per_token_group_quant_fp8,
 )
 from .cutlass_scaled_mm import SM_VERSION_NUM, cutlass_scaled_mm, get_sm_version_num  # noqa: F401
+from .fp8_einsum import fp8_einsum, w8a8_block_fp8_bmm  # noqa: F401
 from .grouped_block_fp8_matmul import grouped_w8a8_block_fp8_matmul  # noqa: F401
 from .registration import (  # noqa: F401
     all_registered_keys,
@@ -38,14 +40,17 @@ __all__ = [
     "apply_gems_patches_to_vllm",
     "cutlass_scaled_mm",
     "enable",
+    "fp8_einsum",
     "fp8_matmul",
     "grouped_w8a8_block_fp8_matmul",
     "only_enable",
     "patch_empty_vllm",
     "per_block_cast_to_fp8",
+    "per_token_cast_to_fp8",
     "per_token_group_quant_fp8",
     "scaled_mm",
     "scaled_mm_out",
     "use_gems",
+    "w8a8_block_fp8_bmm",
     "w8a8_block_fp8_matmul",
 ]

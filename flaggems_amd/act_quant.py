@@ -242,3 +242,34 @@ def per_block_cast_to_fp8(
         )
     _lib.check(status, "fg_block_quant_fp8")
     return q, sf
+
+
+def per_token_cast_to_fp8(
+    x: torch.Tensor, use_ue8m0: bool = True, gran_k: int = 128
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Quantize a 2-D activation to e4m3fn with one fp32 scale per ``1 x gran_k`` group.
+
+    Same parameters, defaults and results (bit for bit) as the torch helper of the reference's einsum test
+    (tests/test_fp8_einsum.py:70-86): amax floored at 1e-4, scale = amax / 448 (rounded up to a power of two when
+    ``use_ue8m0``), codes = x * (1 / scale).  The last dimension must be a multiple of ``gran_k`` (the reference
+    pads with zeros otherwise; not implemented here).  Returns (codes [m, n], scales [m, n / gran_k] fp32).
+    """
+    logger.debug("GEMS PER_TOKEN_CAST_TO_FP8")
+    assert x.dim() == 2
+    if x.dtype not in _IN_DTYPES:
+        raise NotImplementedError(f"per_token_cast_to_fp8: unsupported input dtype {x.dtype}")
+    m, n = x.shape
+    if n % gran_k != 0:
+        raise NotImplementedError(f"per_token_cast_to_fp8: last dimension {n} is not a multiple of {gran_k}")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    q = torch.empty((m, n), dtype=torch.float8_e4m3fn, device=x.device)
+    sf = torch.empty((m, n // gran_k), dtype=torch.float32, device=x.device)
+    if x.numel() == 0:
+        return q, sf
+    _launch_group_quant(
+        x, q, sf, gran_k, floor=1e-4, fp8_min=-448.0, fp8_max=448.0,
+        scale_rule=_lib.FG_SCALE_DIV, quotient_rule=_lib.FG_QUOT_RECIP_MUL,
+        pow2_rule=_lib.FG_POW2_BITS_CLAMPED if use_ue8m0 else _lib.FG_POW2_NONE,
+    )
+    return q, sf

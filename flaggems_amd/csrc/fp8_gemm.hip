@@ -616,6 +616,32 @@ extern "C" int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int6
   return launch_gemm<kModeBlock>(a, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
+extern "C" int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_batch_stride,
+                                         const void* B, int64_t ldb, int64_t b_batch_stride,
+                                         const float* As, int64_t as_row_stride, int64_t as_col_stride, int64_t as_batch_stride,
+                                         const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride, int64_t bs_batch_stride,
+                                         void* C, int64_t ldc, int64_t c_batch_stride, int c_dtype,
+                                         int64_t batch, int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
+                                         void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace fg;
+  if (batch < 0) FG_FAIL(FG_ERR_INVALID_ARG, "fg_batched_block_fp8_gemm: negative batch count");
+  if (a_batch_stride < 0 || b_batch_stride < 0 || as_batch_stride < 0 || bs_batch_stride < 0 || c_batch_stride < 0)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_batched_block_fp8_gemm: negative batch stride");
+  const size_t c_elem = c_dtype == FG_F32 ? 4 : 2;
+  // One launch per matrix, in batch order on the caller's stream: each is the plain GEMM of its operands (same
+  // kernels, same bits), and launches that follow each other on a stream may share the workspace.
+  for (int64_t i = 0; i < batch; ++i) {
+    const int rc = fg_block_fp8_gemm(
+        A ? (const uint8_t*)A + i * a_batch_stride : nullptr, lda, B ? (const uint8_t*)B + i * b_batch_stride : nullptr, ldb,
+        As ? As + i * as_batch_stride : nullptr, as_row_stride, as_col_stride,
+        Bs ? Bs + i * bs_batch_stride : nullptr, bs_row_stride, bs_col_stride,
+        C ? (uint8_t*)C + (size_t)(i * c_batch_stride) * c_elem : nullptr, ldc, c_dtype, M, N, K, block_n, block_k,
+        workspace, workspace_bytes, stream);
+    if (rc != FG_OK) return rc;
+  }
+  return FG_OK;
+}
+
 extern "C" size_t fg_grouped_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   (void)N;
   return fg::grouped_workspace_bytes(M, K);

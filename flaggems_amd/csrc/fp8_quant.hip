@@ -87,6 +87,16 @@ __device__ __forceinline__ float quantize_value(float x, float s, float r, const
   return (y != y) ? y : c;
 }
 
+// The reference helpers that round scales with FG_POW2_BITS_CLAMPED cast the quotient without clamping it
+// (tests/test_fp8_einsum.py:70-103), and an e4m3fn cast has no infinity: what lies past the last finite code's
+// rounding interval (|y| > 464) becomes NaN.  Only an infinite input under a scale held at 2^127 gets there, so the
+// callers apply this to groups that hold an Inf or NaN only.
+__device__ __forceinline__ float unclamped_overflow(float x, float s, float r, float y, const QuantArgs& a) {
+  if (a.pow2_rule != FG_POW2_BITS_CLAMPED || a.e5m2) return y;
+  const float raw = (a.quotient_rule == FG_QUOT_RECIP_MUL) ? x * r : x / s;
+  return fabsf(raw) > 464.0f ? bits_to_float(0x7FC00000u | (float_to_bits(raw) & 0x80000000u)) : y;
+}
+
 template <bool HI>
 __device__ __forceinline__ uint32_t pack2(float v0, float v1, uint32_t old, int e5m2) {
   if (e5m2) return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(v0, v1, (int)old, HI);
@@ -185,6 +195,10 @@ __global__ __launch_bounds__(kQuantThreads) void group_quant_vec_kernel(QuantArg
     float y[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) y[i] = quantize_value(xv[i], s, r, a);
+    if (special) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = unclamped_overflow(xv[i], s, r, y[i], a);
+    }
     uint32_t w0 = pack2<false>(y[0], y[1], 0u, a.e5m2);
     w0 = pack2<true>(y[2], y[3], w0, a.e5m2);
     uint32_t w1 = pack2<false>(y[4], y[5], 0u, a.e5m2);
@@ -229,6 +243,7 @@ __global__ __launch_bounds__(kQuantThreads) void group_quant_generic_kernel(Quan
   const float r = 1.0f / s;
   for (uint32_t i = lane; i < a.group_size; i += 64) {
     float y = quantize_value(E::widen((uint32_t)xp[i]), s, r, a);
+    if (m >= E::kInf) y = unclamped_overflow(E::widen((uint32_t)xp[i]), s, r, y, a);
     uint32_t wd = pack2<false>(y, 0.0f, 0u, a.e5m2);
     wd = fix_nan_byte(wd, 0, y, a.e5m2);
     qp[i] = (uint8_t)(wd & 0xFFu);
@@ -352,12 +367,7 @@ __global__ __launch_bounds__(kQuantThreads) void block_quant_kernel(BlockQuantAr
       if constexpr (kWords == 4) xv = E::widen((w[i][e >> 1] >> (16 * (e & 1))) & 0xFFFFu);
       else xv = E::widen(w[i][e]);
       y[e] = quantize_value(xv, s, r, a);
-      // The reference casts the quotient without clamping it, and an e4m3fn cast has no infinity: what lies
-      // past the last finite code's rounding interval (|y| > 464) becomes NaN.  Only an infinite input gets there.
-      if (special && !a.e5m2) {
-        const float raw = (a.quotient_rule == FG_QUOT_RECIP_MUL) ? xv * r : xv / s;
-        if (fabsf(raw) > 464.0f) y[e] = bits_to_float(0x7FC00000u | (float_to_bits(raw) & 0x80000000u));
-      }
+      if (special) y[e] = unclamped_overflow(xv, s, r, y[e], a);
     }
     uint32_t w0 = pack2<false>(y[0], y[1], 0u, a.e5m2);
     w0 = pack2<true>(y[2], y[3], w0, a.e5m2);

@@ -56,7 +56,9 @@ typedef enum fg_pow2_rule {
   FG_POW2_BITS = 1, /* exponent + (mantissa != 0), 32-bit wrap-around as in fast_round_scale */
   FG_POW2_LOG2 = 2, /* exp2(ceil(log2(max(|s|, 1e-10)))) */
   FG_POW2_BITS_CLAMPED = 3 /* |s|: exponent + (mantissa != 0) held in [1, 254], as in _ceil_to_ue8m0
-                              (tests/test_fp8_einsum.py:63-67): Inf and NaN become 2^127 */
+                              (tests/test_fp8_einsum.py:63-67): Inf and NaN become 2^127; with this rule an
+                              infinite input under such a scale gives the NaN code, as a cast that is not
+                              preceded by a clamp does */
 } fg_pow2_rule;
 
 /* Library version (major*10000 + minor*100 + patch) and last error text (thread-local). */
@@ -150,6 +152,25 @@ int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
 
 #define FG_WORKSPACE_COUNTER_BYTES 16384
 size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Batched block-scaled FP8 GEMM: `batch` independent problems of fg_block_fp8_gemm with the same M, N, K and
+ * strides.  Matrix i of each operand starts i * <its batch stride> after matrix 0 (bytes for A and B, floats for
+ * the scales, elements of c_dtype for C); row strides are free, so a [b, h, r] activation with h as the batch
+ * takes lda = h * r and a_batch_stride = r.  The matrices are launched one after the other on `stream`: the
+ * results are, bit for bit, those of `batch` calls of fg_block_fp8_gemm, and the workspace rules are that entry
+ * point's (fg_block_fp8_gemm_workspace_bytes(M, N, K); one workspace serves the whole batch).
+ *
+ * Stands in for w8a8_block_fp8_bmm (src/flag_gems/runtime/backend/_nvidia/hopper/ops/w8a8_block_fp8_bmm.py:629-779)
+ * and, through it, fp8_einsum("bhr,hdr->bhd") (.../hopper/ops/fp8_einsum.py:22-68).
+ */
+int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_batch_stride,
+                              const void* B, int64_t ldb, int64_t b_batch_stride,
+                              const float* As, int64_t as_row_stride, int64_t as_col_stride, int64_t as_batch_stride,
+                              const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride, int64_t bs_batch_stride,
+                              void* C, int64_t ldc, int64_t c_batch_stride, int c_dtype,
+                              int64_t batch, int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
+                              void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Grouped block-scaled FP8 GEMM (mixture-of-experts layers with the tokens sorted by expert):

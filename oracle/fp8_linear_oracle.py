@@ -29,6 +29,9 @@ the checks live in tests/test_oracle_*.py):
   segments; pinned by the dequantise-then-matmul reference per segment, by "one
   group = the plain GEMM", by "identical weights in every group = the plain GEMM
   whatever the segment ends", and by a float64 loop on a tiny ragged case.
+* fp8_block_einsum_ref -- dequantise-then-einsum over [b, h, r] x [h, d, r]; pinned
+  per head against block_fp8_matmul_tiled_ref (a different order of operations)
+  and by a float64 loop on a tiny case.
 * scaled_mm_ref, scaled_mm_ref_postscale -- pinned against each other, a float64
   loop, and the unit-scale/zero-bias closed form.
 
@@ -295,6 +298,48 @@ def grouped_block_fp8_matmul_ref(
             )
         begin = max(begin, end)
     return c
+
+
+def fp8_block_einsum_ref(
+    x_data: torch.Tensor,
+    x_scale: torch.Tensor,
+    y_data: torch.Tensor,
+    y_scale: torch.Tensor,
+    block_shape: List[int],
+) -> torch.Tensor:
+    """Restates ``torch_fp8_block_einsum_reference`` (reference tests/test_fp8_einsum.py:130-160):
+    x [b, h, r] dequantised per (token, head, K-block), y [h, d, r] per (head, N-block, K-block), then
+    ``einsum("bhr,hdr->bhd")`` in fp32."""
+    block_n, block_k = block_shape
+    b, h, r = x_data.shape
+    d = y_data.shape[1]
+    x_f = x_data.to(torch.float32)
+    y_f = y_data.to(torch.float32)
+    x_deq = torch.empty_like(x_f)
+    for kt in range(x_scale.shape[-1]):
+        ks, ke = kt * block_k, min((kt + 1) * block_k, r)
+        x_deq[:, :, ks:ke] = x_f[:, :, ks:ke] * x_scale[:, :, kt : kt + 1]
+    y_deq = torch.empty_like(y_f)
+    for nt in range(y_scale.shape[1]):
+        ns, ne = nt * block_n, min((nt + 1) * block_n, d)
+        for kt in range(x_scale.shape[-1]):
+            ks, ke = kt * block_k, min((kt + 1) * block_k, r)
+            y_deq[:, ns:ne, ks:ke] = y_f[:, ns:ne, ks:ke] * y_scale[:, nt, kt].view(h, 1, 1)
+    return torch.einsum("bhr,hdr->bhd", x_deq, y_deq)
+
+
+def make_fp8_einsum_inputs(b: int, h: int, r: int, d: int, seed: int = 0):
+    """Inputs as the reference test builds them (tests/test_fp8_einsum.py:105-127): x, y ~ N(0,1) bf16,
+    x cast per token (1 x 128, power-of-two scales), y per head per 128 x 128 block (power-of-two scales)."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((b, h, r), generator=g).bfloat16()
+    y = torch.randn((h, d, r), generator=g).bfloat16()
+    xq, xs = per_token_cast_to_fp8_ref(x.view(-1, r), use_ue8m0=True)
+    yq = torch.empty((h, d, r), dtype=FP8_DTYPE)
+    ys = torch.empty((h, (d + 127) // 128, (r + 127) // 128), dtype=torch.float32)
+    for i in range(h):
+        yq[i], ys[i] = per_block_cast_to_fp8_ref(y[i], use_ue8m0=True)
+    return xq.view(b, h, r), xs.view(b, h, -1), yq, ys
 
 
 def make_moe_rows(tokens: int, experts: int = 8, top_k: int = 2, seed: int = 0) -> torch.Tensor:

@@ -219,3 +219,19 @@ def test_moe_rows_are_cumulative_and_skewed():
     counts = torch.diff(ends, prepend=torch.zeros(1, dtype=torch.int32))
     assert (counts >= 0).all() and counts.max() > 2 * counts.min()
     assert torch.equal(ends, O.make_moe_rows(4096, 8, 2, seed=0))
+
+
+# ---- batched einsum
+
+
+def test_einsum_ref_per_head_and_f64():
+    xq, xs, yq, ys = O.make_fp8_einsum_inputs(5, 3, 256, 256, seed=31)
+    got = O.fp8_block_einsum_ref(xq, xs, yq, ys, [128, 128])
+    assert got.shape == (5, 3, 256)
+    for head in range(3):
+        want = O.block_fp8_matmul_tiled_ref(xq[:, head], yq[head], xs[:, head], ys[head], [128, 128])
+        torch.testing.assert_close(got[:, head], want, rtol=1e-4, atol=1e-5)
+    want = _loop_f64(xq[:2, 1].contiguous(), yq[1, :9].contiguous(), xs[:2, 1], ys[1])
+    np.testing.assert_allclose(got[:2, 1, :9].double().numpy(), want, rtol=1e-5, atol=1e-6)
+    # scales of this input maker are powers of two and every group's largest code is +-448 or the group is tiny
+    assert torch.all(torch.frexp(xs)[0] == 0.5) and torch.all(torch.frexp(ys)[0] == 0.5)
