@@ -261,6 +261,28 @@ def main():
                     "frac_hbm": round(wq_gbs / PEAK_HBM_GBPS, 4)}
     del w_in
 
+    # ---- activation fused into the quantizer (HBM bound): bf16 [8192, 2 x 14336] gate|up -> e4m3fn [8192, 14336],
+    # next to the two separate kernels it replaces
+    gu = torch.randn(8192, 2 * 14336, device=dev, generator=gen).bfloat16()
+
+    def time_calls(fn, reps=20):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(reps):
+            fn()
+        end.record()
+        end.synchronize()
+        return start.elapsed_time(end) * 1e3 / reps
+
+    fused_us = time_calls(lambda: flag_gems.silu_and_mul_per_token_group_quant_fp8(gu, 128))
+    apart_us = time_calls(lambda: flag_gems.per_token_group_quant_fp8(flag_gems.silu_and_mul_packed(gu), 128))
+    fused_gbs = (5.0 + 4.0 / 128) * 8192 * 14336 / (fused_us * 1e-6) / 1e9
+    fused = {"shape": [8192, 28672], "us": round(fused_us, 2), "gbps": round(fused_gbs, 1),
+             "frac_hbm": round(fused_gbs / PEAK_HBM_GBPS, 4), "two_kernels_us": round(apart_us, 2)}
+    del gu
+
     # ---- the other configurations of the path, each shape timed alone: HIP events around the replay of a graph
     # of `reps` launches (as above: decode-sized launches are shorter than a Python call)
     def time_eager(fn, reps):
@@ -386,6 +408,7 @@ def main():
         "roofline_small_m": roofline_small,
         "quantizer": quant,
         "weight_quantizer_128x128": weight_quant,
+        "silu_mul_quantizer": fused,
         "cutlass_scaled_mm_n8192_k8192_bias": scaled,
         "llama3_8b_linears": llama,
         "mixtral_moe_grouped_gemm": moe,

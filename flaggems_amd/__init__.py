@@ -12,6 +12,8 @@ from .act_quant import (  # noqa: F401
     per_block_cast_to_fp8,
     per_token_cast_to_fp8,
     per_token_group_quant_fp8,
+    silu_and_mul_packed,
+    silu_and_mul_per_token_group_quant_fp8,
 )
 from .cutlass_scaled_mm import SM_VERSION_NUM, cutlass_scaled_mm, get_sm_version_num  # noqa: F401
 from .fp8_einsum import fp8_einsum, w8a8_block_fp8_bmm  # noqa: F401
@@ -50,6 +52,8 @@ __all__ = [
     "per_token_group_quant_fp8",
     "scaled_mm",
     "scaled_mm_out",
+    "silu_and_mul_packed",
+    "silu_and_mul_per_token_group_quant_fp8",
     "use_gems",
     "w8a8_block_fp8_bmm",
     "w8a8_block_fp8_matmul",

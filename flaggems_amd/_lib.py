@@ -46,6 +46,12 @@ SIGNATURES = {
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64,
          c_int64, c_int64, c_float, c_float, c_float, c_float, c_int, c_int, c_int, c_void_p],
     ),
+    "fg_silu_mul_group_quant_fp8": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64,
+         c_int64, c_float, c_float, c_float, c_float, c_int, c_int, c_int, c_void_p],
+    ),
+    "fg_silu_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p]),
     "fg_act_quant_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "fg_block_fp8_gemm": (
         c_int,

@@ -273,3 +273,81 @@ def per_token_cast_to_fp8(
         pow2_rule=_lib.FG_POW2_BITS_CLAMPED if use_ue8m0 else _lib.FG_POW2_NONE,
     )
     return q, sf
+
+
+def silu_and_mul_packed(x: torch.Tensor) -> torch.Tensor:
+    """``silu(x[..., :d]) * x[..., d:]`` with d = x.shape[-1] // 2, in x's dtype.
+
+    The arithmetic of the reference's activation kernel (src/flag_gems/fused/silu_and_mul.py:13-18 and
+    src/flag_gems/fused/fused_moe.py:795-800): fp32 ``g / (1 + exp(-g)) * u``, rounded once to the output type,
+    applied to the gate and up halves of one tensor the way the expert layers hold them."""
+    logger.debug("GEMS SILU_AND_MUL")
+    assert x.shape[-1] % 2 == 0 and x.stride(-1) == 1
+    if x.dtype not in _IN_DTYPES:
+        raise NotImplementedError(f"silu_and_mul_packed: unsupported input dtype {x.dtype}")
+    d = x.shape[-1] // 2
+    out = torch.empty(x.shape[:-1] + (d,), dtype=x.dtype, device=x.device)
+    if out.numel() == 0:
+        return out
+    x2d = _as_rows(x)
+    _lib.require_gpu(x2d, "silu_and_mul")
+    rows = x2d.shape[0]
+    with torch.cuda.device(x.device):
+        status = _lib.load().fg_silu_mul(
+            x2d.data_ptr(), _lib.DTYPE_CODE[x.dtype], rows, d, x2d.stride(0) if rows > 1 else max(2 * d, x2d.stride(0)), d,
+            out.data_ptr(), d, _lib.current_stream_ptr(x.device))
+    _lib.check(status, "fg_silu_mul")
+    return out
+
+
+def silu_and_mul_per_token_group_quant_fp8(
+    x: torch.Tensor,
+    group_size: int,
+    eps: float = 1e-10,
+    dtype: Optional[torch.dtype] = None,
+    column_major_scales: bool = False,
+    scale_ue8m0: bool = False,
+    *,
+    scale_rule: Optional[str] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``per_token_group_quant_fp8(silu_and_mul_packed(x), group_size, ...)`` in one pass over x.
+
+    The step between the two GEMMs of an expert or MLP layer (src/flag_gems/fused/fused_moe.py:2108-2122): the
+    activated tensor is rounded to x's dtype as the separate kernel would store it, but never written.
+    Same codes and scales, bit for bit, as the two calls.  x [..., 2 d]; returns (x_q [..., d], x_s [..., d / group_size]).
+    """
+    logger.debug("GEMS SILU_AND_MUL PER TOKEN GROUP QUANT FP8")
+    fp8_dtype = SUPPORTED_FP8_DTYPE if dtype is None else dtype
+    assert x.shape[-1] % 2 == 0 and x.stride(-1) == 1
+    d = x.shape[-1] // 2
+    assert d % group_size == 0, f"half of the last dimension of `x` {d} must be divisible by `group_size` {group_size}"
+    if fp8_dtype not in _FP8_DTYPES:
+        raise NotImplementedError(f"silu_and_mul_per_token_group_quant_fp8: unsupported output dtype {fp8_dtype}")
+    if x.dtype not in _IN_DTYPES:
+        raise NotImplementedError(f"silu_and_mul_per_token_group_quant_fp8: unsupported input dtype {x.dtype}")
+    finfo = torch.finfo(fp8_dtype)
+    lead = x.shape[:-1]
+    x_q = torch.empty(lead + (d,), device=x.device, dtype=fp8_dtype)
+    if column_major_scales:
+        if x.dim() != 2:
+            raise NotImplementedError("column_major_scales needs a 2-D input")
+        x_s = torch.empty((d // group_size, x.shape[0]), device=x.device, dtype=torch.float32).permute(-1, -2)
+    else:
+        x_s = torch.empty(lead + (d // group_size,), device=x.device, dtype=torch.float32)
+    if x_q.numel() == 0:
+        return x_q, x_s
+    x2d = _as_rows(x)
+    _lib.require_gpu(x2d, "fused activation + quantizer")
+    rows = x2d.shape[0]
+    q2d = x_q.view(-1, d)
+    s2d = x_s if x_s.dim() == 2 else x_s.view(-1, x_s.shape[-1])
+    with torch.cuda.device(x.device):
+        status = _lib.load().fg_silu_mul_group_quant_fp8(
+            x2d.data_ptr(), _lib.DTYPE_CODE[x.dtype], rows, d, x2d.stride(0) if rows > 1 else max(2 * d, x2d.stride(0)), d,
+            q2d.data_ptr(), _lib.DTYPE_CODE[fp8_dtype], d,
+            s2d.data_ptr(), s2d.stride(0), s2d.stride(1),
+            group_size, _round_to_dtype(float(eps), x.dtype), finfo.min, finfo.max, 1.0 / finfo.max,
+            _scale_rule_code(scale_rule), _lib.FG_QUOT_DIV, _lib.FG_POW2_LOG2 if scale_ue8m0 else _lib.FG_POW2_NONE,
+            _lib.current_stream_ptr(x.device))
+    _lib.check(status, "fg_silu_mul_group_quant_fp8")
+    return x_q, x_s

@@ -25,6 +25,7 @@ struct QuantArgs {
   uint32_t group_size;
   float floor, lo, hi, inv_max;
   int scale_rule, quotient_rule, pow2_rule, e5m2;
+  int64_t up_offset;  // fused SiLU-and-mul producer: elements from a gate value to its up value (same row)
 };
 
 template <int XDT> struct Elem;
@@ -32,6 +33,11 @@ template <> struct Elem<FG_BF16> {
   using raw = uint16_t;
   static constexpr uint32_t kAbs = 0x7FFFu, kInf = 0x7F80u;
   __device__ static float widen(uint32_t b) { return bits_to_float(b << 16); }
+  __device__ static uint32_t narrow(float f) {  // round to nearest even; NaN stays NaN
+    const uint32_t u = float_to_bits(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+  }
 };
 template <> struct Elem<FG_F16> {
   using raw = uint16_t;
@@ -39,12 +45,38 @@ template <> struct Elem<FG_F16> {
   __device__ static float widen(uint32_t b) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
   }
+  __device__ static uint32_t narrow(float f) { return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f); }
 };
 template <> struct Elem<FG_F32> {
   using raw = uint32_t;
   static constexpr uint32_t kAbs = 0x7FFFFFFFu, kInf = 0x7F800000u;
   __device__ static float widen(uint32_t b) { return bits_to_float(b); }
+  __device__ static uint32_t narrow(float f) { return float_to_bits(f); }
 };
+
+// gate * sigmoid(gate) * up in fp32, as the reference's activation kernel computes it
+// (src/flag_gems/fused/fused_moe.py:795-800: x / (1 + exp(-x)) * y), rounded once to the input's type.
+template <int XDT>
+__device__ __forceinline__ uint32_t silu_mul_raw(uint32_t gate, uint32_t up) {
+  using E = Elem<XDT>;
+  const float g = E::widen(gate), u = E::widen(up);
+  return E::narrow(g / (1.0f + expf(-g)) * u);
+}
+
+// eight gate values and eight up values (raw words as loaded) -> eight activated values in the same packing
+template <int XDT, int WORDS>
+__device__ __forceinline__ void silu_mul_words(uint32_t (&w)[WORDS], const uint32_t (&up)[WORDS]) {
+#pragma unroll
+  for (int i = 0; i < WORDS; ++i) {
+    if constexpr (WORDS == 4) {
+      const uint32_t lo = silu_mul_raw<XDT>(w[i] & 0xFFFFu, up[i] & 0xFFFFu);
+      const uint32_t hi = silu_mul_raw<XDT>(w[i] >> 16, up[i] >> 16);
+      w[i] = (lo & 0xFFFFu) | (hi << 16);
+    } else {
+      w[i] = silu_mul_raw<XDT>(w[i], up[i]);
+    }
+  }
+}
 
 // scale from the group's absolute maximum (already floored), following the requested rules
 __device__ __forceinline__ float derive_scale(float amax, const QuantArgs& a) {
@@ -128,7 +160,9 @@ constexpr int kQuantThreads = 256;
 constexpr int kQuantUnroll = 4;
 
 // Vector kernel: group_size == 8 * LPG, rows 16-byte aligned.
-template <int XDT, int LPG>
+// SILU: the value quantized is silu(x[row, c]) * x[row, c + up_offset], rounded to x's type first (what a separate
+// activation kernel would have stored), and x is never re-read.
+template <int XDT, int LPG, bool SILU = false>
 __global__ __launch_bounds__(kQuantThreads) void group_quant_vec_kernel(QuantArgs a) {
   using E = Elem<XDT>;
   constexpr int kWords = sizeof(typename E::raw) * 8 / 4;  // 32-bit words per lane: 4 or 8
@@ -158,6 +192,17 @@ __global__ __launch_bounds__(kQuantThreads) void group_quant_vec_kernel(QuantArg
       if constexpr (kWords == 8) {
         u32x4 v2 = p4[1];
         w[u][4] = v2.x; w[u][5] = v2.y; w[u][6] = v2.z; w[u][7] = v2.w;
+      }
+      if constexpr (SILU) {
+        const u32x4* q4 = reinterpret_cast<const u32x4*>(p + a.up_offset);
+        uint32_t up[kWords];
+        u32x4 t = q4[0];
+        up[0] = t.x; up[1] = t.y; up[2] = t.z; up[3] = t.w;
+        if constexpr (kWords == 8) {
+          u32x4 t2 = q4[1];
+          up[4] = t2.x; up[5] = t2.y; up[6] = t2.z; up[7] = t2.w;
+        }
+        silu_mul_words<XDT, kWords>(w[u], up);
       }
     } else {
 #pragma unroll
@@ -252,12 +297,22 @@ __global__ __launch_bounds__(kQuantThreads) void group_quant_generic_kernel(Quan
 }
 
 template <int XDT>
-int launch_quant(const QuantArgs& a, bool vec_ok, hipStream_t stream) {
+int launch_quant(const QuantArgs& a, bool vec_ok, hipStream_t stream, bool silu = false) {
   const uint32_t g = a.group_size;
   int lpg = 0;
   if (vec_ok && g % 8 == 0) {
     uint32_t l = g / 8;
     if (l == 1 || l == 2 || l == 4 || l == 8 || l == 16 || l == 32 || l == 64) lpg = (int)l;
+  }
+  if (silu) {
+    if (lpg != 16 && lpg != 8)
+      FG_FAIL(FG_ERR_UNSUPPORTED, "fused activation + quantizer: group size 64 or 128 and 16-byte aligned rows only");
+    const uint64_t chunks = (uint64_t)a.total_groups * (uint64_t)lpg;
+    dim3 grid((uint32_t)ceil_div((int64_t)chunks, (int64_t)kQuantThreads * kQuantUnroll));
+    if (lpg == 16) hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, true>), grid, dim3(kQuantThreads), 0, stream, a);
+    else hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 8, true>), grid, dim3(kQuantThreads), 0, stream, a);
+    FG_CHECK_LAUNCH("group_quant_vec_kernel (fused activation)");
+    return FG_OK;
   }
   if (lpg == 0) {
     dim3 grid((uint32_t)ceil_div(a.total_groups, kQuantThreads / 64));
@@ -435,13 +490,15 @@ extern "C" int fg_block_quant_fp8(const void* x, int x_dtype, int64_t rows, int6
   return FG_OK;
 }
 
-extern "C" int fg_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride,
-                                  void* q, int q_dtype, int64_t q_row_stride,
-                                  float* s, int64_t s_row_stride, int64_t s_col_stride,
-                                  int64_t group_size, float amax_floor, float fp8_min, float fp8_max,
-                                  float inv_fp8_max, int scale_rule, int quotient_rule, int pow2_rule,
-                                  void* stream) {
-  using namespace fg;
+namespace fg {
+namespace {
+// silu: the quantized value is silu(x[r, c]) * x[r, c + up_offset] (x then has at least up_offset + cols columns)
+int group_quant_entry(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride,
+                      void* q, int q_dtype, int64_t q_row_stride,
+                      float* s, int64_t s_row_stride, int64_t s_col_stride,
+                      int64_t group_size, float amax_floor, float fp8_min, float fp8_max,
+                      float inv_fp8_max, int scale_rule, int quotient_rule, int pow2_rule,
+                      void* stream, bool silu, int64_t up_offset) {
   if (rows < 0 || cols < 0) FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: negative size");
   if (rows == 0 || cols == 0) return FG_OK;
   if (!x || !q || !s) FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: null pointer");
@@ -456,13 +513,15 @@ extern "C" int fg_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int6
     FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: bad rule selector");
   if (x_row_stride < cols || q_row_stride < cols)
     FG_FAIL(FG_ERR_INVALID_ARG, "fg_group_quant_fp8: row stride smaller than cols");
+  if (silu && (up_offset < cols || x_row_stride < up_offset + cols))
+    FG_FAIL(FG_ERR_INVALID_ARG, "fused activation + quantizer: the up half must follow the gate half inside the row");
   if (group_size > (int64_t)1 << 24) FG_FAIL(FG_ERR_UNSUPPORTED, "fg_group_quant_fp8: group_size too large");
 
   const int64_t groups_per_row = cols / group_size;
   if (groups_per_row > 0x7FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fg_group_quant_fp8: too many groups per row");
   const size_t esz = (x_dtype == FG_F32) ? 4 : 2;
   const bool vec_ok = ((uintptr_t)x % 16 == 0) && ((x_row_stride * esz) % 16 == 0) &&
-                      ((uintptr_t)q % 8 == 0) && (q_row_stride % 8 == 0);
+                      ((uintptr_t)q % 8 == 0) && (q_row_stride % 8 == 0) && (!silu || (up_offset * esz) % 16 == 0);
 
   // Launch in row slabs so that 32-bit chunk indices cannot overflow.
   const int64_t max_groups = (int64_t)1 << 24;
@@ -489,14 +548,92 @@ extern "C" int fg_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int6
     a.quotient_rule = quotient_rule;
     a.pow2_rule = pow2_rule;
     a.e5m2 = (q_dtype == FG_FP8_E5M2);
+    a.up_offset = up_offset;
     int rc;
-    if (x_dtype == FG_BF16) rc = launch_quant<FG_BF16>(a, vec_ok, (hipStream_t)stream);
-    else if (x_dtype == FG_F16) rc = launch_quant<FG_F16>(a, vec_ok, (hipStream_t)stream);
-    else rc = launch_quant<FG_F32>(a, vec_ok, (hipStream_t)stream);
+    if (x_dtype == FG_BF16) rc = launch_quant<FG_BF16>(a, vec_ok, (hipStream_t)stream, silu);
+    else if (x_dtype == FG_F16) rc = launch_quant<FG_F16>(a, vec_ok, (hipStream_t)stream, silu);
+    else rc = launch_quant<FG_F32>(a, vec_ok, (hipStream_t)stream, silu);
     if (rc != FG_OK) return rc;
   }
   return FG_OK;
 }
+
+// out[r, c] = silu(x[r, c]) * x[r, c + up_offset] rounded to x's type; eight elements per thread
+template <int XDT>
+__global__ __launch_bounds__(kQuantThreads) void silu_mul_kernel(const void* x, void* out, int64_t x_row_stride,
+                                                                 int64_t out_row_stride, int64_t up_offset,
+                                                                 uint32_t chunks_per_row, uint32_t total_chunks) {
+  using E = Elem<XDT>;
+  using Raw = typename E::raw;
+  constexpr int kWords = sizeof(Raw) * 8 / 4;
+  const uint32_t c = blockIdx.x * kQuantThreads + threadIdx.x;
+  if (c >= total_chunks) return;
+  const uint32_t row = c / chunks_per_row, col = (c - row * chunks_per_row) * 8u;
+  const Raw* p = reinterpret_cast<const Raw*>(x) + (int64_t)row * x_row_stride + col;
+  uint32_t w[kWords], up[kWords];
+#pragma unroll
+  for (int k = 0; k < kWords / 4; ++k) {
+    const u32x4 v = reinterpret_cast<const u32x4*>(p)[k], t = reinterpret_cast<const u32x4*>(p + up_offset)[k];
+    w[4 * k] = v.x; w[4 * k + 1] = v.y; w[4 * k + 2] = v.z; w[4 * k + 3] = v.w;
+    up[4 * k] = t.x; up[4 * k + 1] = t.y; up[4 * k + 2] = t.z; up[4 * k + 3] = t.w;
+  }
+  silu_mul_words<XDT, kWords>(w, up);
+  Raw* o = reinterpret_cast<Raw*>(out) + (int64_t)row * out_row_stride + col;
+#pragma unroll
+  for (int k = 0; k < kWords / 4; ++k) {
+    const u32x4 v = {w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3]};
+    reinterpret_cast<u32x4*>(o)[k] = v;
+  }
+}
+}  // namespace
+}  // namespace fg
+
+extern "C" int fg_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride,
+                                  void* q, int q_dtype, int64_t q_row_stride,
+                                  float* s, int64_t s_row_stride, int64_t s_col_stride,
+                                  int64_t group_size, float amax_floor, float fp8_min, float fp8_max,
+                                  float inv_fp8_max, int scale_rule, int quotient_rule, int pow2_rule,
+                                  void* stream) {
+  return fg::group_quant_entry(x, x_dtype, rows, cols, x_row_stride, q, q_dtype, q_row_stride, s, s_row_stride,
+                               s_col_stride, group_size, amax_floor, fp8_min, fp8_max, inv_fp8_max, scale_rule,
+                               quotient_rule, pow2_rule, stream, false, 0);
+}
+
+extern "C" int fg_silu_mul_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride,
+                                           int64_t up_offset, void* q, int q_dtype, int64_t q_row_stride,
+                                           float* s, int64_t s_row_stride, int64_t s_col_stride,
+                                           int64_t group_size, float amax_floor, float fp8_min, float fp8_max,
+                                           float inv_fp8_max, int scale_rule, int quotient_rule, int pow2_rule,
+                                           void* stream) {
+  return fg::group_quant_entry(x, x_dtype, rows, cols, x_row_stride, q, q_dtype, q_row_stride, s, s_row_stride,
+                               s_col_stride, group_size, amax_floor, fp8_min, fp8_max, inv_fp8_max, scale_rule,
+                               quotient_rule, pow2_rule, stream, true, up_offset);
+}
+
+extern "C" int fg_silu_mul(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride, int64_t up_offset,
+                           void* out, int64_t out_row_stride, void* stream) {
+  using namespace fg;
+  if (rows < 0 || cols < 0) FG_FAIL(FG_ERR_INVALID_ARG, "fg_silu_mul: negative size");
+  if (rows == 0 || cols == 0) return FG_OK;
+  if (!x || !out) FG_FAIL(FG_ERR_INVALID_ARG, "fg_silu_mul: null pointer");
+  if (x_dtype != FG_BF16 && x_dtype != FG_F16 && x_dtype != FG_F32) FG_FAIL(FG_ERR_INVALID_ARG, "fg_silu_mul: x_dtype %d", x_dtype);
+  if (up_offset < cols || x_row_stride < up_offset + cols || out_row_stride < cols)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_silu_mul: the up half must follow the gate half inside the row");
+  const int64_t esz = (x_dtype == FG_F32) ? 4 : 2;
+  if (cols % 8 != 0 || (uintptr_t)x % 16 != 0 || (uintptr_t)out % 16 != 0 || (x_row_stride * esz) % 16 != 0 ||
+      (out_row_stride * esz) % 16 != 0 || (up_offset * esz) % 16 != 0)
+    FG_FAIL(FG_ERR_UNSUPPORTED, "fg_silu_mul: rows and halves must be 16-byte aligned and cols a multiple of 8");
+  const int64_t chunks = rows * (cols / 8);
+  if (chunks > 0x7FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fg_silu_mul: more than 2^31 chunks");
+  const dim3 grid((uint32_t)ceil_div(chunks, (int64_t)kQuantThreads));
+  const uint32_t cpr = (uint32_t)(cols / 8), total = (uint32_t)chunks;
+  if (x_dtype == FG_BF16) hipLaunchKernelGGL(silu_mul_kernel<FG_BF16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, x, out, x_row_stride, out_row_stride, up_offset, cpr, total);
+  else if (x_dtype == FG_F16) hipLaunchKernelGGL(silu_mul_kernel<FG_F16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, x, out, x_row_stride, out_row_stride, up_offset, cpr, total);
+  else hipLaunchKernelGGL(silu_mul_kernel<FG_F32>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, x, out, x_row_stride, out_row_stride, up_offset, cpr, total);
+  FG_CHECK_LAUNCH("silu_mul_kernel");
+  return FG_OK;
+}
+
 
 extern "C" int fg_act_quant_bf16(const void* x, void* y, float* s, int64_t rows, int64_t cols,
                                  int64_t block_size, int round_scale, void* stream) {

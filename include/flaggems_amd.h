@@ -108,6 +108,35 @@ int fg_block_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, i
                        void* stream);
 
 /*
+ * Activation fused into the quantizer: the value quantized at [r, c] is
+ *     act[r, c] = silu(x[r, c]) * x[r, c + up_offset],   silu(g) = g / (1 + exp(-g)) in fp32,
+ * rounded once to x's type (what a separate activation kernel would have stored) and then quantized exactly as
+ * fg_group_quant_fp8 quantizes a stored act: same codes and scales, bit for bit, as fg_silu_mul followed by
+ * fg_group_quant_fp8, without writing and re-reading act.  x: [rows, >= up_offset + cols]; the gate half starts
+ * at column 0, the up half at column up_offset (>= cols).  group_size 64 or 128; x, its rows and the up half
+ * 16-byte aligned, q rows 8-byte aligned (FG_ERR_UNSUPPORTED otherwise).  Other arguments as fg_group_quant_fp8.
+ *
+ * The reference runs the two steps apart between the two expert GEMMs: _silu_and_mul_kernel
+ * (src/flag_gems/fused/fused_moe.py:795-800; the operator silu_and_mul, src/flag_gems/fused/silu_and_mul.py:13-18)
+ * into intermediate_cache2, then moe_kernel_quantize_input -> per_token_group_quant_fp8
+ * (src/flag_gems/fused/fused_moe.py:2108-2122, 642-659).
+ */
+int fg_silu_mul_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride,
+                                int64_t up_offset, void* q, int q_dtype, int64_t q_row_stride,
+                                float* s, int64_t s_row_stride, int64_t s_col_stride,
+                                int64_t group_size, float amax_floor, float fp8_min, float fp8_max,
+                                float inv_fp8_max, int scale_rule, int quotient_rule, int pow2_rule,
+                                void* stream);
+
+/*
+ * The activation alone: out[r, c] = silu(x[r, c]) * x[r, c + up_offset] in x's type, out [rows, cols] with row
+ * stride out_row_stride.  cols a multiple of 8; x, out, their rows and the up half 16-byte aligned.
+ * Stands in for silu_and_mul_kernel (src/flag_gems/fused/silu_and_mul.py:13-18) on the two halves of one tensor.
+ */
+int fg_silu_mul(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride, int64_t up_offset,
+                void* out, int64_t out_row_stride, void* stream);
+
+/*
  * act_quant with the reference's fixed rules (bf16 in, e4m3fn out, floor 1e-4,
  * scale = amax * fp32(1/448), reciprocal-multiply quotient, power-of-two scale when
  * round_scale != 0), contiguous [rows, cols] input and outputs.

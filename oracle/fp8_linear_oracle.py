@@ -32,6 +32,10 @@ the checks live in tests/test_oracle_*.py):
 * fp8_block_einsum_ref -- dequantise-then-einsum over [b, h, r] x [h, d, r]; pinned
   per head against block_fp8_matmul_tiled_ref (a different order of operations)
   and by a float64 loop on a tiny case.
+* silu_and_mul_ref -- pinned by a float64 evaluation (at most one rounding step of the
+  output type apart), by torch.sigmoid (a different formula), and by the special
+  cases silu(0) = 0, silu(g) = g for large g, silu(g) = -0 for very negative g and
+  silu(g) - silu(-g) = g.
 * scaled_mm_ref, scaled_mm_ref_postscale -- pinned against each other, a float64
   loop, and the unit-scale/zero-bias closed form.
 
@@ -133,6 +137,18 @@ def per_token_group_quant_fp8_div_ref(
     x_quant = x_quant.reshape(x.shape)
     x_scales = x_scales.reshape(x.shape[:-1] + (x.shape[-1] // group_size,))
     return x_quant, x_scales
+
+
+def silu_and_mul_ref(x: torch.Tensor) -> torch.Tensor:
+    """``silu(x[..., :d]) * x[..., d:]`` the way the reference's activation kernel computes it
+    (src/flag_gems/fused/silu_and_mul.py:13-18, src/flag_gems/fused/fused_moe.py:795-800): the gate in
+    fp32, ``g / (1 + exp(-g))``, times the up value, one rounding to the input's dtype.  (The torch
+    expression of the reference's MoE check, tests/test_fused_experts_impl.py:629-633, rounds the
+    activation and the product separately in bf16; the kernel, restated here, rounds once.)"""
+    d = x.shape[-1] // 2
+    g = x[..., :d].to(torch.float32)
+    u = x[..., d:].to(torch.float32)
+    return (g / (1.0 + torch.exp(-g)) * u).to(x.dtype)
 
 
 # --------------------------------------------------------------------------------------

@@ -211,3 +211,26 @@ def test_per_token_cast_matches_group_quant_shape_and_scale():
     amax[:, :300] = x.float()
     want = amax.view(5, 3, 128).abs().amax(-1).clamp(1e-4) / 448.0
     assert torch.equal(sf, want)
+
+
+# ---- activation between the two GEMMs of an expert / MLP layer
+
+
+def test_silu_and_mul_ref_pinned():
+    g = torch.Generator().manual_seed(41)
+    x = (3 * torch.randn(64, 512, generator=g)).bfloat16()
+    got = O.silu_and_mul_ref(x)
+    gate, up = x[:, :256].double(), x[:, 256:].double()
+    exact = gate / (1 + torch.exp(-gate)) * up
+    # one rounding of a bf16 result: at most half a step from the exact value (plus fp32 noise far below that)
+    step = torch.maximum(exact.abs(), torch.tensor(2.0 ** -126, dtype=torch.float64)) * 2.0 ** -7  # a bf16 step is at most 2^-7 of the value
+    assert torch.all((got.double() - exact).abs() <= 0.5 * step + 1e-30)
+    # a different formula for the same function
+    other = (x[:, :256].float() * torch.sigmoid(x[:, :256].float()) * x[:, 256:].float())
+    torch.testing.assert_close(got.float(), other, rtol=2.0 ** -7, atol=1e-30)
+    # special cases
+    sp = torch.tensor([[0.0, 100.0, -100.0, 3.0, -3.0, 1.0, 2.0, 1.0, 1.0, 1.0]], dtype=torch.float32)
+    out = O.silu_and_mul_ref(sp)
+    assert out[0, 0] == 0.0 and out[0, 1] == 200.0 and out[0, 2] == 0.0 and torch.signbit(out[0, 2])
+    torch.testing.assert_close(out[0, 3] - out[0, 4], torch.tensor(3.0), rtol=1e-6, atol=0)
+    assert O.silu_and_mul_ref(torch.zeros(2, 0)).shape == (2, 0)
