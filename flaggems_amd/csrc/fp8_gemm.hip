@@ -349,7 +349,8 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
       for (int i = 0; i < TN; ++i) {
         const v8i wf = (i == 0) ? wf_first : read_fragment(tw, i, frag_off);
 #pragma unroll
-        for (int j = 0; j < TM; ++j) acc[i][j] = mfma_fp8_16x16x128(wf, xf[j], acc[i][j]);
+        for (int j = 0; j < TM; ++j)
+          acc[i][j] = MODE == kModeRowColI8 ? mfma_i8_16x16x128(wf, xf[j], acc[i][j]) : mfma_fp8_16x16x128(wf, xf[j], acc[i][j]);
       }
     }
 
@@ -404,14 +405,19 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
     const int m = m0 + wm0 + j * 16 + l16;
     if (m >= a.M) continue;
     float sa = 1.f;
-    if (MODE == kModeRowCol) sa = a.xs[a.xs_per_row ? m : 0];
+    constexpr bool kRowCol = MODE != kModeBlock;
+    if (kRowCol) sa = a.xs[a.xs_per_row ? m : 0];
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
       const int n = n0 + wn0 + i * 16 + lg * 4;
       if (n >= a.N) continue;
       float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+      if (MODE == kModeRowColI8) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (float)__builtin_bit_cast(int, v[e]);  // int32 sums -> fp32, then as fp8
+      }
       const int nv = (a.N - n < 4) ? a.N - n : 4;
-      if (MODE == kModeRowCol) {
+      if (kRowCol) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int ne = (e < nv) ? n + e : n;
@@ -425,7 +431,7 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           h[e] = float_to_bf16_bits(v[e]);
-          if (MODE == kModeRowCol && a.bias) {
+          if (kRowCol && a.bias) {
             const int ne = (e < nv) ? n + e : n;
             h[e] = float_to_bf16_bits(bf16_bits_to_float(h[e]) + load_as_float(a.bias, ne, a.bias_dtype));
           }
@@ -441,14 +447,14 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
         _Float16* cp = reinterpret_cast<_Float16*>(a.C) + off;
         for (int e = 0; e < nv; ++e) {
           _Float16 h = (_Float16)v[e];
-          if (MODE == kModeRowCol && a.bias) h = (_Float16)((float)h + load_as_float(a.bias, n + e, a.bias_dtype));
+          if (kRowCol && a.bias) h = (_Float16)((float)h + load_as_float(a.bias, n + e, a.bias_dtype));
           cp[e] = h;
         }
       } else if (a.c_dtype == FG_F32) {
         float* cp = reinterpret_cast<float*>(a.C) + off;
         for (int e = 0; e < nv; ++e) {
           float h = v[e];
-          if (MODE == kModeRowCol && a.bias) h = h + load_as_float(a.bias, n + e, a.bias_dtype);
+          if (kRowCol && a.bias) h = h + load_as_float(a.bias, n + e, a.bias_dtype);
           cp[e] = h;
         }
       } else {  // FG_FP8_E4M3FN
@@ -456,7 +462,7 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
         for (int e = 0; e < nv; ++e) {
           float h = v[e];
           uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(h, 0.f, 0, false) & 0xFFu;
-          if (MODE == kModeRowCol && a.bias) {
+          if (kRowCol && a.bias) {
             // the reference adds the bias to the already rounded output, in the output type
             const float back = __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
             h = back + load_as_float(a.bias, n + e, a.bias_dtype);
@@ -707,4 +713,34 @@ extern "C" int fg_scaled_fp8_gemm(const void* A, int64_t lda, const void* B, int
   a.c_dtype = c_dtype; a.bias_dtype = bias_dtype;
   a.xs_per_row = a_scale_per_row; a.ws_per_col = b_scale_per_col;
   return launch_gemm<kModeRowCol>(a, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int fg_scaled_int8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
+                                   const float* a_scale, int a_scale_per_row,
+                                   const float* b_scale, int b_scale_per_col,
+                                   const void* bias, int bias_dtype,
+                                   void* C, int64_t ldc, int c_dtype,
+                                   int64_t M, int64_t N, int64_t K, void* stream) {
+  using namespace fg;
+  if (c_dtype != FG_BF16 && c_dtype != FG_F16 && c_dtype != FG_F32)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_scaled_int8_gemm: c_dtype %d", c_dtype);
+  if (bias && bias_dtype != FG_BF16 && bias_dtype != FG_F16 && bias_dtype != FG_F32)
+    FG_FAIL(FG_ERR_INVALID_ARG, "fg_scaled_int8_gemm: bias_dtype %d", bias_dtype);
+  int rc = check_common(A, B, C, lda, ldb, ldc, M, N, K, "fg_scaled_int8_gemm");
+  if (rc < 0) return rc;
+  if (rc == 1) return FG_OK;
+  if (!a_scale || !b_scale) FG_FAIL(FG_ERR_INVALID_ARG, "fg_scaled_int8_gemm: null scale pointer");
+  GemmArgs a = {};
+  a.X = (const uint8_t*)A; a.W = (const uint8_t*)B; a.C = C;
+  a.xs = a_scale; a.ws = b_scale; a.bias = bias;
+  a.ldx = lda; a.ldw = ldb; a.ldc = ldc;
+  a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)ceil_div(K, 128);
+  a.c_dtype = c_dtype; a.bias_dtype = bias_dtype;
+  a.xs_per_row = a_scale_per_row; a.ws_per_col = b_scale_per_col;
+  const bool direct = (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) && (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
+                      ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
+  hipStream_t st = (hipStream_t)stream;
+  if (M > 128)
+    return direct ? launch_cfg<256, 256, 4, 2, kModeRowColI8, true>(a, st) : launch_cfg<256, 256, 4, 2, kModeRowColI8, false>(a, st);
+  return direct ? launch_cfg<128, 128, 2, 2, kModeRowColI8, true>(a, st) : launch_cfg<128, 128, 2, 2, kModeRowColI8, false>(a, st);
 }

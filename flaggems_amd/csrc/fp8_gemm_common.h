@@ -5,7 +5,9 @@
 
 namespace fg {
 
-enum { kModeBlock = 0, kModeRowCol = 1 };
+// kModeRowColI8: int8 operands, int32 sums (kept as bit patterns in the fp32 accumulator registers), scales and
+// bias as kModeRowCol.  Only the tile kernel has it.
+enum { kModeBlock = 0, kModeRowCol = 1, kModeRowColI8 = 2 };
 
 struct GemmArgs {
   const uint8_t* X;  // activations [M, K]
@@ -78,6 +80,17 @@ __device__ __forceinline__ void store_output(const GemmArgs& a, int m, int n, fl
 __device__ __forceinline__ v4f mfma_fp8_16x16x128(v8i a, v8i b, v4f c) {
   // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled instruction
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+// One K-block (128) of int8 products into int32 sums: two 16x16x64 instructions, each on the half of the fragment
+// registers that holds the same K positions in both operands (the operands share one K layout, whatever it is).
+__device__ __forceinline__ v4f mfma_i8_16x16x128(v8i a, v8i b, v4f c) {
+  v4i acc = __builtin_bit_cast(v4i, c);
+  const v4i a_lo = {a[0], a[1], a[2], a[3]}, a_hi = {a[4], a[5], a[6], a[7]};
+  const v4i b_lo = {b[0], b[1], b[2], b[3]}, b_hi = {b[4], b[5], b[6], b[7]};
+  acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo, b_lo, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi, b_hi, acc, 0, 0, 0);
+  return __builtin_bit_cast(v4f, acc);
 }
 
 // Operands of inline assembly with an "s" constraint must be in scalar registers; this makes the compiler see

@@ -1,5 +1,5 @@
-"""cutlass_scaled_mm (host side): per-tensor / per-token x per-channel scaled FP8 GEMM with optional
-bias, and the 128-block-wise variant, written into a caller-owned output.
+"""cutlass_scaled_mm (host side): per-tensor / per-token x per-channel scaled FP8 or int8 GEMM with optional
+bias, and the 128-block-wise FP8 variant, written into a caller-owned output.
 
 Mirrors src/flag_gems/fused/cutlass_scaled_mm.py:371-431 (dispatch) and :475-526 (entry point) of
 the reference: same argument order, same assertions and messages, returns None.  The reference
@@ -53,6 +53,26 @@ def _launch_scaled_gemm(c, a, b, a_scale, b_scale, bias) -> None:
     _lib.check(status, "fg_scaled_fp8_gemm")
 
 
+def _launch_scaled_int8_gemm(c, a, b, a_scale, b_scale, bias) -> None:
+    _lib.require_gpu(a, "scaled int8 gemm")
+    lib = _lib.load()
+    m, k = a.shape
+    n = b.shape[1]
+    dev = a.device
+    with torch.cuda.device(dev):
+        status = lib.fg_scaled_int8_gemm(
+            a.data_ptr(), a.stride(0) if m > 1 else max(k, a.stride(0)),
+            b.data_ptr(), b.stride(1) if n > 1 else max(k, b.stride(1)),
+            a_scale.data_ptr(), 1 if a_scale.numel() > 1 or m == 1 else 0,
+            b_scale.data_ptr(), 1 if b_scale.numel() > 1 or n == 1 else 0,
+            bias.data_ptr() if bias is not None else None,
+            _lib.DTYPE_CODE[bias.dtype] if bias is not None else _lib.FG_BF16,
+            c.data_ptr(), c.stride(0) if m > 1 else max(n, c.stride(0)), _lib.DTYPE_CODE[c.dtype],
+            m, n, k, _lib.current_stream_ptr(dev),
+        )
+    _lib.check(status, "fg_scaled_int8_gemm")
+
+
 def dispatch_scaled_mm(c, a, b, a_scale, b_scale, bias) -> None:
     assert a_scale.dtype == torch.float32, "a_scale must be float32"
     assert b_scale.dtype == torch.float32, "b_scale must be float32"
@@ -70,10 +90,13 @@ def dispatch_scaled_mm(c, a, b, a_scale, b_scale, bias) -> None:
             _launch_scaled_gemm(c, a, b, a_scale, b_scale, bias)
         else:
             assert a.dtype == torch.int8, f"Unsupported dtype: {a.dtype}"
-            raise NotImplementedError(
-                "cutlass_scaled_mm: int8 operands are not implemented in the gfx950 build; "
-                "use FP8 (float8_e4m3fn) quantization"
-            )
+            if c.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+                raise NotImplementedError(f"cutlass_scaled_mm (int8): unsupported output dtype {c.dtype}")
+            if bias is not None and bias.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+                raise NotImplementedError(f"cutlass_scaled_mm: unsupported bias dtype {bias.dtype}")
+            if b.dtype != torch.int8:
+                raise NotImplementedError(f"cutlass_scaled_mm (int8): b is {b.dtype}")
+            _launch_scaled_int8_gemm(c, a, b, a_scale, b_scale, bias)
     else:
         assert a_scale.dim() == 2, "a_scale must be 2D tensor for blockwise scaling"
         assert b_scale.dim() == 2, "b_scale must be 2D tensor for blockwise scaling"

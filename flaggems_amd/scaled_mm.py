@@ -1,9 +1,9 @@
 """aten::_scaled_mm / aten::_scaled_mm.out (host side).
 
 Mirrors src/flag_gems/ops/scaled_mm.py:214-273 (argument normalisation and RuntimeError messages)
-and :333-452 (entry points) of the reference.  FP8 (e4m3fn) operands run on the HIP scaled GEMM;
-the reference's generic Triton kernel for other operand types is not part of this build and such
-calls raise NotImplementedError.
+and :333-452 (entry points) of the reference.  FP8 (e4m3fn) and int8 operands run on the HIP scaled
+GEMMs (the reference sends both to cutlass_scaled_mm, :289-316); its generic Triton kernel for other
+operand types is not part of this build and such calls raise NotImplementedError.
 """
 from __future__ import annotations
 
@@ -11,7 +11,7 @@ import logging
 
 import torch
 
-from .cutlass_scaled_mm import _launch_scaled_gemm
+from .cutlass_scaled_mm import _launch_scaled_gemm, _launch_scaled_int8_gemm
 
 logger = logging.getLogger("flag_gems." + __name__.split(".")[-1])
 
@@ -82,10 +82,12 @@ def _scaled_mm_impl(self, mat2, scale_a, scale_b, bias, out_dtype, out):
     if M == 0 or N == 0:
         return out
 
-    if self.dtype != torch.float8_e4m3fn:
+    if self.dtype not in (torch.float8_e4m3fn, torch.int8):
         raise NotImplementedError(
-            f"_scaled_mm: only float8_e4m3fn operands are implemented in the gfx950 build, got {self.dtype}"
+            f"_scaled_mm: only float8_e4m3fn and int8 operands are implemented in the gfx950 build, got {self.dtype}"
         )
+    if self.dtype == torch.int8 and out.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise NotImplementedError(f"_scaled_mm: int8 operands need a floating-point out_dtype, got {out.dtype}")
     if scale_a.dtype != torch.float32 or scale_b.dtype != torch.float32:
         scale_a, scale_b = scale_a.to(torch.float32), scale_b.to(torch.float32)
     # the kernel wants K-contiguous rows on both sides: self row-major, mat2 column-major
@@ -94,7 +96,10 @@ def _scaled_mm_impl(self, mat2, scale_a, scale_b, bias, out_dtype, out):
     if mat2.stride(0) != 1:
         mat2 = mat2.t().contiguous().t()
     target = out if out.stride(1) == 1 else torch.empty((M, N), dtype=out.dtype, device=out.device)
-    _launch_scaled_gemm(target, self, mat2, scale_a, scale_b, bias)
+    if self.dtype == torch.int8:
+        _launch_scaled_int8_gemm(target, self, mat2, scale_a, scale_b, bias)
+    else:
+        _launch_scaled_gemm(target, self, mat2, scale_a, scale_b, bias)
     if target is not out:
         out.copy_(target)
     return out

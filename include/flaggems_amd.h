@@ -257,6 +257,21 @@ int fg_scaled_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
 
 size_t fg_scaled_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
+/*
+ * The same with int8 operands: C[m, n] = float(sum_k A[m,k] * B[n,k] in int32) * a_scale[m or 0] * b_scale[n or 0],
+ * rounded to c_dtype (FG_BF16, FG_F16 or FG_F32), then + bias[n] in c_dtype.  A: int8 [M, K] rows lda apart,
+ * B: int8 [N, K] rows ldb apart (the column-major [K, N] operand of the reference).  Served by the tile kernel at
+ * every M (no workspace, no K split): correct at decode sizes, not tuned for them.
+ * Stands in for the int8 branch of cutlass_scaled_mm (src/flag_gems/fused/cutlass_scaled_mm.py:198-344 with an
+ * int32 accumulator, dispatch :394-402).
+ */
+int fg_scaled_int8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
+                        const float* a_scale, int a_scale_per_row,
+                        const float* b_scale, int b_scale_per_col,
+                        const void* bias, int bias_dtype,
+                        void* C, int64_t ldc, int c_dtype,
+                        int64_t M, int64_t N, int64_t K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,89 @@
+"""GPU parity of the int8 branch of cutlass_scaled_mm / aten::_scaled_mm against the CPU oracle.
+
+int8 x int8 sums are exact in int32, so the only rounding is float(sum) * scale_a * scale_b -> out dtype
+(-> + bias): the result must match the oracle to one step of the output type (the reference's own tolerance for
+int8 is rtol 1e-1, atol 1.0, tests/test_cutlass_scaled_mm.py:237-238).  Inputs as the reference builds them
+(:48-49, :205-212): round(clamp(randn * 5, -128, 127))."""
+import pytest
+import torch
+
+import flag_gems
+from oracle import fp8_linear_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _to_int8(t):
+    return torch.round(t.clamp(min=-128, max=127)).to(torch.int8)
+
+
+def _inputs(M, N, K, seed, a_kind, b_kind):
+    g = torch.Generator().manual_seed(seed)
+    a = _to_int8(torch.randn(M, K, generator=g) * 5)
+    b = _to_int8(torch.randn(N, K, generator=g) * 5).t()  # [K, N] column-major
+    sa = torch.rand((M,) if a_kind == "vector" else (1,), generator=g) * 0.02 + 0.001
+    sb = torch.rand((N,) if b_kind == "vector" else (1,), generator=g) * 0.02 + 0.001
+    return a, b, sa, sb
+
+
+def _exact(a, b, sa, sb):
+    """int32-exact sums (float64 holds them exactly), scaled in fp32 in the kernel's order."""
+    acc = (a.double() @ b.double()).float()
+    sa2 = sa.reshape(-1, 1) if sa.numel() > 1 else sa.reshape(1, 1)
+    sb2 = sb.reshape(1, -1) if sb.numel() > 1 else sb.reshape(1, 1)
+    return acc * sa2 * sb2
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 256, 128), (16, 512, 512), (33, 1024, 1024), (100, 640, 4096), (256, 4096, 4096),
+                                   (512, 8192, 1024), (1100, 1300, 2048), (64, 200, 192), (7, 24, 40)])
+@pytest.mark.parametrize("kinds", [("scalar", "scalar"), ("vector", "vector"), ("vector", "scalar")])
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16])
+def test_int8_cutlass_scaled_mm(M, N, K, kinds, out_dtype):
+    a, b, sa, sb = _inputs(M, N, K, 0, *kinds)
+    for use_bias in (False, True):
+        bias = torch.randn(N, generator=torch.Generator().manual_seed(1)).to(out_dtype) if use_bias else None
+        want = O.scaled_mm_ref(a, b, sa, sb, out_dtype, bias)
+        c = torch.empty(M, -(-N // 16) * 16, dtype=out_dtype, device=DEV)[:, :N]  # the reference asserts these strides
+        ld = -(-K // 16) * 16
+        b_dev = torch.zeros(N, ld, dtype=torch.int8, device=DEV)
+        b_dev[:, :K] = b.t().to(DEV)
+        flag_gems.cutlass_scaled_mm(c, a.to(DEV), b_dev[:, :K].t(), sa.to(DEV), sb.to(DEV), bias.to(DEV) if use_bias else None)
+        # the reference's tolerance
+        torch.testing.assert_close(c.cpu(), want, rtol=1e-1, atol=1.0)
+        # this build's: the exact sums, scaled in fp32, rounded once (then the bias added in the output type)
+        mine = _exact(a, b, sa, sb).to(out_dtype)
+        if use_bias:
+            mine = mine + bias
+        eps = torch.finfo(out_dtype).eps
+        err = (c.cpu().double() - mine.double()).abs()
+        assert torch.all(err <= mine.double().abs() * eps + 1e-6), f"max err {err.max().item()}"
+        assert (c.cpu() != mine).float().mean().item() < 2e-3
+
+
+def test_int8_sums_are_exact():
+    """Unit scales and fp32 output: every int32 sum comes back exactly, also at the extremes of int8."""
+    M, N, K = 130, 260, 1024
+    g = torch.Generator().manual_seed(3)
+    a = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+    b = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+    a[0, :] = -128
+    b[0, :] = -128
+    a[1, :] = 127
+    b[1, :] = -128
+    one = torch.ones(1)
+    c = torch.empty(M, 272, dtype=torch.float32, device=DEV)[:, :N]
+    flag_gems.cutlass_scaled_mm(c, a.to(DEV), b.to(DEV).t(), one.to(DEV), one.to(DEV), None)
+    want = a.double() @ b.double().t()
+    assert want.abs().max() <= 2 ** 24  # exactly representable in fp32
+    assert torch.equal(c.cpu().double(), want)
+    assert c[0, 0].item() == 128 * 128 * K and c[1, 0].item() == -127 * 128 * K
+
+
+def test_int8_through_aten_scaled_mm():
+    a, b, sa, sb = _inputs(64, 128, 256, 4, "vector", "vector")
+    want = O.scaled_mm_ref(a, b, sa, sb, torch.bfloat16)
+    got = flag_gems.scaled_mm(a.to(DEV), b.to(DEV), sa.view(-1, 1).to(DEV), sb.view(1, -1).to(DEV), out_dtype=torch.bfloat16)
+    torch.testing.assert_close(got.cpu().float(), want.float(), rtol=2.0 ** -7, atol=1e-3)
+    with pytest.raises(NotImplementedError):
+        flag_gems.scaled_mm(a.to(DEV), b.to(DEV), sa.view(-1, 1).to(DEV), sb.view(1, -1).to(DEV))  # int8 output

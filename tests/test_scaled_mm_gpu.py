@@ -112,10 +112,10 @@ def test_assertions_and_unsupported():
         flag_gems.cutlass_scaled_mm(c, a, b, sa.double(), sb)              # scale dtype
     with pytest.raises(AssertionError):
         flag_gems.cutlass_scaled_mm(c, a, b, sa, sb, torch.zeros(3, dtype=torch.bfloat16, device=DEV))
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(NotImplementedError):  # int8 operands with an fp8 output
         ai = torch.ones(16, 128, dtype=torch.int8, device=DEV)
         bi = torch.ones(256, 128, dtype=torch.int8, device=DEV).t()
-        flag_gems.cutlass_scaled_mm(c, ai, bi, sa, sb)
+        flag_gems.cutlass_scaled_mm(torch.empty(16, 256, dtype=FP8, device=DEV), ai, bi, sa, sb)
 
 
 # ----------------------------------------------------------------- aten::_scaled_mm
