@@ -62,7 +62,8 @@ def test_grouped_gemm_matches_the_oracle(M, N, K, ends):
     got = _run(xq, wq, xs, ws, ends)
     _check(got, xq, wq, xs, ws, ends)
     # a second call gives the same bits (no order of arrival enters the sums)
-    assert torch.equal(got, _run(xq, wq, xs, ws, ends))
+    rows = int(ends[-1])  # rows nobody owns are left as torch.empty made them
+    assert torch.equal(got[:rows], _run(xq, wq, xs, ws, ends)[:rows])
 
 
 def test_grouped_gemm_equals_plain_gemm_where_the_tiles_coincide():
