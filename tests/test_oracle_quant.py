@@ -234,3 +234,26 @@ def test_silu_and_mul_ref_pinned():
     assert out[0, 0] == 0.0 and out[0, 1] == 200.0 and out[0, 2] == 0.0 and torch.signbit(out[0, 2])
     torch.testing.assert_close(out[0, 3] - out[0, 4], torch.tensor(3.0), rtol=1e-6, atol=0)
     assert O.silu_and_mul_ref(torch.zeros(2, 0)).shape == (2, 0)
+
+
+def test_three_operation_division_is_the_correctly_rounded_quotient():
+    """The quantizer kernels replace x / s by q0 = RN(x r), e = RN(x - q0 s) (one fused multiply-add),
+    RN(q0 + e r) with r = RN(1 / s), for scales in [2^-60, 2^100].  Emulated here in numpy (float64 holds the
+    products of two fp32 values exactly) against fp32 division, on quotients spread over the fp8 range and on
+    quotients within a few fp32 steps of the fp8 rounding boundaries."""
+    rng = np.random.default_rng(0)
+    n = 1_500_000
+    for mode in (0, 1):
+        s = (np.exp2(rng.uniform(-60, 60, n)) * rng.uniform(1, 2, n)).astype(np.float32)
+        if mode == 0:
+            x = (s.astype(np.float64) * rng.uniform(-448, 448, n)).astype(np.float32)
+        else:
+            mid = (rng.integers(16, 32, n) + 0.5) / 16.0 * np.exp2(rng.integers(-10, 9, n))
+            x = (s.astype(np.float64) * mid * (1 + rng.integers(-3, 4, n) * 2.0 ** -24)).astype(np.float32)
+        want = (x / s).astype(np.float32)
+        r = (np.float32(1.0) / s).astype(np.float32)
+        q0 = (x * r).astype(np.float32)
+        # the fused multiply-add rounds the exact remainder once (it fits fp32 whenever q0 is within a step)
+        e = (x.astype(np.float64) - q0.astype(np.float64) * s.astype(np.float64)).astype(np.float32)
+        q1 = (q0.astype(np.float64) + e.astype(np.float64) * r.astype(np.float64)).astype(np.float32)
+        assert np.array_equal(q1, want)
