@@ -261,19 +261,30 @@ __global__ __launch_bounds__(kQuantThreads) void group_quant_vec_kernel(QuantArg
     const float s = derive_scale(amax, a);
     const float r = 1.0f / s;
 
+    // Decided once per wavefront (uniform branches): almost every wavefront holds finite inputs under finite
+    // non-zero scales only, where no quotient can be NaN and a plain clamp finishes the job.
+    const bool plain = __builtin_amdgcn_ballot_w64(special || !(s > 0.0f) || !(s < __builtin_huge_valf())) == 0;
     float y[8];
-    const bool short_div = short_division_ok(special, s);
+    if (plain) {
+      if (a.quotient_rule == FG_QUOT_RECIP_MUL) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) y[i] = quantize_value(xv[i], s, r, a, short_div);
-    if (special) {
+        for (int i = 0; i < 8; ++i) y[i] = fminf(fmaxf(xv[i] * r, a.lo), a.hi);
+      } else if (__builtin_amdgcn_ballot_w64(!short_division_ok(false, s)) == 0) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) y[i] = unclamped_overflow(xv[i], s, r, y[i], a);
+        for (int i = 0; i < 8; ++i) y[i] = fminf(fmaxf(short_division(xv[i], s, r), a.lo), a.hi);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = fminf(fmaxf(xv[i] / s, a.lo), a.hi);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = unclamped_overflow(xv[i], s, r, quantize_value(xv[i], s, r, a), a);
     }
     uint32_t w0 = pack2<false>(y[0], y[1], 0u, a.e5m2);
     w0 = pack2<true>(y[2], y[3], w0, a.e5m2);
     uint32_t w1 = pack2<false>(y[4], y[5], 0u, a.e5m2);
     w1 = pack2<true>(y[6], y[7], w1, a.e5m2);
-    if (special || !(s == s)) {
+    if (!plain) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         w0 = fix_nan_byte(w0, i, y[i], a.e5m2);
