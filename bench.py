@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One step = one pass over the DeepSeek-V3 block-fp8 GEMM sweep of BASELINE.json configs[2]:
+One step = one pass over the DeepSeek-V3 block-fp8 GEMM sweep that the headline metric is quoted on:
 M in {1, 8, 64, 512, 2048, 4096} x (N, K) in {(2112,7168), (24576,1536), (32768,512), (7168,16384),
 (4608,7168), (7168,2304)}, e4m3fn operands already resident in HBM (1x128 activation scales,
 128x128 weight scales, bf16 output).  `value` is the sweep's total 2*M*N*K divided by the wall
@@ -21,7 +21,7 @@ Prints ONE JSON line with the driver's fields plus
                 linears as GEMM alone and as act_quant + GEMM), graph replays of one shape at a time with ONE copy
                 of the weights (small-M figures there may be served by the 256 MB Infinity Cache), not part of `value`
   mixtral_moe_grouped_gemm
-                BASELINE.json configs[4]: 8 experts, top-2 over T tokens with Zipf(1.1) expert loads, rows sorted by
+                Mixtral-8x7B expert layers: 8 experts, top-2 over T tokens with Zipf(1.1) expert loads, rows sorted by
                 expert; the grouped block-fp8 GEMM with W1 [8,28672,4096] and W2 [8,4096,14336]; not part of `value`
 """
 from __future__ import annotations
@@ -306,7 +306,7 @@ def main():
         del gr
         return sorted(ts)[1]
 
-    # cutlass_scaled_mm semantics (BASELINE configs[3]): per-token x per-channel scales, bf16 bias, N = K = 8192
+    # cutlass_scaled_mm semantics: per-token x per-channel scales, bf16 bias, N = K = 8192
     scaled = []
     nk = 8192
     b_src = torch.randn(nk, nk, device=dev, generator=gen)
@@ -325,7 +325,7 @@ def main():
                        "gbps": round(nbytes / us / 1e3, 1)})
     del b_q, a_q, c
 
-    # Llama-3-8B linears (BASELINE configs[1]): GEMM alone and act_quant + GEMM from bf16 activations
+    # Llama-3-8B linears: GEMM alone and act_quant + GEMM from bf16 activations
     llama = []
     for (n, k) in [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]:
         wq, ws = make_weight(n, k, gen, dev)
@@ -342,7 +342,7 @@ def main():
                           "tflops": round(gemm_flops(m, n, k) / us_g / 1e6, 1), "gbps": round(gemm_bytes(m, n, k) / us_g / 1e3, 1)})
         del wq, ws
 
-    # Mixtral-8x7B expert layers (BASELINE configs[4]): grouped block-fp8 GEMM over rows sorted by expert
+    # Mixtral-8x7B expert layers: grouped block-fp8 GEMM over rows sorted by expert
     moe = []
     experts = 8
     for (n, k) in [(28672, 4096), (4096, 14336)]:

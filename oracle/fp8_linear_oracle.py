@@ -433,7 +433,7 @@ def scaled_mm_ref_postscale(
 # Synthetic inputs of the benchmark configurations
 # --------------------------------------------------------------------------------------
 def make_config1(seed: int = 0):
-    """BASELINE config 1: X bf16 [64,1024] ~N(0,1), W bf16 [512,1024] ~N(0,0.02),
+    """The CPU-runnable benchmark configuration: X bf16 [64,1024] ~N(0,1), W bf16 [512,1024] ~N(0,0.02),
     generator order X then W, one ``torch.manual_seed(seed)``."""
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(64, 1024, generator=g).bfloat16()

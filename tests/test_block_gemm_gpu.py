@@ -1,6 +1,6 @@
 """GPU parity of the block-scaled FP8 GEMM against the CPU oracle.
 
-Tolerance: BASELINE bar rtol 1e-2 / atol 1e-2 against the fp32-dequantised matmul for bf16 output;
+Tolerance: rtol 1e-2 / atol 1e-2 (the bar this build sets itself) against the fp32-dequantised matmul for bf16 output;
 the reference's own tolerance (fp16 output, atol 1e-4*K, rtol 1e-3,
 tests/test_w8a8_block_fp8_matmul.py:107) is applied to its own shape list as well."""
 import os
