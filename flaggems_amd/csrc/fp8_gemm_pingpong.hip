@@ -959,7 +959,10 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : 0;
   const size_t need = FG_WORKSPACE_COUNTER_BYTES + sk_bytes;
   // workspace: [counters][partial tiles, if the shape is one that shares tiles][transposed activation scales]
+  // (a grouped problem's tile count is an upper bound that a few hundred rows spread over many segments inflate:
+  // there the gathers are few and the transposition, ~5 us whatever the size, does not pay)
   if (mode == kModeBlock && g.xs_rs >= kTransposeMinRowStride && transposition_pays(tiles, g.KB, cus) && workspace != nullptr &&
+      (grouped == nullptr || g.M >= 1024) &&
       (uintptr_t)workspace % 16 == 0 &&
       workspace_bytes >= need + transposed_scales_bytes(g.M, g.KB)) {
     float* const xs_t = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + need);
