@@ -119,3 +119,53 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, os.path.join(dirpath, f)
+
+
+def test_widened_entry_points_validate_and_refuse_the_cpu():
+    """The operators added around the hot path (grouped and batched GEMM, weight quantizer, fused activation, int8):
+    same rules as the rest -- host checks first, no CPU implementation, C-ABI validation before any launch."""
+    for name in ["grouped_w8a8_block_fp8_matmul", "w8a8_block_fp8_bmm", "fp8_einsum", "per_block_cast_to_fp8",
+                 "per_token_cast_to_fp8", "silu_and_mul_packed", "silu_and_mul_per_token_group_quant_fp8"]:
+        assert hasattr(flag_gems, name), name
+    a = torch.zeros(4, 256, dtype=torch.float8_e4m3fn)
+    b = torch.zeros(2, 128, 256, dtype=torch.float8_e4m3fn)
+    ends = torch.tensor([1, 4], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        flag_gems.grouped_w8a8_block_fp8_matmul(a, b, torch.ones(4, 2), torch.ones(2, 1, 2), ends, [128, 128])
+    with pytest.raises(AssertionError):  # the group table must be int32
+        flag_gems.grouped_w8a8_block_fp8_matmul(a, b, torch.ones(4, 2), torch.ones(2, 1, 2), ends.long(), [128, 128])
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        flag_gems.fp8_einsum("bhr,hdr->bhd", torch.zeros(3, 2, 256, dtype=torch.float8_e4m3fn), torch.ones(3, 2, 2),
+                             b, torch.ones(2, 1, 2))
+    with pytest.raises(AssertionError, match="only supports"):
+        flag_gems.fp8_einsum("bhr,hrd->bhd", torch.zeros(3, 2, 256, dtype=torch.float8_e4m3fn), torch.ones(3, 2, 2),
+                             b, torch.ones(2, 1, 2))
+    x = torch.zeros(4, 512, dtype=torch.bfloat16)
+    for fn in (lambda: flag_gems.per_block_cast_to_fp8(x), lambda: flag_gems.per_token_cast_to_fp8(x),
+               lambda: flag_gems.silu_and_mul_packed(x), lambda: flag_gems.silu_and_mul_per_token_group_quant_fp8(x, 128)):
+        with pytest.raises(RuntimeError, match="no CPU implementation"):
+            fn()
+    with pytest.raises(AssertionError, match="divisible"):
+        flag_gems.silu_and_mul_per_token_group_quant_fp8(x, 96)
+    ai = torch.zeros(4, 256, dtype=torch.int8)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        flag_gems.cutlass_scaled_mm(torch.zeros(4, 16, dtype=torch.bfloat16), ai, torch.zeros(16, 256, dtype=torch.int8).t(),
+                                    torch.ones(1), torch.ones(1))
+    if not os.path.exists(_lib.LIB_PATH):
+        return
+    lib = _lib.load()
+    # grouped GEMM: K that is not a multiple of 128, a non-bf16 result, a missing table
+    args = lambda k, dt, tab: (1, k, 1, k, 128 * k, 1, 2, 1, 1, 2, 1, 2, tab, 2, 1, 128, dt, 4, 128, k, 128, 128, None, 0, None)
+    assert lib.fg_grouped_block_fp8_gemm(*args(192, _lib.FG_BF16, 1)) == _lib.FG_ERR_UNSUPPORTED
+    assert lib.fg_grouped_block_fp8_gemm(*args(256, _lib.FG_F32, 1)) == _lib.FG_ERR_UNSUPPORTED
+    assert lib.fg_grouped_block_fp8_gemm(*args(256, _lib.FG_BF16, None)) == _lib.FG_ERR_INVALID_ARG
+    # block quantizer: only 128 x 128 blocks; empty input is accepted
+    q = lambda rows, blk: lib.fg_block_quant_fp8(1, _lib.FG_BF16, rows, 256, 256, 1, _lib.FG_FP8_E4M3FN, 256, 1, 2, 1,
+                                                 blk, blk, 1e-4, -448.0, 448.0, 1.0 / 448.0, 1, 0, 0, None)
+    assert q(4, 64) == _lib.FG_ERR_UNSUPPORTED and q(0, 128) == 0
+    # fused activation: the up half must lie inside the row
+    rc = lib.fg_silu_mul_group_quant_fp8(1, _lib.FG_BF16, 4, 256, 300, 256, 1, _lib.FG_FP8_E4M3FN, 256, 1, 2, 1,
+                                         128, 1e-10, -448.0, 448.0, 1.0 / 448.0, 0, 1, 0, None)
+    assert rc == _lib.FG_ERR_INVALID_ARG
+    assert lib.fg_batched_block_fp8_gemm(None, 0, 0, None, 0, 0, None, 0, 0, 0, None, 0, 0, 0, None, 0, 0, _lib.FG_BF16,
+                                         -1, 4, 4, 128, 128, 128, None, 0, None) == _lib.FG_ERR_INVALID_ARG
