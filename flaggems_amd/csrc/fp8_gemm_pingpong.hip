@@ -101,6 +101,10 @@ struct PpArgs {
   // sk_q or sk_q + 1 steps (the first sk_r ranges get the extra step).  A tile that straddles ranges is
   // finished through the workspace: fp32 partial tiles and one arrival counter per (range, wavefront).
   int sk, sk_q, sk_r;
+  // sk_split != 0: every tile is cut into sk_split ranges of sk_q steps (sk_q * sk_split = KB, sk_r = 0, grid =
+  // tiles * sk_split), and the blocks of one XCD take the same cut of consecutive tiles: they walk the same K
+  // offsets at the same time and share operand panels in their L2, as whole-tile launches do.
+  int sk_split;
   float* partials;
   unsigned int* counters;
   // Start-up delay of block b: (b mod 16) * stagger sleeps of about 1000 cycles.  With short K loops all compute
@@ -546,7 +550,15 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   int pos = (int)blockIdx.x, first_idx = (int)blockIdx.x, first_kb = 0, total;
   if (SK) {
     // ranges that are neighbours in the step order go to one XCD (block ids congruent mod 8)
-    if ((gridDim.x & 7) == 0) pos = (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3);
+    if (a.sk_split) {
+      // position of this block in XCD-major order (block b runs on XCD b mod 8), then (cut, tile) in that order
+      const int x = (int)(blockIdx.x & 7), per = (int)(gridDim.x >> 3), extra = (int)(gridDim.x & 7);
+      const int idx = x * per + (x < extra ? x : extra) + (int)(blockIdx.x >> 3);
+      const int cut = idx / a.n_tiles;
+      pos = (idx - cut * a.n_tiles) * a.sk_split + cut;
+    } else if ((gridDim.x & 7) == 0) {
+      pos = (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3);
+    }
     const int s0 = sk_range_begin(a, pos);
     total = a.sk_q + (pos < a.sk_r ? 1 : 0);
     first_idx = s0 / g.KB;
@@ -855,14 +867,40 @@ int cu_count() {
 struct SkPlan {
   bool use;
   int grid, q, r;
+  int split;  // != 0: tiles cut into `split` equal ranges each (grid = tiles * split), see PpArgs::sk_split
 };
 SkPlan plan_stream_k(int64_t tiles, int KB, int cus) {
-  SkPlan p = {false, 0, 0, 0};
+  SkPlan p = {false, 0, 0, 0, 0};
   const int64_t total = tiles * KB;
   if (cus < 8 || total < cus || total > 0x7FFFFFFF) return p;
+#ifdef FG_DEV_KNOBS
+  if (const char* e = getenv("FG_SK_SPLIT")) {
+    const int S = atoi(e);
+    if (S >= 2 && KB % S == 0 && tiles * S <= cus) {
+      p.use = true; p.grid = (int)(tiles * S); p.q = KB / S; p.r = 0; p.split = S;
+      return p;
+    }
+  }
+#endif
   const int64_t dp_grid = tiles < cus ? tiles : cus;
   const int64_t dp_steps = ceil_div(tiles, dp_grid) * KB;
   const int64_t q = total / cus;
+  // Equal cuts of every tile (PpArgs::sk_split) keep the operand sharing of whole-tile launches, which contiguous
+  // ranges of total / cus steps lose unless they happen to cut every tile alike.  They pay when the cuts are long
+  // and nearly fill the GPU: measured M = 512, N = 7168, K = 16384 (56 tiles): 4 cuts of 32 steps on 224 units
+  // 86 us against 110 us for 256 ranges of 28 steps; M = 1024, same N and K: 2 cuts of 64 steps 125 us against
+  // 174 us.  Cuts of 8 or 28 steps lose to the contiguous ranges (the partial tiles dominate either way).
+  const bool ranges_cut_tiles_alike = total % cus == 0 && q > 0 && KB % q == 0;
+  if (!ranges_cut_tiles_alike) {
+    for (int64_t S = cus / tiles; S >= 2; --S) {
+      if (KB % S != 0) continue;
+      const int64_t cut = KB / S;
+      if (cut < 32 || tiles * S * 5 < (int64_t)cus * 4) break;  // shorter cuts or emptier grids only get worse
+      if ((cut + 16) >= dp_steps) break;                         // ~16 steps to publish and add the partial tiles
+      p.use = true; p.grid = (int)(tiles * S); p.q = (int)cut; p.r = 0; p.split = (int)S;
+      return p;
+    }
+  }
   // Measured on DeepSeek-V3 shapes, M = 128 ... 4096, in units of a whole-tile K-block: ranges that start at
   // different K offsets stop sharing operand panels in their XCD's L2, which makes a K-block about 1.35 times as
   // expensive, and the tiles are finished only after the slowest of their ranges, which adds about 14 K-blocks
@@ -973,7 +1011,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   }
   if (mode == kModeBlock && sk.use && workspace != nullptr && workspace_bytes >= need && (size_t)sk.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
       (uintptr_t)workspace % 16 == 0) {
-    a.sk = 1; a.sk_q = sk.q; a.sk_r = sk.r;
+    a.sk = 1; a.sk_q = sk.q; a.sk_r = sk.r; a.sk_split = sk.split;
     a.counters = reinterpret_cast<unsigned int*>(workspace);
     a.partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
     grid = sk.grid;

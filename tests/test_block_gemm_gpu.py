@@ -107,6 +107,23 @@ def test_few_tiles_split_along_k(M, N, K, dtype):
         assert torch.equal(again.view(torch.int8), got.view(torch.int8))
 
 
+@pytest.mark.parametrize("M,N,K", [(1024, 7168, 8192), (300, 7000, 16384)])
+def test_tiles_cut_into_equal_ranges_along_k(M, N, K):
+    """112 tiles x 64 K-blocks and 56 tiles x 128 K-blocks (ragged in M and N): the persistent kernel cuts every
+    tile into ranges of at least 32 K-blocks that fill most of the GPU, one block per range, and the last
+    wavefront to arrive adds the ranges' partial sums in range order.  Against the oracle, and bit-identical on
+    reruns."""
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=11)
+    want = O.block_fp8_matmul_tiled_ref(xq, wq, xs, ws, [128, 128], torch.float32)
+    args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    got = flag_gems.w8a8_block_fp8_matmul(*args)
+    torch.testing.assert_close(got.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    err = (got.cpu().double() - want.double()).abs()
+    assert float((err / (want.double().abs() / 128 + 2e-3)).max()) < 1.0
+    for _ in range(3):
+        assert torch.equal(flag_gems.w8a8_block_fp8_matmul(*args), got)
+
+
 @pytest.mark.parametrize("M,N,K", [(1100, 1300, 8192), (1200, 3000, 4096)])
 def test_activation_scales_in_either_layout_give_the_same_bits(M, N, K):
     """The persistent kernel reads activation scales K-block by K-block for 64 rows at a time.  Row-major
