@@ -548,12 +548,26 @@ int launch_tile_split(GemmArgs a, const TileSplitPlan& plan, void* workspace, hi
   return FG_OK;
 }
 
+// Whether the 33..64-row kernel is the one to take for the shape (it is compared with the K-split tile kernel and
+// the decode kernels, which take the same shapes).
+bool mid_m_preferred(const MidMPlan& mid, int64_t M, int64_t N, int64_t K) {
+  (void)M; (void)N; (void)K;
+#ifdef FG_DEV_KNOBS
+  if (const char* e = getenv("FG_MIDM")) return mid.use && atoi(e) != 0;
+#endif
+  return mid.use;
+}
+
 template <int MODE>
 int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   const bool direct = (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) &&
                       (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
                       ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
   if (direct) {
+    const MidMPlan mid = plan_mid_m(a.M, a.N, a.K);
+    if (mid_m_preferred(mid, a.M, a.N, a.K) && (mid.splits == 1 || (workspace != nullptr && workspace_bytes >= mid.workspace_bytes &&
+                                                                       (uintptr_t)workspace % 16 == 0)))
+      return launch_mid_m(a, MODE, mid, workspace, workspace_bytes, stream);
     const TileSplitPlan ts = plan_tile_split(a.M, a.N, a.K);
     if (ts.use && workspace != nullptr && workspace_bytes >= ts.workspace_bytes && (uintptr_t)workspace % 16 == 0)
       return launch_tile_split<MODE>(a, ts, workspace, stream);
@@ -589,6 +603,8 @@ extern "C" size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_
   size_t need = fg::plan_tile_split(M, N, K).workspace_bytes;
   const fg::SmallMPlan plan = fg::plan_small_m(M, N, K);
   if (plan.use && plan.workspace_bytes > need) need = plan.workspace_bytes;
+  const fg::MidMPlan mid = fg::plan_mid_m(M, N, K);
+  if (mid.use && mid.workspace_bytes > need) need = mid.workspace_bytes;
   const size_t pp = fg::pingpong_workspace_bytes(M, N, K);
   return pp > need ? pp : need;
 }

@@ -131,6 +131,20 @@ int launch_small_m(const GemmArgs& a, int mode, const SmallMPlan& plan, void* wo
                    hipStream_t stream);
 
 
+// 33 <= M <= 64 rows, fp8_gemm_midm.hip: activations staged in LDS once per block, weights streamed.
+struct MidMPlan {
+  bool use;
+  int rg;            // 16-row weight groups per wavefront: 1, 2 or 4
+  int waves;         // wavefronts per block: 4 or 8
+  int kb_per_split;  // K-blocks per block (<= 16)
+  int splits;        // blocks along K
+  int n_chunks;      // ceil(N / (16 * rg))
+  size_t workspace_bytes;
+};
+MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K);
+int launch_mid_m(const GemmArgs& a, int mode, const MidMPlan& plan, void* workspace, size_t workspace_bytes,
+                 hipStream_t stream);
+
 // Persistent 256x256 kernel, fp8_gemm_pingpong.hip: bf16 output with 16-byte aligned rows, M > 128 (or M > 64 when
 // the workspace lets it share tiles along K);
 // the caller has checked that the operands qualify for direct global->LDS loads.

@@ -1,0 +1,301 @@
+// FP8 GEMM for 33 <= M <= 64 activation rows on gfx950: the weight is read once, straight from global memory
+// into MFMA operand registers, and the activations come out of LDS.
+//
+// With up to 64 rows the activation slice of a K-block (64 x 128 bytes) is as large as the 64 weight rows a
+// wavefront multiplies it with, so a wavefront that fetches both from global memory moves two bytes for every
+// weight byte (the decode kernels do that; they were built for <= 32 rows).  Here a block first copies the
+// activation rows of its K range into LDS once (swizzled 16-byte chunks, conflict-free as MFMA fragments) and
+// its 4 or 8 wavefronts, each with weight rows of its own, read their fragments from there: no wavefront
+// shares an output element with another, so nothing is reduced across wavefronts, and the loop has no barrier.
+//
+//  * A wavefront owns 16 * RG weight rows (RG = 1, 2, 4) and the K-blocks [split * kb_per_split, ...): per K-block
+//    2 * RG 16-byte loads per lane (DEPTH K-blocks in flight, 64 VGPRs), 8 LDS reads, 4 * RG MFMAs.
+//  * K is split over gridDim.y blocks only as far as LDS (16 K-blocks = 128 KB of activations) or the number
+//    of wavefronts requires; each wavefront then publishes its sums and the one that arrives last adds the
+//    splits' sums in split order (a fixed order: results do not depend on timing) and resets the counter.
+//
+// Arithmetic as in the other kernels: per K-block products accumulated by the fp8 MFMA, multiplied by
+// As[m, kb] * Bs[n / 128, kb] in fp32 (block mode) or accumulated unscaled and scaled at the end (row/column mode).
+
+#include "fp8_gemm_common.h"
+
+namespace fg {
+namespace {
+
+constexpr int kMidRows = 64;            // activation rows staged (rows past M repeat the last one; never stored)
+constexpr int kMidKbMax = 16;           // K-blocks of activations a block keeps in LDS
+constexpr int kMidStageBytes = kMidRows * 128;
+
+struct MidArgs {
+  GemmArgs g;
+  int kb_per_split, splits, n_chunks;  // n_chunks = ceil(N / (16 * RG))
+  float* partials;                     // [n_chunks][splits][RG * 4][64 lanes] x 4 floats
+  unsigned int* counters;              // one per chunk
+};
+
+template <int RG>
+struct WUnit {  // one K-block of a wavefront's weight rows in MFMA operand layout, and its weight-block scale
+  u32x4 lo[RG], hi[RG];
+  float ws;
+};
+
+__device__ __forceinline__ v8i join8(u32x4 lo, u32x4 hi) {
+  v8i f;
+  f[0] = (int)lo.x; f[1] = (int)lo.y; f[2] = (int)lo.z; f[3] = (int)lo.w;
+  f[4] = (int)hi.x; f[5] = (int)hi.y; f[6] = (int)hi.z; f[7] = (int)hi.w;
+  return f;
+}
+
+template <int RG, int WAVES, int DEPTH, int MODE>
+__global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
+  constexpr int NT = WAVES * 64;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [kb][64 rows][128 B], then As [kb][64]
+  const GemmArgs& g = a.g;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, lg = lane >> 4;
+  const int split = (int)blockIdx.y;
+  const int kb0 = split * a.kb_per_split;
+  const int kbs = (g.KB - kb0 < a.kb_per_split) ? g.KB - kb0 : a.kb_per_split;  // >= 1: splits = ceil(KB / kb_per_split)
+  const int chunk = (int)blockIdx.x * WAVES + wave;
+  const bool active = chunk < a.n_chunks;  // uniform over the wavefront
+  const int n0 = active ? chunk * 16 * RG : 0;
+
+  // this lane's weight rows (rows past the edge alias the last valid row; never stored)
+  const uint8_t* wrow[RG];
+#pragma unroll
+  for (int r = 0; r < RG; ++r) {
+    int n = n0 + r * 16 + l16;
+    n = n < g.N ? n : g.N - 1;
+    wrow[r] = g.W + (int64_t)n * g.ldw + (int64_t)kb0 * 128 + lg * 16;
+  }
+  const float* const ws_ptr =
+      (MODE == kModeBlock) ? uniform_ptr(g.ws + (int64_t)(n0 >> 7) * g.ws_rs + (int64_t)kb0 * g.ws_cs) : nullptr;
+  auto load_unit = [&](WUnit<RG>& u, int k) __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < RG; ++r) {
+      u.lo[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[r] + (int64_t)k * 128));
+      u.hi[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[r] + (int64_t)k * 128 + 64));
+    }
+    u.ws = (MODE == kModeBlock) ? ws_ptr[(int64_t)k * g.ws_cs] : 1.f;
+  };
+
+  // the first DEPTH K-blocks of weights are on their way while the activations are staged
+  WUnit<RG> ring[DEPTH];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (active && d < kbs) load_unit(ring[d], d);
+
+  // ---- activations of this block's K range -> LDS: row R, logical 16-byte chunk c at R * 128 + ((c ^ (R & 7)) << 4).
+  // Direct global -> LDS loads (no registers, nothing to wait for until the barrier): one instruction moves a
+  // slab of 8 rows x 128 bytes, lane L landing at byte 16 L of the slab, i.e. row L >> 3, physical chunk L & 7; the
+  // lane therefore fetches logical chunk (L & 7) ^ (row & 7) of its row.  Wavefront w takes the slabs w, w + WAVES, ...
+  {
+    constexpr int kPer = 8 / WAVES;  // slabs per wavefront and K-block
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+    uint32_t xoff[kPer];
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      const int row = (wave + i * WAVES) * 8 + (lane >> 3);
+      const int src = row < g.M ? row : g.M - 1;
+      xoff[i] = (uint32_t)src * (uint32_t)g.ldx + (uint32_t)((((lane & 7) ^ ((lane >> 3) & 7))) << 4);  // ldx < 2^23
+    }
+    const uint8_t* const xbase = uniform_ptr(g.X + (int64_t)kb0 * 128);
+    for (int kb = 0; kb < kbs; ++kb) {
+#pragma unroll
+      for (int i = 0; i < kPer; ++i) {
+        const uint8_t* const src = xbase + (int64_t)kb * 128;
+        const uint32_t dst = lds_base + (uint32_t)(kb * kMidStageBytes + (wave + i * WAVES) * 1024);
+        asm volatile("s_mov_b32 m0, %2\n\t"
+                     "s_nop 0\n\t"
+                     "global_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(xoff[i]), "s"(src), "s"(dst)
+                     : "memory", "m0");
+      }
+    }
+  }
+  float* const xs_lds = reinterpret_cast<float*>(lds + a.kb_per_split * kMidStageBytes);
+  if (MODE == kModeBlock) {
+    for (int i = tid; i < kbs * kMidRows; i += NT) {
+      const int kb = i >> 6, row = i & 63;
+      const int src = row < g.M ? row : g.M - 1;
+      xs_lds[i] = g.xs[(int64_t)src * g.xs_rs + (int64_t)(kb0 + kb) * g.xs_cs];
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // the direct loads are not tracked by the compiler
+  __syncthreads();
+  if (!active) return;  // no barrier below
+
+  v4f acc[RG][4];
+#pragma unroll
+  for (int r = 0; r < RG; ++r)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[r][t] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  // fragment of the 16-row group t for this lane: row t * 16 + l16, logical chunks lg and lg + 4
+  const int frag_off = l16 * 128 + ((lg ^ (l16 & 7)) << 4);
+  // the ring index is static: the body is written out once per register set
+  int kb = 0;
+  while (kb < kbs) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (kb < kbs) {
+        WUnit<RG>& u = ring[d];
+        const uint8_t* const xt = lds + kb * kMidStageBytes;
+        v8i xf[4];
+        float sc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const u32x4 lo = *reinterpret_cast<const u32x4*>(xt + t * 2048 + frag_off);
+          const u32x4 hi = *reinterpret_cast<const u32x4*>(xt + t * 2048 + (frag_off ^ 64));
+          xf[t] = join8(lo, hi);
+          sc[t] = (MODE == kModeBlock) ? xs_lds[kb * kMidRows + t * 16 + l16] * u.ws : 1.f;
+        }
+#pragma unroll
+        for (int r = 0; r < RG; ++r) {
+          const v8i wf = join8(u.lo[r], u.hi[r]);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            if (MODE == kModeBlock) {
+              const v4f p = mfma_fp8_16x16x128(wf, xf[t], v4f{0.f, 0.f, 0.f, 0.f});
+              acc[r][t][0] = __builtin_fmaf(p[0], sc[t], acc[r][t][0]);
+              acc[r][t][1] = __builtin_fmaf(p[1], sc[t], acc[r][t][1]);
+              acc[r][t][2] = __builtin_fmaf(p[2], sc[t], acc[r][t][2]);
+              acc[r][t][3] = __builtin_fmaf(p[3], sc[t], acc[r][t][3]);
+            } else {
+              acc[r][t] = mfma_fp8_16x16x128(wf, xf[t], acc[r][t]);
+            }
+          }
+        }
+        if (kb + DEPTH < kbs) load_unit(u, kb + DEPTH);
+        ++kb;
+      }
+    }
+  }
+
+  // ---- K split over blocks: publish, count in, and let the wavefront that arrives last add the splits in order
+  if (a.splits > 1) {
+    constexpr int kSlotFloats = RG * 4 * 64 * 4;
+    const uint32_t l_off = (uint32_t)lane * 16u;
+    float* const mine = uniform_ptr(a.partials + ((size_t)chunk * a.splits + split) * kSlotFloats);
+#pragma unroll
+    for (int r = 0; r < RG; ++r)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) store_x4_agent(mine + (r * 4 + t) * 256, l_off, acc[r][t]);
+    wait_vmem_all();
+    unsigned int* const cnt = a.counters + chunk;
+    unsigned int prev = 0;
+    if (lane == 0) prev = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    prev = (unsigned int)__builtin_amdgcn_readfirstlane((int)prev);
+    if (prev != (unsigned int)(a.splits - 1)) return;
+    for (int s = 0; s < a.splits; ++s) {
+      const float* const src = uniform_ptr(a.partials + ((size_t)chunk * a.splits + s) * kSlotFloats);
+      v4f tmp[RG][4];
+#pragma unroll
+      for (int r = 0; r < RG; ++r)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) load_x4_agent(tmp[r][t], src + (r * 4 + t) * 256, l_off);
+#pragma unroll
+      for (int r = 0; r < RG; ++r)  // the values are operands of the wait, so no use can move above it
+#pragma unroll
+        for (int t = 0; t < 4; ++t) asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[r][t]) : : "memory");
+#pragma unroll
+      for (int r = 0; r < RG; ++r)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          if (s == 0) acc[r][t] = tmp[r][t]; else acc[r][t] += tmp[r][t];  // no "0 + x" in the sum
+        }
+    }
+    if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+  }
+
+  // ---- results: the lane holds m = t * 16 + l16, n = n0 + r * 16 + 4 * lg + [0, 4)
+  const bool pack_ok = MODE == kModeBlock && g.c_dtype == FG_BF16 && (g.ldc & 3) == 0 && ((uintptr_t)g.C & 7) == 0;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int m = t * 16 + l16;
+    if (m >= g.M) continue;
+#pragma unroll
+    for (int r = 0; r < RG; ++r) {
+      const int n = n0 + r * 16 + lg * 4;
+      if (pack_ok && n + 4 <= g.N) {
+        const u32x2 o = {(uint32_t)float_to_bf16_bits(acc[r][t][0]) | ((uint32_t)float_to_bf16_bits(acc[r][t][1]) << 16),
+                         (uint32_t)float_to_bf16_bits(acc[r][t][2]) | ((uint32_t)float_to_bf16_bits(acc[r][t][3]) << 16)};
+        *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(g.C) + (int64_t)m * g.ldc + n) = o;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < g.N) store_output<MODE>(g, m, n + e, acc[r][t][e]);
+      }
+    }
+  }
+}
+
+template <int RG, int WAVES, int DEPTH>
+int launch_mid(const MidArgs& ma, int mode, hipStream_t stream) {
+  const int lds_bytes = ma.kb_per_split * (kMidStageBytes + kMidRows * 4);
+  auto kb = fp8_gemm_midm_kernel<RG, WAVES, DEPTH, kModeBlock>;
+  auto kr = fp8_gemm_midm_kernel<RG, WAVES, DEPTH, kModeRowCol>;
+  static bool attr_set = false;  // per instantiation; benign if raced
+  if (!attr_set) {
+    constexpr int kMax = kMidKbMax * (kMidStageBytes + kMidRows * 4);
+    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(kb), hipFuncAttributeMaxDynamicSharedMemorySize, kMax);
+    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(kr), hipFuncAttributeMaxDynamicSharedMemorySize, kMax);
+    if (e1 != hipSuccess || e2 != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS) failed", kMax);
+    attr_set = true;
+  }
+  const dim3 grid((uint32_t)ceil_div(ma.n_chunks, WAVES), (uint32_t)ma.splits), block(WAVES * 64);
+  if (mode == kModeBlock) hipLaunchKernelGGL(kb, grid, block, lds_bytes, stream, ma);
+  else hipLaunchKernelGGL(kr, grid, block, lds_bytes, stream, ma);
+  FG_CHECK_LAUNCH("fp8_gemm_midm_kernel");
+  return FG_OK;
+}
+
+}  // namespace
+
+MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K) {
+  MidMPlan p = {};
+  if (M <= 32 || M > kMidRows || N < 1 || K < 128 || K % 128 != 0) return p;
+  const int64_t KB = K / 128;
+  // as few splits as LDS allows, then the widest row group that still gives ~3 wavefronts per compute unit;
+  // narrow weights get more splits instead (their partial sums are small)
+  int64_t splits = ceil_div(KB, (int64_t)kMidKbMax);
+  int rg = 4;
+  const int64_t want = 700;
+  while (rg > 1 && ceil_div(N, 16 * rg) * splits < want) rg >>= 1;
+  while (ceil_div(N, 16 * rg) * splits < want && ceil_div(KB, splits + 1) >= 4) ++splits;
+  const int64_t kbps = ceil_div(KB, splits);
+  splits = ceil_div(KB, kbps);
+  p.rg = rg;
+  p.kb_per_split = (int)kbps;
+  p.splits = (int)splits;
+  p.n_chunks = (int)ceil_div(N, 16 * rg);
+  if (p.n_chunks > FG_WORKSPACE_COUNTER_BYTES / 4 || splits > 65535) return p;
+  p.waves = ceil_div(p.n_chunks, 8) * splits >= 200 ? 8 : 4;
+  p.workspace_bytes = splits > 1 ? (size_t)FG_WORKSPACE_COUNTER_BYTES + (size_t)p.n_chunks * splits * rg * 4 * 64 * 16 : 0;
+  p.use = true;
+  return p;
+}
+
+int launch_mid_m(const GemmArgs& g, int mode, const MidMPlan& plan, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  MidArgs ma;
+  ma.g = g;
+  ma.kb_per_split = plan.kb_per_split;
+  ma.splits = plan.splits;
+  ma.n_chunks = plan.n_chunks;
+  ma.partials = nullptr;
+  ma.counters = nullptr;
+  if (plan.splits > 1) {
+    if (!workspace || workspace_bytes < plan.workspace_bytes)
+      FG_FAIL(FG_ERR_WORKSPACE, "fp8 gemm (33..64 rows): workspace of %zu bytes needed, %zu given", plan.workspace_bytes, workspace_bytes);
+    if ((uintptr_t)workspace % 16 != 0) FG_FAIL(FG_ERR_INVALID_ARG, "fp8 gemm (33..64 rows): workspace must be 16-byte aligned");
+    ma.counters = reinterpret_cast<unsigned int*>(workspace);
+    ma.partials = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
+  }
+  if (plan.rg == 4) return plan.waves == 8 ? launch_mid<4, 8, 2>(ma, mode, stream) : launch_mid<4, 4, 2>(ma, mode, stream);
+  if (plan.rg == 2) return plan.waves == 8 ? launch_mid<2, 8, 4>(ma, mode, stream) : launch_mid<2, 4, 4>(ma, mode, stream);
+  return plan.waves == 8 ? launch_mid<1, 8, 8>(ma, mode, stream) : launch_mid<1, 4, 8>(ma, mode, stream);
+}
+
+}  // namespace fg
