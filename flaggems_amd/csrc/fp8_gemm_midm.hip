@@ -258,13 +258,21 @@ MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K) {
   MidMPlan p = {};
   if (M <= 32 || M > kMidRows || N < 1 || K < 128 || K % 128 != 0) return p;
   const int64_t KB = K / 128;
-  // as few splits as LDS allows, then the widest row group that still gives ~3 wavefronts per compute unit;
-  // narrow weights get more splits instead (their partial sums are small)
-  int64_t splits = ceil_div(KB, (int64_t)kMidKbMax);
-  int rg = 4;
-  const int64_t want = 700;
-  while (rg > 1 && ceil_div(N, 16 * rg) * splits < want) rg >>= 1;
-  while (ceil_div(N, 16 * rg) * splits < want && ceil_div(KB, splits + 1) >= 4) ++splits;
+  // Measured on the DeepSeek-V3 shapes with 64 rows (weights rotated through 512 MB): the narrowest row group
+  // wins almost everywhere (more wavefronts, each with 16 KB of weights in flight); K is split until there are
+  // ~1800 wavefronts but not below 8 K-blocks per block (every split writes and reads N x 64 fp32 sums: +50 % of the
+  // weight bytes at 8 K-blocks, +25 % at 16), and never less than LDS requires.
+  const int64_t min_splits = ceil_div(KB, (int64_t)kMidKbMax);
+  int rg = 1;
+  if (ceil_div(N, 16) * min_splits >= 3000) rg = 2;  // plenty of wavefronts: N = 7168, K = 16384: 43 -> 39 us
+  while (rg < 4 && ceil_div(N, 16 * rg) > FG_WORKSPACE_COUNTER_BYTES / 4) rg <<= 1;
+  int64_t splits = ceil_div((int64_t)1800, ceil_div(N, 16 * rg));
+  const int64_t max_splits = KB / 8 > min_splits ? KB / 8 : min_splits;
+  splits = splits < min_splits ? min_splits : (splits > max_splits ? max_splits : splits);
+#ifdef FG_DEV_KNOBS
+  if (const char* e = getenv("FG_MID_RG")) rg = atoi(e);
+  if (const char* e = getenv("FG_MID_SPLITS")) splits = atoi(e) < ceil_div(KB, (int64_t)kMidKbMax) ? ceil_div(KB, (int64_t)kMidKbMax) : atoi(e);
+#endif
   const int64_t kbps = ceil_div(KB, splits);
   splits = ceil_div(KB, kbps);
   p.rg = rg;
@@ -272,7 +280,11 @@ MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K) {
   p.splits = (int)splits;
   p.n_chunks = (int)ceil_div(N, 16 * rg);
   if (p.n_chunks > FG_WORKSPACE_COUNTER_BYTES / 4 || splits > 65535) return p;
-  p.waves = ceil_div(p.n_chunks, 8) * splits >= 200 ? 8 : 4;
+  // one block per compute unit when its activations take more than half of LDS: then it should bring 8 wavefronts
+  p.waves = kbps * (kMidStageBytes + kMidRows * 4) > 80 * 1024 ? 8 : 4;
+#ifdef FG_DEV_KNOBS
+  if (const char* e = getenv("FG_MID_WAVES")) p.waves = atoi(e);
+#endif
   p.workspace_bytes = splits > 1 ? (size_t)FG_WORKSPACE_COUNTER_BYTES + (size_t)p.n_chunks * splits * rg * 4 * 64 * 16 : 0;
   p.use = true;
   return p;

@@ -107,6 +107,26 @@ def test_few_tiles_split_along_k(M, N, K, dtype):
         assert torch.equal(again.view(torch.int8), got.view(torch.int8))
 
 
+@pytest.mark.parametrize("M,N,K", [(33, 100, 384), (64, 2112, 7168), (50, 7168, 16384), (40, 24584, 1536), (64, 4104, 2304)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_33_to_64_rows(M, N, K, dtype):
+    """33 <= M <= 64 takes the kernel that keeps the activations in LDS and streams the weights: one K range or
+    several (partial sums added in split order), N that ends inside a 16-row group, fewer than 64 rows, every
+    output type, column-major scales; against the oracle and bit-identical on reruns."""
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=13)
+    want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
+    args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    got = flag_gems.w8a8_block_fp8_matmul(*args, output_dtype=dtype)
+    assert got.dtype == dtype and got.shape == (M, N)
+    tol = dict(rtol=1e-4, atol=2e-4) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(got.cpu().float(), want, **tol)
+    for _ in range(2):
+        assert torch.equal(flag_gems.w8a8_block_fp8_matmul(*args, output_dtype=dtype).view(torch.int8), got.view(torch.int8))
+    xs_cm = xs.to(DEV).t().contiguous().t()
+    cm = flag_gems.w8a8_block_fp8_matmul(args[0], args[1], xs_cm, args[3], [128, 128], output_dtype=dtype)
+    assert torch.equal(cm.view(torch.int8), got.view(torch.int8))
+
+
 @pytest.mark.parametrize("M,N,K", [(1024, 7168, 8192), (300, 7000, 16384)])
 def test_tiles_cut_into_equal_ranges_along_k(M, N, K):
     """112 tiles x 64 K-blocks and 56 tiles x 128 K-blocks (ragged in M and N): the persistent kernel cuts every
