@@ -551,11 +551,14 @@ int launch_tile_split(GemmArgs a, const TileSplitPlan& plan, void* workspace, hi
 // Whether the 33..64-row kernel is the one to take for the shape (it is compared with the K-split tile kernel and
 // the decode kernels, which take the same shapes).
 bool mid_m_preferred(const MidMPlan& mid, int64_t M, int64_t N, int64_t K) {
-  (void)M; (void)N; (void)K;
+  (void)M;
 #ifdef FG_DEV_KNOBS
   if (const char* e = getenv("FG_MIDM")) return mid.use && atoi(e) != 0;
 #endif
-  return mid.use;
+  // 33..64 rows: always (measured against both alternatives on every DeepSeek-V3 and Llama-3 shape).  65..128 rows:
+  // the splits' partial sums cost as much as the weights, which pays only while the weights are small: M = 128,
+  // N = 6144, K = 4096: 31 -> 20 us; N = 7168, K = 2304: 19 -> 16 us; but N = 24576, K = 1536: 23 -> 28 us.
+  return mid.use && (mid.tmx == 4 || N * K <= (int64_t)28 << 20);
 }
 
 template <int MODE>

@@ -1,5 +1,5 @@
-// FP8 GEMM for 33 <= M <= 64 activation rows on gfx950: the weight is read once, straight from global memory
-// into MFMA operand registers, and the activations come out of LDS.
+// FP8 GEMM for 33 <= M <= 64 activation rows on gfx950 (and up to 128 rows against small weights): the weight is
+// read once, straight from global memory into MFMA operand registers, and the activations come out of LDS.
 //
 // With up to 64 rows the activation slice of a K-block (64 x 128 bytes) is as large as the 64 weight rows a
 // wavefront multiplies it with, so a wavefront that fetches both from global memory moves two bytes for every
@@ -10,8 +10,8 @@
 //
 //  * A wavefront owns 16 * RG weight rows (RG = 1, 2, 4) and the K-blocks [split * kb_per_split, ...): per K-block
 //    2 * RG 16-byte loads per lane (DEPTH K-blocks in flight, 64 VGPRs), 8 LDS reads, 4 * RG MFMAs.
-//  * K is split over gridDim.y blocks only as far as LDS (16 K-blocks = 128 KB of activations) or the number
-//    of wavefronts requires; each wavefront then publishes its sums and the one that arrives last adds the
+//  * K is split over gridDim.y blocks only as far as LDS (128 KB of activations: 16 K-blocks of 64 rows, 8 of
+//    128 rows) or the number of wavefronts requires; each wavefront then publishes its sums and the one that arrives last adds the
 //    splits' sums in split order (a fixed order: results do not depend on timing) and resets the counter.
 //
 // Arithmetic as in the other kernels: per K-block products accumulated by the fp8 MFMA, multiplied by
@@ -22,14 +22,16 @@
 namespace fg {
 namespace {
 
-constexpr int kMidRows = 64;            // activation rows staged (rows past M repeat the last one; never stored)
-constexpr int kMidKbMax = 16;           // K-blocks of activations a block keeps in LDS
-constexpr int kMidStageBytes = kMidRows * 128;
+// TMX 16-row groups of activations are staged (64 or 128 rows; rows past M repeat the last one and are never
+// stored); a block keeps at most 128 KB of them in LDS: 16 K-blocks of 64 rows, 8 of 128.
+constexpr int mid_rows(int tmx) { return 16 * tmx; }
+constexpr int mid_stage_bytes(int tmx) { return mid_rows(tmx) * 128; }
+constexpr int mid_kb_max(int tmx) { return 64 / tmx; }
 
 struct MidArgs {
   GemmArgs g;
   int kb_per_split, splits, n_chunks;  // n_chunks = ceil(N / (16 * RG))
-  float* partials;                     // [n_chunks][splits][RG * 4][64 lanes] x 4 floats
+  float* partials;                     // [n_chunks][splits][RG * TMX][64 lanes] x 4 floats
   unsigned int* counters;              // one per chunk
 };
 
@@ -46,9 +48,10 @@ __device__ __forceinline__ v8i join8(u32x4 lo, u32x4 hi) {
   return f;
 }
 
-template <int RG, int WAVES, int DEPTH, int MODE>
+template <int TMX, int RG, int WAVES, int DEPTH, int MODE>
 __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
   constexpr int NT = WAVES * 64;
+  constexpr int kMidRows = mid_rows(TMX), kMidStageBytes = mid_stage_bytes(TMX);
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [kb][64 rows][128 B], then As [kb][64]
   const GemmArgs& g = a.g;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -91,7 +94,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
   // slab of 8 rows x 128 bytes, lane L landing at byte 16 L of the slab, i.e. row L >> 3, physical chunk L & 7; the
   // lane therefore fetches logical chunk (L & 7) ^ (row & 7) of its row.  Wavefront w takes the slabs w, w + WAVES, ...
   {
-    constexpr int kPer = 8 / WAVES;  // slabs per wavefront and K-block
+    constexpr int kPer = 2 * TMX / WAVES;  // slabs per wavefront and K-block
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
     uint32_t xoff[kPer];
 #pragma unroll
@@ -118,7 +121,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
   float* const xs_lds = reinterpret_cast<float*>(lds + a.kb_per_split * kMidStageBytes);
   if (MODE == kModeBlock) {
     for (int i = tid; i < kbs * kMidRows; i += NT) {
-      const int kb = i >> 6, row = i & 63;
+      const int kb = i / kMidRows, row = i % kMidRows;
       const int src = row < g.M ? row : g.M - 1;
       xs_lds[i] = g.xs[(int64_t)src * g.xs_rs + (int64_t)(kb0 + kb) * g.xs_cs];
     }
@@ -127,11 +130,11 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
   __syncthreads();
   if (!active) return;  // no barrier below
 
-  v4f acc[RG][4];
+  v4f acc[RG][TMX];
 #pragma unroll
   for (int r = 0; r < RG; ++r)
 #pragma unroll
-    for (int t = 0; t < 4; ++t) acc[r][t] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < TMX; ++t) acc[r][t] = v4f{0.f, 0.f, 0.f, 0.f};
 
   // fragment of the 16-row group t for this lane: row t * 16 + l16, logical chunks lg and lg + 4
   const int frag_off = l16 * 128 + ((lg ^ (l16 & 7)) << 4);
@@ -143,10 +146,10 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
       if (kb < kbs) {
         WUnit<RG>& u = ring[d];
         const uint8_t* const xt = lds + kb * kMidStageBytes;
-        v8i xf[4];
-        float sc[4];
+        v8i xf[TMX];
+        float sc[TMX];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < TMX; ++t) {
           const u32x4 lo = *reinterpret_cast<const u32x4*>(xt + t * 2048 + frag_off);
           const u32x4 hi = *reinterpret_cast<const u32x4*>(xt + t * 2048 + (frag_off ^ 64));
           xf[t] = join8(lo, hi);
@@ -156,7 +159,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
         for (int r = 0; r < RG; ++r) {
           const v8i wf = join8(u.lo[r], u.hi[r]);
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
+          for (int t = 0; t < TMX; ++t) {
             if (MODE == kModeBlock) {
               const v4f p = mfma_fp8_16x16x128(wf, xf[t], v4f{0.f, 0.f, 0.f, 0.f});
               acc[r][t][0] = __builtin_fmaf(p[0], sc[t], acc[r][t][0]);
@@ -176,13 +179,13 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
 
   // ---- K split over blocks: publish, count in, and let the wavefront that arrives last add the splits in order
   if (a.splits > 1) {
-    constexpr int kSlotFloats = RG * 4 * 64 * 4;
+    constexpr int kSlotFloats = RG * TMX * 64 * 4;
     const uint32_t l_off = (uint32_t)lane * 16u;
     float* const mine = uniform_ptr(a.partials + ((size_t)chunk * a.splits + split) * kSlotFloats);
 #pragma unroll
     for (int r = 0; r < RG; ++r)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) store_x4_agent(mine + (r * 4 + t) * 256, l_off, acc[r][t]);
+      for (int t = 0; t < TMX; ++t) store_x4_agent(mine + (r * TMX + t) * 256, l_off, acc[r][t]);
     wait_vmem_all();
     unsigned int* const cnt = a.counters + chunk;
     unsigned int prev = 0;
@@ -191,19 +194,19 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
     if (prev != (unsigned int)(a.splits - 1)) return;
     for (int s = 0; s < a.splits; ++s) {
       const float* const src = uniform_ptr(a.partials + ((size_t)chunk * a.splits + s) * kSlotFloats);
-      v4f tmp[RG][4];
+      v4f tmp[RG][TMX];
 #pragma unroll
       for (int r = 0; r < RG; ++r)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) load_x4_agent(tmp[r][t], src + (r * 4 + t) * 256, l_off);
+        for (int t = 0; t < TMX; ++t) load_x4_agent(tmp[r][t], src + (r * TMX + t) * 256, l_off);
 #pragma unroll
       for (int r = 0; r < RG; ++r)  // the values are operands of the wait, so no use can move above it
 #pragma unroll
-        for (int t = 0; t < 4; ++t) asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[r][t]) : : "memory");
+        for (int t = 0; t < TMX; ++t) asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[r][t]) : : "memory");
 #pragma unroll
       for (int r = 0; r < RG; ++r)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < TMX; ++t) {
           if (s == 0) acc[r][t] = tmp[r][t]; else acc[r][t] += tmp[r][t];  // no "0 + x" in the sum
         }
     }
@@ -213,7 +216,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
   // ---- results: the lane holds m = t * 16 + l16, n = n0 + r * 16 + 4 * lg + [0, 4)
   const bool pack_ok = MODE == kModeBlock && g.c_dtype == FG_BF16 && (g.ldc & 3) == 0 && ((uintptr_t)g.C & 7) == 0;
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
+  for (int t = 0; t < TMX; ++t) {
     const int m = t * 16 + l16;
     if (m >= g.M) continue;
 #pragma unroll
@@ -232,14 +235,15 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
   }
 }
 
-template <int RG, int WAVES, int DEPTH>
+template <int TMX, int RG, int WAVES, int DEPTH>
 int launch_mid(const MidArgs& ma, int mode, hipStream_t stream) {
-  const int lds_bytes = ma.kb_per_split * (kMidStageBytes + kMidRows * 4);
-  auto kb = fp8_gemm_midm_kernel<RG, WAVES, DEPTH, kModeBlock>;
-  auto kr = fp8_gemm_midm_kernel<RG, WAVES, DEPTH, kModeRowCol>;
+  constexpr int kPerKb = mid_stage_bytes(TMX) + mid_rows(TMX) * 4;
+  const int lds_bytes = ma.kb_per_split * kPerKb;
+  auto kb = fp8_gemm_midm_kernel<TMX, RG, WAVES, DEPTH, kModeBlock>;
+  auto kr = fp8_gemm_midm_kernel<TMX, RG, WAVES, DEPTH, kModeRowCol>;
   static bool attr_set = false;  // per instantiation; benign if raced
   if (!attr_set) {
-    constexpr int kMax = kMidKbMax * (kMidStageBytes + kMidRows * 4);
+    constexpr int kMax = mid_kb_max(TMX) * kPerKb;
     hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(kb), hipFuncAttributeMaxDynamicSharedMemorySize, kMax);
     hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(kr), hipFuncAttributeMaxDynamicSharedMemorySize, kMax);
     if (e1 != hipSuccess || e2 != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS) failed", kMax);
@@ -256,36 +260,50 @@ int launch_mid(const MidArgs& ma, int mode, hipStream_t stream) {
 
 MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K) {
   MidMPlan p = {};
-  if (M <= 32 || M > kMidRows || N < 1 || K < 128 || K % 128 != 0) return p;
+  if (M <= 32 || M > 128 || N < 1 || K < 128 || K % 128 != 0) return p;
   const int64_t KB = K / 128;
-  // Measured on the DeepSeek-V3 shapes with 64 rows (weights rotated through 512 MB): the narrowest row group
-  // wins almost everywhere (more wavefronts, each with 16 KB of weights in flight); K is split until there are
-  // ~1800 wavefronts but not below 8 K-blocks per block (every split writes and reads N x 64 fp32 sums: +50 % of the
-  // weight bytes at 8 K-blocks, +25 % at 16), and never less than LDS requires.
-  const int64_t min_splits = ceil_div(KB, (int64_t)kMidKbMax);
-  int rg = 1;
-  if (ceil_div(N, 16) * min_splits >= 3000) rg = 2;  // plenty of wavefronts: N = 7168, K = 16384: 43 -> 39 us
+  const int tmx = M <= 64 ? 4 : 8;
+  const int64_t kb_max = mid_kb_max(tmx);
+  const int64_t min_splits = ceil_div(KB, kb_max);
+  int rg;
+  int64_t splits;
+  if (tmx == 4) {
+    // Measured on the DeepSeek-V3 shapes with 64 rows (weights rotated through 512 MB): the narrowest row group
+    // wins almost everywhere (more wavefronts, each with 16 KB of weights in flight); K is split until there are
+    // ~1800 wavefronts but not below 8 K-blocks per block (every split writes and reads N x 64 fp32 sums: +50 % of
+    // the weight bytes at 8 K-blocks, +25 % at 16), and never less than LDS requires.
+    rg = 1;
+    if (ceil_div(N, 16) * min_splits >= 3000) rg = 2;  // plenty of wavefronts: N = 7168, K = 16384: 43 -> 39 us
+    splits = ceil_div((int64_t)1800, ceil_div(N, 16 * rg));
+    const int64_t max_splits = KB / 8 > min_splits ? KB / 8 : min_splits;
+    splits = splits < min_splits ? min_splits : (splits > max_splits ? max_splits : splits);
+  } else {
+    // 65..128 rows: a K-block of activations is 16 KB, so LDS holds 8 and every split costs as many bytes as the
+    // weights of 8 K-blocks.  Measured (M = 128): one row group per wavefront beats two wherever this kernel
+    // beats the tile kernel at all, which is for weights of up to ~28 MB (see the caller's rule).
+    rg = 1;
+    splits = min_splits;
+  }
   while (rg < 4 && ceil_div(N, 16 * rg) > FG_WORKSPACE_COUNTER_BYTES / 4) rg <<= 1;
-  int64_t splits = ceil_div((int64_t)1800, ceil_div(N, 16 * rg));
-  const int64_t max_splits = KB / 8 > min_splits ? KB / 8 : min_splits;
-  splits = splits < min_splits ? min_splits : (splits > max_splits ? max_splits : splits);
+  if (tmx == 8 && rg > 2) return p;
 #ifdef FG_DEV_KNOBS
   if (const char* e = getenv("FG_MID_RG")) rg = atoi(e);
-  if (const char* e = getenv("FG_MID_SPLITS")) splits = atoi(e) < ceil_div(KB, (int64_t)kMidKbMax) ? ceil_div(KB, (int64_t)kMidKbMax) : atoi(e);
+  if (const char* e = getenv("FG_MID_SPLITS")) splits = atoi(e) < min_splits ? min_splits : atoi(e);
 #endif
   const int64_t kbps = ceil_div(KB, splits);
   splits = ceil_div(KB, kbps);
+  p.tmx = tmx;
   p.rg = rg;
   p.kb_per_split = (int)kbps;
   p.splits = (int)splits;
   p.n_chunks = (int)ceil_div(N, 16 * rg);
   if (p.n_chunks > FG_WORKSPACE_COUNTER_BYTES / 4 || splits > 65535) return p;
   // one block per compute unit when its activations take more than half of LDS: then it should bring 8 wavefronts
-  p.waves = kbps * (kMidStageBytes + kMidRows * 4) > 80 * 1024 ? 8 : 4;
+  p.waves = kbps * (mid_stage_bytes(tmx) + mid_rows(tmx) * 4) > 80 * 1024 ? 8 : 4;
 #ifdef FG_DEV_KNOBS
   if (const char* e = getenv("FG_MID_WAVES")) p.waves = atoi(e);
 #endif
-  p.workspace_bytes = splits > 1 ? (size_t)FG_WORKSPACE_COUNTER_BYTES + (size_t)p.n_chunks * splits * rg * 4 * 64 * 16 : 0;
+  p.workspace_bytes = splits > 1 ? (size_t)FG_WORKSPACE_COUNTER_BYTES + (size_t)p.n_chunks * splits * rg * tmx * 64 * 16 : 0;
   p.use = true;
   return p;
 }
@@ -300,14 +318,18 @@ int launch_mid_m(const GemmArgs& g, int mode, const MidMPlan& plan, void* worksp
   ma.counters = nullptr;
   if (plan.splits > 1) {
     if (!workspace || workspace_bytes < plan.workspace_bytes)
-      FG_FAIL(FG_ERR_WORKSPACE, "fp8 gemm (33..64 rows): workspace of %zu bytes needed, %zu given", plan.workspace_bytes, workspace_bytes);
-    if ((uintptr_t)workspace % 16 != 0) FG_FAIL(FG_ERR_INVALID_ARG, "fp8 gemm (33..64 rows): workspace must be 16-byte aligned");
+      FG_FAIL(FG_ERR_WORKSPACE, "fp8 gemm (33..128 rows): workspace of %zu bytes needed, %zu given", plan.workspace_bytes, workspace_bytes);
+    if ((uintptr_t)workspace % 16 != 0) FG_FAIL(FG_ERR_INVALID_ARG, "fp8 gemm (33..128 rows): workspace must be 16-byte aligned");
     ma.counters = reinterpret_cast<unsigned int*>(workspace);
     ma.partials = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
   }
-  if (plan.rg == 4) return plan.waves == 8 ? launch_mid<4, 8, 2>(ma, mode, stream) : launch_mid<4, 4, 2>(ma, mode, stream);
-  if (plan.rg == 2) return plan.waves == 8 ? launch_mid<2, 8, 4>(ma, mode, stream) : launch_mid<2, 4, 4>(ma, mode, stream);
-  return plan.waves == 8 ? launch_mid<1, 8, 8>(ma, mode, stream) : launch_mid<1, 4, 8>(ma, mode, stream);
+  if (plan.tmx == 8) {
+    if (plan.rg == 2) return plan.waves == 8 ? launch_mid<8, 2, 8, 4>(ma, mode, stream) : launch_mid<8, 2, 4, 4>(ma, mode, stream);
+    return plan.waves == 8 ? launch_mid<8, 1, 8, 8>(ma, mode, stream) : launch_mid<8, 1, 4, 8>(ma, mode, stream);
+  }
+  if (plan.rg == 4) return plan.waves == 8 ? launch_mid<4, 4, 8, 2>(ma, mode, stream) : launch_mid<4, 4, 4, 2>(ma, mode, stream);
+  if (plan.rg == 2) return plan.waves == 8 ? launch_mid<4, 2, 8, 4>(ma, mode, stream) : launch_mid<4, 2, 4, 4>(ma, mode, stream);
+  return plan.waves == 8 ? launch_mid<4, 1, 8, 8>(ma, mode, stream) : launch_mid<4, 1, 4, 8>(ma, mode, stream);
 }
 
 }  // namespace fg

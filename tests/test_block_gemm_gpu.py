@@ -107,12 +107,14 @@ def test_few_tiles_split_along_k(M, N, K, dtype):
         assert torch.equal(again.view(torch.int8), got.view(torch.int8))
 
 
-@pytest.mark.parametrize("M,N,K", [(33, 100, 384), (64, 2112, 7168), (50, 7168, 16384), (40, 24584, 1536), (64, 4104, 2304)])
+@pytest.mark.parametrize("M,N,K", [(33, 100, 384), (64, 2112, 7168), (50, 7168, 16384), (40, 24584, 1536), (64, 4104, 2304),
+                                   (65, 520, 1024), (100, 2112, 4096), (128, 4096, 4096), (128, 7000, 2304)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-def test_33_to_64_rows(M, N, K, dtype):
-    """33 <= M <= 64 takes the kernel that keeps the activations in LDS and streams the weights: one K range or
-    several (partial sums added in split order), N that ends inside a 16-row group, fewer than 64 rows, every
-    output type, column-major scales; against the oracle and bit-identical on reruns."""
+def test_33_to_128_rows(M, N, K, dtype):
+    """33 <= M <= 64 (and 65 <= M <= 128 with small weights) takes the kernel that keeps the activations in LDS and
+    streams the weights: one K range or several (partial sums added in split order), N that ends inside a 16-row
+    group, fewer rows than are staged, every output type, column-major scales; against the oracle and bit-identical
+    on reruns."""
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=13)
     want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
     args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
