@@ -192,23 +192,39 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
     if (lane == 0) prev = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     prev = (unsigned int)__builtin_amdgcn_readfirstlane((int)prev);
     if (prev != (unsigned int)(a.splits - 1)) return;
-    for (int s = 0; s < a.splits; ++s) {
-      const float* const src = uniform_ptr(a.partials + ((size_t)chunk * a.splits + s) * kSlotFloats);
-      v4f tmp[RG][TMX];
+    // The splits' sums are fetched kBatch splits at a time (one round trip to memory per batch instead of one per
+    // split) and added one split after the other, in split order.  Every batch is loaded, waited for and consumed
+    // inside one iteration: the loads are not tracked by the compiler, so no register may be in flight across the
+    // loop's back edge.
+    constexpr int kBatch = RG * TMX <= 8 ? 4 : 2;
+    for (int s0 = 0; s0 < a.splits; s0 += kBatch) {
+      v4f tmp[kBatch][RG][TMX];
 #pragma unroll
-      for (int r = 0; r < RG; ++r)
+      for (int b = 0; b < kBatch; ++b) {
+        const int s = s0 + b < a.splits ? s0 + b : a.splits - 1;  // past the end: re-read the last split, unused
+        const float* const src = uniform_ptr(a.partials + ((size_t)chunk * a.splits + s) * kSlotFloats);
 #pragma unroll
-        for (int t = 0; t < TMX; ++t) load_x4_agent(tmp[r][t], src + (r * TMX + t) * 256, l_off);
+        for (int r = 0; r < RG; ++r)
 #pragma unroll
-      for (int r = 0; r < RG; ++r)  // the values are operands of the wait, so no use can move above it
+          for (int t = 0; t < TMX; ++t) load_x4_agent(tmp[b][r][t], src + (r * TMX + t) * 256, l_off);
+      }
 #pragma unroll
-        for (int t = 0; t < TMX; ++t) asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[r][t]) : : "memory");
+      for (int b = 0; b < kBatch; ++b)  // the values are operands of the wait, so no use can move above it
 #pragma unroll
-      for (int r = 0; r < RG; ++r)
+        for (int r = 0; r < RG; ++r)
 #pragma unroll
-        for (int t = 0; t < TMX; ++t) {
-          if (s == 0) acc[r][t] = tmp[r][t]; else acc[r][t] += tmp[r][t];  // no "0 + x" in the sum
+          for (int t = 0; t < TMX; ++t) asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[b][r][t]) : : "memory");
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        if (s0 + b < a.splits) {
+#pragma unroll
+          for (int r = 0; r < RG; ++r)
+#pragma unroll
+            for (int t = 0; t < TMX; ++t) {
+              if (s0 + b == 0) acc[r][t] = tmp[b][r][t]; else acc[r][t] += tmp[b][r][t];  // no "0 + x" in the sum
+            }
         }
+      }
     }
     if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
   }
