@@ -33,10 +33,11 @@ template <> struct Elem<FG_BF16> {
   using raw = uint16_t;
   static constexpr uint32_t kAbs = 0x7FFFu, kInf = 0x7F80u;
   __device__ static float widen(uint32_t b) { return bits_to_float(b << 16); }
-  __device__ static uint32_t narrow(float f) {  // round to nearest even; NaN stays NaN
-    const uint32_t u = float_to_bits(f);
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
-    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+  // two values -> two bf16 in one word, round to nearest even (one v_cvt_pk_bf16_f32; NaN stays NaN)
+  __device__ static uint32_t narrow2(float lo, float hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
   }
 };
 template <> struct Elem<FG_F16> {
@@ -45,26 +46,27 @@ template <> struct Elem<FG_F16> {
   __device__ static float widen(uint32_t b) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
   }
-  __device__ static uint32_t narrow(float f) { return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f); }
+  __device__ static uint32_t narrow2(float lo, float hi) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+  }
 };
 template <> struct Elem<FG_F32> {
   using raw = uint32_t;
   static constexpr uint32_t kAbs = 0x7FFFFFFFu, kInf = 0x7F800000u;
   __device__ static float widen(uint32_t b) { return bits_to_float(b); }
-  __device__ static uint32_t narrow(float f) { return float_to_bits(f); }
 };
 
 // gate * sigmoid(gate) * up in fp32, as the reference's activation kernel computes it
 // (src/flag_gems/fused/fused_moe.py:795-800: x / (1 + exp(-x)) * y), rounded once to the input's type.
 template <int XDT>
-__device__ __forceinline__ uint32_t silu_mul_raw(uint32_t gate, uint32_t up) {
+__device__ __forceinline__ float silu_mul_f32(uint32_t gate, uint32_t up) {
   using E = Elem<XDT>;
   const float g = E::widen(gate), u = E::widen(up);
-  if constexpr (XDT == FG_F32) return E::narrow(g / (1.0f + expf(-g)) * u);
+  if constexpr (XDT == FG_F32) return g / (1.0f + expf(-g)) * u;
   // 16-bit results: the hardware exponential and reciprocal (what the reference's tl.exp and tl.fdiv compile to)
   // are wrong by a few fp32 steps, thousands of times below the step of the result; the correctly rounded
   // routines cost more instructions than the rest of the quantizer together and would bind the kernel.
-  return E::narrow(__fdividef(g, 1.0f + __expf(-g)) * u);
+  return __fdividef(g, 1.0f + __expf(-g)) * u;
 }
 
 // eight gate values and eight up values (raw words as loaded) -> eight activated values in the same packing
@@ -73,11 +75,9 @@ __device__ __forceinline__ void silu_mul_words(uint32_t (&w)[WORDS], const uint3
 #pragma unroll
   for (int i = 0; i < WORDS; ++i) {
     if constexpr (WORDS == 4) {
-      const uint32_t lo = silu_mul_raw<XDT>(w[i] & 0xFFFFu, up[i] & 0xFFFFu);
-      const uint32_t hi = silu_mul_raw<XDT>(w[i] >> 16, up[i] >> 16);
-      w[i] = (lo & 0xFFFFu) | (hi << 16);
+      w[i] = Elem<XDT>::narrow2(silu_mul_f32<XDT>(w[i] & 0xFFFFu, up[i] & 0xFFFFu), silu_mul_f32<XDT>(w[i] >> 16, up[i] >> 16));
     } else {
-      w[i] = silu_mul_raw<XDT>(w[i], up[i]);
+      w[i] = float_to_bits(silu_mul_f32<XDT>(w[i], up[i]));
     }
   }
 }
