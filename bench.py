@@ -47,12 +47,12 @@ CACHE_BYTES = 512 << 20   # rotate small-M weights through at least this much me
 # scaled by what the same counter read for the 256 MiB device copy issued first in that run (FETCH_SIZE read
 # half of the copied bytes, factor 2.0; WRITE_SIZE read all of them, factor 1.0).  (N, K) -> (fetch, write) KiB.
 TRAFFIC_M4096_KIB = {
-    (2112, 7168): (2.0 * 63344.3, 17792.0),
-    (24576, 1536): (2.0 * 111905.0, 196800.1),
-    (32768, 512): (2.0 * 46694.2, 262144.0),
-    (7168, 16384): (2.0 * 365859.2, 59392.1),
-    (4608, 7168): (2.0 * 124241.8, 37760.0),
-    (7168, 2304): (2.0 * 51546.6, 57632.0),
+    (2112, 7168): (2.0 * 63344.2, 17792.0),
+    (24576, 1536): (2.0 * 111901.5, 196800.2),
+    (32768, 512): (2.0 * 46648.1, 262145.6),
+    (7168, 16384): (2.0 * 365815.6, 59392.0),
+    (4608, 7168): (2.0 * 124243.6, 37760.0),
+    (7168, 2304): (2.0 * 51546.4, 57632.0),
 }
 
 
