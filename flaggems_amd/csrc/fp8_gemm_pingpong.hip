@@ -105,6 +105,9 @@ struct PpArgs {
   // tiles * sk_split), and the blocks of one XCD take the same cut of consecutive tiles: they walk the same K
   // offsets at the same time and share operand panels in their L2, as whole-tile launches do.
   int sk_split;
+  // Stream-K over the last n_tiles tiles of a larger problem (the whole rounds before them ran in a launch of their
+  // own): tile t of this launch is the tile that whole-tile launches number t + tile_base.
+  int tile_base;
   float* partials;
   unsigned int* counters;
   // Start-up delay of block b: (b mod 16) * stagger sleeps of about 1000 cycles.  With short K loops all compute
@@ -190,7 +193,8 @@ struct WalkT {
   __device__ __forceinline__ void locate(const PpArgs& a) {
     int tm = 0, tn = 0;
     if (idx < n_tiles) {
-      if (a.sk) tile_of_sid(idx, tiles_m, a.g.tiles_n, tm, tn);
+      if (a.sk && a.tile_base == 0) tile_of_sid(idx, tiles_m, a.g.tiles_n, tm, tn);
+      else if (a.sk) tile_of_index(idx + a.tile_base, tiles_m, a.g.tiles_n, tm, tn);
       else tile_of_index(idx, tiles_m, a.g.tiles_n, tm, tn);
     }
     m0 = tm * kBM; n0 = tn * kBN;
@@ -916,6 +920,40 @@ SkPlan plan_stream_k(int64_t tiles, int KB, int cus) {
   return p;
 }
 
+// Whole rounds plus a few tiles: the last round would keep tiles % cus units busy for a whole K loop.  Those tiles
+// go to a second launch instead, every one cut into `split` equal ranges (PpArgs::sk_split, tile_base) so that
+// more units share them.  What limits it is the exchange of partial tiles (256 KB each way per block, through
+// memory): measured ~0.25 K-block times per block of the second launch, so it gets at most 128 blocks and is taken
+// only when the sum still comes out 5 % ahead.  M = 4096, N = 4608, K = 7168 (288 tiles on 256 units, 32 x 4
+// ranges of 14): 169 -> 149 us; M = 2304, N = 8192, K = 8192: 192 -> 168 us; with 8 ranges of 7 (256 blocks) the
+// first shape takes 176 us.
+struct TailPlan {
+  bool use;
+  int full, tail, split, cut, grid;
+};
+TailPlan plan_tail(int64_t tiles, int KB, int cus) {
+  TailPlan p = {false, 0, 0, 0, 0, 0};
+  if (cus < 8 || tiles <= cus || tiles > 0x3FFFFFFF) return p;
+  const int64_t tail = tiles % cus;
+  if (tail == 0 || tail * 4 > cus) return p;
+  int64_t S = (cus / 2) / tail;
+  if (S > 16) S = 16;
+#ifdef FG_DEV_KNOBS
+  if (const char* e = getenv("FG_TAIL_S")) { S = atoi(e); if (S < 2) return p; }
+#endif
+  while (S >= 2 && KB % S != 0) --S;
+  if (S < 2 || KB / S < 4) return p;
+  const int64_t rounds = ceil_div(tiles, (int64_t)cus);
+  const int64_t now = rounds * KB, then = (rounds - 1) * KB + KB / S + tail * S / 4;
+#ifdef FG_DEV_KNOBS
+  if (getenv("FG_TAIL_S") == nullptr)
+#endif
+  if (then * 100 > now * 95) return p;
+  p.use = true;
+  p.full = (int)(tiles - tail); p.tail = (int)tail; p.split = (int)S; p.cut = (int)(KB / S); p.grid = (int)(tail * S);
+  return p;
+}
+
 // Activation scales [M, K/128] -> [K/128, M].  The GEMM reads four scales per lane and K-block, for rows 16
 // apart; with K-major rows that is a separate 128-byte line from L2 for every row and K-block (the tile loads
 // keep sweeping the L1), as many line requests as the tiles themselves need, and the tile loads queue behind
@@ -994,7 +1032,9 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   // Stream-K is an optimisation the workspace enables: without one (or with a small one) whole tiles go round-robin.
   SkPlan sk = plan_stream_k(tiles, g.KB, cus);
   if (grouped != nullptr) sk.use = false;  // ranges of steps would need the tile count on the host
-  const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : 0;
+  TailPlan tp = plan_tail(tiles, g.KB, cus);
+  if (sk.use || grouped != nullptr || mode != kModeBlock) tp.use = false;
+  const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : (tp.use ? (size_t)tp.grid * 2 * kPartialSlotBytes : 0);
   const size_t need = FG_WORKSPACE_COUNTER_BYTES + sk_bytes;
   // workspace: [counters][partial tiles, if the shape is one that shares tiles][transposed activation scales]
   // (a grouped problem's tile count is an upper bound that a few hundred rows spread over many segments inflate:
@@ -1034,6 +1074,25 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     kern = aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true> : fp8_gemm_pingpong_kernel<true, kModeBlock, false>;
   else
     kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeBlock, true> : fp8_gemm_pingpong_kernel<false, kModeBlock, false>;
+  if (tp.use && !a.sk && workspace != nullptr && workspace_bytes >= need && (size_t)tp.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
+      (uintptr_t)workspace % 16 == 0) {
+    PpArgs whole = a;
+    whole.n_tiles = tp.full;
+    whole.stagger = 0;
+    hipLaunchKernelGGL(kern, dim3((uint32_t)cus), dim3(kThreads), kLdsBytes, stream, whole);
+    FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel (whole rounds)");
+    PpArgs rest = a;
+    rest.stagger = 0;
+    rest.n_tiles = tp.tail; rest.tile_base = tp.full;
+    rest.sk = 1; rest.sk_q = tp.cut; rest.sk_r = 0; rest.sk_split = tp.split;
+    rest.counters = reinterpret_cast<unsigned int*>(workspace);
+    rest.partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
+    void (*shared)(PpArgs) = fp8_gemm_pingpong_kernel<true, kModeBlock, false>;
+    if (aligned) shared = fp8_gemm_pingpong_kernel<true, kModeBlock, true>;
+    hipLaunchKernelGGL(shared, dim3((uint32_t)tp.grid), dim3(kThreads), kLdsBytes, stream, rest);
+    FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel (last tiles)");
+    return FG_OK;
+  }
   hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
   FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel");
   return FG_OK;
@@ -1059,7 +1118,8 @@ size_t pingpong_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 64 || K <= 0 || K % 128 != 0) return 0;
   const SkPlan sk = plan_stream_k(ceil_div(M, kBM) * ceil_div(N, kBN), (int)(K / 128), cu_count());
   const int64_t KB = K / 128;
-  const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : 0;
+  const TailPlan tp = plan_tail(ceil_div(M, kBM) * ceil_div(N, kBN), (int)(K / 128), cu_count());
+  const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : (tp.use ? (size_t)tp.grid * 2 * kPartialSlotBytes : 0);
   const size_t tr_bytes = transposition_pays(ceil_div(M, kBM) * ceil_div(N, kBN), KB, cu_count())
                               ? transposed_scales_bytes(M, KB) : 0;  // for row-major scales
   return sk_bytes + tr_bytes != 0 ? FG_WORKSPACE_COUNTER_BYTES + sk_bytes + tr_bytes : 0;

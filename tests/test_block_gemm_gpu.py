@@ -146,6 +146,22 @@ def test_tiles_cut_into_equal_ranges_along_k(M, N, K):
         assert torch.equal(flag_gems.w8a8_block_fp8_matmul(*args), got)
 
 
+@pytest.mark.parametrize("M,N,K", [(2304, 8192, 8192), (2250, 8104, 8192)])
+def test_whole_rounds_then_the_last_tiles_shared(M, N, K):
+    """288 tiles on 256 compute units: one launch computes 256 whole tiles, a second one cuts the other 32 into 4
+    ranges each so that half of the units take part (aligned and ragged shapes).  Against the oracle, bit-identical
+    on reruns."""
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=17)
+    want = O.block_fp8_matmul_tiled_ref(xq, wq, xs, ws, [128, 128], torch.float32)
+    args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    got = flag_gems.w8a8_block_fp8_matmul(*args)
+    torch.testing.assert_close(got.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    err = (got.cpu().double() - want.double()).abs()
+    assert float((err / (want.double().abs() / 128 + 2e-3)).max()) < 1.0
+    for _ in range(2):
+        assert torch.equal(flag_gems.w8a8_block_fp8_matmul(*args), got)
+
+
 @pytest.mark.parametrize("M,N,K", [(1100, 1300, 8192), (1200, 3000, 4096)])
 def test_activation_scales_in_either_layout_give_the_same_bits(M, N, K):
     """The persistent kernel reads activation scales K-block by K-block for 64 rows at a time.  Row-major
