@@ -94,7 +94,8 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
   // slab of 8 rows x 128 bytes, lane L landing at byte 16 L of the slab, i.e. row L >> 3, physical chunk L & 7; the
   // lane therefore fetches logical chunk (L & 7) ^ (row & 7) of its row.  Wavefront w takes the slabs w, w + WAVES, ...
   {
-    constexpr int kPer = 2 * TMX / WAVES;  // slabs per wavefront and K-block
+    constexpr int kSlabs = 2 * TMX;                          // per K-block
+    constexpr int kPer = (kSlabs + WAVES - 1) / WAVES;       // slabs per wavefront and K-block (some wavefronts none)
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
     uint32_t xoff[kPer];
 #pragma unroll
@@ -107,14 +108,16 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
     for (int kb = 0; kb < kbs; ++kb) {
 #pragma unroll
       for (int i = 0; i < kPer; ++i) {
-        const uint8_t* const src = xbase + (int64_t)kb * 128;
-        const uint32_t dst = lds_base + (uint32_t)(kb * kMidStageBytes + (wave + i * WAVES) * 1024);
-        asm volatile("s_mov_b32 m0, %2\n\t"
-                     "s_nop 0\n\t"
-                     "global_load_lds_dwordx4 %0, %1"
-                     :
-                     : "v"(xoff[i]), "s"(src), "s"(dst)
-                     : "memory", "m0");
+        if (wave + i * WAVES < kSlabs) {  // uniform over the wavefront
+          const uint8_t* const src = xbase + (int64_t)kb * 128;
+          const uint32_t dst = lds_base + (uint32_t)(kb * kMidStageBytes + (wave + i * WAVES) * 1024);
+          asm volatile("s_mov_b32 m0, %2\n\t"
+                       "s_nop 0\n\t"
+                       "global_load_lds_dwordx4 %0, %1"
+                       :
+                       : "v"(xoff[i]), "s"(src), "s"(dst)
+                       : "memory", "m0");
+        }
       }
     }
   }
@@ -276,6 +279,8 @@ int launch_mid(const MidArgs& ma, int mode, hipStream_t stream) {
 
 MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K) {
   MidMPlan p = {};
+  // (16- and 32-row variants of this kernel were measured against the decode kernels: slower on every shape for
+  // M <= 16, mixed for 17..32 -- 8192 x 8192: 25.9 -> 20.7 us, but 7168 x 16384 at M = 24: 33.5 -> 47 us -- so those M stay there)
   if (M <= 32 || M > 128 || N < 1 || K < 128 || K % 128 != 0) return p;
   const int64_t KB = K / 128;
   const int tmx = M <= 64 ? 4 : 8;
