@@ -283,6 +283,25 @@ def main():
              "frac_hbm": round(fused_gbs / PEAK_HBM_GBPS, 4), "two_kernels_us": round(apart_us, 2)}
     del gu
 
+    # ---- RMSNorm fused into the quantizer (HBM bound): bf16 [4096, 7168] -> e4m3fn codes + 1x128 scales, with and
+    # without the residual add; algorithmic bytes per element: 2 read + 1 written (+ 4 / 128 of scales), and another
+    # 2 read + 2 written for the residual
+    hx = torch.randn(4096, 7168, device=dev, generator=gen).bfloat16()
+    hr = torch.randn(4096, 7168, device=dev, generator=gen).bfloat16()
+    hw = torch.ones(7168, device=dev, dtype=torch.bfloat16)
+    norm_us = time_calls(lambda: flag_gems.rms_norm_per_token_group_quant_fp8(hx, hw, 128, eps=1e-6), 50)
+    norm_apart_us = time_calls(lambda: flag_gems.per_token_group_quant_fp8(flag_gems.rms_norm(hx, (7168,), hw, 1e-6), 128), 50)
+    hr.zero_()  # the residual accumulates x at every call: keep it finite
+    add_us = time_calls(lambda: flag_gems.rms_norm_per_token_group_quant_fp8(hx, hw, 128, eps=1e-6, residual=hr.zero_()), 50)
+    zero_us = time_calls(lambda: hr.zero_(), 50)
+    norm_gbs = (3.0 + 4.0 / 128) * 4096 * 7168 / (norm_us * 1e-6) / 1e9
+    add_gbs = (7.0 + 4.0 / 128) * 4096 * 7168 / ((add_us - zero_us) * 1e-6) / 1e9
+    norm_quant = {"shape": [4096, 7168], "us": round(norm_us, 2), "gbps": round(norm_gbs, 1),
+                  "frac_hbm": round(norm_gbs / PEAK_HBM_GBPS, 4), "two_kernels_us": round(norm_apart_us, 2),
+                  "with_residual_us": round(add_us - zero_us, 2), "with_residual_gbps": round(add_gbs, 1),
+                  "with_residual_frac_hbm": round(add_gbs / PEAK_HBM_GBPS, 4)}
+    del hx, hr, hw
+
     # ---- the other configurations of the path, each shape timed alone: HIP events around the replay of a graph
     # of `reps` launches (as above: decode-sized launches are shorter than a Python call)
     def time_eager(fn, reps):
@@ -409,6 +428,7 @@ def main():
         "quantizer": quant,
         "weight_quantizer_128x128": weight_quant,
         "silu_mul_quantizer": fused,
+        "rms_norm_quantizer": norm_quant,
         "cutlass_scaled_mm_n8192_k8192_bias": scaled,
         "llama3_8b_linears": llama,
         "mixtral_moe_grouped_gemm": moe,

@@ -51,6 +51,12 @@ SIGNATURES = {
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64,
          c_int64, c_float, c_float, c_float, c_float, c_int, c_int, c_int, c_void_p],
     ),
+    "fg_rms_norm_group_quant_fp8": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int64,
+         c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64,
+         c_int64, c_float, c_float, c_float, c_float, c_int, c_int, c_int, c_void_p],
+    ),
     "fg_silu_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p]),
     "fg_act_quant_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "fg_block_fp8_gemm": (

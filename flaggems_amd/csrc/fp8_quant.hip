@@ -10,175 +10,11 @@
 // codes and scales are bit-identical to the torch reference implementations:
 //   tests/test_act_quant.py:48-98 and tests/test_per_token_group_quant_fp8.py:23-48 of the reference.
 
-#include "fg_common.h"
+#include "fp8_quant_device.h"
 
 namespace fg {
 namespace {
 
-struct QuantArgs {
-  const void* x;
-  uint8_t* q;
-  float* s;
-  int64_t x_row_stride, q_row_stride, s_row_stride, s_col_stride;
-  uint32_t groups_per_row;
-  uint32_t total_groups;
-  uint32_t group_size;
-  float floor, lo, hi, inv_max;
-  int scale_rule, quotient_rule, pow2_rule, e5m2;
-  int64_t up_offset;  // fused SiLU-and-mul producer: elements from a gate value to its up value (same row)
-};
-
-template <int XDT> struct Elem;
-template <> struct Elem<FG_BF16> {
-  using raw = uint16_t;
-  static constexpr uint32_t kAbs = 0x7FFFu, kInf = 0x7F80u;
-  __device__ static float widen(uint32_t b) { return bits_to_float(b << 16); }
-  // two values -> two bf16 in one word, round to nearest even (one v_cvt_pk_bf16_f32; NaN stays NaN)
-  __device__ static uint32_t narrow2(float lo, float hi) {
-    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-    typedef float f32x2 __attribute__((ext_vector_type(2)));
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
-  }
-};
-template <> struct Elem<FG_F16> {
-  using raw = uint16_t;
-  static constexpr uint32_t kAbs = 0x7FFFu, kInf = 0x7C00u;
-  __device__ static float widen(uint32_t b) {
-    return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
-  }
-  __device__ static uint32_t narrow2(float lo, float hi) {
-    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
-  }
-};
-template <> struct Elem<FG_F32> {
-  using raw = uint32_t;
-  static constexpr uint32_t kAbs = 0x7FFFFFFFu, kInf = 0x7F800000u;
-  __device__ static float widen(uint32_t b) { return bits_to_float(b); }
-};
-
-// gate * sigmoid(gate) * up in fp32, as the reference's activation kernel computes it
-// (src/flag_gems/fused/fused_moe.py:795-800: x / (1 + exp(-x)) * y), rounded once to the input's type.
-template <int XDT>
-__device__ __forceinline__ float silu_mul_f32(uint32_t gate, uint32_t up) {
-  using E = Elem<XDT>;
-  const float g = E::widen(gate), u = E::widen(up);
-  if constexpr (XDT == FG_F32) return g / (1.0f + expf(-g)) * u;
-  // 16-bit results: the hardware exponential and reciprocal (what the reference's tl.exp and tl.fdiv compile to)
-  // are wrong by a few fp32 steps, thousands of times below the step of the result; the correctly rounded
-  // routines cost more instructions than the rest of the quantizer together and would bind the kernel.
-  return __fdividef(g, 1.0f + __expf(-g)) * u;
-}
-
-// eight gate values and eight up values (raw words as loaded) -> eight activated values in the same packing
-template <int XDT, int WORDS>
-__device__ __forceinline__ void silu_mul_words(uint32_t (&w)[WORDS], const uint32_t (&up)[WORDS]) {
-#pragma unroll
-  for (int i = 0; i < WORDS; ++i) {
-    if constexpr (WORDS == 4) {
-      w[i] = Elem<XDT>::narrow2(silu_mul_f32<XDT>(w[i] & 0xFFFFu, up[i] & 0xFFFFu), silu_mul_f32<XDT>(w[i] >> 16, up[i] >> 16));
-    } else {
-      w[i] = float_to_bits(silu_mul_f32<XDT>(w[i], up[i]));
-    }
-  }
-}
-
-// scale from the group's absolute maximum (already floored), following the requested rules
-__device__ __forceinline__ float derive_scale(float amax, const QuantArgs& a) {
-  float s = (a.scale_rule == FG_SCALE_MUL_INV) ? amax * a.inv_max : amax / a.hi;
-  if (a.pow2_rule == FG_POW2_BITS) {
-    // exponent + (mantissa != 0) re-assembled with 32-bit wrap-around
-    // (reference src/flag_gems/fused/act_quant.py:22-41)
-    uint32_t b = float_to_bits(s);
-    uint32_t e = (b >> 23) & 0xFFu;
-    uint32_t m = b & 0x7FFFFFu;
-    uint32_t l = e - 127u + (m != 0u ? 1u : 0u);
-    s = bits_to_float((l + 127u) << 23);
-  } else if (a.pow2_rule == FG_POW2_BITS_CLAMPED) {
-    // the same on |s| with the exponent field held in [1, 254] (reference tests/test_fp8_einsum.py:63-67)
-    const uint32_t b = float_to_bits(s) & 0x7FFFFFFFu;
-    uint32_t e = (b >> 23) + ((b & 0x7FFFFFu) != 0u ? 1u : 0u);
-    e = e < 1u ? 1u : (e > 254u ? 254u : e);
-    s = bits_to_float(e << 23);
-  } else if (a.pow2_rule == FG_POW2_LOG2) {
-    // exp2(ceil(log2(max(|s|, 1e-10)))) with log2 rounded to fp32 the way a correctly rounded
-    // libm does it (reference src/flag_gems/ops/per_token_group_quant_fp8.py:65-66)
-    float t = fmaxf(fabsf(s), 1e-10f);
-    if (s != s) {
-      // NaN stays NaN
-    } else if (t < __builtin_huge_valf()) {
-      float l = (float)log2((double)t);
-      int k = (int)ceilf(l);
-      s = (k >= -126) ? bits_to_float((uint32_t)(k + 127) << 23) : ldexpf(1.0f, k);
-    } else {
-      s = t;
-    }
-  }
-  return s;
-}
-
-// Whether x / s may be computed as below for every x of a group with scale s: no Inf or NaN in the group, and s
-// far enough from the ends of the exponent range that neither r = 1 / s nor the remainder goes subnormal.
-__device__ __forceinline__ bool short_division_ok(bool special, float s) {
-  return !special && s >= 0x1p-60f && s <= 0x1p100f;
-}
-
-// x / s, correctly rounded, in three operations given the correctly rounded reciprocal r = RN(1 / s)
-// (Markstein's sequence): q0 = RN(x r) is within a step of the quotient, the remainder e = x - q0 s is exact in
-// one fused multiply-add, and RN(q0 + e r) is the correctly rounded quotient.  With s in [2^-60, 2^100] every
-// quotient that can produce a non-zero fp8 code (|y| >= 2^-20) has a normal remainder; below that the last bit may
-// differ from the division instruction sequence's, the code is a zero either way, and its sign is x's.
-// The full sequence (v_div_scale, v_rcp, four fmas, v_div_fmas, v_div_fixup per element) made the quantizer
-// VALU-bound: 115 us against 69 us with a reciprocal multiply on bf16 [8192, 14336].
-__device__ __forceinline__ float short_division(float x, float s, float r) {
-  const float q0 = x * r;
-  const float e = __builtin_fmaf(-q0, s, x);
-  const float q1 = __builtin_fmaf(e, r, q0);
-  return bits_to_float((float_to_bits(q1) & 0x7FFFFFFFu) | (float_to_bits(x) & 0x80000000u));
-}
-
-__device__ __forceinline__ float quantize_value(float x, float s, float r, const QuantArgs& a, bool short_div = false) {
-  float y = (a.quotient_rule == FG_QUOT_RECIP_MUL) ? x * r : (short_div ? short_division(x, s, r) : x / s);
-  // clamp that lets NaN through, as torch.clamp does
-  float c = fminf(fmaxf(y, a.lo), a.hi);
-  return (y != y) ? y : c;
-}
-
-// The reference helpers that round scales with FG_POW2_BITS_CLAMPED cast the quotient without clamping it
-// (tests/test_fp8_einsum.py:70-103), and an e4m3fn cast has no infinity: what lies past the last finite code's
-// rounding interval (|y| > 464) becomes NaN.  Only an infinite input under a scale held at 2^127 gets there, so the
-// callers apply this to groups that hold an Inf or NaN only.
-__device__ __forceinline__ float unclamped_overflow(float x, float s, float r, float y, const QuantArgs& a) {
-  if (a.pow2_rule != FG_POW2_BITS_CLAMPED || a.e5m2) return y;
-  const float raw = (a.quotient_rule == FG_QUOT_RECIP_MUL) ? x * r : x / s;
-  return fabsf(raw) > 464.0f ? bits_to_float(0x7FC00000u | (float_to_bits(raw) & 0x80000000u)) : y;
-}
-
-template <bool HI>
-__device__ __forceinline__ uint32_t pack2(float v0, float v1, uint32_t old, int e5m2) {
-  if (e5m2) return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(v0, v1, (int)old, HI);
-  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, (int)old, HI);
-}
-
-// NaN keeps its sign and takes the all-ones magnitude, whatever the converter does with it
-__device__ __forceinline__ uint32_t fix_nan_byte(uint32_t word, int byte, float v, int e5m2) {
-  if (v != v) {
-    uint32_t code = ((float_to_bits(v) >> 24) & 0x80u) | (e5m2 ? 0x7Fu : 0x7Fu);
-    word = (word & ~(0xFFu << (8 * byte))) | (code << (8 * byte));
-  }
-  return word;
-}
-
-template <int LPG>
-__device__ __forceinline__ uint32_t group_max_u32(uint32_t v) {
-  // max over LPG adjacent lanes; every lane ends with the group's value
-  if (LPG >= 2) v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-  if (LPG >= 4) v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
-  if (LPG >= 8) v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x141, 0xF, 0xF, true));  // row_half_mirror
-  if (LPG >= 16) v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x140, 0xF, 0xF, true)); // row_mirror
-  if (LPG >= 32) v = max(v, (uint32_t)__shfl_xor((int)v, 16, 64));
-  if (LPG >= 64) v = max(v, (uint32_t)__shfl_xor((int)v, 32, 64));
-  return v;
-}
 
 constexpr int kQuantThreads = 256;
 // Independent 8-element chunks per thread (UNROLL of the vector kernel), loaded before any is converted.  Measured,
@@ -241,61 +77,10 @@ __global__ __launch_bounds__(kQuantThreads) void group_quant_vec_kernel(QuantArg
 
 #pragma unroll
   for (int u = 0; u < kQuantUnroll; ++u) {
-    // absolute maximum on the raw bit patterns: NaN patterns compare above everything
-    uint32_t m = 0u;
     float xv[8];
-    if constexpr (kWords == 4) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        uint32_t lo = w[u][i] & 0xFFFFu, hi = w[u][i] >> 16;
-        m = max(m, max(lo & E::kAbs, hi & E::kAbs));
-        xv[2 * i] = E::widen(lo);
-        xv[2 * i + 1] = E::widen(hi);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        m = max(m, w[u][i] & E::kAbs);
-        xv[i] = E::widen(w[u][i]);
-      }
-    }
-    m = group_max_u32<LPG>(m);
-    float amax = E::widen(m);
-    const bool special = m >= E::kInf;  // Inf or NaN somewhere in the group
-    if (!(amax != amax)) amax = fmaxf(amax, a.floor);
-    const float s = derive_scale(amax, a);
-    const float r = 1.0f / s;
-
-    // Decided once per wavefront (uniform branches): almost every wavefront holds finite inputs under finite
-    // non-zero scales only, where no quotient can be NaN and a plain clamp finishes the job.
-    const bool plain = __builtin_amdgcn_ballot_w64(special || !(s > 0.0f) || !(s < __builtin_huge_valf())) == 0;
-    float y[8];
-    if (plain) {
-      if (a.quotient_rule == FG_QUOT_RECIP_MUL) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) y[i] = fminf(fmaxf(xv[i] * r, a.lo), a.hi);
-      } else if (__builtin_amdgcn_ballot_w64(!short_division_ok(false, s)) == 0) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) y[i] = fminf(fmaxf(short_division(xv[i], s, r), a.lo), a.hi);
-      } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) y[i] = fminf(fmaxf(xv[i] / s, a.lo), a.hi);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) y[i] = unclamped_overflow(xv[i], s, r, quantize_value(xv[i], s, r, a), a);
-    }
-    uint32_t w0 = pack2<false>(y[0], y[1], 0u, a.e5m2);
-    w0 = pack2<true>(y[2], y[3], w0, a.e5m2);
-    uint32_t w1 = pack2<false>(y[4], y[5], 0u, a.e5m2);
-    w1 = pack2<true>(y[6], y[7], w1, a.e5m2);
-    if (!plain) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        w0 = fix_nan_byte(w0, i, y[i], a.e5m2);
-        w1 = fix_nan_byte(w1, i, y[4 + i], a.e5m2);
-      }
-    }
+    const uint32_t m = group_max_u32<LPG>(widen_chunk<XDT, kWords>(w[u], xv));
+    uint32_t w0, w1;
+    const float s = quantize_chunk<XDT>(xv, m, a, w0, w1);
     if (live[u]) {
       uint32_t c = first + (uint32_t)u * stride;
       uint32_t lig = c % LPG;

@@ -137,6 +137,37 @@ int fg_silu_mul(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t 
                 void* out, int64_t out_row_stride, void* stream);
 
 /*
+ * RMSNorm (optionally preceded by the residual add) fused into the quantizer: every row of x [rows, cols] is
+ * normalised, multiplied by weight [cols] (x's type), rounded to x's type as a separate norm kernel would have
+ * stored it, and quantized exactly as fg_group_quant_fp8 quantizes that stored tensor (same codes and scales, bit
+ * for bit), without writing and re-reading it.
+ *   residual == NULL (src/flag_gems/ops/rms_norm.py:54-66):
+ *       var = sum(x^2) / cols, rrms = 1 / sqrt(var + eps), y = T(T(x * rrms) * weight), T = rounding to x's type;
+ *   residual != NULL, [rows, cols] of x's type, updated in place
+ *   (src/flag_gems/fused/fused_add_rms_norm.py:92-118, the kernel the reference uses for rows over 4096 elements;
+ *   its kernel for shorter rows, lines 42-56, rounds differently and is not followed):
+ *       t = x + residual in fp32, residual <- T(t), var = sum(t^2) / cols over the unrounded t,
+ *       y = T(T(t) * rrms * weight).
+ * All of it in individually rounded fp32 operations; the sum of squares runs per thread over the 8-element chunks
+ * t, t + 256, ... of the row in order, then over lanes at distances 1, 2, 4, 8, 16, 32, then over the four
+ * wavefronts in order (the reference leaves the order to its compiler).
+ * y: NULL, or [rows, cols] that receives the normalised rows (may be x itself: the reference's fused operator
+ * writes into its input).  q and s: both NULL to normalise only, else as in fg_group_quant_fp8 with group_size
+ * 8, 16, 32, 64, 128, 256 or 512.  cols a multiple of 8 and at most 16384; x, residual, weight, y and their rows
+ * 16-byte aligned, q rows 8-byte aligned (FG_ERR_UNSUPPORTED otherwise).
+ * The reference runs the steps apart: rms_norm or fused_add_rms_norm, then the quantizer inside the linear
+ * layer (src/flag_gems/ops/per_token_group_quant_fp8.py:203-297).
+ */
+int fg_rms_norm_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t x_row_stride,
+                                void* residual, int64_t residual_row_stride, const void* weight, float eps,
+                                void* y, int64_t y_row_stride,
+                                void* q, int q_dtype, int64_t q_row_stride,
+                                float* s, int64_t s_row_stride, int64_t s_col_stride,
+                                int64_t group_size, float amax_floor, float fp8_min, float fp8_max,
+                                float inv_fp8_max, int scale_rule, int quotient_rule, int pow2_rule,
+                                void* stream);
+
+/*
  * act_quant with the reference's fixed rules (bf16 in, e4m3fn out, floor 1e-4,
  * scale = amax * fp32(1/448), reciprocal-multiply quotient, power-of-two scale when
  * round_scale != 0), contiguous [rows, cols] input and outputs.

@@ -36,6 +36,12 @@ the checks live in tests/test_oracle_*.py):
   output type apart), by torch.sigmoid (a different formula), and by the special
   cases silu(0) = 0, silu(g) = g for large g, silu(g) = -0 for very negative g and
   silu(g) - silu(-g) = g.
+* rms_norm_ref, fused_add_rms_norm_ref, row_sum_of_squares_f32 -- pinned by a float64
+  evaluation (one or two rounding steps of the output type apart), by
+  torch.nn.functional.rms_norm on fp32 inputs, by rows of small integers (whose sum of
+  squares is exact in any order, so a dropped or repeated element shows), by rows of
+  one repeated value (closed form), and by the exact invariance under scaling x by a
+  power of two with eps = 0.
 * scaled_mm_ref, scaled_mm_ref_postscale -- pinned against each other, a float64
   loop, and the unit-scale/zero-bias closed form.
 
@@ -149,6 +155,67 @@ def silu_and_mul_ref(x: torch.Tensor) -> torch.Tensor:
     g = x[..., :d].to(torch.float32)
     u = x[..., d:].to(torch.float32)
     return (g / (1.0 + torch.exp(-g)) * u).to(x.dtype)
+
+
+def row_sum_of_squares_f32(t: torch.Tensor) -> torch.Tensor:
+    """Sum of squares of every row of a float32 [rows, cols] tensor (cols a multiple of 8) in fp32, every
+    multiply and add rounded on its own, in the order the HIP library documents for its RMSNorm kernel
+    (the reference leaves the order to its compiler, src/flag_gems/ops/rms_norm.py:64): 256 accumulators
+    take the 8-element chunks t, t + 256, ... of the row element by element; accumulators 64 k .. 64 k + 63
+    are folded with a butterfly at distances 1, 2, 4, 8, 16, 32; the four results are added in order."""
+    assert t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] % 8 == 0
+    rows, cols = t.shape
+    per = -(-(cols // 8) // 256)
+    padded = torch.zeros((rows, per * 2048), dtype=torch.float32)
+    padded[:, :cols] = t
+    v = padded.view(rows, per, 256, 8)
+    acc = torch.zeros((rows, 256), dtype=torch.float32)
+    for i in range(per):
+        for e in range(8):
+            sq = v[:, i, :, e] * v[:, i, :, e]
+            acc = acc + sq
+    acc = acc.view(rows, 4, 64)
+    lanes = torch.arange(64)
+    for mask in (1, 2, 4, 8, 16, 32):
+        acc = acc + acc[:, :, lanes ^ mask]
+    w = acc[:, :, 0]
+    return ((w[:, 0] + w[:, 1]) + w[:, 2]) + w[:, 3]
+
+
+def _inverse_rms(t: torch.Tensor, eps: float) -> torch.Tensor:
+    """``1 / sqrt(sum / N + eps)`` with every operation correctly rounded to fp32.  Division, square root and
+    reciprocal go through float64 and are rounded once more (for these three operations on fp32 operands that
+    second rounding cannot change the result: 53 >= 2 * 24 + 2 bits): the vectorised fp32 reciprocal of some
+    hosts is an approximation, one or two steps off, which would make this oracle depend on the machine."""
+    var = (row_sum_of_squares_f32(t).double() / float(t.shape[1])).float()
+    shifted = var + torch.tensor(eps, dtype=torch.float32)
+    root = torch.sqrt(shifted.double()).float()
+    return (1.0 / root.double()).float()
+
+
+def rms_norm_ref(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5) -> torch.Tensor:
+    """RMSNorm over the last dimension of a 2-D x as the reference's kernel computes it
+    (src/flag_gems/ops/rms_norm.py:54-66): fp32 throughout, ``var = sum(x^2) / N``,
+    ``rrms = 1 / sqrt(var + eps)``, the normalised value rounded to x's dtype *before* the multiplication
+    by the weight, the product rounded again."""
+    xf = x.to(torch.float32)
+    x_normed = (xf * _inverse_rms(xf, eps)[:, None]).to(x.dtype)
+    return (x_normed.to(torch.float32) * weight.to(torch.float32)).to(x.dtype)
+
+
+def fused_add_rms_norm_ref(
+    x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Residual add + RMSNorm as the reference's looped kernel computes it
+    (src/flag_gems/fused/fused_add_rms_norm.py:92-118; the reference uses it for rows over 4096 elements, and its
+    single-pass kernel for shorter rows, lines 42-56, rounds differently): ``t = x + residual`` in fp32, the
+    new residual is t rounded to the dtype, the variance is ``sum(t^2) / N`` of the *unrounded* t, the
+    second pass reads the rounded t back: ``y = T(t) * rrms * w`` rounded once.
+    Returns (y, new_residual); the reference writes them over x and residual."""
+    t = x.to(torch.float32) + residual.to(torch.float32)
+    stored = t.to(x.dtype)
+    y = ((stored.to(torch.float32) * _inverse_rms(t, eps)[:, None]) * weight.to(torch.float32)).to(x.dtype)
+    return y, stored
 
 
 # --------------------------------------------------------------------------------------
