@@ -176,6 +176,9 @@ __device__ __forceinline__ uint32_t group_max_u32(uint32_t v) {
   return v;
 }
 
+// clamp of a value that is not NaN, in one instruction (the median of the three)
+__device__ __forceinline__ float clamp_finite(float v, float lo, float hi) { return __builtin_amdgcn_fmed3f(v, lo, hi); }
+
 // A lane's eight values (raw words as loaded) widened to fp32; returns the largest absolute bit pattern among them
 // (NaN patterns compare above everything).
 template <int XDT, int WORDS>
@@ -214,18 +217,20 @@ __device__ __forceinline__ float quantize_chunk(const float (&xv)[8], uint32_t m
 
   // Decided once per wavefront (uniform branches): almost every wavefront holds finite inputs under finite
   // non-zero scales only, where no quotient can be NaN and a plain clamp finishes the job.
-  const bool plain = __builtin_amdgcn_ballot_w64(special || !(s > 0.0f) || !(s < __builtin_huge_valf())) == 0;
+  // (a scale so small that its reciprocal overflows makes 0 * inf = NaN under the reciprocal rule: not plain either)
+  const bool plain = __builtin_amdgcn_ballot_w64(special || !(s > 0.0f) || !(s < __builtin_huge_valf()) ||
+                                                 !(r < __builtin_huge_valf())) == 0;
   float y[8];
   if (plain) {
     if (a.quotient_rule == FG_QUOT_RECIP_MUL) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) y[i] = fminf(fmaxf(xv[i] * r, a.lo), a.hi);
+      for (int i = 0; i < 8; ++i) y[i] = clamp_finite(xv[i] * r, a.lo, a.hi);
     } else if (__builtin_amdgcn_ballot_w64(!short_division_ok(false, s)) == 0) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) y[i] = fminf(fmaxf(short_division(xv[i], s, r), a.lo), a.hi);
+      for (int i = 0; i < 8; ++i) y[i] = clamp_finite(short_division(xv[i], s, r), a.lo, a.hi);
     } else {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) y[i] = fminf(fmaxf(xv[i] / s, a.lo), a.hi);
+      for (int i = 0; i < 8; ++i) y[i] = clamp_finite(xv[i] / s, a.lo, a.hi);
     }
   } else {
 #pragma unroll

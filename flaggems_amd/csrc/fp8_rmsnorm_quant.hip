@@ -80,6 +80,11 @@ __device__ __forceinline__ void narrow_chunk(const float (&v)[8], uint32_t (&w)[
   }
 }
 
+// Measured on bf16 [4096, 7168]: 25 us for the norm alone (4.7 TB/s), 36 us with the quantizer (the quantizer alone:
+// 18 us): with both in one kernel the vector ALU is the limit, not memory.  A variant with as many workgroups as stay
+// resident, each loading its next row (raw words) before working on the current one, was measured and not kept: the
+// norm alone went to 22.5 us, the fused call stayed at 37 us, and rows of 16384 elements got slower (150 us against
+// 101) because the second row in registers left one wavefront per SIMD.
 template <int XDT, int CHUNKS>
 __global__ __launch_bounds__(kNormThreads) void rms_norm_quant_kernel(NormQuantArgs a) {
   using E = Elem<XDT>;
