@@ -83,6 +83,11 @@ SIGNATURES = {
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
          c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p],
     ),
+    "fg_scaled_gemm": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+         c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p],
+    ),
     "fg_scaled_int8_gemm": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,

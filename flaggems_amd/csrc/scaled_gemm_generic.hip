@@ -1,0 +1,199 @@
+// aten::_scaled_mm for operands that are not quantized (bf16, fp16, fp32) on gfx950:
+//     C[m, n] = cast( (sum_k A[m, k] * B[n, k]) * a_scale[m or 0] * b_scale[n or 0] + bias[n] )
+// with the sum, the scales and the bias in fp32 and one rounding at the end, which is what the reference's generic
+// kernel computes (src/flag_gems/ops/scaled_mm.py:77-133: tl.dot with an fp32 accumulator and allow_tf32 = False,
+// acc * scale_a * scale_b, + bias, store).
+//
+// The quantized operand types have tuned kernels of their own; this one keeps the operator on the GPU for the
+// other types.  A workgroup of four wavefronts computes a 128 x 128 tile of C, each wavefront a 64 x 64 quarter as
+// 4 x 4 MFMA tiles (v_mfma_f32_16x16x32_bf16 / _f16, v_mfma_f32_16x16x4_f32).  Both operands are K-contiguous rows,
+// and an MFMA operand is "row (lane % 16), eight consecutive k at 8 (lane / 16)": one 16-byte load per lane and
+// tile straight from global memory, no LDS; the next K step's operands are loaded before the current step's
+// MFMAs.  The two wavefronts that share a row or column panel meet in the L1/L2 caches.
+
+#include "fg_common.h"
+
+namespace fg {
+namespace {
+
+constexpr int kGenThreads = 256;
+constexpr int kGenTile = 128;    // rows and columns of C per workgroup
+constexpr int kGenWaveTile = 64; // per wavefront
+constexpr int kGenFrags = kGenWaveTile / 16;
+
+struct GenericArgs {
+  const void* A;
+  const void* B;
+  int64_t lda, ldb, ldc;  // elements
+  const float* a_scale;
+  const float* b_scale;
+  int a_per_row, b_per_col;
+  const void* bias;
+  int bias_dtype;
+  void* C;
+  int c_dtype;
+  int M, N, K;
+  int tiles_n;
+};
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+template <int DT> struct GenElem;
+template <> struct GenElem<FG_BF16> {
+  static constexpr int kBytes = 2, kStep = 32;  // K per 16-byte load round: 4 lane groups x 8 elements
+  __device__ static v4f mma(u32x4 a, u32x4 b, v4f c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct GenElem<FG_F16> {
+  static constexpr int kBytes = 2, kStep = 32;
+  __device__ static v4f mma(u32x4 a, u32x4 b, v4f c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct GenElem<FG_F32> {
+  static constexpr int kBytes = 4, kStep = 16;  // 4 lane groups x 4 elements; element j of every lane feeds MFMA j
+  __device__ static v4f mma(u32x4 a, u32x4 b, v4f c) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) c = __builtin_amdgcn_mfma_f32_16x16x4f32(bits_to_float(a[j]), bits_to_float(b[j]), c, 0, 0, 0);
+    return c;
+  }
+};
+
+__device__ __forceinline__ float load_scalar_as_float(const void* p, int64_t i, int dtype) {
+  if (dtype == FG_F32) return reinterpret_cast<const float*>(p)[i];
+  if (dtype == FG_F16) return (float)reinterpret_cast<const _Float16*>(p)[i];
+  return bits_to_float((uint32_t)reinterpret_cast<const uint16_t*>(p)[i] << 16);
+}
+
+__device__ __forceinline__ void store_rounded(void* C, int64_t off, float v, int dtype) {
+  if (dtype == FG_F32) {
+    reinterpret_cast<float*>(C)[off] = v;
+  } else if (dtype == FG_F16) {
+    reinterpret_cast<_Float16*>(C)[off] = (_Float16)v;
+  } else {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{v, 0.0f}, bf16x2));
+    reinterpret_cast<uint16_t*>(C)[off] = (uint16_t)(w & 0xFFFFu);
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kGenThreads) void scaled_gemm_generic_kernel(GenericArgs a) {
+  using E = GenElem<DT>;
+  constexpr int kPerLane = 16 / E::kBytes;  // elements of one 16-byte load
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile_m = blockIdx.x / a.tiles_n, tile_n = blockIdx.x - tile_m * a.tiles_n;
+  const int m0 = tile_m * kGenTile + (wave >> 1) * kGenWaveTile;
+  const int n0 = tile_n * kGenTile + (wave & 1) * kGenWaveTile;
+  // a wavefront whose quarter lies outside C has nothing to do (there is no barrier in this kernel)
+  if (m0 >= a.M || n0 >= a.N) return;
+
+  const int r = lane & 15, kq = (lane >> 4) * kPerLane;
+  // rows past the edge read the last valid row (their results are not stored)
+  const char* ap[kGenFrags];
+  const char* bp[kGenFrags];
+#pragma unroll
+  for (int f = 0; f < kGenFrags; ++f) {
+    const int am = min(m0 + 16 * f + r, a.M - 1), bn = min(n0 + 16 * f + r, a.N - 1);
+    ap[f] = reinterpret_cast<const char*>(a.A) + ((int64_t)am * a.lda + kq) * E::kBytes;
+    bp[f] = reinterpret_cast<const char*>(a.B) + ((int64_t)bn * a.ldb + kq) * E::kBytes;
+  }
+
+  v4f acc[kGenFrags][kGenFrags];
+#pragma unroll
+  for (int i = 0; i < kGenFrags; ++i)
+#pragma unroll
+    for (int j = 0; j < kGenFrags; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  u32x4 fa[kGenFrags], fb[kGenFrags], na[kGenFrags], nb[kGenFrags];
+  // K is a multiple of the elements per load, so a lane's load lies wholly inside or wholly outside the row
+  auto load_step = [&](int k, u32x4 (&xa)[kGenFrags], u32x4 (&xb)[kGenFrags]) {
+    const bool inside = k + kq < a.K;
+#pragma unroll
+    for (int f = 0; f < kGenFrags; ++f) {
+      xa[f] = inside ? *reinterpret_cast<const u32x4*>(ap[f] + (int64_t)k * E::kBytes) : zero;
+      xb[f] = inside ? *reinterpret_cast<const u32x4*>(bp[f] + (int64_t)k * E::kBytes) : zero;
+    }
+  };
+
+  load_step(0, fa, fb);
+  for (int k = 0; k < a.K; k += E::kStep) {
+    const bool more = k + E::kStep < a.K;  // uniform
+    if (more) load_step(k + E::kStep, na, nb);
+#pragma unroll
+    for (int i = 0; i < kGenFrags; ++i)
+#pragma unroll
+      for (int j = 0; j < kGenFrags; ++j) acc[i][j] = E::mma(fa[i], fb[j], acc[i][j]);
+    if (more) {
+#pragma unroll
+      for (int f = 0; f < kGenFrags; ++f) { fa[f] = na[f]; fb[f] = nb[f]; }
+    }
+  }
+
+  // lane holds C[16 i + 4 (lane / 16) + e][16 j + lane % 16], e < 4
+  const int crow = (lane >> 4) * 4, ccol = lane & 15;
+#pragma unroll
+  for (int j = 0; j < kGenFrags; ++j) {
+    const int n = n0 + 16 * j + ccol;
+    if (n >= a.N) continue;
+    const float sb = a.b_scale[a.b_per_col ? n : 0];
+    const float bias = a.bias ? load_scalar_as_float(a.bias, n, a.bias_dtype) : 0.0f;
+#pragma unroll
+    for (int i = 0; i < kGenFrags; ++i) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int m = m0 + 16 * i + crow + e;
+        if (m >= a.M) continue;
+        float v = (acc[i][j][e] * a.a_scale[a.a_per_row ? m : 0]) * sb;
+        if (a.bias) v = v + bias;
+        store_rounded(a.C, (int64_t)m * a.ldc + n, v, a.c_dtype);
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace fg
+
+extern "C" int fg_scaled_gemm(const void* A, int64_t lda, const void* B, int64_t ldb, int ab_dtype,
+                              const float* a_scale, int a_scale_per_row,
+                              const float* b_scale, int b_scale_per_col,
+                              const void* bias, int bias_dtype,
+                              void* C, int64_t ldc, int c_dtype,
+                              int64_t M, int64_t N, int64_t K, void* stream) {
+  using namespace fg;
+  const char* me = "fg_scaled_gemm";
+  if (M < 0 || N < 0 || K < 0) FG_FAIL(FG_ERR_INVALID_ARG, "%s: negative size", me);
+  if (M == 0 || N == 0) return FG_OK;
+  if (!A || !B || !C || !a_scale || !b_scale) FG_FAIL(FG_ERR_INVALID_ARG, "%s: null pointer", me);
+  if (ab_dtype != FG_BF16 && ab_dtype != FG_F16 && ab_dtype != FG_F32) FG_FAIL(FG_ERR_INVALID_ARG, "%s: operand dtype %d", me, ab_dtype);
+  if (c_dtype != FG_BF16 && c_dtype != FG_F16 && c_dtype != FG_F32) FG_FAIL(FG_ERR_UNSUPPORTED, "%s: output dtype %d", me, c_dtype);
+  if (bias && bias_dtype != FG_BF16 && bias_dtype != FG_F16 && bias_dtype != FG_F32)
+    FG_FAIL(FG_ERR_INVALID_ARG, "%s: bias dtype %d", me, bias_dtype);
+  if (lda < K || ldb < K || ldc < N) FG_FAIL(FG_ERR_INVALID_ARG, "%s: row stride smaller than the row", me);
+  if (M > 0x3FFFFFFF || N > 0x3FFFFFFF || K > 0x3FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "%s: dimension above 2^30", me);
+  const int64_t esz = ab_dtype == FG_F32 ? 4 : 2, per_load = 16 / esz;
+  if (K % per_load != 0 || (uintptr_t)A % 16 != 0 || (uintptr_t)B % 16 != 0 || (lda * esz) % 16 != 0 || (ldb * esz) % 16 != 0)
+    FG_FAIL(FG_ERR_UNSUPPORTED, "%s: K must be a multiple of %lld and operand rows 16-byte aligned", me, (long long)per_load);
+  const int64_t tiles_m = ceil_div(M, kGenTile), tiles_n = ceil_div(N, kGenTile);
+  if (tiles_m * tiles_n > 0x7FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "%s: too many tiles", me);
+
+  GenericArgs g;
+  g.A = A; g.B = B; g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+  g.a_scale = a_scale; g.b_scale = b_scale;
+  g.a_per_row = a_scale_per_row != 0; g.b_per_col = b_scale_per_col != 0;
+  g.bias = bias; g.bias_dtype = bias_dtype;
+  g.C = C; g.c_dtype = c_dtype;
+  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  g.tiles_n = (int)tiles_n;
+  const dim3 grid((uint32_t)(tiles_m * tiles_n)), block(kGenThreads);
+  if (ab_dtype == FG_BF16) hipLaunchKernelGGL(scaled_gemm_generic_kernel<FG_BF16>, grid, block, 0, (hipStream_t)stream, g);
+  else if (ab_dtype == FG_F16) hipLaunchKernelGGL(scaled_gemm_generic_kernel<FG_F16>, grid, block, 0, (hipStream_t)stream, g);
+  else hipLaunchKernelGGL(scaled_gemm_generic_kernel<FG_F32>, grid, block, 0, (hipStream_t)stream, g);
+  FG_CHECK_LAUNCH("scaled_gemm_generic_kernel");
+  return FG_OK;
+}

@@ -73,6 +73,27 @@ def _launch_scaled_int8_gemm(c, a, b, a_scale, b_scale, bias) -> None:
     _lib.check(status, "fg_scaled_int8_gemm")
 
 
+def _launch_scaled_generic_gemm(c, a, b, a_scale, b_scale, bias) -> None:
+    """bf16 / fp16 / fp32 operands: a [M, K] with unit column stride, b [K, N] with unit row stride (column-major)."""
+    _lib.require_gpu(a, "scaled gemm")
+    lib = _lib.load()
+    m, k = a.shape
+    n = b.shape[1]
+    dev = a.device
+    with torch.cuda.device(dev):
+        status = lib.fg_scaled_gemm(
+            a.data_ptr(), a.stride(0) if m > 1 else max(k, a.stride(0)),
+            b.data_ptr(), b.stride(1) if n > 1 else max(k, b.stride(1)), _lib.DTYPE_CODE[a.dtype],
+            a_scale.data_ptr(), 1 if a_scale.numel() > 1 or m == 1 else 0,
+            b_scale.data_ptr(), 1 if b_scale.numel() > 1 or n == 1 else 0,
+            bias.data_ptr() if bias is not None else None,
+            _lib.DTYPE_CODE[bias.dtype] if bias is not None else _lib.FG_BF16,
+            c.data_ptr(), c.stride(0) if m > 1 else max(n, c.stride(0)), _lib.DTYPE_CODE[c.dtype],
+            m, n, k, _lib.current_stream_ptr(dev),
+        )
+    _lib.check(status, "fg_scaled_gemm")
+
+
 def dispatch_scaled_mm(c, a, b, a_scale, b_scale, bias) -> None:
     assert a_scale.dtype == torch.float32, "a_scale must be float32"
     assert b_scale.dtype == torch.float32, "b_scale must be float32"

@@ -289,6 +289,24 @@ int fg_scaled_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
 size_t fg_scaled_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
+ * The same operator for operands that are not quantized (aten::_scaled_mm on bf16, fp16 or fp32 matrices):
+ *     C[m, n] = cast( (sum_k A[m,k] * B[n,k]) * a_scale[m or 0] * b_scale[n or 0] + bias[n] )
+ * with the sum, the scaling and the bias in fp32 and one rounding to c_dtype at the end (here the bias is added
+ * BEFORE the rounding: that is what the reference's generic kernel does, unlike its cutlass path above).
+ * A: [M, K] rows lda elements apart; B: N rows of K contiguous elements, ldb apart (the column-major [K, N] operand);
+ * both of ab_dtype in {FG_BF16, FG_F16, FG_F32}.  c_dtype and bias_dtype in {FG_BF16, FG_F16, FG_F32}; bias may be
+ * null.  K a multiple of 8 (bf16, fp16) or 4 (fp32) and operand rows 16-byte aligned, else FG_ERR_UNSUPPORTED (the
+ * host pads or copies).  No workspace.
+ * Stands in for scaled_mm_kernel (src/flag_gems/ops/scaled_mm.py:37-133, launched from :365-422).
+ */
+int fg_scaled_gemm(const void* A, int64_t lda, const void* B, int64_t ldb, int ab_dtype,
+                   const float* a_scale, int a_scale_per_row,
+                   const float* b_scale, int b_scale_per_col,
+                   const void* bias, int bias_dtype,
+                   void* C, int64_t ldc, int c_dtype,
+                   int64_t M, int64_t N, int64_t K, void* stream);
+
+/*
  * The same with int8 operands: C[m, n] = float(sum_k A[m,k] * B[n,k] in int32) * a_scale[m or 0] * b_scale[n or 0],
  * rounded to c_dtype (FG_BF16, FG_F16 or FG_F32), then + bias[n] in c_dtype.  A: int8 [M, K] rows lda apart,
  * B: int8 [N, K] rows ldb apart (the column-major [K, N] operand of the reference).  Served by the tile kernel at
