@@ -344,6 +344,20 @@ def main():
                        "gbps": round(nbytes / us / 1e3, 1)})
     del b_q, a_q, c
 
+    # aten::_scaled_mm on operands that are not quantized (the generic kernel): per-row x per-column scales, N = K = 4096
+    generic = []
+    for dt, peak in ((torch.bfloat16, 2500.0), (torch.float16, 2500.0), (torch.float32, 157.3)):
+        gb = torch.randn(4096, 4096, device=dev, generator=gen).to(dt).t()
+        g_sb = torch.rand(1, 4096, device=dev, generator=gen) + 0.5
+        for m in (64, 4096):
+            ga = torch.randn(m, 4096, device=dev, generator=gen).to(dt)
+            g_sa = torch.rand(m, 1, device=dev, generator=gen) + 0.5
+            us = time_eager(lambda: flag_gems.scaled_mm(ga, gb, g_sa, g_sb), 10)
+            tf = gemm_flops(m, 4096, 4096) / us / 1e6
+            generic.append({"dtype": str(dt)[6:], "M": m, "N": 4096, "K": 4096, "us": round(us, 2), "tflops": round(tf, 1),
+                            "frac_mfma": round(tf / peak, 4)})
+        del ga, gb
+
     # Llama-3-8B linears: GEMM alone and act_quant + GEMM from bf16 activations
     llama = []
     for (n, k) in [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]:
@@ -430,6 +444,7 @@ def main():
         "silu_mul_quantizer": fused,
         "rms_norm_quantizer": norm_quant,
         "cutlass_scaled_mm_n8192_k8192_bias": scaled,
+        "scaled_mm_unquantized_operands": generic,
         "llama3_8b_linears": llama,
         "mixtral_moe_grouped_gemm": moe,
         "cpu_baseline": cpu,
