@@ -27,6 +27,10 @@ struct GemmArgs {
   int splits, kb_per_split;
   float* split_partials;
   unsigned int* split_counters;
+  // tile kernel over a batch of equal problems in one launch: blockIdx.y is the batch entry, whose operands lie
+  // these many bytes (X, W, C) or floats (xs, ws) after the previous entry's; batch <= 1: one problem
+  int batch;
+  int64_t x_batch_bytes, w_batch_bytes, c_batch_bytes, xs_batch_stride, ws_batch_stride;
 };
 
 // s_waitcnt vmcnt(0) with expcnt/lgkmcnt left at their maxima (gfx9 encoding)
