@@ -217,9 +217,10 @@ size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * Batched block-scaled FP8 GEMM: `batch` independent problems of fg_block_fp8_gemm with the same M, N, K and
  * strides.  Matrix i of each operand starts i * <its batch stride> after matrix 0 (bytes for A and B, floats for
  * the scales, elements of c_dtype for C); row strides are free, so a [b, h, r] activation with h as the batch
- * takes lda = h * r and a_batch_stride = r.  The matrices are launched one after the other on `stream`: the
- * results are, bit for bit, those of `batch` calls of fg_block_fp8_gemm, and the workspace rules are that entry
- * point's (fg_block_fp8_gemm_workspace_bytes(M, N, K); one workspace serves the whole batch).
+ * takes lda = h * r and a_batch_stride = r.  Matrices too small to fill the GPU on their own go out in one launch
+ * (the batch entry in the grid), larger ones one after the other on `stream`; either way the results are, bit for
+ * bit, those of `batch` calls of fg_block_fp8_gemm, and the workspace rules are that entry point's
+ * (fg_block_fp8_gemm_workspace_bytes(M, N, K); one workspace serves the whole batch).
  *
  * Stands in for w8a8_block_fp8_bmm (src/flag_gems/runtime/backend/_nvidia/hopper/ops/w8a8_block_fp8_bmm.py:629-779)
  * and, through it, fp8_einsum("bhr,hdr->bhd") (.../hopper/ops/fp8_einsum.py:22-68).
