@@ -358,6 +358,22 @@ def main():
                             "frac_mfma": round(tf / peak, 4)})
         del ga, gb
 
+    # fp8_einsum("bhr,hdr->bhd") at the first shape group of the reference's benchmark (h = 8, r = 4096, d = 1024)
+    einsum = []
+    eh, er, ed = 8, 4096, 1024
+    ey = torch.randn(eh, ed, er, device=dev, generator=gen).to(torch.float8_e4m3fn)
+    eys = torch.rand(eh, ed // 128, er // 128, device=dev, generator=gen) + 0.5
+    for eb in (1, 128, 4096):
+        ex = torch.randn(eb, eh, er, device=dev, generator=gen).to(torch.float8_e4m3fn)
+        exs = torch.rand(eb, eh, er // 128, device=dev, generator=gen) + 0.5
+        us = time_eager(lambda: flag_gems.fp8_einsum("bhr,hdr->bhd", ex, exs, ey, eys), 10)
+        nbytes = eh * ed * er + eb * eh * er + 2 * eb * eh * ed + 4 * (eh * (ed // 128) * (er // 128) + eb * eh * (er // 128))
+        tf = 2.0 * eb * eh * ed * er / us / 1e6
+        einsum.append({"b": eb, "h": eh, "r": er, "d": ed, "us": round(us, 2), "tflops": round(tf, 1),
+                       "gbps": round(nbytes / us / 1e3, 1), "frac_mfma": round(tf / PEAK_FP8_TFLOPS, 4),
+                       "frac_hbm": round(nbytes / us / 1e3 / PEAK_HBM_GBPS, 4)})
+    del ey, eys, ex, exs
+
     # Llama-3-8B linears: GEMM alone and act_quant + GEMM from bf16 activations
     llama = []
     for (n, k) in [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]:
@@ -445,6 +461,7 @@ def main():
         "rms_norm_quantizer": norm_quant,
         "cutlass_scaled_mm_n8192_k8192_bias": scaled,
         "scaled_mm_unquantized_operands": generic,
+        "fp8_einsum_bhr_hdr": einsum,
         "llama3_8b_linears": llama,
         "mixtral_moe_grouped_gemm": moe,
         "cpu_baseline": cpu,
