@@ -46,8 +46,7 @@ __global__ __launch_bounds__(kQuantThreads) void group_quant_vec_kernel(QuantArg
     uint32_t cc = live[u] ? c : 0u;
     gid[u] = cc / LPG;
     uint32_t lig = cc % LPG;
-    row[u] = gid[u] / a.groups_per_row;
-    gcol[u] = gid[u] - row[u] * a.groups_per_row;
+    row[u] = divide_below_2_24(gid[u], a.groups_per_row, a.inv_groups_per_row, gcol[u]);
     const typename E::raw* p = reinterpret_cast<const typename E::raw*>(a.x) +
                                (int64_t)row[u] * a.x_row_stride + (int64_t)gcol[u] * (LPG * 8) + lig * 8;
     const u32x4* p4 = reinterpret_cast<const u32x4*>(p);
@@ -383,6 +382,7 @@ int group_quant_entry(const void* x, int x_dtype, int64_t rows, int64_t cols, in
     a.pow2_rule = pow2_rule;
     a.e5m2 = (q_dtype == FG_FP8_E5M2);
     a.up_offset = up_offset;
+    a.inv_groups_per_row = nr == 1 ? 0.0f : 1.0f / (float)groups_per_row;  // nr > 1 implies fewer than 2^24 groups in all
     int rc;
     if (x_dtype == FG_BF16) rc = launch_quant<FG_BF16>(a, vec_ok, (hipStream_t)stream, silu);
     else if (x_dtype == FG_F16) rc = launch_quant<FG_F16>(a, vec_ok, (hipStream_t)stream, silu);

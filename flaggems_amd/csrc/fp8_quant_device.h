@@ -18,7 +18,21 @@ struct QuantArgs {
   float floor, lo, hi, inv_max;
   int scale_rule, quotient_rule, pow2_rule, e5m2;
   int64_t up_offset;  // fused SiLU-and-mul producer: elements from a gate value to its up value (same row)
+  float inv_groups_per_row;  // fp32(1 / groups_per_row), or 0 when the launch covers a single row
 };
+
+// n / d for n < 2^24 and 1 <= d < 2^24, given inv = fp32(1 / d): the fp32 product is within one of the quotient
+// ((n / d) 2^-23 < 1 for d >= 2, exact for d = 1), and one step either way from the remainder makes it exact.
+// With inv = 0 and n < d the result is 0 whatever d is.  About ten instructions where the compiler's 32-bit
+// division takes about thirty, once per 8-element chunk.
+__device__ __forceinline__ uint32_t divide_below_2_24(uint32_t n, uint32_t d, float inv, uint32_t& remainder) {
+  uint32_t q = (uint32_t)((float)n * inv);
+  int32_t r = (int32_t)(n - q * d);
+  if (r < 0) { q -= 1u; r += (int32_t)d; }
+  else if ((uint32_t)r >= d) { q += 1u; r -= (int32_t)d; }
+  remainder = (uint32_t)r;
+  return q;
+}
 
 template <int XDT> struct Elem;
 template <> struct Elem<FG_BF16> {

@@ -260,6 +260,7 @@ extern "C" int fg_rms_norm_group_quant_fp8(const void* x, int x_dtype, int64_t r
   a.q.pow2_rule = pow2_rule;
   a.q.e5m2 = (q_dtype == FG_FP8_E5M2);
   a.q.up_offset = 0;
+  a.q.inv_groups_per_row = 0.0f;
   a.lanes_per_group = 1;
   if (q) {
     if (q_dtype != FG_FP8_E4M3FN && q_dtype != FG_FP8_E5M2) FG_FAIL(FG_ERR_INVALID_ARG, "%s: q_dtype %d", me, q_dtype);

@@ -257,3 +257,36 @@ def test_three_operation_division_is_the_correctly_rounded_quotient():
         e = (x.astype(np.float64) - q0.astype(np.float64) * s.astype(np.float64)).astype(np.float32)
         q1 = (q0.astype(np.float64) + e.astype(np.float64) * r.astype(np.float64)).astype(np.float32)
         assert np.array_equal(q1, want)
+
+
+def test_fast_index_division_is_exact():
+    """The quantizer kernel splits a group index n < 2^24 into (row, column) with q = uint(fp32(n) * fp32(1 / d)) and one
+    corrective step from the remainder, instead of a 32-bit division.  Emulated here in numpy against integer
+    division: every d up to 4096 at the n next to multiples of d and at the top of the range, and random (n, d)."""
+    rng = np.random.default_rng(1)
+
+    def fast(n, d):
+        inv = (np.float32(1.0) / d.astype(np.float32)).astype(np.float32)
+        q = (n.astype(np.float32) * inv).astype(np.float32).astype(np.int64)
+        r = n.astype(np.int64) - q * d.astype(np.int64)
+        low, high = r < 0, r >= d
+        q = q - low + (high & ~low)
+        return q, n.astype(np.int64) - q * d.astype(np.int64)
+
+    top = (1 << 24) - 1
+    for d0 in range(1, 4097):
+        mult = (rng.integers(0, top // d0 + 1, 64) * d0).astype(np.int64)
+        n = np.unique(np.clip(np.concatenate([mult - 1, mult, mult + 1, [top, top - 1, 0, d0 - 1]]), 0, top))
+        d = np.full_like(n, d0)
+        q, r = fast(n, d)
+        assert np.array_equal(q, n // d0) and np.array_equal(r, n % d0), d0
+    d = rng.integers(1, 1 << 23, 2_000_000)
+    n = rng.integers(0, 1 << 24, 2_000_000)
+    q, r = fast(n, d)
+    assert np.array_equal(q, n // d) and np.array_equal(r, n % d)
+    # multiples of large divisors, where the product lands next to an integer
+    k = rng.integers(1, 64, 500_000)
+    d = rng.integers(1 << 10, 1 << 18, 500_000)
+    n = np.minimum(k * d + rng.integers(-1, 2, 500_000), top)
+    q, r = fast(n, d)
+    assert np.array_equal(q, n // d) and np.array_equal(r, n % d)
