@@ -94,6 +94,7 @@ SIGNATURES = {
          c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p],
     ),
     "fg_scaled_fp8_gemm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
+    "fg_batched_block_fp8_gemm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
 }
 
 _lib = None

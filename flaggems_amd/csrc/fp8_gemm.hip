@@ -650,6 +650,18 @@ extern "C" int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int6
   return launch_gemm<kModeBlock>(a, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
+extern "C" size_t fg_batched_block_fp8_gemm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K) {
+  size_t need = fg_block_fp8_gemm_workspace_bytes(M, N, K);
+  if (batch > 1 && M >= 1 && M <= 32) {
+    const fg::SmallMPlan plan = fg::plan_small_m(M, N, K, batch);
+    if (plan.use && plan.splits > 1) {
+      const size_t all = FG_WORKSPACE_COUNTER_BYTES + (size_t)batch * (plan.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES);
+      if (all > need) need = all;
+    }
+  }
+  return need;
+}
+
 extern "C" int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_batch_stride,
                                          const void* B, int64_t ldb, int64_t b_batch_stride,
                                          const float* As, int64_t as_row_stride, int64_t as_col_stride, int64_t as_batch_stride,
@@ -685,6 +697,17 @@ extern "C" int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_b
       a.batch = (int)batch;
       a.x_batch_bytes = a_batch_stride; a.w_batch_bytes = b_batch_stride; a.c_batch_bytes = c_batch_stride * (int64_t)c_elem;
       a.xs_batch_stride = as_batch_stride; a.ws_batch_stride = bs_batch_stride;
+      // up to 32 rows: the weight-streaming kernels with the entry in blockIdx.y, when the workspace holds every
+      // entry's partial sums and the counter area every entry's counters; else (and above 32 rows) the tile kernel
+      if (M <= 32) {
+        const SmallMPlan plan = plan_small_m(M, N, K, batch);
+        const size_t per_entry = plan.splits > 1 ? plan.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES : 0;
+        const bool fits = plan.splits == 1 ||
+                          (workspace != nullptr && (uintptr_t)workspace % 16 == 0 &&
+                           workspace_bytes >= FG_WORKSPACE_COUNTER_BYTES + (size_t)batch * per_entry &&
+                           (size_t)batch * plan.n_chunks * sizeof(unsigned int) <= FG_WORKSPACE_COUNTER_BYTES);
+        if (plan.use && fits) return launch_small_m(a, kModeBlock, plan, workspace, workspace_bytes, (hipStream_t)stream);
+      }
       return launch_cfg<128, 128, 2, 2, kModeBlock, true>(a, (hipStream_t)stream);
     }
   }

@@ -130,7 +130,7 @@ struct SmallMPlan {
   int n_chunks;   // ceil(N / (16 * rg))
   size_t workspace_bytes;
 };
-SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K);
+SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries = 1);
 int launch_small_m(const GemmArgs& a, int mode, const SmallMPlan& plan, void* workspace, size_t workspace_bytes,
                    hipStream_t stream);
 

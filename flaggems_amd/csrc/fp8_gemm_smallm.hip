@@ -32,7 +32,22 @@ struct SmallArgs {
   int kpw, splits, n_chunks;
   float* partials;      // [n_chunks][splits][16 * TMX][64]
   unsigned int* counters;
+  int64_t partials_per_entry;  // floats; a batch (g.batch > 1, entry = blockIdx.y) keeps one such array and n_chunks counters per entry
 };
+
+// blockIdx.y-th problem of a batch: operands, partial sums and counters of that entry
+__device__ __forceinline__ void select_batch_entry(SmallArgs& a) {
+  if (a.g.batch > 1) {  // uniform
+    const int64_t z = blockIdx.y;
+    a.g.X += z * a.g.x_batch_bytes;
+    a.g.W += z * a.g.w_batch_bytes;
+    a.g.C = reinterpret_cast<uint8_t*>(a.g.C) + z * a.g.c_batch_bytes;
+    a.g.xs += z * a.g.xs_batch_stride;
+    a.g.ws += z * a.g.ws_batch_stride;
+    if (a.partials) a.partials += z * a.partials_per_entry;
+    if (a.counters) a.counters += z * a.n_chunks;
+  }
+}
 
 __device__ __forceinline__ v8i join(u32x4 lo, u32x4 hi) {
   v8i f;
@@ -163,6 +178,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_smallm_kernel(SmallArgs a
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  select_batch_entry(a);
   const int chunk = blockIdx.x % a.n_chunks;
   const int split = blockIdx.x / a.n_chunks;
   const int n0 = chunk * kChunkRows;
@@ -243,6 +259,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  select_batch_entry(a);
   const int chunk = blockIdx.x % a.n_chunks;
   const int split = blockIdx.x / a.n_chunks;
   const int n0 = chunk * kRows;
@@ -364,7 +381,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
 
 template <int TMX, int WAVES>
 int launch_t(const SmallArgs& sa, int mode, hipStream_t stream) {
-  const dim3 grid((uint32_t)(sa.n_chunks * sa.splits)), block(WAVES * 64);
+  const dim3 grid((uint32_t)(sa.n_chunks * sa.splits), (uint32_t)(sa.g.batch > 1 ? sa.g.batch : 1)), block(WAVES * 64);
   if (mode == kModeBlock) hipLaunchKernelGGL((fp8_gemm_smallm_kernel<TMX, WAVES, kModeBlock>), grid, block, 0, stream, sa);
   else hipLaunchKernelGGL((fp8_gemm_smallm_kernel<TMX, WAVES, kModeRowCol>), grid, block, 0, stream, sa);
   FG_CHECK_LAUNCH("fp8_gemm_smallm_kernel");
@@ -377,7 +394,7 @@ int launch_transpose(const SmallArgs& sa, int mode, hipStream_t stream) {
   constexpr int kSlabs = WAVES * 16 * RG * 256;
   constexpr int kRed = WAVES * 16 * TMX * 16 * RG * 4;
   constexpr int kLds = kSlabs > kRed ? kSlabs : kRed;
-  const dim3 grid((uint32_t)(sa.n_chunks * sa.splits)), block(WAVES * 64);
+  const dim3 grid((uint32_t)(sa.n_chunks * sa.splits), (uint32_t)(sa.g.batch > 1 ? sa.g.batch : 1)), block(WAVES * 64);
   auto kb = fp8_gemm_transpose_kernel<TMX, RG, DEPTH, WAVES, kModeBlock>;
   auto kr = fp8_gemm_transpose_kernel<TMX, RG, DEPTH, WAVES, kModeRowCol>;
   static bool attr_set = false;
@@ -395,7 +412,8 @@ int launch_transpose(const SmallArgs& sa, int mode, hipStream_t stream) {
 
 }  // namespace
 
-SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K) {
+SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
+  if (entries < 1) entries = 1;  // equal problems launched together: their blocks fill the GPU together
   SmallMPlan p = {};
   p.use = false;
   if (M < 1 || M > 64 || N < 1 || K < 128 || K % 128 != 0) return p;
@@ -409,7 +427,7 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K) {
     // split across blocks only for very narrow weights (a split costs a round trip of partial tiles
     // through memory: measured 6.1 us unsplit against 8.6 us split in two for N = 2112, K = 7168).
     p.rg = 4;
-    while (p.rg > 1 && ceil_div(N, 16 * p.rg) < 140) p.rg >>= 1;
+    while (p.rg > 1 && ceil_div(N, 16 * p.rg) * entries < 140) p.rg >>= 1;
     p.waves = (p.tmx == 2 && p.rg == 4) ? 4 : 8;
   } else {
     p.waves = p.tmx == 4 ? 4 : 8;  // LDS reduction buffer is 4 KB * tmx per wavefront
@@ -422,11 +440,11 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K) {
   if (p.staged) {
     const int64_t pairs = (KB + 1) / 2;
     splits = 1;
-    while (p.n_chunks * splits < 100 && splits * 2 <= max_splits && splits * 2 * p.waves <= pairs) splits *= 2;
+    while (p.n_chunks * entries * splits < 100 && splits * 2 <= max_splits && splits * 2 * p.waves <= pairs) splits *= 2;
     kpw = ceil_div(pairs, splits * p.waves);
   } else {
     // aim for ~8 wavefronts per CU on 256 CUs, each with at least one K-block
-    const int64_t units = (int64_t)p.n_chunks * KB;
+    const int64_t units = (int64_t)p.n_chunks * entries * KB;
     kpw = units / 2048;
     if (kpw < 1) kpw = 1;
     splits = ceil_div(KB, kpw * p.waves);
@@ -454,9 +472,16 @@ int launch_small_m(const GemmArgs& g, int mode, const SmallMPlan& plan, void* wo
   sa.n_chunks = plan.n_chunks;
   sa.partials = nullptr;
   sa.counters = nullptr;
+  sa.partials_per_entry = 0;
   if (plan.splits > 1) {
-    if (!workspace || workspace_bytes < plan.workspace_bytes)
-      FG_FAIL(FG_ERR_WORKSPACE, "fp8 gemm (small M): workspace of %zu bytes needed, %zu given", plan.workspace_bytes,
+    const size_t entries = g.batch > 1 ? (size_t)g.batch : 1;
+    const size_t per_entry = plan.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES;
+    const size_t need = FG_WORKSPACE_COUNTER_BYTES + entries * per_entry;
+    sa.partials_per_entry = (int64_t)(per_entry / sizeof(float));
+    if (entries * (size_t)plan.n_chunks * sizeof(unsigned int) > FG_WORKSPACE_COUNTER_BYTES)
+      FG_FAIL(FG_ERR_WORKSPACE, "fp8 gemm (small M): %zu batch entries of %d chunks do not fit the counter area", entries, plan.n_chunks);
+    if (!workspace || workspace_bytes < need)
+      FG_FAIL(FG_ERR_WORKSPACE, "fp8 gemm (small M): workspace of %zu bytes needed, %zu given", need,
               workspace_bytes);
     if ((uintptr_t)workspace % 16 != 0) FG_FAIL(FG_ERR_INVALID_ARG, "fp8 gemm (small M): workspace must be 16-byte aligned");
     sa.counters = reinterpret_cast<unsigned int*>(workspace);

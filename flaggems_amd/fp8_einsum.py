@@ -63,7 +63,7 @@ def w8a8_block_fp8_bmm(
     lib = _lib.load()
     dev = x.device
     with torch.cuda.device(dev):
-        ws_bytes = lib.fg_block_fp8_gemm_workspace_bytes(M, N, K)
+        ws_bytes = lib.fg_batched_block_fp8_gemm_workspace_bytes(B, M, N, K)
         ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
         status = lib.fg_batched_block_fp8_gemm(
             x.data_ptr(), x.stride(1) if M > 1 else max(K, x.stride(1)), x.stride(0),

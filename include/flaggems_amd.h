@@ -220,11 +220,14 @@ size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * takes lda = h * r and a_batch_stride = r.  Matrices too small to fill the GPU on their own go out in one launch
  * (the batch entry in the grid), larger ones one after the other on `stream`; either way the results are, bit for
  * bit, those of `batch` calls of fg_block_fp8_gemm, and the workspace rules are that entry point's
- * (fg_block_fp8_gemm_workspace_bytes(M, N, K); one workspace serves the whole batch).
+ * (one workspace serves the whole batch; fg_batched_block_fp8_gemm_workspace_bytes(batch, M, N, K) is what the
+ * kernels can use: at most 32 rows per matrix, every entry keeps its own partial sums, and with less than that
+ * the call takes a slower kernel instead of failing).
  *
  * Stands in for w8a8_block_fp8_bmm (src/flag_gems/runtime/backend/_nvidia/hopper/ops/w8a8_block_fp8_bmm.py:629-779)
  * and, through it, fp8_einsum("bhr,hdr->bhd") (.../hopper/ops/fp8_einsum.py:22-68).
  */
+size_t fg_batched_block_fp8_gemm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K);
 int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_batch_stride,
                               const void* B, int64_t ldb, int64_t b_batch_stride,
                               const float* As, int64_t as_row_stride, int64_t as_col_stride, int64_t as_batch_stride,
