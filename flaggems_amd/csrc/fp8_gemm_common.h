@@ -146,7 +146,7 @@ struct MidMPlan {
   int n_chunks;      // ceil(N / (16 * rg))
   size_t workspace_bytes;
 };
-MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K);
+MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K, int64_t entries = 1);
 int launch_mid_m(const GemmArgs& a, int mode, const MidMPlan& plan, void* workspace, size_t workspace_bytes,
                  hipStream_t stream);
 

@@ -33,6 +33,7 @@ struct MidArgs {
   int kb_per_split, splits, n_chunks;  // n_chunks = ceil(N / (16 * RG))
   float* partials;                     // [n_chunks][splits][RG * TMX][64 lanes] x 4 floats
   unsigned int* counters;              // one per chunk
+  int64_t partials_per_entry;          // floats; a batch (g.batch > 1, entry = blockIdx.z) keeps one such array and n_chunks counters per entry
 };
 
 template <int RG>
@@ -53,6 +54,16 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
   constexpr int NT = WAVES * 64;
   constexpr int kMidRows = mid_rows(TMX), kMidStageBytes = mid_stage_bytes(TMX);
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [kb][64 rows][128 B], then As [kb][64]
+  if (a.g.batch > 1) {  // uniform: this workgroup's entry of the batch
+    const int64_t z = blockIdx.z;
+    a.g.X += z * a.g.x_batch_bytes;
+    a.g.W += z * a.g.w_batch_bytes;
+    a.g.C = reinterpret_cast<uint8_t*>(a.g.C) + z * a.g.c_batch_bytes;
+    a.g.xs += z * a.g.xs_batch_stride;
+    a.g.ws += z * a.g.ws_batch_stride;
+    if (a.partials) a.partials += z * a.partials_per_entry;
+    if (a.counters) a.counters += z * a.n_chunks;
+  }
   const GemmArgs& g = a.g;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -268,7 +279,7 @@ int launch_mid(const MidArgs& ma, int mode, hipStream_t stream) {
     if (e1 != hipSuccess || e2 != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS) failed", kMax);
     attr_set = true;
   }
-  const dim3 grid((uint32_t)ceil_div(ma.n_chunks, WAVES), (uint32_t)ma.splits), block(WAVES * 64);
+  const dim3 grid((uint32_t)ceil_div(ma.n_chunks, WAVES), (uint32_t)ma.splits, (uint32_t)(ma.g.batch > 1 ? ma.g.batch : 1)), block(WAVES * 64);
   if (mode == kModeBlock) hipLaunchKernelGGL(kb, grid, block, lds_bytes, stream, ma);
   else hipLaunchKernelGGL(kr, grid, block, lds_bytes, stream, ma);
   FG_CHECK_LAUNCH("fp8_gemm_midm_kernel");
@@ -277,8 +288,9 @@ int launch_mid(const MidArgs& ma, int mode, hipStream_t stream) {
 
 }  // namespace
 
-MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K) {
+MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   MidMPlan p = {};
+  if (entries < 1) entries = 1;  // equal problems launched together: their wavefronts fill the GPU together
   // (16- and 32-row variants of this kernel were measured against the decode kernels: slower on every shape for
   // M <= 16, mixed for 17..32 -- 8192 x 8192: 25.9 -> 20.7 us, but 7168 x 16384 at M = 24: 33.5 -> 47 us -- so those M stay there)
   if (M <= 32 || M > 128 || N < 1 || K < 128 || K % 128 != 0) return p;
@@ -294,8 +306,8 @@ MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K) {
     // ~1800 wavefronts but not below 8 K-blocks per block (every split writes and reads N x 64 fp32 sums: +50 % of
     // the weight bytes at 8 K-blocks, +25 % at 16), and never less than LDS requires.
     rg = 1;
-    if (ceil_div(N, 16) * min_splits >= 3000) rg = 2;  // plenty of wavefronts: N = 7168, K = 16384: 43 -> 39 us
-    splits = ceil_div((int64_t)1800, ceil_div(N, 16 * rg));
+    if (ceil_div(N, 16) * entries * min_splits >= 3000) rg = 2;  // plenty of wavefronts: N = 7168, K = 16384: 43 -> 39 us
+    splits = ceil_div((int64_t)1800, ceil_div(N, 16 * rg) * entries);
     const int64_t max_splits = KB / 8 > min_splits ? KB / 8 : min_splits;
     splits = splits < min_splits ? min_splits : (splits > max_splits ? max_splits : splits);
   } else {
@@ -337,9 +349,16 @@ int launch_mid_m(const GemmArgs& g, int mode, const MidMPlan& plan, void* worksp
   ma.n_chunks = plan.n_chunks;
   ma.partials = nullptr;
   ma.counters = nullptr;
+  ma.partials_per_entry = 0;
   if (plan.splits > 1) {
-    if (!workspace || workspace_bytes < plan.workspace_bytes)
-      FG_FAIL(FG_ERR_WORKSPACE, "fp8 gemm (33..128 rows): workspace of %zu bytes needed, %zu given", plan.workspace_bytes, workspace_bytes);
+    const size_t entries = g.batch > 1 ? (size_t)g.batch : 1;
+    const size_t per_entry = plan.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES;
+    const size_t need = FG_WORKSPACE_COUNTER_BYTES + entries * per_entry;
+    ma.partials_per_entry = (int64_t)(per_entry / sizeof(float));
+    if (entries * (size_t)plan.n_chunks * sizeof(unsigned int) > FG_WORKSPACE_COUNTER_BYTES)
+      FG_FAIL(FG_ERR_WORKSPACE, "fp8 gemm (33..128 rows): %zu batch entries of %d chunks do not fit the counter area", entries, plan.n_chunks);
+    if (!workspace || workspace_bytes < need)
+      FG_FAIL(FG_ERR_WORKSPACE, "fp8 gemm (33..128 rows): workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     if ((uintptr_t)workspace % 16 != 0) FG_FAIL(FG_ERR_INVALID_ARG, "fp8 gemm (33..128 rows): workspace must be 16-byte aligned");
     ma.counters = reinterpret_cast<unsigned int*>(workspace);
     ma.partials = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);

@@ -43,6 +43,23 @@ def test_einsum_large_batch_and_per_head_bits():
         assert torch.equal(got[:, head], plain)
 
 
+@pytest.mark.parametrize("M", [1, 5, 17, 32, 33, 48, 64, 100, 128])
+@pytest.mark.parametrize("B,N,K", [(3, 384, 640), (12, 1024, 2048), (40, 128, 512), (2, 7168, 2304)])
+def test_batches_of_few_rows_go_out_in_one_launch(M, B, N, K):
+    """Up to 128 rows per matrix the weight-streaming kernels take the whole batch in one launch (the entry in the
+    grid, every entry with its own partial sums and counters); strided operands and outputs, and a second call on the
+    same workspace."""
+    xq, xs, yq, ys = O.make_fp8_einsum_inputs(M, B, K, N, seed=M + B)
+    want = O.fp8_block_einsum_ref(xq, xs, yq, ys, [128, 128]).permute(1, 0, 2)       # [B, M, N]
+    x, x_s = xq.permute(1, 0, 2).to(DEV), xs.permute(1, 0, 2).to(DEV)                # strided views, as fp8_einsum passes them
+    z = torch.full((B, M, N + 3), 3.0, dtype=torch.bfloat16, device=DEV)
+    for _ in range(2):
+        flag_gems.w8a8_block_fp8_bmm(x, yq.to(DEV), x_s, ys.to(DEV), [128, 128], z=z[:, :, :N])
+        top = want.abs().max().item()
+        torch.testing.assert_close(z[:, :, :N].cpu().float(), want, rtol=1e-2, atol=1e-2 * max(1.0, top / 8))
+        assert torch.all(z[:, :, N:] == 3.0)
+
+
 def test_bmm_into_callers_buffer_and_other_dtypes():
     B, M, N, K = 3, 200, 384, 512
     xq, xs, yq, ys = O.make_fp8_einsum_inputs(M, B, K, N, seed=2)
