@@ -218,8 +218,9 @@ size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * strides.  Matrix i of each operand starts i * <its batch stride> after matrix 0 (bytes for A and B, floats for
  * the scales, elements of c_dtype for C); row strides are free, so a [b, h, r] activation with h as the batch
  * takes lda = h * r and a_batch_stride = r.  Matrices too small to fill the GPU on their own go out in one launch
- * (the batch entry in the grid), larger ones one after the other on `stream`; either way the results are, bit for
- * bit, those of `batch` calls of fg_block_fp8_gemm, and the workspace rules are that entry point's
+ * (the batch entry in the grid), larger ones one after the other on `stream`; the results are those of `batch`
+ * calls of fg_block_fp8_gemm (the same bits, except that up to 128 rows K may be split over fewer blocks than for
+ * a lone matrix, which changes the order of the fp32 partial sums), and the workspace rules are that entry point's
  * (one workspace serves the whole batch; fg_batched_block_fp8_gemm_workspace_bytes(batch, M, N, K) is what the
  * kernels can use: at most 32 rows per matrix, every entry keeps its own partial sums, and with less than that
  * the call takes a slower kernel instead of failing).
