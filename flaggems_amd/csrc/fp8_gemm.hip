@@ -504,7 +504,7 @@ int launch_cfg(GemmArgs a, hipStream_t stream) {
   return FG_OK;
 }
 
-// M > 32 with at most 128 tiles of 128 x 128: K split over blocks so that more than one block per compute unit is
+// M > 32 with at most 128 tiles of 128 x 128 (256 when K <= 8192): K split over blocks so that more than one block per compute unit is
 // resident (a K-block of one tile costs a full load latency, ~1.8 us; the loads of several blocks overlap).
 // Measured against the persistent kernel (which has a quarter of the tiles, and stream-K): M = 256, N = 2112,
 // K = 7168: 79 -> 31 us; M = 512, N = 4096, K = 4096: 50 -> 28 us; M = 512, N = 1024, K = 8192: 83 -> 26 us.
@@ -520,11 +520,15 @@ TileSplitPlan plan_tile_split(int64_t M, int64_t N, int64_t K) {
   const int64_t KB = K / 128;
   const int64_t tiles = ceil_div(M, kSplitTile) * ceil_div(N, kSplitTile);
   if (tiles * kSplitWaves * 4 > FG_WORKSPACE_COUNTER_BYTES) return p;
-  if (tiles > 128) return p;  // enough tiles to go round
+  // 129..256 tiles: one block per compute unit, which waits out every K-block's load; two blocks per tile help while
+  // K is at most 8192 (measured M = 512: N = 6144, K = 4096: 54 -> 33 us; 4608 x 7168: 56 -> 44; 7168 x 2304: 35 -> 27;
+  // M = 1024: 4096 x 4096: 51 -> 38; but 4096 x 14336: 85 -> 97, so long K stays with the persistent kernel)
+  if (tiles > 256 || (tiles > 128 && KB > 64)) return p;
   // up to 64 rows the decode kernels are the alternative: they win unless K is long (measured: K = 7168 and
   // 16384 faster here, K = 1024 ... 2304 faster there)
   if (M <= 64 && KB < 32) return p;
   int64_t splits = (320 + tiles / 2) / tiles;  // ~1.25 blocks per compute unit
+  if (tiles > 128) splits = 2;
   if (splits > KB / 4) splits = KB / 4;  // at least four K-blocks per block
   if (splits > 8) splits = 8;            // the wavefront that finishes a tile reads the splits one after another
   if (splits < 2) return p;

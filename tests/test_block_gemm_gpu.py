@@ -107,6 +107,21 @@ def test_few_tiles_split_along_k(M, N, K, dtype):
         assert torch.equal(again.view(torch.int8), got.view(torch.int8))
 
 
+@pytest.mark.parametrize("M,N,K", [(700, 4000, 4096), (512, 6144, 4096), (1000, 3200, 8192), (300, 10000, 1024)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_129_to_256_tiles_with_k_split_in_two(M, N, K, dtype):
+    """129..256 tiles of 128 x 128 with K <= 8192: two blocks per tile, the second half's sums added in split order;
+    ragged M and N; against the oracle and bit-identical on reruns."""
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=17)
+    want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
+    args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    got = flag_gems.w8a8_block_fp8_matmul(*args, output_dtype=dtype)
+    tol = dict(rtol=1e-4, atol=4e-4) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(got.cpu().float(), want, **tol)
+    for _ in range(2):
+        assert torch.equal(flag_gems.w8a8_block_fp8_matmul(*args, output_dtype=dtype).view(torch.int8), got.view(torch.int8))
+
+
 @pytest.mark.parametrize("M,N,K", [(33, 100, 384), (64, 2112, 7168), (50, 7168, 16384), (40, 24584, 1536), (64, 4104, 2304),
                                    (65, 520, 1024), (100, 2112, 4096), (128, 4096, 4096), (128, 7000, 2304)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
