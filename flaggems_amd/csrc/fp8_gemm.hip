@@ -592,11 +592,11 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
   }
   {
     const int64_t tiles128 = ceil_div(a.M, 128) * ceil_div(a.N, 128);
-    // 257..640 tiles of 128 x 128 with short K (up to 448 tiles for K up to 8192): one to two and a half tiles per
-    // compute unit, two workgroups resident on each; the persistent kernel has a quarter of the tiles and spends its
+    // 257..512 tiles of 128 x 128 with short K (up to 448 tiles for K up to 8192): at most the 512 workgroups that are
+    // resident at a time, two on each compute unit (560 tiles: M = 1280, N = 7168, K = 2304 went from 36 to 51 us); the persistent kernel has a quarter of the tiles and spends its
     // time filling and draining.  Measured: M = 256, N = 24576, K = 1536: 27.7 -> 23.4 us; M = 768, N = 7168, K = 2304:
     // 34.8 -> 28.9; N = 6144, K = 4096: 50.0 -> 43.4; M = 1024, N = 7168, K = 2304: 35.3 -> 29.6 (N = K = 8192: 86 -> 89).
-    if (direct && a.M > 128 && a.M <= 1024 && tiles128 > 256 && ((tiles128 <= 640 && a.KB <= 32) || (tiles128 <= 448 && a.KB <= 64)))
+    if (direct && a.M > 128 && a.M <= 1024 && tiles128 > 256 && ((tiles128 <= 512 && a.KB <= 32) || (tiles128 <= 448 && a.KB <= 64)))
       return launch_cfg<128, 128, 2, 2, MODE, true>(a, stream);
   }
   const bool big = a.M > 128;
