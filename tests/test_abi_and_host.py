@@ -169,3 +169,15 @@ def test_widened_entry_points_validate_and_refuse_the_cpu():
     assert rc == _lib.FG_ERR_INVALID_ARG
     assert lib.fg_batched_block_fp8_gemm(None, 0, 0, None, 0, 0, None, 0, 0, 0, None, 0, 0, 0, None, 0, 0, _lib.FG_BF16,
                                          -1, 4, 4, 128, 128, 128, None, 0, None) == _lib.FG_ERR_INVALID_ARG
+
+
+def test_batched_workspace_query_is_host_only_and_never_below_the_single_problem():
+    """fg_batched_block_fp8_gemm_workspace_bytes needs no GPU; it is at least the single-problem figure (with less the
+    batched call takes a slower kernel, it never fails) and does not shrink when the batch grows past one entry's plan."""
+    lib = _lib.load()
+    for (M, N, K) in [(1, 1024, 4096), (8, 1024, 7168), (32, 128, 512), (64, 1024, 7168), (128, 1024, 4096), (4096, 1024, 4096)]:
+        single = lib.fg_block_fp8_gemm_workspace_bytes(M, N, K)
+        assert lib.fg_batched_block_fp8_gemm_workspace_bytes(1, M, N, K) == single
+        for batch in (2, 8, 16, 128):
+            assert lib.fg_batched_block_fp8_gemm_workspace_bytes(batch, M, N, K) >= single
+    assert lib.fg_batched_block_fp8_gemm_workspace_bytes(16, 64, 1024, 7168) > lib.fg_block_fp8_gemm_workspace_bytes(64, 1024, 7168)
