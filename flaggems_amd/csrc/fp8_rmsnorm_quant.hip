@@ -85,8 +85,17 @@ __device__ __forceinline__ void narrow_chunk(const float (&v)[8], uint32_t (&w)[
 // resident, each loading its next row (raw words) before working on the current one, was measured and not kept: the
 // norm alone went to 22.5 us, the fused call stayed at 37 us, and rows of 16384 elements got slower (150 us against
 // 101) because the second row in registers left one wavefront per SIMD.
-template <int XDT, int CHUNKS>
+// QUANT: 0 = the norm alone, 1 = with the quantizer and its rules taken from the arguments, 2 = with the quantizer
+// under the rules of per_token_group_quant_fp8's defaults (scale = amax * (1 / max), true division, no power-of-two
+// rounding, e4m3), which lets the compiler drop every rule switch from the loop.
+template <int XDT, int CHUNKS, int QUANT>
 __global__ __launch_bounds__(kNormThreads) void rms_norm_quant_kernel(NormQuantArgs a) {
+  if (QUANT == 2) {
+    a.q.scale_rule = FG_SCALE_MUL_INV;
+    a.q.quotient_rule = FG_QUOT_DIV;
+    a.q.pow2_rule = FG_POW2_NONE;
+    a.q.e5m2 = 0;
+  }
   using E = Elem<XDT>;
   using Raw = typename E::raw;
   constexpr int kWords = sizeof(Raw) * 8 / 4;
@@ -94,7 +103,7 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_quant_kernel(NormQuantA
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const bool add_residual = a.residual != nullptr;
-  const bool quantize = a.q.q != nullptr;
+  constexpr bool quantize = QUANT != 0;
   const Raw* wp = reinterpret_cast<const Raw*>(a.weight);
   uint32_t parity = 0;
 
@@ -198,10 +207,19 @@ int launch_norm(const NormQuantArgs& a, int cus, hipStream_t stream) {
   // enough workgroups to hold every compute unit's wave slots a few times over; beyond that, rows are walked
   const uint32_t grid = a.rows < (uint32_t)cus * 16u ? a.rows : (uint32_t)cus * 16u;
   const dim3 g(grid), b(kNormThreads);
-  if (per_thread <= 1) hipLaunchKernelGGL((rms_norm_quant_kernel<XDT, 1>), g, b, 0, stream, a);
-  else if (per_thread <= 2) hipLaunchKernelGGL((rms_norm_quant_kernel<XDT, 2>), g, b, 0, stream, a);
-  else if (per_thread <= 4) hipLaunchKernelGGL((rms_norm_quant_kernel<XDT, 4>), g, b, 0, stream, a);
-  else hipLaunchKernelGGL((rms_norm_quant_kernel<XDT, 8>), g, b, 0, stream, a);
+  const int quant = a.q.q == nullptr ? 0
+                    : (a.q.scale_rule == FG_SCALE_MUL_INV && a.q.quotient_rule == FG_QUOT_DIV && a.q.pow2_rule == FG_POW2_NONE && !a.q.e5m2) ? 2 : 1;
+#define FG_NORM_LAUNCH(C)                                                                                            \
+  do {                                                                                                               \
+    if (quant == 0) hipLaunchKernelGGL((rms_norm_quant_kernel<XDT, C, 0>), g, b, 0, stream, a);                      \
+    else if (quant == 1) hipLaunchKernelGGL((rms_norm_quant_kernel<XDT, C, 1>), g, b, 0, stream, a);                 \
+    else hipLaunchKernelGGL((rms_norm_quant_kernel<XDT, C, 2>), g, b, 0, stream, a);                                 \
+  } while (0)
+  if (per_thread <= 1) FG_NORM_LAUNCH(1);
+  else if (per_thread <= 2) FG_NORM_LAUNCH(2);
+  else if (per_thread <= 4) FG_NORM_LAUNCH(4);
+  else FG_NORM_LAUNCH(8);
+#undef FG_NORM_LAUNCH
   FG_CHECK_LAUNCH("rms_norm_quant_kernel");
   return FG_OK;
 }
