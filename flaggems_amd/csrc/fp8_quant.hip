@@ -27,8 +27,17 @@ constexpr uint64_t kQuantSmallChunks = 512ull * 1024;  // up to this many chunks
 // Vector kernel: group_size == 8 * LPG, rows 16-byte aligned.
 // SILU: the value quantized is silu(x[row, c]) * x[row, c + up_offset], rounded to x's type first (what a separate
 // activation kernel would have stored), and x is never re-read.
-template <int XDT, int LPG, int kQuantUnroll, bool SILU = false>
+// RULES: 0 = scale, quotient and rounding rules from the arguments; 1 = act_quant's defaults (amax * (1 / max),
+// x * (1 / s), no power-of-two rounding, e4m3); 2 = per_token_group_quant_fp8's (the same with true division): the
+// compiler then drops every rule switch from the loop.
+template <int XDT, int LPG, int kQuantUnroll, bool SILU = false, int RULES = 0>
 __global__ __launch_bounds__(kQuantThreads) void group_quant_vec_kernel(QuantArgs a) {
+  if (RULES != 0) {
+    a.scale_rule = FG_SCALE_MUL_INV;
+    a.quotient_rule = RULES == 1 ? FG_QUOT_RECIP_MUL : FG_QUOT_DIV;
+    a.pow2_rule = FG_POW2_NONE;
+    a.e5m2 = 0;
+  }
   using E = Elem<XDT>;
   constexpr int kWords = sizeof(typename E::raw) * 8 / 4;  // 32-bit words per lane: 4 or 8
   const uint32_t total_chunks = a.total_groups * (uint32_t)LPG;  // host guarantees no overflow
@@ -129,13 +138,18 @@ int launch_quant(const QuantArgs& a, bool vec_ok, hipStream_t stream, bool silu 
     uint32_t l = g / 8;
     if (l == 1 || l == 2 || l == 4 || l == 8 || l == 16 || l == 32 || l == 64) lpg = (int)l;
   }
+  const int rules = (a.scale_rule == FG_SCALE_MUL_INV && a.pow2_rule == FG_POW2_NONE && !a.e5m2)
+                        ? (a.quotient_rule == FG_QUOT_RECIP_MUL ? 1 : 2) : 0;
   if (silu) {
     if (lpg != 16 && lpg != 8)
       FG_FAIL(FG_ERR_UNSUPPORTED, "fused activation + quantizer: group size 64 or 128 and 16-byte aligned rows only");
     const uint64_t chunks = (uint64_t)a.total_groups * (uint64_t)lpg;
     const bool small = chunks <= kQuantSmallChunks;
     dim3 grid((uint32_t)ceil_div((int64_t)chunks, (int64_t)kQuantThreads * (small ? 1 : kQuantUnrollLarge)));
-    if (lpg == 16) {
+    if (lpg == 16 && rules == 2) {
+      if (small) hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, 1, true, 2>), grid, dim3(kQuantThreads), 0, stream, a);
+      else hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, true, 2>), grid, dim3(kQuantThreads), 0, stream, a);
+    } else if (lpg == 16) {
       if (small) hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, 1, true>), grid, dim3(kQuantThreads), 0, stream, a);
       else hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, true>), grid, dim3(kQuantThreads), 0, stream, a);
     } else {
@@ -154,6 +168,17 @@ int launch_quant(const QuantArgs& a, bool vec_ok, hipStream_t stream, bool silu 
   const uint64_t chunks = (uint64_t)a.total_groups * (uint64_t)lpg;
   const bool small = chunks <= kQuantSmallChunks;
   dim3 grid((uint32_t)ceil_div((int64_t)chunks, (int64_t)kQuantThreads * (small ? 1 : kQuantUnrollLarge)));
+  if (lpg == 16 && rules != 0) {  // group size 128 under either operator's default rules
+    if (rules == 1) {
+      if (small) hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, 1, false, 1>), grid, dim3(kQuantThreads), 0, stream, a);
+      else hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, false, 1>), grid, dim3(kQuantThreads), 0, stream, a);
+    } else {
+      if (small) hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, 1, false, 2>), grid, dim3(kQuantThreads), 0, stream, a);
+      else hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, false, 2>), grid, dim3(kQuantThreads), 0, stream, a);
+    }
+    FG_CHECK_LAUNCH("group_quant_vec_kernel");
+    return FG_OK;
+  }
   switch (lpg) {
 #define FG_CASE(L)                                                                                                       \
   case L:                                                                                                                \
