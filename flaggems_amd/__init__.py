@@ -29,7 +29,7 @@ from .registration import (  # noqa: F401
     use_gems,
 )
 from .scaled_mm import scaled_mm, scaled_mm_out  # noqa: F401
-from .w8a8_block_fp8_matmul import fp8_matmul, w8a8_block_fp8_matmul  # noqa: F401
+from .w8a8_block_fp8_matmul import fp8_matmul, fp8_matmul_noop, w8a8_block_fp8_matmul  # noqa: F401
 
 __version__ = "0.1.0"
 device = "cuda"  # PyTorch-ROCm device type of an MI355X
@@ -45,6 +45,7 @@ __all__ = [
     "enable",
     "fp8_einsum",
     "fp8_matmul",
+    "fp8_matmul_noop",
     "fused_add_rms_norm",
     "grouped_w8a8_block_fp8_matmul",
     "only_enable",

@@ -8,7 +8,7 @@ from __future__ import annotations
 import ctypes
 import os
 import threading
-from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint64, c_void_p
 
 import torch
 
@@ -36,6 +36,7 @@ DTYPE_CODE = {
 SIGNATURES = {
     "fg_version": (c_int, []),
     "fg_last_error_string": (c_char_p, []),
+    "fg_stream_capture_id": (c_uint64, [c_void_p]),
     "fg_group_quant_fp8": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64,
@@ -149,16 +150,38 @@ def current_stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
-# per-(device, stream) workspace, zero-filled once at creation, grown on demand
-_workspaces = {}
+# Workspace of the GEMM kernels (arrival counters, split-K partial sums, transposed scales): one zero-filled buffer
+# per (device, stream), grown on demand.  Launches recorded into a HIP graph keep the raw address they were given, so
+#   * a buffer that is replaced is retired, not released: a graph captured earlier may still write to it;
+#   * a buffer allocated while a capture is in progress comes from that graph's private memory pool and is handed out
+#     to launches of the same capture only (its zero fill is a kernel recorded in the graph; the counters are zero
+#     again after every launch, so refilling them on every replay changes nothing).
+# Growth at least doubles the size, so retired buffers add up to less than the live one.
+_workspaces = {}   # (device index, stream handle) -> (buffer, id of the capture it was allocated in, or 0)
+_retired = []
 
 
 def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    key = (device.index if device.index is not None else torch.cuda.current_device(),
-           torch.cuda.current_stream(device).cuda_stream)
-    buf = _workspaces.get(key)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    capture = int(load().fg_stream_capture_id(stream))
     need = max(int(nbytes), FG_WORKSPACE_COUNTER_BYTES)
+    buf, made_in = _workspaces.get(key, (None, 0))
+    if buf is not None and made_in not in (0, capture):
+        buf = None  # belongs to another graph's pool: that graph keeps the memory, this table must not hand it out
     if buf is None or buf.numel() < need:
+        if buf is not None:
+            if made_in == 0:
+                _retired.append(buf)
+            need = max(need, 2 * buf.numel())
         buf = torch.zeros(need, dtype=torch.uint8, device=device)
-        _workspaces[key] = buf
+        # buffers of captures that have ended stay with their graphs; this table only drops its references
+        for other in [k for k, (_, cap) in _workspaces.items() if cap not in (0, capture)]:
+            del _workspaces[other]
+        _workspaces[key] = (buf, capture)
     return buf
+
+
+def reserve_workspace(device: torch.device, nbytes: int) -> None:
+    """Size the current stream's workspace ahead of time (for example before capturing a graph on this stream)."""
+    workspace(torch.device(device), nbytes)

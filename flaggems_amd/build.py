@@ -27,7 +27,9 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # MFMA results land in architectural VGPRs, where the scale FMAs can read them directly
     "-mllvm", "-amdgpu-mfma-vgpr-form=1",
-    "-w",
+    "-Wall",
+    # the global->LDS loads are written in assembly and name m0, which the compiler reports on every expansion
+    "-Wno-inline-asm",
 ]
 
 
@@ -49,6 +51,8 @@ def _run(cmd):
     )
     if proc.returncode != 0:
         raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    if out and "warning" in out:
+        print(out, flush=True)
     return out
 
 

@@ -28,11 +28,45 @@ constexpr size_t kErrorBufferBytes = 512;
     return (code);                                                      \
   } while (0)
 
+// Status of the most recent kernel launch made by this thread through FG_LAUNCH.  The launch call's own return
+// value is kept, so that an error some other library left in the process-wide "last error" slot is neither taken
+// for this launch's nor cleared.
+hipError_t& launch_status();
+
+template <typename T>
+struct same_type { using type = T; };
+
+// Launches `kern` with the given arguments (converted to the kernel's parameter types) and records the status.
+template <typename... KArgs>
+inline void launch(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream,
+                   typename same_type<KArgs>::type... args) {
+  void* params[] = {const_cast<void*>(static_cast<const void*>(&args))...};
+  launch_status() = hipLaunchKernel(reinterpret_cast<const void*>(kern), grid, block, params, lds_bytes, stream);
+}
+
+#define FG_LAUNCH(kern, grid, block, lds_bytes, stream, ...) ::fg::launch(kern, grid, block, lds_bytes, stream, __VA_ARGS__)
+
 #define FG_CHECK_LAUNCH(what)                                                       \
   do {                                                                              \
-    hipError_t e_ = hipGetLastError();                                              \
+    hipError_t e_ = ::fg::launch_status();                                          \
     if (e_ != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e_)); \
   } while (0)
+
+// Kernels that use more than 64 KB of dynamic LDS need the limit raised once per device (the attribute belongs to
+// the device's copy of the kernel).  `done` is one flag array per kernel set; a race sets the attribute twice.
+constexpr int kMaxDevices = 64;
+struct PerDeviceFlags { bool done[kMaxDevices]; };
+inline hipError_t raise_dynamic_lds_limit(PerDeviceFlags& flags, int bytes, const void* k0, const void* k1 = nullptr) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const bool tracked = dev >= 0 && dev < kMaxDevices;
+  if (tracked && flags.done[dev]) return hipSuccess;
+  e = hipFuncSetAttribute(k0, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && k1) e = hipFuncSetAttribute(k1, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && tracked) flags.done[dev] = true;
+  return e;
+}
 
 __host__ __device__ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

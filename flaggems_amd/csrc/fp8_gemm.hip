@@ -135,7 +135,7 @@ __device__ __forceinline__ v8i read_fragment(const uint8_t* lds_tile, int rg, in
 
 // One K-block partial product with a zero accumulator input, result in architectural VGPRs.
 __device__ __forceinline__ v4f mfma_fp8_block_partial(v8i a, v8i b) {
-  v4f p;
+  v4f p = {};
   asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=&v"(p) : "v"(a), "v"(b));
   return p;
 }
@@ -489,17 +489,15 @@ int launch_cfg(GemmArgs a, hipStream_t stream) {
   a.tiles_m = (int)ceil_div(a.M, BM);
   a.tiles_n = (int)ceil_div(a.N, BN);
   auto kern = fp8_gemm_kernel<BM, BN, WM, WN, MODE, DIRECT>;
-  static bool attr_set = false;  // per instantiation; benign if raced
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
+  static PerDeviceFlags lds_limit_raised = {};  // per instantiation
+  {
+    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, Cfg::kLdsBytes, reinterpret_cast<const void*>(kern));
     if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
-    attr_set = true;
   }
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
   if (blocks > 0x7FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: too many tiles");
   if (a.batch > 65535) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: more than 65535 batch entries in one launch");
-  hipLaunchKernelGGL(kern, dim3((uint32_t)blocks, (uint32_t)(a.batch > 1 ? a.batch : 1)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, a);
+  FG_LAUNCH(kern, dim3((uint32_t)blocks, (uint32_t)(a.batch > 1 ? a.batch : 1)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, a);
   FG_CHECK_LAUNCH("fp8_gemm_kernel");
   return FG_OK;
 }
@@ -549,14 +547,13 @@ int launch_tile_split(GemmArgs a, const TileSplitPlan& plan, void* workspace, hi
   a.split_counters = reinterpret_cast<unsigned int*>(workspace);
   a.split_partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
   auto kern = fp8_gemm_kernel<kSplitTile, kSplitTile, 2, 2, MODE, true, true>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
+  static PerDeviceFlags lds_limit_raised = {};
+  {
+    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, Cfg::kLdsBytes, reinterpret_cast<const void*>(kern));
     if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
-    attr_set = true;
   }
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n * a.splits;
-  hipLaunchKernelGGL(kern, dim3((uint32_t)blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, a);
+  FG_LAUNCH(kern, dim3((uint32_t)blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, a);
   FG_CHECK_LAUNCH("fp8_gemm_kernel (K split)");
   return FG_OK;
 }
@@ -565,9 +562,6 @@ int launch_tile_split(GemmArgs a, const TileSplitPlan& plan, void* workspace, hi
 // the decode kernels, which take the same shapes).
 bool mid_m_preferred(const MidMPlan& mid, int64_t M, int64_t N, int64_t K) {
   (void)M;
-#ifdef FG_DEV_KNOBS
-  if (const char* e = getenv("FG_MIDM")) return mid.use && atoi(e) != 0;
-#endif
   // 33..64 rows: always (measured against both alternatives on every DeepSeek-V3 and Llama-3 shape).  65..128 rows:
   // the splits' partial sums cost as much as the weights, which pays only while the weights are small: M = 128,
   // N = 6144, K = 4096: 31 -> 20 us; N = 7168, K = 2304: 19 -> 16 us; but N = 24576, K = 1536: 23 -> 28 us.
@@ -576,7 +570,9 @@ bool mid_m_preferred(const MidMPlan& mid, int64_t M, int64_t N, int64_t K) {
 
 template <int MODE>
 int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-  const bool direct = (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) &&
+  // K == 0 (an empty sum: zeros, or the bias) goes to the guarded tile kernel, whose K loop may be empty; the
+  // kernels below all assume at least one K-block
+  const bool direct = (a.K > 0) && (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) &&
                       (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
                       ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
   if (direct) {

@@ -271,17 +271,15 @@ int launch_mid(const MidArgs& ma, int mode, hipStream_t stream) {
   const int lds_bytes = ma.kb_per_split * kPerKb;
   auto kb = fp8_gemm_midm_kernel<TMX, RG, WAVES, DEPTH, kModeBlock>;
   auto kr = fp8_gemm_midm_kernel<TMX, RG, WAVES, DEPTH, kModeRowCol>;
-  static bool attr_set = false;  // per instantiation; benign if raced
-  if (!attr_set) {
+  static PerDeviceFlags lds_limit_raised = {};  // per instantiation
+  {
     constexpr int kMax = mid_kb_max(TMX) * kPerKb;
-    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(kb), hipFuncAttributeMaxDynamicSharedMemorySize, kMax);
-    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(kr), hipFuncAttributeMaxDynamicSharedMemorySize, kMax);
-    if (e1 != hipSuccess || e2 != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS) failed", kMax);
-    attr_set = true;
+    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, kMax, reinterpret_cast<const void*>(kb), reinterpret_cast<const void*>(kr));
+    if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kMax, hipGetErrorString(e));
   }
   const dim3 grid((uint32_t)ceil_div(ma.n_chunks, WAVES), (uint32_t)ma.splits, (uint32_t)(ma.g.batch > 1 ? ma.g.batch : 1)), block(WAVES * 64);
-  if (mode == kModeBlock) hipLaunchKernelGGL(kb, grid, block, lds_bytes, stream, ma);
-  else hipLaunchKernelGGL(kr, grid, block, lds_bytes, stream, ma);
+  if (mode == kModeBlock) FG_LAUNCH(kb, grid, block, lds_bytes, stream, ma);
+  else FG_LAUNCH(kr, grid, block, lds_bytes, stream, ma);
   FG_CHECK_LAUNCH("fp8_gemm_midm_kernel");
   return FG_OK;
 }
@@ -319,10 +317,6 @@ MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   }
   while (rg < 4 && ceil_div(N, 16 * rg) > FG_WORKSPACE_COUNTER_BYTES / 4) rg <<= 1;
   if (tmx == 8 && rg > 2) return p;
-#ifdef FG_DEV_KNOBS
-  if (const char* e = getenv("FG_MID_RG")) rg = atoi(e);
-  if (const char* e = getenv("FG_MID_SPLITS")) splits = atoi(e) < min_splits ? min_splits : atoi(e);
-#endif
   const int64_t kbps = ceil_div(KB, splits);
   splits = ceil_div(KB, kbps);
   p.tmx = tmx;
@@ -333,9 +327,6 @@ MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   if (p.n_chunks > FG_WORKSPACE_COUNTER_BYTES / 4 || splits > 65535) return p;
   // one block per compute unit when its activations take more than half of LDS: then it should bring 8 wavefronts
   p.waves = kbps * (mid_stage_bytes(tmx) + mid_rows(tmx) * 4) > 80 * 1024 ? 8 : 4;
-#ifdef FG_DEV_KNOBS
-  if (const char* e = getenv("FG_MID_WAVES")) p.waves = atoi(e);
-#endif
   p.workspace_bytes = splits > 1 ? (size_t)FG_WORKSPACE_COUNTER_BYTES + (size_t)p.n_chunks * splits * rg * tmx * 64 * 16 : 0;
   p.use = true;
   return p;

@@ -44,41 +44,6 @@
 
 #include "fp8_gemm_common.h"
 
-#ifdef FG_PP_TRACE
-#ifndef FG_PP_TRACE_PHASE
-#define FG_PP_TRACE_PHASE 1
-#endif
-// development aid: per-slot timestamps of block 0, wavefronts 0 and 4; every fourth step is recorded and
-// written out a step later, so that the stores do not disturb the step they describe
-__device__ unsigned long long fg_pp_trace_buf[2][64][20];
-// the clock reads stay in scalar registers until the end of the step, so that a stamp costs one issue slot
-#define FG_PP_STAMP(id) fg_ts[id] = __builtin_amdgcn_s_memtime()
-#define FG_PP_STAMPS_DECLARE unsigned long long fg_ts[18] = {}
-#define FG_PP_STAMPS_STORE                                                                          \
-  do {                                                                                              \
-    if (blockIdx.x == 0 && (wave & 3) == 0 && lane == 0 && (T & 3) == ((FG_PP_TRACE_PHASE + 1) & 3) && T > 0 && T <= 64)                 \
-      for (int i = 0; i < 18; ++i) if (i < 8 || i >= 10) fg_pp_trace_buf[grp][T - 1][i] = fg_ts[i];  \
-    fg_ts[0] = fg_ts[8]; fg_ts[1] = fg_ts[9];                                                       \
-  } while (0)
-extern "C" void fg_pp_trace_dump() {
-  static unsigned long long h[2][64][20];
-  hipMemcpyFromSymbol(h, HIP_SYMBOL(fg_pp_trace_buf), sizeof(h));
-  unsigned long long t0 = h[0][0][0];
-  for (int T = FG_PP_TRACE_PHASE; T < 64; T += 4)
-    for (int g = 0; g < 2; ++g) {
-      printf("T=%2d %c:", T, g ? 'B' : 'A');
-      for (int i = 0; i < 8; ++i) printf(" %8lld", (long long)(h[g][T][i] - t0));
-      printf("  issue:");
-      for (int i = 10; i < 18; ++i) printf(" %5lld", (long long)(h[g][T][i] - h[g][T][1]));
-      printf("\n");
-    }
-}
-#else
-#define FG_PP_STAMP(id) do {} while (0)
-#define FG_PP_STAMPS_DECLARE do {} while (0)
-#define FG_PP_STAMPS_STORE do {} while (0)
-#endif
-
 namespace fg {
 namespace {
 
@@ -163,7 +128,6 @@ __device__ __forceinline__ void tile_of_sid(int sid, int tiles_m, int tiles_n, i
 // A block visits the virtual ids blockIdx.x, blockIdx.x + gridDim.x, ...  The grid is either the tile count
 // (one round) or the number of compute units, a multiple of 8, so a block stays on its XCD's run of tiles.
 // tile_of_index maps [0, n_tiles) onto the tiles one-to-one.
-__device__ __forceinline__ bool valid_vid(int vid, int n_tiles) { return vid < n_tiles; }
 
 // weight row (within the wavefront's 128) held by LDS row rho of the wavefront's region
 __device__ __forceinline__ int weight_row_of_lds_row(int rho) {
@@ -286,7 +250,7 @@ __device__ __forceinline__ v8i read_frag(const uint8_t* region, int rg, int lane
 
 // MFMA with a zero accumulator input, result in architectural VGPRs
 __device__ __forceinline__ v4f mfma_partial(const v8i& w, const v8i& x) {
-  v4f p;
+  v4f p = {};
   asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=&v"(p) : "v"(w), "v"(x));
   return p;
 }
@@ -701,14 +665,12 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   // several microseconds to drain.
   constexpr bool kRelaxedStoreWaits = ALIGNED && MODE == kModeBlock;
   bool flushed_prev = false;  // this wavefront stored a tile in its previous fetch phase
-  FG_PP_STAMPS_DECLARE;
   auto run_steps = [&](int t_begin, int t_end) __attribute__((always_inline)) {
   flushed_prev = false;  // every instance of this loop ends with all vector-memory operations complete
   for (int T = t_begin; T < t_end; ++T) {
     // ================= fetch(T)
     // Scales of this step were requested a step ago; the only younger vector-memory operations are the eight
     // tile loads that followed them (for A those have landed as well: it waited at the end of its multiply).
-    FG_PP_STAMP(8);
     float xs[kTM], sc[kTM];
     const bool more = T + 1 < total;
     float ws = 1.f;
@@ -718,8 +680,6 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
       if (more) request_scales();  // of step T+1; the pointer was moved there a step ago
       ws = *(const __attribute__((address_space(4))) float*)ws_ptr;
     }
-    FG_PP_STAMP(9);
-    FG_PP_STAMPS_STORE;  // of the previous step, behind this step's first wait
     const uint8_t* const tw = lds + rw_slot * kWStageBytes + (wn0 >> 4) * 2048;
     const uint8_t* const tx = lds + kXRegion + rx_slot * kXStageBytes + (wm0 >> 4) * 2048;
     // All activation fragments and the first two weight fragments (the other six follow during the multiply,
@@ -732,34 +692,24 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     // cheaper than a branch per load, and the wait counts below stay the same on every step.
     v8i xf[kTM], wr[3];
     issue_stage_part(0);
-    FG_PP_STAMP(10);
     xf[0] = read_frag(tx, 0, frag_off);
     issue_stage_part(1);
-    FG_PP_STAMP(11);
     xf[1] = read_frag(tx, 1, frag_off);
     issue_stage_part(2);
-    FG_PP_STAMP(12);
     xf[2] = read_frag(tx, 2, frag_off);
     issue_stage_part(3);
-    FG_PP_STAMP(13);
     xf[3] = read_frag(tx, 3, frag_off);
     issue_stage_part(4);
-    FG_PP_STAMP(14);
     wr[0] = read_frag(tw, 0, frag_off);
     issue_stage_part(5);
-    FG_PP_STAMP(15);
     wr[1] = read_frag(tw, 1, frag_off);
     issue_stage_part(6);
-    FG_PP_STAMP(16);
     issue_stage_part(7);
-    FG_PP_STAMP(17);
-    FG_PP_STAMP(2);
     // scalar bookkeeping of the next step, under the latency of the LDS reads (in the multiply phase every
     // extra instruction delays the MFMAs: a wavefront issues one instruction in ~6 cycles, and the MFMA with
     // its four FMAs fills the 32 cycles the matrix pipe takes)
     if (loaded < total) finish_stage();
     if (MODE == kModeBlock && T + 2 < total) advance_scales();
-    FG_PP_STAMP(3);
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): fragments are in registers
     // B's weights of stage T+1, issued a step ago, must have landed before the barrier; the scale requests
     // and the tile loads of this slot are younger.
@@ -774,11 +724,9 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
 #pragma unroll
       for (int j = 0; j < kTM; ++j) sc[j] = xs[j] * ws;
     }
-    FG_PP_STAMP(4);
     const bool flushed_now = pending;
     if (pending) flush_whole_tile();  // after the waits, so that no wait of this slot covers the stores
     __builtin_amdgcn_s_barrier();
-    FG_PP_STAMP(5);
 
     // ================= multiply(T)
     __builtin_amdgcn_s_setprio(kMultiplyPrio);
@@ -806,12 +754,10 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
       scale_into<4>(acc[(L - 1) / kTM][(L - 1) % kTM], p[(L - 1) % 3], sc[(L - 1) % kTM]);
     }
     __builtin_amdgcn_s_setprio(kFetchPrio);
-    FG_PP_STAMP(6);
     if (grp == 0) {  // A's share of stage T+1 has landed
       if (kRelaxedStoreWaits && flushed_now) wait_vmem<kStoresPerTile>(); else wait_vmem_all();
     }
     flushed_prev = flushed_now;
-    FG_PP_STAMP(7);
     __builtin_amdgcn_s_barrier();
 
     // ================= next step; a finished tile is stored in this wavefront's next fetch slot
@@ -877,15 +823,6 @@ SkPlan plan_stream_k(int64_t tiles, int KB, int cus) {
   SkPlan p = {false, 0, 0, 0, 0};
   const int64_t total = tiles * KB;
   if (cus < 8 || total < cus || total > 0x7FFFFFFF) return p;
-#ifdef FG_DEV_KNOBS
-  if (const char* e = getenv("FG_SK_SPLIT")) {
-    const int S = atoi(e);
-    if (S >= 2 && KB % S == 0 && tiles * S <= cus) {
-      p.use = true; p.grid = (int)(tiles * S); p.q = KB / S; p.r = 0; p.split = S;
-      return p;
-    }
-  }
-#endif
   const int64_t dp_grid = tiles < cus ? tiles : cus;
   const int64_t dp_steps = ceil_div(tiles, dp_grid) * KB;
   const int64_t q = total / cus;
@@ -938,16 +875,10 @@ TailPlan plan_tail(int64_t tiles, int KB, int cus) {
   if (tail == 0 || tail * 4 > cus) return p;
   int64_t S = (cus / 2) / tail;
   if (S > 16) S = 16;
-#ifdef FG_DEV_KNOBS
-  if (const char* e = getenv("FG_TAIL_S")) { S = atoi(e); if (S < 2) return p; }
-#endif
   while (S >= 2 && KB % S != 0) --S;
   if (S < 2 || KB / S < 4) return p;
   const int64_t rounds = ceil_div(tiles, (int64_t)cus);
   const int64_t now = rounds * KB, then = (rounds - 1) * KB + KB / S + tail * S / 4;
-#ifdef FG_DEV_KNOBS
-  if (getenv("FG_TAIL_S") == nullptr)
-#endif
   if (then * 100 > now * 95) return p;
   p.use = true;
   p.full = (int)(tiles - tail); p.tail = (int)tail; p.split = (int)S; p.cut = (int)(KB / S); p.grid = (int)(tail * S);
@@ -1013,19 +944,17 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   const int64_t tiles = (int64_t)a.g.tiles_m * a.g.tiles_n;
   if (tiles > 0x3FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: too many tiles");
   a.n_tiles = (int)tiles;
-  static bool attr_set = false;  // benign if raced
-  if (!attr_set) {
-    for (const void* k : {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false>),
-                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, true>),
-                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false>),
-                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true>),
-                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, false>),
-                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, true>),
-                          reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false, true>)}) {
-      hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-      if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
-    }
-    attr_set = true;
+  static PerDeviceFlags lds_limit_raised[7] = {};
+  const void* const kernels[7] = {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, true>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, false>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, true>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false, true>)};
+  for (int i = 0; i < 7; ++i) {
+    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised[i], kLdsBytes, kernels[i]);
+    if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
   }
   const int cus = cu_count();
   int grid = tiles < cus ? (int)tiles : cus;
@@ -1044,7 +973,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
       (uintptr_t)workspace % 16 == 0 &&
       workspace_bytes >= need + transposed_scales_bytes(g.M, g.KB)) {
     float* const xs_t = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + need);
-    hipLaunchKernelGGL(transpose_scales_kernel, dim3((uint32_t)ceil_div(g.M, 256), (uint32_t)ceil_div(g.KB, kTransposeKbPerBlock)),
+    FG_LAUNCH(transpose_scales_kernel, dim3((uint32_t)ceil_div(g.M, 256), (uint32_t)ceil_div(g.KB, kTransposeKbPerBlock)),
                        dim3(256), 0, stream, g.xs, g.xs_rs, g.xs_cs, g.M, g.KB, xs_t);
     FG_CHECK_LAUNCH("transpose_scales_kernel");
     a.g.xs = xs_t; a.g.xs_rs = 1; a.g.xs_cs = g.M;
@@ -1079,7 +1008,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     PpArgs whole = a;
     whole.n_tiles = tp.full;
     whole.stagger = 0;
-    hipLaunchKernelGGL(kern, dim3((uint32_t)cus), dim3(kThreads), kLdsBytes, stream, whole);
+    FG_LAUNCH(kern, dim3((uint32_t)cus), dim3(kThreads), kLdsBytes, stream, whole);
     FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel (whole rounds)");
     PpArgs rest = a;
     rest.stagger = 0;
@@ -1089,11 +1018,11 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     rest.partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
     void (*shared)(PpArgs) = fp8_gemm_pingpong_kernel<true, kModeBlock, false>;
     if (aligned) shared = fp8_gemm_pingpong_kernel<true, kModeBlock, true>;
-    hipLaunchKernelGGL(shared, dim3((uint32_t)tp.grid), dim3(kThreads), kLdsBytes, stream, rest);
+    FG_LAUNCH(shared, dim3((uint32_t)tp.grid), dim3(kThreads), kLdsBytes, stream, rest);
     FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel (last tiles)");
     return FG_OK;
   }
-  hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
+  FG_LAUNCH(kern, dim3((uint32_t)grid), dim3(kThreads), kLdsBytes, stream, a);
   FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel");
   return FG_OK;
 }

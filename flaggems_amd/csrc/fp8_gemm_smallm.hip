@@ -148,8 +148,9 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
   }
   // A device-scope fence here would write back and invalidate the whole L2 (measured ~50 us per
   // launch).  The partial tiles bypass the L2 on both sides instead, so it is enough that every
-  // store of this block has been acknowledged before the counter moves.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  // store of this block has been acknowledged before the counter moves: every thread waits for its
+  // own stores (a workgroup-scope fence emits no such wait), then the barrier collects the block.
+  wait_vmem_all();
   __syncthreads();
   if (tid == 0) {
     const unsigned int prev = __hip_atomic_fetch_add(&a.counters[chunk], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -171,7 +172,6 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
 
 template <int TMX, int WAVES, int MODE>
 __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_smallm_kernel(SmallArgs a) {
-  constexpr int NT = WAVES * 64;
   constexpr int MROWS = 16 * TMX;
   __shared__ float red[WAVES][MROWS][kChunkRows];  // 4 KB * TMX per wavefront
   __shared__ int last_flag;
@@ -382,8 +382,8 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
 template <int TMX, int WAVES>
 int launch_t(const SmallArgs& sa, int mode, hipStream_t stream) {
   const dim3 grid((uint32_t)(sa.n_chunks * sa.splits), (uint32_t)(sa.g.batch > 1 ? sa.g.batch : 1)), block(WAVES * 64);
-  if (mode == kModeBlock) hipLaunchKernelGGL((fp8_gemm_smallm_kernel<TMX, WAVES, kModeBlock>), grid, block, 0, stream, sa);
-  else hipLaunchKernelGGL((fp8_gemm_smallm_kernel<TMX, WAVES, kModeRowCol>), grid, block, 0, stream, sa);
+  if (mode == kModeBlock) FG_LAUNCH((fp8_gemm_smallm_kernel<TMX, WAVES, kModeBlock>), grid, block, 0, stream, sa);
+  else FG_LAUNCH((fp8_gemm_smallm_kernel<TMX, WAVES, kModeRowCol>), grid, block, 0, stream, sa);
   FG_CHECK_LAUNCH("fp8_gemm_smallm_kernel");
   return FG_OK;
 }
@@ -397,15 +397,13 @@ int launch_transpose(const SmallArgs& sa, int mode, hipStream_t stream) {
   const dim3 grid((uint32_t)(sa.n_chunks * sa.splits), (uint32_t)(sa.g.batch > 1 ? sa.g.batch : 1)), block(WAVES * 64);
   auto kb = fp8_gemm_transpose_kernel<TMX, RG, DEPTH, WAVES, kModeBlock>;
   auto kr = fp8_gemm_transpose_kernel<TMX, RG, DEPTH, WAVES, kModeRowCol>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(kb), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(kr), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e1 != hipSuccess || e2 != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS) failed", kLds);
-    attr_set = true;
+  static PerDeviceFlags lds_limit_raised = {};  // per instantiation
+  {
+    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, kLds, reinterpret_cast<const void*>(kb), reinterpret_cast<const void*>(kr));
+    if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLds, hipGetErrorString(e));
   }
-  if (mode == kModeBlock) hipLaunchKernelGGL(kb, grid, block, kLds, stream, sa);
-  else hipLaunchKernelGGL(kr, grid, block, kLds, stream, sa);
+  if (mode == kModeBlock) FG_LAUNCH(kb, grid, block, kLds, stream, sa);
+  else FG_LAUNCH(kr, grid, block, kLds, stream, sa);
   FG_CHECK_LAUNCH("fp8_gemm_transpose_kernel");
   return FG_OK;
 }

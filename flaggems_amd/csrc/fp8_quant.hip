@@ -147,21 +147,21 @@ int launch_quant(const QuantArgs& a, bool vec_ok, hipStream_t stream, bool silu 
     const bool small = chunks <= kQuantSmallChunks;
     dim3 grid((uint32_t)ceil_div((int64_t)chunks, (int64_t)kQuantThreads * (small ? 1 : kQuantUnrollLarge)));
     if (lpg == 16 && rules == 2) {
-      if (small) hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, 1, true, 2>), grid, dim3(kQuantThreads), 0, stream, a);
-      else hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, true, 2>), grid, dim3(kQuantThreads), 0, stream, a);
+      if (small) FG_LAUNCH((group_quant_vec_kernel<XDT, 16, 1, true, 2>), grid, dim3(kQuantThreads), 0, stream, a);
+      else FG_LAUNCH((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, true, 2>), grid, dim3(kQuantThreads), 0, stream, a);
     } else if (lpg == 16) {
-      if (small) hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, 1, true>), grid, dim3(kQuantThreads), 0, stream, a);
-      else hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, true>), grid, dim3(kQuantThreads), 0, stream, a);
+      if (small) FG_LAUNCH((group_quant_vec_kernel<XDT, 16, 1, true>), grid, dim3(kQuantThreads), 0, stream, a);
+      else FG_LAUNCH((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, true>), grid, dim3(kQuantThreads), 0, stream, a);
     } else {
-      if (small) hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 8, 1, true>), grid, dim3(kQuantThreads), 0, stream, a);
-      else hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 8, kQuantUnrollLarge, true>), grid, dim3(kQuantThreads), 0, stream, a);
+      if (small) FG_LAUNCH((group_quant_vec_kernel<XDT, 8, 1, true>), grid, dim3(kQuantThreads), 0, stream, a);
+      else FG_LAUNCH((group_quant_vec_kernel<XDT, 8, kQuantUnrollLarge, true>), grid, dim3(kQuantThreads), 0, stream, a);
     }
     FG_CHECK_LAUNCH("group_quant_vec_kernel (fused activation)");
     return FG_OK;
   }
   if (lpg == 0) {
     dim3 grid((uint32_t)ceil_div(a.total_groups, kQuantThreads / 64));
-    hipLaunchKernelGGL(group_quant_generic_kernel<XDT>, grid, dim3(kQuantThreads), 0, stream, a);
+    FG_LAUNCH(group_quant_generic_kernel<XDT>, grid, dim3(kQuantThreads), 0, stream, a);
     FG_CHECK_LAUNCH("group_quant_generic_kernel");
     return FG_OK;
   }
@@ -170,11 +170,11 @@ int launch_quant(const QuantArgs& a, bool vec_ok, hipStream_t stream, bool silu 
   dim3 grid((uint32_t)ceil_div((int64_t)chunks, (int64_t)kQuantThreads * (small ? 1 : kQuantUnrollLarge)));
   if (lpg == 16 && rules != 0) {  // group size 128 under either operator's default rules
     if (rules == 1) {
-      if (small) hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, 1, false, 1>), grid, dim3(kQuantThreads), 0, stream, a);
-      else hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, false, 1>), grid, dim3(kQuantThreads), 0, stream, a);
+      if (small) FG_LAUNCH((group_quant_vec_kernel<XDT, 16, 1, false, 1>), grid, dim3(kQuantThreads), 0, stream, a);
+      else FG_LAUNCH((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, false, 1>), grid, dim3(kQuantThreads), 0, stream, a);
     } else {
-      if (small) hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, 1, false, 2>), grid, dim3(kQuantThreads), 0, stream, a);
-      else hipLaunchKernelGGL((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, false, 2>), grid, dim3(kQuantThreads), 0, stream, a);
+      if (small) FG_LAUNCH((group_quant_vec_kernel<XDT, 16, 1, false, 2>), grid, dim3(kQuantThreads), 0, stream, a);
+      else FG_LAUNCH((group_quant_vec_kernel<XDT, 16, kQuantUnrollLarge, false, 2>), grid, dim3(kQuantThreads), 0, stream, a);
     }
     FG_CHECK_LAUNCH("group_quant_vec_kernel");
     return FG_OK;
@@ -182,8 +182,8 @@ int launch_quant(const QuantArgs& a, bool vec_ok, hipStream_t stream, bool silu 
   switch (lpg) {
 #define FG_CASE(L)                                                                                                       \
   case L:                                                                                                                \
-    if (small) hipLaunchKernelGGL((group_quant_vec_kernel<XDT, L, 1>), grid, dim3(kQuantThreads), 0, stream, a);         \
-    else hipLaunchKernelGGL((group_quant_vec_kernel<XDT, L, kQuantUnrollLarge>), grid, dim3(kQuantThreads), 0, stream, a); \
+    if (small) FG_LAUNCH((group_quant_vec_kernel<XDT, L, 1>), grid, dim3(kQuantThreads), 0, stream, a);         \
+    else FG_LAUNCH((group_quant_vec_kernel<XDT, L, kQuantUnrollLarge>), grid, dim3(kQuantThreads), 0, stream, a); \
     break;
     FG_CASE(1) FG_CASE(2) FG_CASE(4) FG_CASE(8) FG_CASE(16) FG_CASE(32) FG_CASE(64)
 #undef FG_CASE
@@ -341,9 +341,9 @@ extern "C" int fg_block_quant_fp8(const void* x, int x_dtype, int64_t rows, int6
   b.rows = (uint32_t)rows; b.cols = (uint32_t)cols;
   b.vec = ((uintptr_t)x % 16 == 0) && ((x_row_stride * esz) % 16 == 0) && ((uintptr_t)q % 8 == 0) && (q_row_stride % 8 == 0);
   const dim3 grid((uint32_t)block_cols_n, (uint32_t)block_rows_n);
-  if (x_dtype == FG_BF16) hipLaunchKernelGGL(block_quant_kernel<FG_BF16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, b);
-  else if (x_dtype == FG_F16) hipLaunchKernelGGL(block_quant_kernel<FG_F16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, b);
-  else hipLaunchKernelGGL(block_quant_kernel<FG_F32>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, b);
+  if (x_dtype == FG_BF16) FG_LAUNCH(block_quant_kernel<FG_BF16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, b);
+  else if (x_dtype == FG_F16) FG_LAUNCH(block_quant_kernel<FG_F16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, b);
+  else FG_LAUNCH(block_quant_kernel<FG_F32>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, b);
   FG_CHECK_LAUNCH("block_quant_kernel");
   return FG_OK;
 }
@@ -486,9 +486,9 @@ extern "C" int fg_silu_mul(const void* x, int x_dtype, int64_t rows, int64_t col
   if (chunks > 0x7FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fg_silu_mul: more than 2^31 chunks");
   const dim3 grid((uint32_t)ceil_div(chunks, (int64_t)kQuantThreads));
   const uint32_t cpr = (uint32_t)(cols / 8), total = (uint32_t)chunks;
-  if (x_dtype == FG_BF16) hipLaunchKernelGGL(silu_mul_kernel<FG_BF16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, x, out, x_row_stride, out_row_stride, up_offset, cpr, total);
-  else if (x_dtype == FG_F16) hipLaunchKernelGGL(silu_mul_kernel<FG_F16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, x, out, x_row_stride, out_row_stride, up_offset, cpr, total);
-  else hipLaunchKernelGGL(silu_mul_kernel<FG_F32>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, x, out, x_row_stride, out_row_stride, up_offset, cpr, total);
+  if (x_dtype == FG_BF16) FG_LAUNCH(silu_mul_kernel<FG_BF16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, x, out, x_row_stride, out_row_stride, up_offset, cpr, total);
+  else if (x_dtype == FG_F16) FG_LAUNCH(silu_mul_kernel<FG_F16>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, x, out, x_row_stride, out_row_stride, up_offset, cpr, total);
+  else FG_LAUNCH(silu_mul_kernel<FG_F32>, grid, dim3(kQuantThreads), 0, (hipStream_t)stream, x, out, x_row_stride, out_row_stride, up_offset, cpr, total);
   FG_CHECK_LAUNCH("silu_mul_kernel");
   return FG_OK;
 }

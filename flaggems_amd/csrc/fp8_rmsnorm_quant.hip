@@ -211,9 +211,9 @@ int launch_norm(const NormQuantArgs& a, int cus, hipStream_t stream) {
                     : (a.q.scale_rule == FG_SCALE_MUL_INV && a.q.quotient_rule == FG_QUOT_DIV && a.q.pow2_rule == FG_POW2_NONE && !a.q.e5m2) ? 2 : 1;
 #define FG_NORM_LAUNCH(C)                                                                                            \
   do {                                                                                                               \
-    if (quant == 0) hipLaunchKernelGGL((rms_norm_quant_kernel<XDT, C, 0>), g, b, 0, stream, a);                      \
-    else if (quant == 1) hipLaunchKernelGGL((rms_norm_quant_kernel<XDT, C, 1>), g, b, 0, stream, a);                 \
-    else hipLaunchKernelGGL((rms_norm_quant_kernel<XDT, C, 2>), g, b, 0, stream, a);                                 \
+    if (quant == 0) FG_LAUNCH((rms_norm_quant_kernel<XDT, C, 0>), g, b, 0, stream, a);                      \
+    else if (quant == 1) FG_LAUNCH((rms_norm_quant_kernel<XDT, C, 1>), g, b, 0, stream, a);                 \
+    else FG_LAUNCH((rms_norm_quant_kernel<XDT, C, 2>), g, b, 0, stream, a);                                 \
   } while (0)
   if (per_thread <= 1) FG_NORM_LAUNCH(1);
   else if (per_thread <= 2) FG_NORM_LAUNCH(2);

@@ -302,11 +302,11 @@ extern "C" int fg_scaled_gemm(const void* A, int64_t lda, const void* B, int64_t
   const dim3 grid((uint32_t)(tiles_m * tiles_n)), block(kGenThreads);
   // 16-bit operands with enough rows to fill tiles go through LDS; fp32 and short problems load straight into registers
   const bool staged = ab_dtype != FG_F32 && M > 32 && K >= kLdsStepElems;
-  if (staged && ab_dtype == FG_BF16) hipLaunchKernelGGL(scaled_gemm_lds_kernel<FG_BF16>, grid, block, 0, (hipStream_t)stream, g);
-  else if (staged) hipLaunchKernelGGL(scaled_gemm_lds_kernel<FG_F16>, grid, block, 0, (hipStream_t)stream, g);
-  else if (ab_dtype == FG_BF16) hipLaunchKernelGGL(scaled_gemm_generic_kernel<FG_BF16>, grid, block, 0, (hipStream_t)stream, g);
-  else if (ab_dtype == FG_F16) hipLaunchKernelGGL(scaled_gemm_generic_kernel<FG_F16>, grid, block, 0, (hipStream_t)stream, g);
-  else hipLaunchKernelGGL(scaled_gemm_generic_kernel<FG_F32>, grid, block, 0, (hipStream_t)stream, g);
+  if (staged && ab_dtype == FG_BF16) FG_LAUNCH(scaled_gemm_lds_kernel<FG_BF16>, grid, block, 0, (hipStream_t)stream, g);
+  else if (staged) FG_LAUNCH(scaled_gemm_lds_kernel<FG_F16>, grid, block, 0, (hipStream_t)stream, g);
+  else if (ab_dtype == FG_BF16) FG_LAUNCH(scaled_gemm_generic_kernel<FG_BF16>, grid, block, 0, (hipStream_t)stream, g);
+  else if (ab_dtype == FG_F16) FG_LAUNCH(scaled_gemm_generic_kernel<FG_F16>, grid, block, 0, (hipStream_t)stream, g);
+  else FG_LAUNCH(scaled_gemm_generic_kernel<FG_F32>, grid, block, 0, (hipStream_t)stream, g);
   FG_CHECK_LAUNCH("scaled_gemm_generic_kernel");
   return FG_OK;
 }

@@ -15,70 +15,41 @@ from .cutlass_scaled_mm import _launch_scaled_gemm, _launch_scaled_generic_gemm,
 
 logger = logging.getLogger("flag_gems." + __name__.split(".")[-1])
 
-SCALAR_SCALE = 0
-VECTOR_SCALE = 1
-
-
-def _resolve_out_dtype(self, out_dtype, out=None):
-    if out_dtype is not None:
-        if out is not None and out.dtype != out_dtype:
-            raise RuntimeError("out_dtype must be the same as the dtype of the provided out tensor")
-        return out_dtype
-    if out is not None:
-        return out.dtype
-    return self.dtype
-
-
-def _normalize_scale(scale, expected_size, *, is_left_scale):
-    if scale.numel() == 1:
-        return scale.reshape(1).contiguous(), SCALAR_SCALE
-    valid = scale.ndim == 1 and scale.shape[0] == expected_size
-    if is_left_scale:
-        valid = valid or (scale.ndim == 2 and tuple(scale.shape) == (expected_size, 1))
-    else:
-        valid = valid or (scale.ndim == 2 and tuple(scale.shape) == (1, expected_size))
-    if valid:
-        return scale.reshape(expected_size).contiguous(), VECTOR_SCALE
-    name = "scale_a" if is_left_scale else "scale_b"
-    shape = f"({expected_size}, 1)" if is_left_scale else f"(1, {expected_size})"
-    raise RuntimeError(f"{name} must be a scalar tensor or have shape {shape}")
-
-
-def _normalize_bias(bias, cols):
-    if bias is None:
-        return None
-    if bias.numel() != cols:
-        raise RuntimeError(f"Bias must be size {cols} but got {bias.numel()}")
-    return bias.reshape(cols).contiguous()
-
-
-def _check_inputs(self, mat2):
-    if self.ndim != 2:
-        raise RuntimeError("self must be a matrix")
-    if mat2.ndim != 2:
-        raise RuntimeError("mat2 must be a matrix")
-    if self.shape[1] != mat2.shape[0]:
+def _scale_vector(scale, count, name, matrix_shape):
+    """One scale (any tensor with a single element) or `count` of them, given as ``[count]`` or as the
+    matrix-shaped column / row ``matrix_shape``; returned as a contiguous 1-D tensor.  The launchers tell the two
+    kinds apart by the element count.  Error text: src/flag_gems/ops/scaled_mm.py:245-249."""
+    if scale.numel() != 1 and tuple(scale.shape) not in ((count,), matrix_shape):
         raise RuntimeError(
-            f"mat1 and mat2 shapes cannot be multiplied ({self.shape[0]}x{self.shape[1]} "
-            f"and {mat2.shape[0]}x{mat2.shape[1]})"
+            f"{name} must be a scalar tensor or have shape ({matrix_shape[0]}, {matrix_shape[1]})"
         )
-    if self.dtype != mat2.dtype:
-        raise RuntimeError(f"self and mat2 must have the same dtype, but got {self.dtype} and {mat2.dtype}")
+    return scale.reshape(-1).contiguous()
 
 
 def _scaled_mm_impl(self, mat2, scale_a, scale_b, bias, out_dtype, out):
-    _check_inputs(self, mat2)
-    M, K = self.shape
-    _, N = mat2.shape
-    output_dtype = _resolve_out_dtype(self, out_dtype, out)
+    # argument errors in the reference's order and wording (src/flag_gems/ops/scaled_mm.py:214-273, 350-351)
+    for name, operand in (("self", self), ("mat2", mat2)):
+        if operand.dim() != 2:
+            raise RuntimeError(f"{name} must be a matrix")
+    (M, K), (K2, N) = self.shape, mat2.shape
+    if K != K2:
+        raise RuntimeError(f"mat1 and mat2 shapes cannot be multiplied ({M}x{K} and {K2}x{N})")
+    if self.dtype != mat2.dtype:
+        raise RuntimeError(f"self and mat2 must have the same dtype, but got {self.dtype} and {mat2.dtype}")
+    # result type: the explicit out_dtype, else that of the tensor to fill, else the operands'
     if out is None:
-        out = torch.empty((M, N), dtype=output_dtype, device=self.device)
-    elif tuple(out.shape) != (M, N):
-        raise RuntimeError("Incompatible output shape")
-
-    scale_a, _ = _normalize_scale(scale_a, M, is_left_scale=True)
-    scale_b, _ = _normalize_scale(scale_b, N, is_left_scale=False)
-    bias = _normalize_bias(bias, N)
+        out = torch.empty((M, N), dtype=out_dtype if out_dtype is not None else self.dtype, device=self.device)
+    else:
+        if out_dtype is not None and out.dtype != out_dtype:
+            raise RuntimeError("out_dtype must be the same as the dtype of the provided out tensor")
+        if tuple(out.shape) != (M, N):
+            raise RuntimeError("Incompatible output shape")
+    scale_a = _scale_vector(scale_a, M, "scale_a", (M, 1))
+    scale_b = _scale_vector(scale_b, N, "scale_b", (1, N))
+    if bias is not None:
+        if bias.numel() != N:
+            raise RuntimeError(f"Bias must be size {N} but got {bias.numel()}")
+        bias = bias.reshape(N).contiguous()
     if M == 0 or N == 0:
         return out
 

@@ -3,6 +3,7 @@
 Mirrors the reference entry points
   w8a8_block_fp8_matmul  src/flag_gems/ops/w8a8_block_fp8_matmul.py:173-232
   fp8_matmul             src/flag_gems/ops/fp8_matmul.py:137-205
+  fp8_matmul_noop        cpp/lib/fp8_matmul.cpp:104-125 (checks and allocation only: a probe of the host overhead)
 with the same parameters, defaults and assertions.  The reference picks a Triton tile from a
 per-device YAML table; here the C library picks the HIP kernel variant from (M, N, K).
 """
@@ -122,3 +123,19 @@ def fp8_matmul(
         return C.view(out_shape)
     _launch_block_gemm(a.view(M, K), b, a_s.view(M, -1), b_s, C, GROUP_SIZE, GROUP_SIZE)
     return C.view(out_shape)
+
+
+def fp8_matmul_noop(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Tensor) -> torch.Tensor:
+    """Everything ``fp8_matmul`` does on the host and nothing on the device: the same checks, the same
+    allocation, no launch.  The returned bf16 tensor ``[..., N]`` is uninitialised.  Timing it next to
+    ``fp8_matmul`` separates the binding's overhead from the kernel's launch."""
+    assert b.ndim == 2, "b must be 2D"
+    assert a.is_contiguous() and b.is_contiguous(), "a and b must be contiguous"
+    assert a_s.is_contiguous() and b_s.is_contiguous(), "a_s and b_s must be contiguous"
+    K = a.size(-1)
+    M = a.numel() // K if K else 0
+    N = b.size(0)
+    assert b.size(1) == K, "a and b must have the same K dimension"
+    a_s.view(M, -1)  # the scales must fold to one row per activation row, as the launch would require
+    C = torch.empty((M, N), device=a.device, dtype=torch.bfloat16)
+    return C.view(*a.size()[:-1], N)

@@ -66,6 +66,14 @@ int fg_version(void);
 const char* fg_last_error_string(void);
 
 /*
+ * Capture state of a stream: 0 when `stream` is not being captured into a HIP graph, otherwise a non-zero id of the
+ * capture in progress.  No reference counterpart (the reference leaves graph capture to PyTorch); the Python binding
+ * uses it to decide which workspace buffer a launch may be given: a buffer allocated inside a capture belongs to that
+ * graph only, and a buffer a captured launch has seen must never be released.
+ */
+unsigned long long fg_stream_capture_id(void* stream);
+
+/*
  * Per-token-group FP8 quantization: for every row r and every group g of `group_size`
  * consecutive columns,
  *     amax  = max |x[r, g*G : (g+1)*G]|          (NaN propagates)

@@ -290,3 +290,74 @@ def test_fast_index_division_is_exact():
     n = np.minimum(k * d + rng.integers(-1, 2, 500_000), top)
     q, r = fast(n, d)
     assert np.array_equal(q, n // d) and np.array_equal(r, n % d)
+
+
+# ---- DeepGEMM-style helpers (inputs of the batched GEMM and of the weight quantizer)
+
+
+def test_ceil_to_ue8m0_is_the_least_power_of_two_not_below():
+    """The smallest power of two >= |s|, held in [2^-126, 2^127]: checked with math.frexp (no bit tricks) on
+    random scales over the whole exponent range, on exact powers of two (which must map to themselves: a floor
+    would pass "is a power of two" but not this), on their neighbours, and at the clamp edges."""
+    import math
+
+    rng = np.random.default_rng(3)
+    s = (np.exp2(rng.uniform(-126, 127, 20000)) * rng.choice([-1.0, 1.0], 20000)).astype(np.float32)
+    pw = np.exp2(np.arange(-126, 128)).astype(np.float32)
+    up = np.nextafter(pw, np.float32(np.inf)).astype(np.float32)
+    down = np.nextafter(pw, np.float32(0)).astype(np.float32)
+    vals = np.concatenate([s, pw, -pw, up, down[1:]])
+    got = O._ceil_to_ue8m0(torch.from_numpy(vals)).numpy()
+    for v, g in zip(vals.tolist(), got.tolist()):
+        m, e = math.frexp(abs(v))                 # |v| = m * 2^e, 0.5 <= m < 1
+        want = 2.0 ** (e - 1) if m == 0.5 else 2.0 ** e
+        want = min(max(want, 2.0 ** -126), 2.0 ** 127)
+        assert g == want, (v, g, want)
+        assert g >= min(abs(v), 2.0 ** 127) and (g < 2 * abs(v) or g == 2.0 ** -126)
+    # clamp edges: zero and subnormals go to the smallest normal, Inf and NaN (exponent field 255) to 2^127
+    edge = torch.tensor([0.0, -0.0, 1e-45, 1.1e-38, float("inf"), float("-inf"), float("nan"), 3.4e38])
+    out = O._ceil_to_ue8m0(edge).tolist()
+    assert out[:4] == [2.0 ** -126] * 4 and out[4:] == [2.0 ** 127] * 4
+
+
+@pytest.mark.parametrize("use_ue8m0", [False, True])
+def test_per_token_cast_codes_vs_brute_force(use_ue8m0):
+    """Codes and scales of per_token_cast_to_fp8_ref against numpy scalar arithmetic and the bit-level encoder:
+    ragged last group (zero padding takes part in no maximum that matters and yields no code), both scale kinds."""
+    x = _rand_bf16(6, 300, 21, "wide")
+    xq, sf = O.per_token_cast_to_fp8_ref(x, use_ue8m0=use_ue8m0)
+    assert xq.shape == (6, 300) and sf.shape == (6, 3)
+    xn = x.float().numpy()
+    for r in range(6):
+        for g in range(3):
+            seg = xn[r, g * 128 : min((g + 1) * 128, 300)]
+            amax = max(F32(np.abs(seg).max()), F32(1e-4))
+            s = F32(amax) / F32(448.0)
+            if use_ue8m0:
+                m, e = np.frexp(s)
+                s = F32(np.ldexp(1.0, e - 1 if m == 0.5 else e))
+            assert sf[r, g].item() == s
+            codes = e4m3.encode((seg * (F32(1.0) / s)).astype(np.float32))
+            assert np.array_equal(codes, xq.view(torch.uint8).numpy()[r, g * 128 : g * 128 + seg.size])
+
+
+def test_per_block_cast_ue8m0_vs_brute_force():
+    """The use_ue8m0=True branch of per_block_cast_to_fp8_ref, as test_per_block_cast_vs_brute_force does for the
+    other: scale = least power of two >= amax / 448 (frexp, not the oracle's bit test), codes from the bit-level
+    encoder of the fp32 products."""
+    g = torch.Generator().manual_seed(18)
+    w = (0.02 * torch.randn(200, 300, generator=g) * torch.logspace(-2, 1, 300)).bfloat16()
+    wq, ws = O.per_block_cast_to_fp8_ref(w, use_ue8m0=True)
+    assert wq.shape == (200, 300) and ws.shape == (2, 3)
+    wn = w.float().numpy()
+    for bi in range(2):
+        for bj in range(3):
+            blk = wn[bi * 128 : (bi + 1) * 128, bj * 128 : (bj + 1) * 128]
+            amax = max(F32(np.abs(blk).max()), F32(1e-4))
+            s = F32(amax) / F32(448.0)
+            m, e = np.frexp(s)
+            s = F32(np.ldexp(1.0, e - 1 if m == 0.5 else e))
+            assert ws[bi, bj].item() == s
+            codes = e4m3.encode((blk * (F32(1.0) / s)).astype(np.float32))
+            got = wq.view(torch.uint8).numpy()[bi * 128 : (bi + 1) * 128, bj * 128 : (bj + 1) * 128]
+            assert np.array_equal(codes, got)
