@@ -23,6 +23,7 @@ FG_SCALE_MUL_INV, FG_SCALE_DIV = 0, 1
 FG_QUOT_RECIP_MUL, FG_QUOT_DIV = 0, 1
 FG_POW2_NONE, FG_POW2_BITS, FG_POW2_LOG2, FG_POW2_BITS_CLAMPED = 0, 1, 2, 3
 FG_WORKSPACE_COUNTER_BYTES = 16384
+FG_NOALLOC_SCRATCH_BYTES = 32 << 20
 
 DTYPE_CODE = {
     torch.bfloat16: FG_BF16,
@@ -66,6 +67,11 @@ SIGNATURES = {
          c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p],
     ),
     "fg_block_fp8_gemm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
+    "fg_block_fp8_gemm_noalloc": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
+         c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p],
+    ),
     "fg_batched_block_fp8_gemm": (
         c_int,
         [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64,

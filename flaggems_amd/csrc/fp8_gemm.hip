@@ -18,6 +18,8 @@
 
 #include "fp8_gemm_common.h"
 
+#include <mutex>
+
 namespace fg {
 namespace {
 
@@ -657,6 +659,80 @@ extern "C" int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int6
   a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)ceil_div(K, 128);
   a.c_dtype = c_dtype;
   return launch_gemm<kModeBlock>(a, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// fg_block_fp8_gemm for callers that cannot allocate: the workspace is a device array built into the library.
+// ---------------------------------------------------------------------------------------------
+namespace fg {
+namespace {
+
+constexpr size_t kScratchBytes = FG_NOALLOC_SCRATCH_BYTES;
+// Counters (first FG_WORKSPACE_COUNTER_BYTES), split-K partial sums and transposed activation scales of the
+// launches made through fg_block_fp8_gemm_noalloc.  One copy per GPU, at an address of its own on each; in host
+// code the name is only a handle for hipGetSymbolAddress.
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+__global__ __launch_bounds__(256) void clear_counters_kernel(uint32_t* p, int n) {
+  const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+  if (i < n) p[i] = 0u;
+}
+
+// device address of `scratch` on each device, looked up on the first call made with that device current
+struct ScratchTable {
+  std::mutex lock;
+  void* ptr[kMaxDevices] = {};
+};
+ScratchTable& scratch_table() {
+  static ScratchTable t;
+  return t;
+}
+
+// Address of the current device's copy (looked up once per device).  On the first use the counter area is cleared
+// by a kernel on the caller's stream, ahead of the launch that follows: a fill kernel, not a memset, so that the
+// call may be recorded into a graph.
+int scratch_of_current_device(hipStream_t stream, void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "fg_block_fp8_gemm_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) FG_FAIL(FG_ERR_UNSUPPORTED, "fg_block_fp8_gemm_noalloc: device index %d (at most %d devices)", dev, kMaxDevices);
+  ScratchTable& t = scratch_table();
+  std::lock_guard<std::mutex> guard(t.lock);
+  if (t.ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      FG_FAIL(FG_ERR_LAUNCH, "fg_block_fp8_gemm_noalloc: hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    constexpr int kWords = FG_WORKSPACE_COUNTER_BYTES / 4;
+    FG_LAUNCH(clear_counters_kernel, dim3(kWords / 256), dim3(256), 0, stream, reinterpret_cast<uint32_t*>(p), kWords);
+    FG_CHECK_LAUNCH("clear_counters_kernel");
+    t.ptr[dev] = p;
+  }
+  *out = t.ptr[dev];
+  return FG_OK;
+}
+
+}  // namespace
+}  // namespace fg
+
+extern "C" int fg_block_fp8_gemm_noalloc(const void* A, int64_t lda, const void* B, int64_t ldb,
+                                         const float* As, int64_t as_row_stride, int64_t as_col_stride,
+                                         const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride,
+                                         void* C, int64_t ldc, int c_dtype,
+                                         int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k, void* stream) {
+  using namespace fg;
+  if (M < 0 || N < 0 || K < 0) FG_FAIL(FG_ERR_INVALID_ARG, "fg_block_fp8_gemm_noalloc: negative size");
+  const size_t need = fg_block_fp8_gemm_workspace_bytes(M, N, K);
+  if (need > kScratchBytes)
+    FG_FAIL(FG_ERR_WORKSPACE,
+            "fg_block_fp8_gemm_noalloc: M = %lld, N = %lld, K = %lld wants %zu bytes of workspace and the built-in buffer has "
+            "%zu; call fg_block_fp8_gemm with a workspace of the caller's",
+            (long long)M, (long long)N, (long long)K, need, kScratchBytes);
+  void* ws = nullptr;
+  const int rc = scratch_of_current_device((hipStream_t)stream, &ws);
+  if (rc != FG_OK) return rc;
+  return fg_block_fp8_gemm(A, lda, B, ldb, As, as_row_stride, as_col_stride, Bs, bs_row_stride, bs_col_stride, C, ldc, c_dtype,
+                           M, N, K, block_n, block_k, ws, kScratchBytes, stream);
 }
 
 extern "C" size_t fg_batched_block_fp8_gemm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K) {

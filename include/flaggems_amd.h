@@ -222,6 +222,25 @@ int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
 size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
+ * fg_block_fp8_gemm without the workspace arguments, for callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose
+ * wrappers allocate through torch).  The workspace is an array of FG_NOALLOC_SCRATCH_BYTES built into the library's
+ * device code, one copy per GPU, held until the process ends; the call allocates nothing and frees nothing.  Same
+ * kernels and same results as fg_block_fp8_gemm given a workspace of that size.  A shape for which
+ * fg_block_fp8_gemm_workspace_bytes(M, N, K) exceeds FG_NOALLOC_SCRATCH_BYTES is refused with FG_ERR_WORKSPACE (use
+ * fg_block_fp8_gemm with a workspace of the caller's).  All calls on one GPU share that GPU's array: calls that may
+ * overlap on one GPU (two streams, two threads) race on the counters and partial sums and must be serialised by the
+ * caller.  The first call on a device looks the array's address up and clears its counter area with a kernel on
+ * `stream`; every launch leaves the counters zero for the next.
+ */
+#define FG_NOALLOC_SCRATCH_BYTES (32u << 20)
+int fg_block_fp8_gemm_noalloc(const void* A, int64_t lda, const void* B, int64_t ldb,
+                              const float* As, int64_t as_row_stride, int64_t as_col_stride,
+                              const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride,
+                              void* C, int64_t ldc, int c_dtype,
+                              int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k, void* stream);
+
+/*
  * Batched block-scaled FP8 GEMM: `batch` independent problems of fg_block_fp8_gemm with the same M, N, K and
  * strides.  Matrix i of each operand starts i * <its batch stride> after matrix 0 (bytes for A and B, floats for
  * the scales, elements of c_dtype for C); row strides are free, so a [b, h, r] activation with h as the batch
