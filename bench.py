@@ -3,7 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One step = one pass over the DeepSeek-V3 block-fp8 GEMM sweep that the headline metric is quoted on:
+One step = SWEEPS_PER_STEP (16) passes over the DeepSeek-V3 block-fp8 GEMM sweep that the headline metric is quoted on
+(a single pass takes about 2 ms, so 20 steps of one pass would be a 40 ms timed region):
 M in {1, 8, 64, 512, 2048, 4096} x (N, K) in {(2112,7168), (24576,1536), (32768,512), (7168,16384),
 (4608,7168), (7168,2304)}, e4m3fn operands already resident in HBM (1x128 activation scales,
 128x128 weight scales, bf16 output).  `value` is the sweep's total 2*M*N*K divided by the wall
@@ -39,7 +40,11 @@ PEAK_FP8_TFLOPS = 5000.0  # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E, published
 DSV3_NK = [(2112, 7168), (24576, 1536), (32768, 512), (7168, 16384), (4608, 7168), (7168, 2304)]
 DSV3_M = [1, 8, 64, 512, 2048, 4096]
+DETAIL_M = [1, 8, 16, 64, 512, 2048, 4096]  # per-shape timings also cover M = 16 (decode bar: M <= 16)
 CACHE_BYTES = 512 << 20   # rotate small-M weights through at least this much memory
+SWEEPS_PER_STEP = 16      # passes over the 36-GEMM sweep in one step
+LAUNCHES = 100            # back-to-back launches per timed graph replay
+REPEATS = 6               # timed replays per shape; the first is dropped, the median of the other five is reported
 
 # Bytes that crossed the L2 <-> memory-fabric boundary in one M = 4096 call (the persistent kernel and, where the
 # call makes one, the transposition of the activation scales before it), from two
@@ -125,7 +130,7 @@ def main():
         copies = max(1, -(-CACHE_BYTES // (n * k)))
         pool = [(wq, ws)] + [(wq.clone(), ws.clone()) for _ in range(copies - 1)]
         weights[(n, k)] = pool
-        for m in DSV3_M:
+        for m in DETAIL_M:
             if (m, k) not in acts:
                 x = torch.randn(m, k, device=dev, generator=gen).bfloat16()
                 acts[(m, k)] = flag_gems.act_quant_triton(x, 128)
@@ -135,7 +140,7 @@ def main():
 
     def run_one(m, n, k, rot):
         pool = weights[(n, k)]
-        wq, ws = pool[rot % len(pool)] if m <= 64 else pool[0]
+        wq, ws = pool[rot % len(pool)] if m <= 128 else pool[0]
         xq, xs = acts[(m, k)]
         return flag_gems.w8a8_block_fp8_matmul(xq, wq, xs, ws, [128, 128])
 
@@ -174,42 +179,54 @@ def main():
             step_graphs.append(g)
     torch.cuda.synchronize()
 
+    def run_step(i):
+        for r in range(SWEEPS_PER_STEP):
+            step_graphs[(i * SWEEPS_PER_STEP + r) % NG].replay()
+
     for i in range(args.warmup):
-        step_graphs[i % NG].replay()
+        run_step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step_graphs[i % NG].replay()
+        run_step(i)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
-    total_flops = sum(gemm_flops(*c) for c in calls)
+    total_flops = SWEEPS_PER_STEP * sum(gemm_flops(*c) for c in calls)
     value = total_flops / (ms_per_step * 1e-3) / 1e12
 
-    # ---- per-shape kernel time: HIP events (on the replay stream) around a graph of `reps` launches
-    detail = []
-    for (m, n, k) in calls:
-        reps = 10 if m >= 512 else 40
+    # ---- per-shape kernel time: HIP events (on the replay stream) around a graph of LAUNCHES back-to-back launches,
+    # REPEATS replays, the first dropped, median of the rest
+    def time_graph(fn_of_launch, launches=LAUNCHES, repeats=REPEATS):
         with torch.cuda.stream(side):
+            fn_of_launch(0)
+            fn_of_launch(1)
+            torch.cuda.synchronize()
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=side):
-                for r in range(reps):
-                    run_one(m, n, k, r)
+                for r in range(launches):
+                    fn_of_launch(r)
         torch.cuda.synchronize()
         times = []
-        for _ in range(4):
+        for _ in range(repeats):
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record()
             g.replay()
             end.record()
             end.synchronize()
-            times.append(start.elapsed_time(end) * 1e3 / reps)
-        us = sorted(times[1:])[1]  # median of the last three replays
+            times.append(start.elapsed_time(end) * 1e3 / launches)
         del g
-        tf = gemm_flops(m, n, k) / (us * 1e-6) / 1e12
-        gbs = gemm_bytes(m, n, k) / (us * 1e-6) / 1e9
-        detail.append({"M": m, "N": n, "K": k, "us": round(us, 2), "tflops": round(tf, 1), "gbps": round(gbs, 1),
-                       "frac_mfma": round(tf / PEAK_FP8_TFLOPS, 4), "frac_hbm": round(gbs / PEAK_HBM_GBPS, 4)})
+        rest = sorted(times[1:])
+        return rest[len(rest) // 2]
+
+    detail = []
+    for (n, k) in DSV3_NK:
+        for m in DETAIL_M:
+            us = time_graph(lambda r: run_one(m, n, k, r))
+            tf = gemm_flops(m, n, k) / (us * 1e-6) / 1e12
+            gbs = gemm_bytes(m, n, k) / (us * 1e-6) / 1e9
+            detail.append({"M": m, "N": n, "K": k, "us": round(us, 2), "tflops": round(tf, 1), "gbps": round(gbs, 1),
+                           "frac_mfma": round(tf / PEAK_FP8_TFLOPS, 4), "frac_hbm": round(gbs / PEAK_HBM_GBPS, 4)})
 
     big = [d for d in detail if d["M"] == 4096]
     big_flops = sum(gemm_flops(d["M"], d["N"], d["K"]) for d in big)
@@ -218,17 +235,19 @@ def main():
     traffic = sum(f + w for (f, w) in TRAFFIC_M4096_KIB.values()) * 1024.0 / len(TRAFFIC_M4096_KIB)
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": round(traffic),
-                "traffic_unit": "bytes per launch (mean of the six launches; counters of an earlier run)",
+                "traffic_unit": "bytes per launch, mean of the six launches",
+                "traffic_source": "profiles/fp8_gemm_dsv3_hbm_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of "
+                                  "`bench.py --counter-pass`, scaled by a 256 MiB copy in the same run; not re-measured in this run)",
                 "flops_per_launch": big_flops / len(big), "algorithmic_bytes_per_launch":
                     sum(gemm_bytes(d["M"], d["N"], d["K"]) for d in big) / len(big),
                 "avg_launch_us": round(big_time * 1e6 / len(big), 2),
                 "kernel": "fp8_gemm_pingpong_kernel (with the scale transposition that precedes it), the six M=4096 calls of the sweep"}
-    small = [d for d in detail if d["M"] <= 8]
+    small = [d for d in detail if d["M"] <= 16]
     small_bytes = sum(gemm_bytes(d["M"], d["N"], d["K"]) for d in small)
     small_time = sum(d["us"] for d in small) * 1e-6
     roofline_small = {"bound": "hbm", "achieved": round(small_bytes / small_time / 1e9, 1), "peak": PEAK_HBM_GBPS,
                       "unit": "GB/s", "frac": round(small_bytes / small_time / 1e9 / PEAK_HBM_GBPS, 4),
-                      "kernel": "the twelve M in {1, 8} launches of the sweep, weights rotated through 512 MB"}
+                      "kernel": "the eighteen M in {1, 8, 16} launches of the six DSv3 (N,K), weights rotated through 512 MB"}
 
     # ---- quantizer (HBM bound): act_quant on bf16 [4096, 7168]
     xq_in = torch.randn(4096, 7168, device=dev, generator=gen).bfloat16()
@@ -305,25 +324,7 @@ def main():
     # ---- the other configurations of the path, each shape timed alone: HIP events around the replay of a graph
     # of `reps` launches (as above: decode-sized launches are shorter than a Python call)
     def time_eager(fn, reps):
-        with torch.cuda.stream(side):
-            for _ in range(2):
-                fn()
-            torch.cuda.synchronize()
-            gr = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(gr, stream=side):
-                for _ in range(reps):
-                    fn()
-        torch.cuda.synchronize()
-        ts = []
-        for _ in range(3):
-            s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            s_.record()
-            gr.replay()
-            e_.record()
-            e_.synchronize()
-            ts.append(s_.elapsed_time(e_) * 1e3 / reps)
-        del gr
-        return sorted(ts)[1]
+        return time_graph(lambda r: fn(), launches=max(reps, 20))
 
     # cutlass_scaled_mm semantics: per-token x per-channel scales, bf16 bias, N = K = 8192
     scaled = []
@@ -374,22 +375,29 @@ def main():
                        "frac_hbm": round(nbytes / us / 1e3 / PEAK_HBM_GBPS, 4)})
     del ey, eys, ex, exs
 
-    # Llama-3-8B linears: GEMM alone and act_quant + GEMM from bf16 activations
+    # Llama-3-8B linears: GEMM alone and act_quant + GEMM from bf16 activations; for M <= 128 every launch reads another
+    # copy of the weights out of a pool of at least 512 MB, as in the sweep above
     llama = []
     for (n, k) in [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]:
         wq, ws = make_weight(n, k, gen, dev)
+        copies = max(1, -(-CACHE_BYTES // (n * k)))
+        pool = [wq] + [wq.clone() for _ in range(copies - 1)]
         for m in (1, 16, 128, 1024, 4096):
             x = torch.randn(m, k, device=dev, generator=gen).bfloat16()
             xq, xs = flag_gems.act_quant_triton(x, 128)
-            reps = 10 if m >= 1024 else 30
-            us_g = time_eager(lambda: flag_gems.w8a8_block_fp8_matmul(xq, wq, xs, ws, [128, 128]), reps)
-            def e2e():
+            use = pool if m <= 128 else pool[:1]
+            launches = LAUNCHES if m <= 1024 else 20
+            us_g = time_graph(lambda r: flag_gems.w8a8_block_fp8_matmul(xq, use[r % len(use)], xs, ws, [128, 128]), launches)
+
+            def e2e(r):
                 q, s2 = flag_gems.act_quant_triton(x, 128)
-                return flag_gems.w8a8_block_fp8_matmul(q, wq, s2, ws, [128, 128])
-            us_e = time_eager(e2e, reps)
+                return flag_gems.w8a8_block_fp8_matmul(q, use[r % len(use)], s2, ws, [128, 128])
+
+            us_e = time_graph(e2e, launches)
             llama.append({"M": m, "N": n, "K": k, "gemm_us": round(us_g, 2), "quant_gemm_us": round(us_e, 2),
-                          "tflops": round(gemm_flops(m, n, k) / us_g / 1e6, 1), "gbps": round(gemm_bytes(m, n, k) / us_g / 1e3, 1)})
-        del wq, ws
+                          "tflops": round(gemm_flops(m, n, k) / us_g / 1e6, 1), "gbps": round(gemm_bytes(m, n, k) / us_g / 1e3, 1),
+                          "weight_copies": len(use)})
+        del wq, ws, pool
 
     # Mixtral-8x7B expert layers: grouped block-fp8 GEMM over rows sorted by expert
     moe = []
@@ -411,8 +419,9 @@ def main():
                         "frac_mfma": round(tf / PEAK_FP8_TFLOPS, 4), "frac_hbm": round(nbytes / us / 1e3 / PEAK_HBM_GBPS, 4)})
         del wq, ws
 
-    # ---- CPU baseline: the oracle on the host cores, bounded sample
+    # ---- CPU baseline: the oracle on the host cores, bounded samples
     cpu = None
+    cpu_configs = None
     if not args.no_cpu:
         from oracle import fp8_linear_oracle as O
 
@@ -425,7 +434,7 @@ def main():
             xq, xs = acts[(4096, k)]
             wq, ws = weights[(n, k)][0]
             cpu_in.append((n, k, xq[:sample_m].cpu(), xs[:sample_m].cpu(), wq.cpu(), ws.cpu()))
-        while cpu_time < 12.0 and passes < 8:  # whole passes over the six GEMMs, about 10-30 s in all
+        while cpu_time < 10.0 and passes < 8:  # whole passes over the six GEMMs
             for (n, k, a, a_s, b, b_s) in cpu_in:
                 t0 = time.perf_counter()
                 O.block_fp8_matmul_tiled_ref(a, b, a_s, b_s, [128, 128], torch.bfloat16)
@@ -435,6 +444,43 @@ def main():
         cpu = {"value": round(cpu_flops / cpu_time / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                "sample": f"oracle block_fp8_matmul_tiled_ref (per-K-tile fp32 matmul, torch CPU) on the M={sample_m} "
                          f"GEMMs of the six DSv3 (N,K) shapes, {passes} passes, {cpu_time:.1f} s"}
+
+        # the other configurations on the host, each timed once after one warm-up call (decode-sized M only: larger
+        # ones take seconds per call on a CPU and say nothing new)
+        def cpu_time_of(fn):
+            fn()
+            t0 = time.perf_counter()
+            fn()
+            return time.perf_counter() - t0
+
+        cpu_configs = []
+        x1, w1 = O.make_config1(0)
+        t = cpu_time_of(lambda: O.run_config1(0))
+        cpu_configs.append({"config": "1: act_quant + 128x128 weight quantizer + block-fp8 GEMM, M=64 N=512 K=1024, end to end",
+                            "ms": round(t * 1e3, 3), "tflops": round(gemm_flops(64, 512, 1024) / t / 1e12, 5)})
+        del x1, w1
+        for (n, k, a, a_s, b, b_s) in cpu_in:
+            m = 64
+            t = cpu_time_of(lambda: O.block_fp8_matmul_tiled_ref(a[:m], b, a_s[:m], b_s, [128, 128], torch.bfloat16))
+            cpu_configs.append({"config": f"3: DSv3 block-fp8 GEMM M={m} N={n} K={k}", "ms": round(t * 1e3, 3),
+                                "tflops": round(gemm_flops(m, n, k) / t / 1e12, 5)})
+        del cpu_in
+        gcpu = torch.Generator().manual_seed(0)
+        for (n, k) in [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]:
+            m = 128
+            xq_c, xs_c = O.act_quant_ref(torch.randn(m, k, generator=gcpu).bfloat16(), 128)
+            wq_c, ws_c = O.per_block_cast_to_fp8_ref((0.02 * torch.randn(n, k, generator=gcpu)).bfloat16())
+            t = cpu_time_of(lambda: O.block_fp8_matmul_tiled_ref(xq_c, wq_c, xs_c, ws_c, [128, 128], torch.bfloat16))
+            cpu_configs.append({"config": f"2: Llama-3-8B linear M={m} N={n} K={k}", "ms": round(t * 1e3, 3),
+                                "tflops": round(gemm_flops(m, n, k) / t / 1e12, 5)})
+        m, nk_c = 32, 8192
+        a_c = torch.randn(m, nk_c, generator=gcpu).clamp(-448, 448).to(torch.float8_e4m3fn)
+        b_c = torch.randn(nk_c, nk_c, generator=gcpu).clamp(-448, 448).to(torch.float8_e4m3fn).t()
+        sa_c, sb_c = torch.rand(m, 1, generator=gcpu), torch.rand(1, nk_c, generator=gcpu)
+        bias_c = torch.randn(nk_c, generator=gcpu).bfloat16()
+        t = cpu_time_of(lambda: O.scaled_mm_ref(a_c, b_c, sa_c, sb_c, torch.bfloat16, bias_c))
+        cpu_configs.append({"config": f"4: cutlass_scaled_mm M={m} N={nk_c} K={nk_c} with bias", "ms": round(t * 1e3, 3),
+                            "tflops": round(gemm_flops(m, nk_c, nk_c) / t / 1e12, 5)})
 
     out = {
         "metric": "block_fp8_gemm_tflops",
@@ -450,9 +496,11 @@ def main():
         "dtype": "fp8_e4m3fn x fp8_e4m3fn -> f32 accumulate -> bf16",
         "data": "synthetic",
         "config": {"workload": "DeepSeek-V3 block-fp8 GEMM sweep: M in {1,8,64,512,2048,4096} x 6 (N,K); "
-                               "1x128 activation scales, 128x128 weight scales, bf16 out; one step = all 36 GEMMs, replayed from a HIP graph",
+                               "1x128 activation scales, 128x128 weight scales, bf16 out; one step = 16 passes over all 36 GEMMs, each pass one HIP graph replay "
+                               "(weights of the M <= 64 calls rotated through 512 MB)",
+                   "sweeps_per_step": SWEEPS_PER_STEP,
                    "pct_fp8_mfma_peak_at_M4096": round(100 * achieved / PEAK_FP8_TFLOPS, 2),
-                   "pct_hbm_at_M_le_8": round(100 * roofline_small["frac"], 2)},
+                   "pct_hbm_at_M_le_16": round(100 * roofline_small["frac"], 2)},
         "roofline": roofline,
         "roofline_small_m": roofline_small,
         "quantizer": quant,
@@ -465,6 +513,7 @@ def main():
         "llama3_8b_linears": llama,
         "mixtral_moe_grouped_gemm": moe,
         "cpu_baseline": cpu,
+        "cpu_baseline_other_configs": cpu_configs,
         "detail": detail,
     }
     print(json.dumps(out), flush=True)

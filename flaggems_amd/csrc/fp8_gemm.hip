@@ -19,6 +19,9 @@
 #include "fp8_gemm_common.h"
 
 #include <mutex>
+#ifdef FG_DEV_KNOBS
+#include <stdlib.h>
+#endif
 
 namespace fg {
 namespace {
@@ -162,14 +165,41 @@ __device__ __forceinline__ void scale_accumulate(v4f& acc, const v4f& p, float s
   acc[0] = a0; acc[1] = a1; acc[2] = a2; acc[3] = a3;
 }
 
-template <int BM, int BN, int WM, int WN>
+// Global -> LDS copies the compiler does not see (it would otherwise order every later LDS read behind them):
+// 16 bytes per lane to lds_addr + 16 * lane, or 4 bytes per lane to lds_addr + 4 * lane.  `base` and `lds_addr`
+// are wave-uniform; the copy counts in vmcnt and has landed in LDS when the counter says so.
+__device__ __forceinline__ void copy_to_lds_16(uint32_t byte_off, const void* base, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\t"
+               "s_nop 0\n\t"
+               "global_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(byte_off), "s"(base), "s"(lds_addr)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void copy_to_lds_4(uint32_t byte_off, const void* base, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\t"
+               "s_nop 0\n\t"
+               "global_load_lds_dword %0, %1"
+               :
+               : "v"(byte_off), "s"(base), "s"(lds_addr)
+               : "memory", "m0");
+}
+template <int PENDING>
+__device__ __forceinline__ void wait_vmem_at_most() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PENDING) : "memory");
+}
+
+// NST: LDS stages.  2: the next K-block is loaded while the current one is multiplied.  More: NST - 1 K-blocks
+// are in flight while one is multiplied (see "deep pipeline" in the kernel).
+template <int BM, int BN, int WM, int WN, int NST = 2>
 struct TileCfg {
   static constexpr int kThreads = WM * WN * 64;
   static constexpr int kWaveM = BM / WM, kWaveN = BN / WN;
   static constexpr int TM = kWaveM / 16, TN = kWaveN / 16;
   static constexpr int kStageBytes = (BM + BN) * 128;
-  static constexpr int kScaleBytes = 2 * BM * 4;
-  static constexpr int kLdsBytes = 2 * kStageBytes + kScaleBytes;
+  // activation scales of a stage: one per row (two stages), or one per thread (deep pipeline: every thread copies one)
+  static constexpr int kScaleBytes = NST == 2 ? 2 * BM * 4 : NST * kThreads * 4;
+  static constexpr int kLdsBytes = NST * kStageBytes + kScaleBytes;
   static_assert(BM <= kThreads, "one thread per activation row stages the row scales");
   static_assert(kWaveN <= 128 && 128 % kWaveN == 0, "a wavefront's N extent must stay inside one 128-wide scale block");
 };
@@ -182,9 +212,10 @@ struct TileCfg {
 // the one that arrives last adds the sums of all splits in split order -- the same order whoever comes last --
 // and runs the epilogue.  For problems with few tiles, which would leave most of the GPU idle while every
 // K-block of a tile costs a full load latency.
-template <int BM, int BN, int WM, int WN, int MODE, bool DIRECT, bool SPLIT = false>
+template <int BM, int BN, int WM, int WN, int MODE, bool DIRECT, bool SPLIT = false, int NST = 2>
 __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
-  using Cfg = TileCfg<BM, BN, WM, WN>;
+  using Cfg = TileCfg<BM, BN, WM, WN, NST>;
+  static_assert(NST == 2 || (DIRECT && MODE != kModeRowColI8 && NST >= 3 && NST <= 5), "deep pipeline: direct fp8 loads, 3..5 stages");
   if (!SPLIT && a.batch > 1) {  // uniform: this workgroup's entry of the batch
     const int64_t z = blockIdx.y;
     a.X += z * a.x_batch_bytes;
@@ -198,7 +229,7 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   auto lds_w = [&](int stage) -> uint8_t* { return lds + stage * Cfg::kStageBytes; };
   auto lds_x = [&](int stage) -> uint8_t* { return lds + stage * Cfg::kStageBytes + BN * 128; };
-  float* const lds_xs = reinterpret_cast<float*>(lds + 2 * Cfg::kStageBytes);  // [2][BM]
+  float* const lds_xs = reinterpret_cast<float*>(lds + NST * Cfg::kStageBytes);  // [2][BM], or [NST][NT]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -248,6 +279,121 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
   const int wn_blk = ((n0 + wn0) >> 7) < nb_last ? ((n0 + wn0) >> 7) : nb_last;
   const float* ws_ptr = a.ws + (int64_t)wn_blk * a.ws_rs;
 
+  if constexpr (NST > 2) {
+    // ---- deep pipeline.  NST - 1 K-blocks are on their way into LDS while one is multiplied, so a K-block costs
+    // 1 / (NST - 1) of a load latency instead of a whole one (a block that owns a compute unit alone -- few tiles,
+    // K split over blocks -- is otherwise bound by exactly that latency).  Per K-block a wavefront issues
+    // kPerStage copies in a fixed order (its thread's activation scale, then its slabs of the two tiles); vmcnt
+    // retires them in order, so "at most p * kPerStage pending" means that all but the youngest p stages have
+    // landed.  One barrier per K-block: behind it every wavefront's share of the stage is in LDS and nobody reads
+    // the slot that the stage issued next overwrites.
+    // (Measured and not kept: reading the fragments of K-block kb + 1 into a second register set under the MFMAs of
+    // K-block kb.  With one wavefront per SIMD everything it issues is serial anyway; 3-8 % slower.)
+    constexpr int kLoadsW = DirectTile<BN, NT>::kPerWave, kLoadsX = DirectTile<BM, NT>::kPerWave;
+    constexpr int kPerStage = kLoadsW + kLoadsX + (MODE == kModeBlock ? 1 : 0);
+    static_assert((NST - 2) * kPerStage <= 63, "vmcnt holds 6 bits");
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+    const uint32_t lds_scales = lds_base + NST * Cfg::kStageBytes;
+    // this thread's activation row (threads past the tile copy the last row's scale; nobody reads it)
+    int xs_rel = tid < BM ? tid : BM - 1;
+    xs_rel = (m0 + xs_rel < a.M) ? xs_rel : a.M - 1 - m0;
+    const uint32_t xs_off = (uint32_t)xs_rel * (uint32_t)a.xs_rs * 4u;  // the host checks that 256 rows of scales fit 32 bits
+    const float* const xs_tile = MODE == kModeBlock ? a.xs + (int64_t)m0 * a.xs_rs : nullptr;
+    auto issue_scale = [&](int kb_load, int slot) __attribute__((always_inline)) {
+      if (MODE != kModeBlock) return;
+      copy_to_lds_4(xs_off, uniform_ptr(xs_tile + (int64_t)kb_load * a.xs_cs), lds_scales + (uint32_t)((slot * NT + wave * 64) * 4));
+    };
+    auto issue_tile_part = [&](int kb_load, int slot, int q) __attribute__((always_inline)) {
+      if (q < kLoadsW) {
+        const int slab = wave + q * (NT / 64);
+        copy_to_lds_16(dt_w.off[q], uniform_ptr(w_base + (int64_t)kb_load * 128), lds_base + (uint32_t)(slot * Cfg::kStageBytes + slab * 1024));
+      } else {
+        const int slab = wave + (q - kLoadsW) * (NT / 64);
+        copy_to_lds_16(dt_x.off[q - kLoadsW], uniform_ptr(x_base + (int64_t)kb_load * 128),
+                       lds_base + (uint32_t)(slot * Cfg::kStageBytes + BN * 128 + slab * 1024));
+      }
+    };
+    // (read through the constant address space: next to assembly that clobbers memory the compiler would otherwise
+    // use a vector load, and its wait for that load would wait for every copy in flight)
+    auto weight_scale = [&](int kb_) __attribute__((always_inline)) -> float {
+      return *(const __attribute__((address_space(4))) float*)(ws_ptr + (int64_t)kb_ * a.ws_cs);
+    };
+    float ws_pend = 1.f, ws_cur = 1.f;
+    for (int st = 0; st < NST - 1; ++st) {
+      if (kb_begin + st < kb_end) {
+        issue_scale(kb_begin + st, st);
+#pragma unroll
+        for (int q = 0; q < kLoadsW + kLoadsX; ++q) issue_tile_part(kb_begin + st, st, q);
+      }
+    }
+    if (MODE == kModeBlock && kb_begin < kb_end) ws_pend = weight_scale(kb_begin);
+    int cur = 0, load_slot = NST - 1;
+    for (int kb = kb_begin; kb < kb_end; ++kb) {
+      const int rem = kb_end - 1 - kb;  // stages issued after this one that may still be on their way
+      if (rem >= NST - 2) wait_vmem_at_most<(NST - 2) * kPerStage>();
+      else if (NST > 3 && rem == 1) wait_vmem_at_most<kPerStage>();
+      else if (NST > 4 && rem == 2) wait_vmem_at_most<2 * kPerStage>();
+      else wait_vmem_at_most<0>();
+      // (a bare barrier: __syncthreads() carries a fence for which the compiler waits for every copy in flight.
+      // The LDS reads of the previous K-block have returned: their values were consumed by its MFMAs.)
+      __builtin_amdgcn_s_barrier();
+      const int kb_load = kb + NST - 1;
+      const bool more = kb_load < kb_end;
+      if (MODE == kModeBlock) {
+        ws_cur = ws_pend;
+        if (kb + 1 < kb_end) ws_pend = weight_scale(kb + 1);
+      }
+      if (more) issue_scale(kb_load, load_slot);
+      const uint8_t* const tw = lds_w(cur) + (wn0 >> 4) * 2048;
+      const uint8_t* const tx = lds_x(cur) + (wm0 >> 4) * 2048;
+      v8i xf[TM];
+      xf[0] = read_fragment(tx, 0, frag_off);
+      v8i wf = read_fragment(tw, 0, frag_off);
+#pragma unroll
+      for (int j = 1; j < TM; ++j) xf[j] = read_fragment(tx, j, frag_off);
+      constexpr int kLoadEvery = (TN * TM) / (kLoadsW + kLoadsX);
+      static_assert(kLoadEvery >= 1, "more tile loads than MFMA steps");
+      if (MODE == kModeBlock) {
+        float sc[TM];
+#pragma unroll
+        for (int j = 0; j < TM; ++j) sc[j] = lds_xs[cur * NT + wm0 + j * 16 + l16] * ws_cur;
+        v4f p_prev = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+          v8i wf_next = wf;
+          if (i + 1 < TN) wf_next = read_fragment(tw, i + 1, frag_off);
+#pragma unroll
+          for (int j = 0; j < TM; ++j) {
+            const v4f p = mfma_fp8_block_partial(wf, xf[j]);
+            if (i > 0 || j > 0) {
+              const int pi = (j == 0) ? i - 1 : i, pj = (j == 0) ? TM - 1 : j - 1;
+              scale_accumulate(acc[pi][pj], p_prev, sc[pj]);
+            }
+            p_prev = p;
+            const int t = i * TM + j;
+            if (t % kLoadEvery == 0 && t / kLoadEvery < kLoadsW + kLoadsX && more) issue_tile_part(kb_load, load_slot, t / kLoadEvery);
+          }
+          wf = wf_next;
+        }
+        scale_accumulate(acc[TN - 1][TM - 1], p_prev, sc[TM - 1]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+          v8i wf_next = wf;
+          if (i + 1 < TN) wf_next = read_fragment(tw, i + 1, frag_off);
+#pragma unroll
+          for (int j = 0; j < TM; ++j) {
+            acc[i][j] = mfma_fp8_16x16x128(wf, xf[j], acc[i][j]);
+            const int t = i * TM + j;
+            if (t % kLoadEvery == 0 && t / kLoadEvery < kLoadsW + kLoadsX && more) issue_tile_part(kb_load, load_slot, t / kLoadEvery);
+          }
+          wf = wf_next;
+        }
+      }
+      cur = (cur + 1 == NST) ? 0 : cur + 1;
+      load_slot = (load_slot + 1 == NST) ? 0 : load_slot + 1;
+    }
+  } else {
   // ---- prologue: stage 0
   if (kb_begin >= kb_end) {
     // K == 0 (or an empty range): nothing to stage, the accumulators stay zero
@@ -370,6 +516,8 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
         st_x.store(lds_x(nxt), tid);
       }
     }
+  }
+
   }
 
   if (SPLIT && a.splits > 1) {
@@ -560,6 +708,67 @@ int launch_tile_split(GemmArgs a, const TileSplitPlan& plan, void* workspace, hi
   return FG_OK;
 }
 
+// 65 <= M <= 1024 with at most one 128 x 128 tile per compute unit: the tile kernel with four LDS stages, one block
+// per compute unit, K split over blocks while blocks are fewer than compute units.  With two stages a block that
+// has a compute unit to itself pays a whole load latency per K-block.
+struct PipePlan {
+  bool use;
+  int splits, kb_per_split;
+  size_t workspace_bytes;
+};
+constexpr int kPipeStages = 4;
+PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs) {
+  PipePlan p = {false, 1, 0, 0};
+  if (M <= 64 || M > 1024 || K <= 0 || K % 128 != 0) return p;
+  if (xs_rs < 0 || xs_rs >= (1 << 21)) return p;  // 256 rows of scales addressed with 32-bit byte offsets
+  const int64_t KB = K / 128;
+  const int64_t tiles = ceil_div(M, kSplitTile) * ceil_div(N, kSplitTile);
+  const int cus = cu_count();
+  if (tiles > cus || KB < 4) return p;
+  // One block per compute unit (its four stages take 129 KB of LDS), where the two-stage kernel fits two: with
+  // tiles for 50..70 % of the units the latter, with K cut in two, keeps all units busy and wins (measured M = 512,
+  // N = 4608, K = 7168, 144 tiles: 43 us against 48).
+  if (tiles * 2 > cus && tiles * 10 < (int64_t)cus * 7) return p;
+  if (tiles * kSplitWaves * 4 > FG_WORKSPACE_COUNTER_BYTES) return p;
+  int64_t splits = cus / tiles;
+  if (splits > KB / 5) splits = KB / 5;  // at least five K-blocks per block: a block starts with a full load latency
+  if (splits > 8) splits = 8;            // the wavefront that finishes a tile reads the splits one after another
+  if (splits < 1) splits = 1;
+#ifdef FG_DEV_KNOBS
+  if (const char* e = getenv("FG_PIPE")) { if (atoi(e) == 0) return p; }
+  if (const char* e = getenv("FG_PIPE_SPLITS")) { splits = atoi(e); if (splits < 1) splits = 1; if (splits > KB) splits = KB; }
+#endif
+  p.kb_per_split = (int)ceil_div(KB, splits);
+  p.splits = (int)ceil_div(KB, (int64_t)p.kb_per_split);
+  // A K-block of a 128 x 128 tile takes ~0.85 us here against ~0.4 us per quarter of a 256 x 256 tile in the
+  // persistent kernel: long K loops stay there (measured M = 512, N = 7168, K = 16384: 109 us here, 86 us there).
+  if (p.kb_per_split > 32) return p;
+  p.workspace_bytes = p.splits > 1 ? FG_WORKSPACE_COUNTER_BYTES + (size_t)tiles * p.splits * kSplitTile * kSplitTile * sizeof(float) : 0;
+  p.use = true;
+  return p;
+}
+
+template <int MODE>
+int launch_pipe(GemmArgs a, const PipePlan& plan, void* workspace, hipStream_t stream) {
+  using Cfg = TileCfg<kSplitTile, kSplitTile, 2, 2, kPipeStages>;
+  a.tiles_m = (int)ceil_div(a.M, kSplitTile);
+  a.tiles_n = (int)ceil_div(a.N, kSplitTile);
+  a.splits = plan.splits;
+  a.kb_per_split = plan.kb_per_split;
+  a.split_counters = reinterpret_cast<unsigned int*>(workspace);
+  a.split_partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES) : nullptr;
+  auto kern = fp8_gemm_kernel<kSplitTile, kSplitTile, 2, 2, MODE, true, true, kPipeStages>;
+  static PerDeviceFlags lds_limit_raised = {};
+  {
+    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, Cfg::kLdsBytes, reinterpret_cast<const void*>(kern));
+    if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
+  }
+  const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n * a.splits;
+  FG_LAUNCH(kern, dim3((uint32_t)blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, a);
+  FG_CHECK_LAUNCH("fp8_gemm_kernel (four stages)");
+  return FG_OK;
+}
+
 // Whether the 33..64-row kernel is the one to take for the shape (it is compared with the K-split tile kernel and
 // the decode kernels, which take the same shapes).
 bool mid_m_preferred(const MidMPlan& mid, int64_t M, int64_t N, int64_t K) {
@@ -582,6 +791,11 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
     if (mid_m_preferred(mid, a.M, a.N, a.K) && (mid.splits == 1 || (workspace != nullptr && workspace_bytes >= mid.workspace_bytes &&
                                                                        (uintptr_t)workspace % 16 == 0)))
       return launch_mid_m(a, MODE, mid, workspace, workspace_bytes, stream);
+    if (MODE != kModeRowColI8) {
+      const PipePlan pp = plan_pipe(a.M, a.N, a.K, MODE == kModeBlock ? a.xs_rs : 0);
+      const bool ws_ok = pp.splits == 1 || (workspace != nullptr && workspace_bytes >= pp.workspace_bytes && (uintptr_t)workspace % 16 == 0);
+      if (pp.use && ws_ok && !(mid_m_preferred(mid, a.M, a.N, a.K))) return launch_pipe<MODE>(a, pp, workspace, stream);
+    }
     const TileSplitPlan ts = plan_tile_split(a.M, a.N, a.K);
     if (ts.use && workspace != nullptr && workspace_bytes >= ts.workspace_bytes && (uintptr_t)workspace % 16 == 0)
       return launch_tile_split<MODE>(a, ts, workspace, stream);
@@ -624,6 +838,8 @@ int check_common(const void* A, const void* B, const void* C, int64_t lda, int64
 extern "C" size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   // the largest any kernel that may take the shape can use
   size_t need = fg::plan_tile_split(M, N, K).workspace_bytes;
+  const fg::PipePlan pipe = fg::plan_pipe(M, N, K, 0);
+  if (pipe.use && pipe.workspace_bytes > need) need = pipe.workspace_bytes;
   const fg::SmallMPlan plan = fg::plan_small_m(M, N, K);
   if (plan.use && plan.workspace_bytes > need) need = plan.workspace_bytes;
   const fg::MidMPlan mid = fg::plan_mid_m(M, N, K);

@@ -118,6 +118,9 @@ __device__ __forceinline__ void load_x4_agent(v4f& v, const float* base, uint32_
 }
 
 
+// Compute units of the current device (256 when it cannot be asked, e.g. on a host without a GPU).
+int cu_count();
+
 // Small-M (decode) path, fp8_gemm_smallm.hip.  `use` reports whether the kernel takes the problem.
 struct SmallMPlan {
   bool use;

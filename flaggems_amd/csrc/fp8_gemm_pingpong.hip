@@ -89,40 +89,41 @@ struct PpArgs {
   const int* groups;
   int n_groups;
   int64_t w_group_stride, ws_group_stride;
+  uint64_t group4_magic;  // ceil(2^40 / (4 * tiles_n)) when that divides every tile number exactly, else 0 (see tile_of_sid)
 };
 
 constexpr int kPartialFloatsPerWave = 64 * 128;                      // one wavefront's 64 x 128 results
 constexpr int kPartialFloatsPerSlot = 8 * kPartialFloatsPerWave;     // a whole 256 x 256 tile
 constexpr size_t kPartialSlotBytes = (size_t)kPartialFloatsPerSlot * 4;  // 256 KB
 
+// Tile number -> (tile row, tile column): four tile rows are walked before moving along N.  The division by
+// 4 * tiles_n is a multiplication by a constant the host prepares (`magic` = ceil(2^40 / (4 * tiles_n)), exact while
+// tiles * 4 * tiles_n < 2^40; 0 = divide): a walk crosses a tile boundary once per K / 128 steps, in a phase with
+// little slack, and a 32-bit division by a run-time value costs about a thousand cycles there.
+__device__ __forceinline__ void tile_of_sid(int sid, int tiles_m, int tiles_n, uint64_t magic, int& tm, int& tn) {
+  constexpr int GROUP_M = 4;
+  const int per_group = GROUP_M * tiles_n;
+  const int g = magic != 0 ? (int)(((uint64_t)(uint32_t)sid * magic) >> 40) : sid / per_group;
+  const int first_m = g * GROUP_M;
+  const int gm = (tiles_m - first_m < GROUP_M) ? tiles_m - first_m : GROUP_M;
+  const uint32_t r = (uint32_t)(sid - g * per_group);
+  uint32_t q;  // r / gm
+  if (gm == 4) q = r >> 2;
+  else if (gm == 3) q = r / 3u;
+  else if (gm == 2) q = r >> 1;
+  else q = r;
+  tm = first_m + (int)(r - q * (uint32_t)gm);
+  tn = (int)q;
+}
+
 // Same XCD-aware order as the tile kernel: ids congruent mod 8 (one XCD) walk a contiguous run of tiles,
 // four tile rows at a time.
-__device__ __forceinline__ void tile_of_index(int vid, int tiles_m, int tiles_n, int& tm, int& tn) {
+__device__ __forceinline__ void tile_of_index(int vid, int tiles_m, int tiles_n, uint64_t magic, int& tm, int& tn) {
   const int total = tiles_m * tiles_n;
   const int xcd = vid & 7, local = vid >> 3;
   const int base = total >> 3, rem = total & 7;
   const int sid = xcd * base + (xcd < rem ? xcd : rem) + local;
-  constexpr int GROUP_M = 4;
-  const int per_group = GROUP_M * tiles_n;
-  const int g = sid / per_group;
-  const int first_m = g * GROUP_M;
-  const int gm = (tiles_m - first_m < GROUP_M) ? tiles_m - first_m : GROUP_M;
-  const int r = sid - g * per_group;
-  tm = first_m + r % gm;
-  tn = r / gm;
-}
-
-// Stream-K order: consecutive tile numbers walk four tile rows before moving along N, so the ranges of
-// neighbouring blocks (which the launch places on one XCD) share operand panels.
-__device__ __forceinline__ void tile_of_sid(int sid, int tiles_m, int tiles_n, int& tm, int& tn) {
-  constexpr int GROUP_M = 4;
-  const int per_group = GROUP_M * tiles_n;
-  const int g = sid / per_group;
-  const int first_m = g * GROUP_M;
-  const int gm = (tiles_m - first_m < GROUP_M) ? tiles_m - first_m : GROUP_M;
-  const int r = sid - g * per_group;
-  tm = first_m + r % gm;
-  tn = r / gm;
+  tile_of_sid(sid, tiles_m, tiles_n, magic, tm, tn);
 }
 
 // A block visits the virtual ids blockIdx.x, blockIdx.x + gridDim.x, ...  The grid is either the tile count
@@ -157,9 +158,9 @@ struct WalkT {
   __device__ __forceinline__ void locate(const PpArgs& a) {
     int tm = 0, tn = 0;
     if (idx < n_tiles) {
-      if (a.sk && a.tile_base == 0) tile_of_sid(idx, tiles_m, a.g.tiles_n, tm, tn);
-      else if (a.sk) tile_of_index(idx + a.tile_base, tiles_m, a.g.tiles_n, tm, tn);
-      else tile_of_index(idx, tiles_m, a.g.tiles_n, tm, tn);
+      if (a.sk && a.tile_base == 0) tile_of_sid(idx, tiles_m, a.g.tiles_n, a.group4_magic, tm, tn);
+      else if (a.sk) tile_of_index(idx + a.tile_base, tiles_m, a.g.tiles_n, a.group4_magic, tm, tn);
+      else tile_of_index(idx, tiles_m, a.g.tiles_n, a.group4_magic, tm, tn);
     }
     m0 = tm * kBM; n0 = tn * kBN;
     m_end = a.g.M; group = 0;
@@ -311,6 +312,17 @@ __device__ __forceinline__ void wait_vmem() {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PENDING) : "memory");
 }
 
+// 16 bytes of results
+__device__ __forceinline__ void store_result_16(uint16_t* p, u32x4 v) {
+#if defined(FG_EXP_NOSTORE)
+  if (v.x == 0x12345678u) *reinterpret_cast<u32x4*>(p) = v;
+#elif defined(FG_EXP_NTSTORE)
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+#else
+  *reinterpret_cast<u32x4*>(p) = v;
+#endif
+}
+
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
@@ -386,7 +398,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
     for (int q = 0; q < 4; ++q) {
       const int n = piece_column(n_base, q, lg);
       if (ALIGNED || n + 8 <= a.N) {
-        *reinterpret_cast<u32x4*>(row + n) = u32x4{w[4 * q], w[4 * q + 1], w[4 * q + 2], w[4 * q + 3]};
+        store_result_16(row + n, u32x4{w[4 * q], w[4 * q + 1], w[4 * q + 2], w[4 * q + 3]});
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
@@ -801,18 +813,6 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   if (grp == 0) __builtin_amdgcn_s_barrier();  // pairs with B's extra barrier at the start
 }
 
-int cu_count() {
-  static int cached[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
-  }
-  return cached[dev];
-}
-
 // Stream-K pays when whole-tile rounds leave compute units idle: `steps` K-blocks per block either way.
 struct SkPlan {
   bool use;
@@ -890,9 +890,9 @@ TailPlan plan_tail(int64_t tiles, int KB, int cus) {
 // keep sweeping the L1), as many line requests as the tiles themselves need, and the tile loads queue behind
 // them in the address unit: measured 20 % of the run time on K = 16384.  From the transposed copy a
 // wavefront's 64 scales of a K-block are 256 contiguous bytes.
-// One thread per row and 16 K-blocks: reads run along a row (16-byte loads where the layout allows), writes
+// One thread per row and 4 K-blocks: reads run along a row (16-byte loads where the layout allows), writes
 // run along M and are contiguous over the threads of a block.
-constexpr int kTransposeKbPerBlock = 16;
+constexpr int kTransposeKbPerBlock = 4;  // (16: a quarter of the blocks and 3 us instead of 2 on [4096, 56])
 __global__ __launch_bounds__(256) void transpose_scales_kernel(const float* __restrict__ xs, int64_t rs, int64_t cs, int M,
                                                                int KB, float* __restrict__ out) {
   const int m = (int)blockIdx.x * 256 + (int)threadIdx.x;
@@ -944,6 +944,11 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   const int64_t tiles = (int64_t)a.g.tiles_m * a.g.tiles_n;
   if (tiles > 0x3FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm: too many tiles");
   a.n_tiles = (int)tiles;
+  {
+    const uint64_t d = 4ull * (uint64_t)a.g.tiles_n;
+    // n * magic >> 40 == n / d for every n with n * d < 2^40 (the tile numbers of whole problems are below `tiles`)
+    a.group4_magic = (d > 0 && (uint64_t)tiles * d < (1ull << 40)) ? ((1ull << 40) + d - 1) / d : 0;
+  }
   static PerDeviceFlags lds_limit_raised[7] = {};
   const void* const kernels[7] = {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, true>),
@@ -1028,6 +1033,18 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
 }
 
 }  // namespace
+
+int cu_count() {
+  static int cached[kMaxDevices] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
 
 bool pingpong_takes(const GemmArgs& g, int mode, const void* workspace, size_t workspace_bytes) {
   // bf16 rows that take 16-byte stores; activation-scale offsets (bytes from the first row) that fit 32 bits
