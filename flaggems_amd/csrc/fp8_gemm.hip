@@ -19,9 +19,6 @@
 #include "fp8_gemm_common.h"
 
 #include <mutex>
-#ifdef FG_DEV_KNOBS
-#include <stdlib.h>
-#endif
 
 namespace fg {
 namespace {
@@ -734,10 +731,6 @@ PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs) {
   if (splits > KB / 5) splits = KB / 5;  // at least five K-blocks per block: a block starts with a full load latency
   if (splits > 8) splits = 8;            // the wavefront that finishes a tile reads the splits one after another
   if (splits < 1) splits = 1;
-#ifdef FG_DEV_KNOBS
-  if (const char* e = getenv("FG_PIPE")) { if (atoi(e) == 0) return p; }
-  if (const char* e = getenv("FG_PIPE_SPLITS")) { splits = atoi(e); if (splits < 1) splits = 1; if (splits > KB) splits = KB; }
-#endif
   p.kb_per_split = (int)ceil_div(KB, splits);
   p.splits = (int)ceil_div(KB, (int64_t)p.kb_per_split);
   // A K-block of a 128 x 128 tile takes ~0.85 us here against ~0.4 us per quarter of a 256 x 256 tile in the

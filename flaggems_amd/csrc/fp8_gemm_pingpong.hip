@@ -314,13 +314,7 @@ __device__ __forceinline__ void wait_vmem() {
 
 // 16 bytes of results
 __device__ __forceinline__ void store_result_16(uint16_t* p, u32x4 v) {
-#if defined(FG_EXP_NOSTORE)
-  if (v.x == 0x12345678u) *reinterpret_cast<u32x4*>(p) = v;
-#elif defined(FG_EXP_NTSTORE)
-  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
-#else
   *reinterpret_cast<u32x4*>(p) = v;
-#endif
 }
 
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));

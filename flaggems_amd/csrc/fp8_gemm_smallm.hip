@@ -20,9 +20,6 @@
 // at the end (row/column mode).
 
 #include "fp8_gemm_common.h"
-#ifdef FG_DEV_KNOBS
-#include <stdlib.h>
-#endif
 
 namespace fg {
 namespace {
@@ -429,9 +426,6 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
     // through memory: measured 6.1 us unsplit against 8.6 us split in two for N = 2112, K = 7168).
     p.rg = 4;
     while (p.rg > 1 && ceil_div(N, 16 * p.rg) * entries < 140) p.rg >>= 1;
-#ifdef FG_DEV_KNOBS
-    if (const char* e = getenv("FG_SM_RG")) p.rg = atoi(e);
-#endif
     p.waves = (p.tmx == 2 && p.rg == 4) ? 4 : 8;
   } else {
     p.waves = p.tmx == 4 ? 4 : 8;  // LDS reduction buffer is 4 KB * tmx per wavefront
@@ -445,9 +439,6 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
     const int64_t pairs = (KB + 1) / 2;
     splits = 1;
     while (p.n_chunks * entries * splits < 100 && splits * 2 <= max_splits && splits * 2 * p.waves <= pairs) splits *= 2;
-#ifdef FG_DEV_KNOBS
-    if (const char* e = getenv("FG_SM_SPLITS")) { splits = atoi(e); if (splits * p.waves > pairs) splits = pairs / p.waves > 0 ? pairs / p.waves : 1; }
-#endif
     kpw = ceil_div(pairs, splits * p.waves);
   } else {
     // aim for ~8 wavefronts per CU on 256 CUs, each with at least one K-block
