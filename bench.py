@@ -106,7 +106,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--counter-pass", action="store_true",
                     help="for hardware-counter runs: one 256 MiB device copy (calibration), then one eager launch of "
-                         "each M=4096 and M=1 GEMM of the sweep and one quantizer launch, no timing, no JSON")
+                         "every (M, N, K) of the per-shape table, an elementwise marker kernel before each, and one "
+                         "quantizer launch; no timing, no JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; run with --gpus 1 "
@@ -147,18 +148,20 @@ def main():
     if args.counter_pass:
         src = torch.randint(0, 255, (256 << 20,), device=dev, dtype=torch.uint8)
         dst = torch.empty_like(src)
-        for (m, n, k) in calls:  # first launches (workspace zero fill etc.) happen before the counted ones
-            if m in (1, 4096):
-                run_one(m, n, k, 0)
+        shapes = [(m, n, k) for (n, k) in DSV3_NK for m in DETAIL_M]
+        for (m, n, k) in shapes:  # first launches (workspace zero fill etc.) happen before the counted ones
+            run_one(m, n, k, 0)
+        mark = torch.zeros(64, device=dev)
         torch.cuda.synchronize()
         dst.copy_(src)
-        for (m, n, k) in calls:
-            if m in (1, 4096):
-                run_one(m, n, k, 1)
+        for (m, n, k) in shapes:
+            mark.add_(1.0)  # an elementwise kernel between two calls: delimits the kernels of a call in the counter files
+            run_one(m, n, k, 1)
+        mark.add_(1.0)
         flag_gems.act_quant_triton(torch.randn(4096, 7168, device=dev, generator=gen).bfloat16(), 128)
         torch.cuda.synchronize()
-        print("counter pass done: copy 268435456 B, then (M,N,K) =",
-              [c for c in calls if c[0] in (1, 4096)], "then act_quant [4096,7168]", flush=True)
+        print("counter pass done: copy 268435456 B, then (M,N,K) =", shapes, "each after one elementwise marker kernel, "
+              "then a marker and act_quant [4096,7168]", flush=True)
         return
 
     # The sweep is replayed from HIP graphs (the reference's benchmark harness has the same mode):
@@ -219,14 +222,35 @@ def main():
         rest = sorted(times[1:])
         return rest[len(rest) // 2]
 
+    # the floor for the weight-streaming kernels: a kernel that only reads a buffer of the weight's size once, launched
+    # and rotated through the same pool exactly like the GEMM (fg_stream_read_probe)
+    from flaggems_amd import _lib as fg_lib
+
+    probe = fg_lib.load().fg_stream_read_probe
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+    def read_probe(n, k, rot):
+        pool = weights[(n, k)]
+        wq = pool[rot % len(pool)][0]
+        rc = probe(wq.data_ptr(), wq.numel(), sink.data_ptr(), torch.cuda.current_stream(dev).cuda_stream)
+        assert rc == 0
+
+    read_floor = {}
+    for (n, k) in DSV3_NK:
+        read_floor[(n, k)] = time_graph(lambda r: read_probe(n, k, r))
+
     detail = []
     for (n, k) in DSV3_NK:
         for m in DETAIL_M:
             us = time_graph(lambda r: run_one(m, n, k, r))
             tf = gemm_flops(m, n, k) / (us * 1e-6) / 1e12
             gbs = gemm_bytes(m, n, k) / (us * 1e-6) / 1e9
-            detail.append({"M": m, "N": n, "K": k, "us": round(us, 2), "tflops": round(tf, 1), "gbps": round(gbs, 1),
-                           "frac_mfma": round(tf / PEAK_FP8_TFLOPS, 4), "frac_hbm": round(gbs / PEAK_HBM_GBPS, 4)})
+            row = {"M": m, "N": n, "K": k, "us": round(us, 2), "tflops": round(tf, 1), "gbps": round(gbs, 1),
+                   "frac_mfma": round(tf / PEAK_FP8_TFLOPS, 4), "frac_hbm": round(gbs / PEAK_HBM_GBPS, 4)}
+            if m <= 64:
+                row["weight_read_floor_us"] = round(read_floor[(n, k)], 2)
+                row["read_floor_over_us"] = round(read_floor[(n, k)] / us, 4)
+            detail.append(row)
 
     big = [d for d in detail if d["M"] == 4096]
     big_flops = sum(gemm_flops(d["M"], d["N"], d["K"]) for d in big)
@@ -247,7 +271,10 @@ def main():
     small_time = sum(d["us"] for d in small) * 1e-6
     roofline_small = {"bound": "hbm", "achieved": round(small_bytes / small_time / 1e9, 1), "peak": PEAK_HBM_GBPS,
                       "unit": "GB/s", "frac": round(small_bytes / small_time / 1e9 / PEAK_HBM_GBPS, 4),
-                      "kernel": "the eighteen M in {1, 8, 16} launches of the six DSv3 (N,K), weights rotated through 512 MB"}
+                      "kernel": "the eighteen M in {1, 8, 16} launches of the six DSv3 (N,K), weights rotated through 512 MB",
+                      "weight_read_floor_gbps": round(sum(n * k for (n, k) in DSV3_NK) / sum(read_floor.values()) / 1e3, 1),
+                      "weight_read_floor_us": {f"{n}x{k}": round(v, 2) for (n, k), v in read_floor.items()},
+                      "time_of_read_floor_over_time": round(3 * sum(read_floor.values()) / (small_time * 1e6), 4)}
 
     # ---- quantizer (HBM bound): act_quant on bf16 [4096, 7168]
     xq_in = torch.randn(4096, 7168, device=dev, generator=gen).bfloat16()

@@ -32,6 +32,7 @@ constexpr size_t kErrorBufferBytes = 512;
 // value is kept, so that an error some other library left in the process-wide "last error" slot is neither taken
 // for this launch's nor cleared.
 hipError_t& launch_status();
+int cu_count_or_default();  // compute units of the current device, 256 when it cannot be asked
 
 template <typename T>
 struct same_type { using type = T; };

@@ -74,6 +74,14 @@ const char* fg_last_error_string(void);
 unsigned long long fg_stream_capture_id(void* stream);
 
 /*
+ * Measurement aid, no reference counterpart: enqueues a kernel that reads `bytes` bytes at `src` once (16-byte
+ * non-temporal loads from every compute unit) and does nothing else.  Its duration is the floor for any kernel that
+ * must stream a buffer of that size from memory, launch cost included; the benchmark reports the decode GEMMs next
+ * to it.  `sink` (4 bytes of device memory, may be NULL) is written only for data no real buffer holds.
+ */
+int fg_stream_read_probe(const void* src, size_t bytes, void* sink, void* stream);
+
+/*
  * Per-token-group FP8 quantization: for every row r and every group g of `group_size`
  * consecutive columns,
  *     amax  = max |x[r, g*G : (g+1)*G]|          (NaN propagates)

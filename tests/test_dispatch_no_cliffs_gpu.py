@@ -1,0 +1,55 @@
+"""The launch planner picks a kernel from (M, N, K) by thresholds that were fitted on the benchmark shapes.  This test
+walks shapes off that grid and checks that none falls into a slow corner: every call must finish within twice a
+deliberately loose cost model (the slower of 1.2 PFLOP/s and 2.5 TB/s, plus 15 us of fixed cost -- about half of what
+the tuned shapes reach), so a rule that sends a shape to a kernel three times too slow for it fails here.  Results
+are checked elsewhere; this file only times."""
+import pytest
+import torch
+
+import flag_gems
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+FP8 = torch.float8_e4m3fn
+
+NK = [(1000, 1024), (2112, 7168), (3000, 3072), (5120, 2048), (7168, 2304), (12288, 1536), (4096, 8192), (1536, 16384),
+      (28672, 4096), (512, 4096)]
+MS = [3, 17, 33, 48, 65, 100, 130, 200, 300, 400, 600, 777, 1000, 1100, 1500, 3000, 5000]
+
+
+def _model_us(M, N, K):
+    flops = 2.0 * M * N * K
+    nbytes = M * K + N * K + 2.0 * M * N + 4.0 * (M + N / 128) * (K / 128)
+    return max(flops / 1.2e15, nbytes / 2.5e12) * 1e6 + 15.0
+
+
+def _time_us(fn):
+    fn()
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(3):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(5):
+            fn()
+        end.record()
+        end.synchronize()
+        best = min(best, start.elapsed_time(end) * 1e3 / 5)
+    return best
+
+
+@pytest.mark.parametrize("N,K", NK)
+def test_no_shape_is_far_off_the_cost_model(N, K):
+    g = torch.Generator(device=DEV).manual_seed(N + K)
+    w = torch.randn(N, K, device=DEV, generator=g).to(FP8)
+    ws = torch.rand((N + 127) // 128, K // 128, device=DEV, generator=g) + 0.5
+    slow = []
+    for M in MS:
+        x = torch.randn(M, K, device=DEV, generator=g).to(FP8)
+        xs = torch.rand(M, K // 128, device=DEV, generator=g) + 0.5
+        us = _time_us(lambda: flag_gems.w8a8_block_fp8_matmul(x, w, xs, ws, [128, 128]))
+        # eager launches from Python cost ~15-20 us of host time each: short kernels are bound by that, not by the GPU
+        limit = 2.0 * _model_us(M, N, K) + 20.0
+        if us > limit:
+            slow.append((M, N, K, round(us, 1), round(limit, 1)))
+    assert not slow, f"(M, N, K, measured us, limit us): {slow}"
