@@ -1051,6 +1051,7 @@ extern "C" int fg_grouped_block_fp8_gemm(const void* A, int64_t lda,
                                          const float* As, int64_t as_row_stride, int64_t as_col_stride,
                                          const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride, int64_t bs_group_stride,
                                          const int32_t* group_ends, int64_t n_groups,
+                                         const int32_t* row_index, int64_t index_div, int64_t a_rows,
                                          void* C, int64_t ldc, int c_dtype,
                                          int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
                                          void* workspace, size_t workspace_bytes, void* stream) {
@@ -1078,7 +1079,7 @@ extern "C" int fg_grouped_block_fp8_gemm(const void* A, int64_t lda,
   a.xs_rs = as_row_stride; a.xs_cs = as_col_stride; a.ws_rs = bs_row_stride; a.ws_cs = bs_col_stride;
   a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)(K / 128);
   a.c_dtype = c_dtype;
-  GroupedGemm grouped = {group_ends, n_groups, b_group_stride, bs_group_stride};
+  GroupedGemm grouped = {group_ends, n_groups, b_group_stride, bs_group_stride, row_index, index_div, row_index ? a_rows : M};
   return launch_grouped(a, grouped, workspace, workspace_bytes, (hipStream_t)stream);
 }
 

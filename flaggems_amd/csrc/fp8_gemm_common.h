@@ -168,6 +168,9 @@ struct GroupedGemm {
   const int* ends;
   int64_t n_groups;
   int64_t w_group_stride, ws_group_stride;
+  // optional gather: row m of the sorted order is row row_index[m] / index_div of X (x_rows rows) and of its scales
+  const int* row_index;
+  int64_t index_div, x_rows;
 };
 int launch_grouped(const GemmArgs& a, const GroupedGemm& grouped, void* workspace, size_t workspace_bytes, hipStream_t stream);
 // workspace that lets launch_grouped read row-major activation scales from a transposed copy

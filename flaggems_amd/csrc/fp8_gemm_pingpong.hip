@@ -89,6 +89,11 @@ struct PpArgs {
   const int* groups;
   int n_groups;
   int64_t w_group_stride, ws_group_stride;
+  // Grouped problem whose rows are gathered (row_index != nullptr): row m of the sorted order is row
+  // row_index[m] / index_div of X and of its scales (the reference's MoE kernel reads its tokens the same way,
+  // sorted_token_ids // top_k, src/flag_gems/fused/fused_moe.py:1111); entries are forced into [0, x_rows).
+  const int* row_index;
+  int index_div, x_rows;
   uint64_t group4_magic;  // ceil(2^40 / (4 * tiles_n)) when that divides every tile number exactly, else 0 (see tile_of_sid)
 };
 
@@ -211,6 +216,23 @@ struct LoadShare {
       row = row < valid ? row : valid - 1;
       off[j] = __umul24((uint32_t)row, ld) + chunk;  // row < 256, ld < 2^23 (checked by the host)
     }
+  }
+  // Activation rows read through an index: offsets are relative to the first row of X (the host checks that
+  // x_rows * ldx fits 32 bits); rows past the segment's end repeat its last row, as above.
+  __device__ __forceinline__ void set_gathered(const GemmArgs& a, const int* row_index, int index_div, int x_rows,
+                                               int m0, int valid, int lane, int wave) {
+    const uint32_t ld = (uint32_t)a.ldx;
+#pragma unroll
+    for (int j = 0; j < kSlabsPerWave; ++j) {
+      const int slab = (wave & 3) + j * 4;
+      const int r = slab * 8 + (lane >> 3);  // LDS row
+      const uint32_t chunk = (uint32_t)(((lane & 7) ^ (r & 7)) << 4);
+      const int row = r < valid ? r : valid - 1;
+      int src = row_index[m0 + row] / index_div;
+      src = src < 0 ? 0 : (src < x_rows ? src : x_rows - 1);
+      off[j] = (uint32_t)src * ld + chunk;
+    }
+    ptr = a.X;
   }
   __device__ __forceinline__ void set_ptr(const GemmArgs& a, int m0, int n0, int wave, int64_t w_group_off = 0) {
     ptr = wave >= 4 ? a.W + w_group_off + (int64_t)n0 * a.ldw : a.X + (int64_t)m0 * a.ldx;
@@ -549,7 +571,15 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   Walk lw;
   lw.start(a, first_idx, first_kb, n_tiles, tiles_m);
   LoadShare share = {};
-  share.set_tile(g, lw.m0, lw.n0, wave, lane, lw.m_end, (int64_t)lw.group * a.w_group_stride);
+  auto set_load_tile = [&]() __attribute__((always_inline)) {
+    if (GROUPED && a.row_index != nullptr && wave < 4) {
+      const int valid = lw.m_end - lw.m0;
+      share.set_gathered(g, a.row_index, a.index_div, a.x_rows, lw.m0, valid < 256 ? valid : 256, lane, wave);
+    } else {
+      share.set_tile(g, lw.m0, lw.n0, wave, lane, lw.m_end, GROUPED ? (int64_t)lw.group * a.w_group_stride : 0);
+    }
+  };
+  set_load_tile();
   share.ptr += (int64_t)first_kb * 128;
   int loaded = 0, w_slot = 0, x_slot = 0;  // stages issued by this wavefront; LDS slots of the next stage
   auto issue_stage_part = [&](int q) __attribute__((always_inline)) {
@@ -564,7 +594,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     if (__builtin_expect(lw.next(a), 0)) {
       if (lw.idx < n_tiles) {
         if (ALIGNED) share.set_ptr(g, lw.m0, lw.n0, wave);
-        else share.set_tile(g, lw.m0, lw.n0, wave, lane, lw.m_end, GROUPED ? (int64_t)lw.group * a.w_group_stride : 0);
+        else set_load_tile();
       }
     } else {
       share.ptr += 128;
@@ -583,18 +613,23 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   uint32_t xs_off[kTM] = {0u, 0u, 0u, 0u};
   const float* xs_ptr = g.xs;
   // offsets are relative to the tile's first row; rows past the edge read the last row's scale
+  const bool gathered = GROUPED && a.row_index != nullptr;  // uniform
   auto set_scale_offsets = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < kTM; ++j) {
       int r = wm0 + j * 16 + l16;
       const int last = sw.m_end - 1 - sw.m0;
       r = r < last ? r : last;
+      if (gathered) {  // the scales of the source row, relative to the first row of the scale matrix
+        int src = a.row_index[sw.m0 + r] / a.index_div;
+        r = src < 0 ? 0 : (src < a.x_rows ? src : a.x_rows - 1);
+      }
       xs_off[j] = (uint32_t)r * (uint32_t)g.xs_rs * 4u;
     }
   };
   auto set_scale_tile = [&]() __attribute__((always_inline)) {
     if (!ALIGNED) set_scale_offsets();
-    xs_ptr = g.xs + (int64_t)sw.m0 * g.xs_rs;
+    xs_ptr = gathered ? g.xs : g.xs + (int64_t)sw.m0 * g.xs_rs;
   };
   if (MODE == kModeBlock) {
     set_scale_offsets();
@@ -933,6 +968,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     a.g.tiles_m = (int)(bound < g.M ? bound : g.M);
     a.groups = grouped->ends; a.n_groups = (int)grouped->n_groups;
     a.w_group_stride = grouped->w_group_stride; a.ws_group_stride = grouped->ws_group_stride;
+    a.row_index = grouped->row_index; a.index_div = (int)grouped->index_div; a.x_rows = (int)grouped->x_rows;
   }
   a.g.tiles_n = (int)ceil_div(g.N, kBN);
   const int64_t tiles = (int64_t)a.g.tiles_m * a.g.tiles_n;
@@ -964,18 +1000,20 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   if (sk.use || grouped != nullptr || mode != kModeBlock) tp.use = false;
   const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : (tp.use ? (size_t)tp.grid * 2 * kPartialSlotBytes : 0);
   const size_t need = FG_WORKSPACE_COUNTER_BYTES + sk_bytes;
+  // rows of the activation-scale matrix: the rows of X, which a gathered problem reads through its index
+  const int64_t scale_rows = (grouped != nullptr && grouped->row_index != nullptr) ? grouped->x_rows : (int64_t)g.M;
   // workspace: [counters][partial tiles, if the shape is one that shares tiles][transposed activation scales]
   // (a grouped problem's tile count is an upper bound that a few hundred rows spread over many segments inflate:
   // there the gathers are few and the transposition, ~5 us whatever the size, does not pay)
   if (mode == kModeBlock && g.xs_rs >= kTransposeMinRowStride && transposition_pays(tiles, g.KB, cus) && workspace != nullptr &&
       (grouped == nullptr || g.M >= 1024) &&
       (uintptr_t)workspace % 16 == 0 &&
-      workspace_bytes >= need + transposed_scales_bytes(g.M, g.KB)) {
+      workspace_bytes >= need + transposed_scales_bytes(scale_rows, g.KB)) {
     float* const xs_t = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + need);
-    FG_LAUNCH(transpose_scales_kernel, dim3((uint32_t)ceil_div(g.M, 256), (uint32_t)ceil_div(g.KB, kTransposeKbPerBlock)),
-                       dim3(256), 0, stream, g.xs, g.xs_rs, g.xs_cs, g.M, g.KB, xs_t);
+    FG_LAUNCH(transpose_scales_kernel, dim3((uint32_t)ceil_div(scale_rows, (int64_t)256), (uint32_t)ceil_div(g.KB, kTransposeKbPerBlock)),
+                       dim3(256), 0, stream, g.xs, g.xs_rs, g.xs_cs, (int)scale_rows, g.KB, xs_t);
     FG_CHECK_LAUNCH("transpose_scales_kernel");
-    a.g.xs = xs_t; a.g.xs_rs = 1; a.g.xs_cs = g.M;
+    a.g.xs = xs_t; a.g.xs_rs = 1; a.g.xs_cs = scale_rows;
   }
   if (mode == kModeBlock && sk.use && workspace != nullptr && workspace_bytes >= need && (size_t)sk.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
       (uintptr_t)workspace % 16 == 0) {
@@ -1076,6 +1114,12 @@ int launch_grouped(const GemmArgs& g, const GroupedGemm& grouped, void* workspac
   if (!(g.xs_rs >= 0 && g.xs_cs >= 0 && g.ws_rs >= 0 && g.ws_cs >= 0 && (int64_t)g.M * g.xs_rs < (1ll << 29)))
     FG_FAIL(FG_ERR_UNSUPPORTED, "grouped fp8 gemm: scale strides must be non-negative and M * row stride below 2^29");
   if (grouped.n_groups <= 0 || grouped.n_groups > 65536) FG_FAIL(FG_ERR_INVALID_ARG, "grouped fp8 gemm: 1..65536 groups");
+  if (grouped.row_index != nullptr) {
+    if (grouped.index_div < 1 || grouped.index_div > 0x7FFFFFFF) FG_FAIL(FG_ERR_INVALID_ARG, "grouped fp8 gemm: index divisor %lld", (long long)grouped.index_div);
+    if (grouped.x_rows < 1 || grouped.x_rows > 0x7FFFFFFF || grouped.x_rows * g.ldx >= (1ll << 32) || grouped.x_rows * g.xs_rs >= (1ll << 29))
+      FG_FAIL(FG_ERR_UNSUPPORTED, "grouped fp8 gemm: %lld gathered rows: the rows of A and of its scales must fit 32-bit byte offsets",
+              (long long)grouped.x_rows);
+  }
   return launch_block(g, kModeBlock, workspace, workspace_bytes, stream, &grouped);
 }
 

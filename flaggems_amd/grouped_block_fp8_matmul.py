@@ -12,7 +12,7 @@ stays on the device; the kernel reads it, so the call never synchronises.
 from __future__ import annotations
 
 import logging
-from typing import List
+from typing import List, Optional
 
 import torch
 
@@ -33,22 +33,34 @@ def grouped_w8a8_block_fp8_matmul(
     offs: torch.Tensor,
     block_size: List[int],
     output_dtype: torch.dtype = torch.bfloat16,
+    row_index: Optional[torch.Tensor] = None,
+    index_divisor: int = 1,
 ) -> torch.Tensor:
     """C[offs[e-1]:offs[e]] = block_fp8_matmul(A[offs[e-1]:offs[e]], B[e]) for every group e.
 
     A [M, K] contiguous e4m3fn (rows sorted by group), As [M, K/block_k] fp32, B [E, N, K] e4m3fn,
     Bs [E, ceil(N/block_n), K/block_k] fp32, offs [E] int32 cumulative row ends on A's device.
     Returns bf16 [M, N]; rows at or past offs[-1] are left unwritten (as ``torch.empty`` made them).
+
+    With ``row_index`` (int32 [M] on A's device) the kernel gathers its rows itself: sorted row m is row
+    ``row_index[m] // index_divisor`` of ``A [T, K]`` and ``As [T, K/block_k]``, the way the reference's MoE kernel
+    reads its tokens (``sorted_token_ids // top_k``, src/flag_gems/fused/fused_moe.py:1111); the result still has
+    M = ``row_index.numel()`` rows in sorted order.
     """
     logger.debug("GEMS GROUPED_W8A8_BLOCK_FP8_MATMUL")
     assert len(block_size) == 2
     block_n, block_k = block_size[0], block_size[1]
     assert A.ndim == 2 and B.ndim == 3 and As.ndim == 2 and Bs.ndim == 3
     assert A.is_contiguous()
-    M, K = A.shape
+    T, K = A.shape  # rows of A: the sorted rows themselves, or the tokens they are gathered from
+    M = T
+    if row_index is not None:
+        assert row_index.ndim == 1 and row_index.dtype == torch.int32 and row_index.is_contiguous()
+        assert row_index.device == A.device and index_divisor >= 1
+        M = row_index.numel()
     E, N, K2 = B.shape
     assert K == K2
-    assert As.shape[0] == M and As.shape[1] == _cdiv(K, block_k)
+    assert As.shape[0] == T and As.shape[1] == _cdiv(K, block_k)
     assert Bs.shape == (E, _cdiv(N, block_n), _cdiv(K, block_k))
     assert offs.ndim == 1 and offs.numel() == E and offs.dtype == torch.int32
     assert offs.device == A.device and offs.is_contiguous()
@@ -68,14 +80,15 @@ def grouped_w8a8_block_fp8_matmul(
     lib = _lib.load()
     dev = A.device
     with torch.cuda.device(dev):
-        ws_bytes = lib.fg_grouped_block_fp8_gemm_workspace_bytes(M, N, K)
+        ws_bytes = lib.fg_grouped_block_fp8_gemm_workspace_bytes(max(M, T), N, K)
         ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
         status = lib.fg_grouped_block_fp8_gemm(
-            A.data_ptr(), A.stride(0) if M > 1 else max(K, A.stride(0)),
+            A.data_ptr(), A.stride(0) if T > 1 else max(K, A.stride(0)),
             B.data_ptr(), B.stride(1) if N > 1 else max(K, B.stride(1)), B.stride(0) if E > 1 else N * K,
             As.data_ptr(), As.stride(0), As.stride(1),
             Bs.data_ptr(), Bs.stride(1), Bs.stride(2), Bs.stride(0),
             offs.data_ptr(), E,
+            row_index.data_ptr() if row_index is not None else None, index_divisor, T,
             C.data_ptr(), C.stride(0), _lib.DTYPE_CODE[C.dtype],
             M, N, K, block_n, block_k,
             ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,

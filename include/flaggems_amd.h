@@ -287,6 +287,11 @@ int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_batch_stride
  * slower general path behind this entry point).
  * `workspace` (optional, 16-byte aligned, fg_grouped_block_fp8_gemm_workspace_bytes(M, N, K) bytes, first
  * FG_WORKSPACE_COUNTER_BYTES zero-filled once) lets row-major As be read from a transposed copy.
+ * row_index (optional DEVICE table of M int32): the kernel gathers its rows itself -- row m of the sorted order
+ * (the order of group_ends and of C) is row row_index[m] / index_div of A and As, which then have a_rows rows
+ * (entries are forced into [0, a_rows); a_rows * lda must fit 32 bits).  This is how the reference's MoE kernel
+ * reads its tokens (rows = sorted_token_ids // top_k, src/flag_gems/fused/fused_moe.py:1111): the caller need not
+ * materialise the activations in expert order.  NULL: A and As are already in sorted order (a_rows ignored).
  *
  * Stands in for the block-wise fp8 branch of fused_moe_kernel (src/flag_gems/fused/fused_moe.py:1378-1450)
  * applied to rows already gathered in expert order, with the group table of aten::_scaled_grouped_mm
@@ -299,6 +304,7 @@ int fg_grouped_block_fp8_gemm(const void* A, int64_t lda,
                               const float* As, int64_t as_row_stride, int64_t as_col_stride,
                               const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride, int64_t bs_group_stride,
                               const int32_t* group_ends, int64_t n_groups,
+                              const int32_t* row_index, int64_t index_div, int64_t a_rows,
                               void* C, int64_t ldc, int c_dtype,
                               int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
                               void* workspace, size_t workspace_bytes, void* stream);

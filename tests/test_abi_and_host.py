@@ -155,7 +155,7 @@ def test_widened_entry_points_validate_and_refuse_the_cpu():
         return
     lib = _lib.load()
     # grouped GEMM: K that is not a multiple of 128, a non-bf16 result, a missing table
-    args = lambda k, dt, tab: (1, k, 1, k, 128 * k, 1, 2, 1, 1, 2, 1, 2, tab, 2, 1, 128, dt, 4, 128, k, 128, 128, None, 0, None)
+    args = lambda k, dt, tab: (1, k, 1, k, 128 * k, 1, 2, 1, 1, 2, 1, 2, tab, 2, None, 1, 4, 1, 128, dt, 4, 128, k, 128, 128, None, 0, None)
     assert lib.fg_grouped_block_fp8_gemm(*args(192, _lib.FG_BF16, 1)) == _lib.FG_ERR_UNSUPPORTED
     assert lib.fg_grouped_block_fp8_gemm(*args(256, _lib.FG_F32, 1)) == _lib.FG_ERR_UNSUPPORTED
     assert lib.fg_grouped_block_fp8_gemm(*args(256, _lib.FG_BF16, None)) == _lib.FG_ERR_INVALID_ARG

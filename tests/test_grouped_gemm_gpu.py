@@ -106,7 +106,7 @@ def test_scale_layouts_and_missing_workspace_through_the_c_abi():
     c = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
     st = _lib.load().fg_grouped_block_fp8_gemm(
         a.data_ptr(), K, b.data_ptr(), K, N * K, a_s.data_ptr(), a_s.stride(0), 1,
-        b_s.data_ptr(), b_s.stride(1), 1, b_s.stride(0), e.data_ptr(), E,
+        b_s.data_ptr(), b_s.stride(1), 1, b_s.stride(0), e.data_ptr(), E, None, 1, M,
         c.data_ptr(), N, _lib.DTYPE_CODE[torch.bfloat16], M, N, K, 128, 128,
         None, 0, _lib.current_stream_ptr(torch.device(DEV)))
     _lib.check(st, "fg_grouped_block_fp8_gemm")
@@ -131,3 +131,41 @@ def test_unsupported_requests_fail_loudly():
     with pytest.raises(NotImplementedError):
         flag_gems.grouped_w8a8_block_fp8_matmul(a, b, torch.ones(64, 2, device=DEV), torch.ones(2, 2, 2, device=DEV),
                                                 ends.to(DEV), [128, 128])
+
+
+@pytest.mark.parametrize("T,N,K,top_k", [(64, 1024, 1024, 2), (700, 2144, 512, 2), (1500, 768, 2048, 1), (333, 640, 256, 4)])
+def test_rows_gathered_through_an_index(T, N, K, top_k):
+    """row_index: the kernel reads row sorted_token_ids[m] // top_k of the token matrix for sorted row m, as the
+    reference's MoE kernel does (src/flag_gems/fused/fused_moe.py:1111), instead of a copy of the activations in
+    expert order.  The result must carry the bits of the call on the materialised copy, and match the oracle."""
+    E = 8
+    g = torch.Generator().manual_seed(T + N)
+    xq, wq, xs, ws = _inputs(T, N, K, E, seed=T)
+    # route every token to top_k experts; sorted_token_ids lists (token * top_k + slot) grouped by expert
+    expert_of = torch.randint(0, E, (T * top_k,), generator=g)
+    order = torch.argsort(expert_of, stable=True).to(torch.int32)          # sorted_token_ids
+    ends = torch.cumsum(torch.bincount(expert_of, minlength=E), 0).to(torch.int32)
+    src = (order // top_k).long()
+    got = flag_gems.grouped_w8a8_block_fp8_matmul(xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), ends.to(DEV), [128, 128],
+                                                  row_index=order.to(DEV), index_divisor=top_k)
+    assert got.shape == (T * top_k, N)
+    a_sorted, s_sorted = xq.view(torch.uint8)[src].view(FP8), xs[src]
+    _check(got, a_sorted, wq, s_sorted, ws, ends)
+    materialised = _run(a_sorted, wq, s_sorted, ws, ends)
+    assert torch.equal(got, materialised)
+    # column-major scales of the token matrix are read in place, through the same index
+    xs_cm = xs.to(DEV).t().contiguous().t()
+    again = flag_gems.grouped_w8a8_block_fp8_matmul(xq.to(DEV), wq.to(DEV), xs_cm, ws.to(DEV), ends.to(DEV), [128, 128],
+                                                    row_index=order.to(DEV), index_divisor=top_k)
+    assert torch.equal(again, got)
+
+
+def test_gather_index_is_forced_into_range():
+    T, N, K, E = 100, 256, 256, 2
+    xq, wq, xs, ws = _inputs(T, N, K, E, seed=3)
+    idx = torch.tensor([5, -7, 99, 100, 10 ** 6, 0, 50, 51], dtype=torch.int32)
+    ends = torch.tensor([3, 8], dtype=torch.int32)
+    got = flag_gems.grouped_w8a8_block_fp8_matmul(xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), ends.to(DEV), [128, 128],
+                                                  row_index=idx.to(DEV))
+    src = idx.long().clamp(0, T - 1)
+    _check(got, xq.view(torch.uint8)[src].view(FP8), wq, xs[src], ws, ends)
