@@ -724,10 +724,6 @@ PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs) {
   const int64_t tiles = ceil_div(M, kSplitTile) * ceil_div(N, kSplitTile);
   const int cus = cu_count();
   if (tiles > cus || KB < 4) return p;
-  // One block per compute unit (its four stages take 129 KB of LDS), where the two-stage kernel fits two: with
-  // tiles for 50..70 % of the units the latter, with K cut in two, keeps all units busy and wins (measured M = 512,
-  // N = 4608, K = 7168, 144 tiles: 43 us against 48).
-  if (tiles * 2 > cus && tiles * 10 < (int64_t)cus * 7) return p;
   if (tiles * kSplitWaves * 4 > FG_WORKSPACE_COUNTER_BYTES) return p;
   int64_t splits = cus / tiles;
   if (splits > KB / 5) splits = KB / 5;  // at least five K-blocks per block: a block starts with a full load latency
@@ -735,9 +731,10 @@ PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs) {
   if (splits < 1) splits = 1;
   p.kb_per_split = (int)ceil_div(KB, splits);
   p.splits = (int)ceil_div(KB, (int64_t)p.kb_per_split);
-  // A K-block of a 128 x 128 tile takes ~0.85 us here against ~0.4 us per quarter of a 256 x 256 tile in the
-  // persistent kernel: long K loops stay there (measured M = 512, N = 7168, K = 16384: 109 us here, 86 us there).
-  if (p.kb_per_split > 32) return p;
+  // Long K loops stay with the persistent kernel, whose 256 x 256 tiles need half the LDS reads per MFMA (measured
+  // with up to 128 K-blocks per block allowed here: M = 1024, N = 4096, K = 14336: 74 -> 82 us; with up to 64: M = 512,
+  // same weights: 53 -> 45 us; N = 7168, K = 16384 at M = 256: 59 -> 50 us).
+  if (p.kb_per_split > 64) return p;
   p.workspace_bytes = p.splits > 1 ? FG_WORKSPACE_COUNTER_BYTES + (size_t)tiles * p.splits * kSplitTile * kSplitTile * sizeof(float) : 0;
   p.use = true;
   return p;
