@@ -707,9 +707,12 @@ int launch_tile_split(GemmArgs a, const TileSplitPlan& plan, void* workspace, hi
   return FG_OK;
 }
 
-// 65 <= M <= 1024 with at most one 128 x 128 tile per compute unit: the tile kernel with four LDS stages, one block
+// M >= 65 with at most one 128 x 128 tile per compute unit: the tile kernel with four LDS stages, one block
 // per compute unit, K split over blocks while blocks are fewer than compute units.  With two stages a block that
-// has a compute unit to itself pays a whole load latency per K-block.
+// has a compute unit to itself pays a whole load latency per K-block.  The tile count decides, not M: tall
+// problems against narrow weights (M = 2048, N = 512, K = 7168: 128 tiles) took 73 us in the persistent kernel, which
+// has a quarter of the tiles and shares them along K, and take 22 us here; with more tiles than compute units a
+// second round of this kernel loses to the persistent kernel (M = 1024, N = 4608, K = 7168, 288 tiles: 62 -> 79 us).
 struct PipePlan {
   bool use;
   int splits, kb_per_split;
@@ -718,7 +721,7 @@ struct PipePlan {
 constexpr int kPipeStages = 4;
 PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs) {
   PipePlan p = {false, 1, 0, 0};
-  if (M <= 64 || M > 1024 || K <= 0 || K % 128 != 0) return p;
+  if (M <= 64 || K <= 0 || K % 128 != 0) return p;
   if (xs_rs < 0 || xs_rs >= (1 << 21)) return p;  // 256 rows of scales addressed with 32-bit byte offsets
   const int64_t KB = K / 128;
   const int64_t tiles = ceil_div(M, kSplitTile) * ceil_div(N, kSplitTile);

@@ -107,6 +107,21 @@ def test_few_tiles_split_along_k(M, N, K, dtype):
         assert torch.equal(again.view(torch.int8), got.view(torch.int8))
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 512, 2048), (1300, 1000, 2304), (4096, 384, 1024), (3000, 1100, 896)])
+def test_tall_problems_against_narrow_weights(M, N, K):
+    """More than 1024 rows but at most one 128 x 128 tile per compute unit: the four-stage tile kernel with K split
+    over blocks, not the persistent kernel.  Ragged M and N, 7 and 18 K-blocks; against the oracle and bit-identical
+    on reruns."""
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=23)
+    want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
+    args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    got = flag_gems.w8a8_block_fp8_matmul(*args)
+    assert got.dtype == torch.bfloat16 and got.shape == (M, N)
+    torch.testing.assert_close(got.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    for _ in range(2):
+        assert torch.equal(flag_gems.w8a8_block_fp8_matmul(*args).view(torch.int16), got.view(torch.int16))
+
+
 @pytest.mark.parametrize("M,N,K", [(700, 4000, 4096), (512, 6144, 4096), (1000, 3200, 8192), (300, 10000, 1024),
                                    (768, 7168, 2304), (256, 24576, 1536), (1000, 6100, 4096), (130, 40000, 512)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])

@@ -13,8 +13,8 @@ DEV = "cuda"
 FP8 = torch.float8_e4m3fn
 
 NK = [(1000, 1024), (2112, 7168), (3000, 3072), (5120, 2048), (7168, 2304), (12288, 1536), (4096, 8192), (1536, 16384),
-      (28672, 4096), (512, 4096)]
-MS = [3, 17, 33, 48, 65, 100, 130, 200, 300, 400, 600, 777, 1000, 1100, 1500, 3000, 5000]
+      (28672, 4096), (512, 4096), (512, 7168), (2048, 16384)]
+MS = [3, 17, 33, 48, 65, 100, 130, 200, 300, 400, 600, 777, 1000, 1100, 1500, 2048, 3000, 5000]
 
 
 def _model_us(M, N, K):
