@@ -17,7 +17,7 @@ from .act_quant import (  # noqa: F401
 )
 from .cutlass_scaled_mm import SM_VERSION_NUM, cutlass_scaled_mm, get_sm_version_num  # noqa: F401
 from .fp8_einsum import fp8_einsum, w8a8_block_fp8_bmm  # noqa: F401
-from .grouped_block_fp8_matmul import grouped_w8a8_block_fp8_matmul  # noqa: F401
+from .grouped_block_fp8_matmul import group_ends_from_expert_ids, grouped_w8a8_block_fp8_matmul  # noqa: F401
 from .norm_quant import fused_add_rms_norm, rms_norm, rms_norm_per_token_group_quant_fp8  # noqa: F401
 from .registration import (  # noqa: F401
     all_registered_keys,
@@ -48,6 +48,7 @@ __all__ = [
     "fp8_matmul_noop",
     "fused_add_rms_norm",
     "grouped_w8a8_block_fp8_matmul",
+    "group_ends_from_expert_ids",
     "only_enable",
     "patch_empty_vllm",
     "per_block_cast_to_fp8",

@@ -82,8 +82,8 @@ SIGNATURES = {
     "fg_grouped_block_fp8_gemm": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64,
-         c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_int64,
-         c_void_p, c_size_t, c_void_p],
+         c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64,
+         c_int64, c_int64, c_void_p, c_size_t, c_void_p],
     ),
     "fg_grouped_block_fp8_gemm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "fg_scaled_fp8_gemm": (

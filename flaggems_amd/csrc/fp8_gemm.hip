@@ -1058,6 +1058,7 @@ extern "C" int fg_grouped_block_fp8_gemm(const void* A, int64_t lda,
                                          const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride, int64_t bs_group_stride,
                                          const int32_t* group_ends, int64_t n_groups,
                                          const int32_t* row_index, int64_t index_div, int64_t a_rows,
+                                         int64_t c_rows, const float* row_weight,
                                          void* C, int64_t ldc, int c_dtype,
                                          int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
                                          void* workspace, size_t workspace_bytes, void* stream) {
@@ -1072,6 +1073,9 @@ extern "C" int fg_grouped_block_fp8_gemm(const void* A, int64_t lda,
   if (rc < 0) return rc;
   if (rc == 1) return FG_OK;
   if (!group_ends) FG_FAIL(FG_ERR_INVALID_ARG, "%s: null group table", who);
+  if (c_rows < 0 || c_rows > 0x7FFFFFFF || (c_rows > 0 && !row_index))
+    FG_FAIL(FG_ERR_INVALID_ARG, "%s: c_rows = %lld (scattered results need row_index)", who, (long long)c_rows);
+  if (row_weight && c_rows == 0) FG_FAIL(FG_ERR_INVALID_ARG, "%s: row_weight needs scattered results (c_rows > 0)", who);
   if (K == 0 || K % 128 != 0) FG_FAIL(FG_ERR_UNSUPPORTED, "%s: K = %lld is not a positive multiple of 128", who, (long long)K);
   if (!As || !Bs) FG_FAIL(FG_ERR_INVALID_ARG, "%s: null scale pointer", who);
   if (b_group_stride < 0 || bs_group_stride < 0) FG_FAIL(FG_ERR_INVALID_ARG, "%s: negative group stride", who);
@@ -1085,7 +1089,8 @@ extern "C" int fg_grouped_block_fp8_gemm(const void* A, int64_t lda,
   a.xs_rs = as_row_stride; a.xs_cs = as_col_stride; a.ws_rs = bs_row_stride; a.ws_cs = bs_col_stride;
   a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)(K / 128);
   a.c_dtype = c_dtype;
-  GroupedGemm grouped = {group_ends, n_groups, b_group_stride, bs_group_stride, row_index, index_div, row_index ? a_rows : M};
+  GroupedGemm grouped = {group_ends, n_groups, b_group_stride, bs_group_stride, row_index, index_div, row_index ? a_rows : M,
+                         c_rows, row_weight};
   return launch_grouped(a, grouped, workspace, workspace_bytes, (hipStream_t)stream);
 }
 

@@ -171,6 +171,10 @@ struct GroupedGemm {
   // optional gather: row m of the sorted order is row row_index[m] / index_div of X (x_rows rows) and of its scales
   const int* row_index;
   int64_t index_div, x_rows;
+  // optional scatter (needs row_index): sorted row m is stored to row row_index[m] of C (c_rows rows; entries outside
+  // [0, c_rows) store nothing), multiplied by row_weight[row_index[m]] when row_weight is given; c_rows = 0: row m
+  int64_t c_rows;
+  const float* row_weight;
 };
 int launch_grouped(const GemmArgs& a, const GroupedGemm& grouped, void* workspace, size_t workspace_bytes, hipStream_t stream);
 // workspace that lets launch_grouped read row-major activation scales from a transposed copy

@@ -94,6 +94,12 @@ struct PpArgs {
   // sorted_token_ids // top_k, src/flag_gems/fused/fused_moe.py:1111); entries are forced into [0, x_rows).
   const int* row_index;
   int index_div, x_rows;
+  // Scattered results (c_rows > 0, with row_index): the result of sorted row m goes to row row_index[m] of C, which
+  // has c_rows rows; entries outside [0, c_rows) are padding and store nothing.  With row_weight the fp32 sums are
+  // multiplied by row_weight[row_index[m]] before the cast.  This is where and how the reference's MoE kernel
+  // writes (offs_token, token_mask, MUL_ROUTED_WEIGHT: src/flag_gems/fused/fused_moe.py:1484-1509).
+  int c_rows;
+  const float* row_weight;
   uint64_t group4_magic;  // ceil(2^40 / (4 * tiles_n)) when that divides every tile number exactly, else 0 (see tile_of_sid)
 };
 
@@ -355,9 +361,11 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 // value, in bf16, as the reference's epilogue does (src/flag_gems/fused/cutlass_scaled_mm.py:288-305).
 // ALIGNED: the tile lies inside the matrix; a wavefront then issues exactly kStoresPerTile store instructions.
 constexpr int kStoresPerTile = 16;
-template <int MODE, bool ALIGNED>
+// SCATTER (grouped problems): rows go where out_index says (see PpArgs::c_rows).
+template <int MODE, bool ALIGNED, bool SCATTER = false>
 __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[kTN][kTM], int m_base, int n_base,
-                                           int l16, int lg, int m_end) {
+                                           int l16, int lg, int m_end, const int* out_index = nullptr, int c_rows = 0,
+                                           const float* row_weight = nullptr) {
   if (MODE == kModeRowCol) {
     // eight columns at a time, so that only eight column scales and bias values are live
 #pragma unroll
@@ -403,12 +411,28 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
   for (int j = 0; j < kTM; ++j) {
     const int m = m_base + j * 16 + l16;
     if (!ALIGNED && m >= m_end) continue;
-    uint16_t* const row = reinterpret_cast<uint16_t*>(a.C) + (int64_t)m * a.ldc;
+    int64_t out_row = m;
+    float wgt = 1.f;
+    if (SCATTER && out_index != nullptr) {
+      const int idx = out_index[m];
+      if (idx < 0 || idx >= c_rows) continue;
+      out_row = idx;
+      if (row_weight != nullptr) wgt = row_weight[idx];
+    }
+    uint16_t* const row = reinterpret_cast<uint16_t*>(a.C) + out_row * a.ldc;
     uint32_t w[16];
+    if (SCATTER && row_weight != nullptr) {
 #pragma unroll
-    for (int t = 0; t < kTN; ++t) {
-      w[2 * t] = pack_bf16(acc[t][j][0], acc[t][j][1]);
-      w[2 * t + 1] = pack_bf16(acc[t][j][2], acc[t][j][3]);
+      for (int t = 0; t < kTN; ++t) {
+        w[2 * t] = pack_bf16(acc[t][j][0] * wgt, acc[t][j][1] * wgt);
+        w[2 * t + 1] = pack_bf16(acc[t][j][2] * wgt, acc[t][j][3] * wgt);
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < kTN; ++t) {
+        w[2 * t] = pack_bf16(acc[t][j][0], acc[t][j][1]);
+        w[2 * t + 1] = pack_bf16(acc[t][j][2], acc[t][j][3]);
+      }
     }
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
@@ -689,7 +713,8 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     pending = false;
   };
   auto flush_whole_tile = [&]() __attribute__((always_inline)) {
-    store_tile<MODE, ALIGNED>(g, acc, pend_m, pend_n, l16, lg, pend_m_end);
+    store_tile<MODE, ALIGNED, GROUPED>(g, acc, pend_m, pend_n, l16, lg, pend_m_end, GROUPED && a.c_rows > 0 ? a.row_index : nullptr,
+                                       a.c_rows, a.row_weight);
     clear_acc();
   };
   auto flush_partial_tile = [&]() __attribute__((always_inline)) {
@@ -969,6 +994,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     a.groups = grouped->ends; a.n_groups = (int)grouped->n_groups;
     a.w_group_stride = grouped->w_group_stride; a.ws_group_stride = grouped->ws_group_stride;
     a.row_index = grouped->row_index; a.index_div = (int)grouped->index_div; a.x_rows = (int)grouped->x_rows;
+    a.c_rows = (int)grouped->c_rows; a.row_weight = grouped->row_weight;
   }
   a.g.tiles_n = (int)ceil_div(g.N, kBN);
   const int64_t tiles = (int64_t)a.g.tiles_m * a.g.tiles_n;

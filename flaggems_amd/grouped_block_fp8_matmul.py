@@ -25,6 +25,20 @@ def _cdiv(a: int, b: int) -> int:
     return (a + b - 1) // b
 
 
+def group_ends_from_expert_ids(expert_ids: torch.Tensor, block_m: int, num_experts: int) -> torch.Tensor:
+    """The ``offs`` table of ``grouped_w8a8_block_fp8_matmul`` from the per-block expert table that the reference's
+    ``moe_align_block_size`` returns (one entry per ``block_m`` sorted rows, -1 for blocks past the padded end;
+    src/flag_gems/fused/moe_align_block_size.py:404-517, consumed at src/flag_gems/fused/fused_moe.py:1105).  Blocks
+    of one expert are consecutive and experts ascend, so expert e ends after ``block_m`` times the number of blocks
+    with an id in [0, e].  Stays on the device of ``expert_ids`` and does not synchronise."""
+    assert expert_ids.ndim == 1 and block_m >= 1 and num_experts >= 1
+    ids = expert_ids.to(torch.int64)
+    used = (ids >= 0) & (ids < num_experts)
+    counts = torch.zeros(num_experts, dtype=torch.int64, device=expert_ids.device)
+    counts.scatter_add_(0, ids.clamp(0, num_experts - 1), used.to(torch.int64))
+    return (torch.cumsum(counts, 0) * block_m).to(torch.int32)
+
+
 def grouped_w8a8_block_fp8_matmul(
     A: torch.Tensor,
     B: torch.Tensor,
@@ -35,6 +49,8 @@ def grouped_w8a8_block_fp8_matmul(
     output_dtype: torch.dtype = torch.bfloat16,
     row_index: Optional[torch.Tensor] = None,
     index_divisor: int = 1,
+    scatter_rows: Optional[int] = None,
+    row_weights: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """C[offs[e-1]:offs[e]] = block_fp8_matmul(A[offs[e-1]:offs[e]], B[e]) for every group e.
 
@@ -46,6 +62,13 @@ def grouped_w8a8_block_fp8_matmul(
     ``row_index[m] // index_divisor`` of ``A [T, K]`` and ``As [T, K/block_k]``, the way the reference's MoE kernel
     reads its tokens (``sorted_token_ids // top_k``, src/flag_gems/fused/fused_moe.py:1111); the result still has
     M = ``row_index.numel()`` rows in sorted order.
+
+    With ``scatter_rows`` = R as well, the result has R rows and sorted row m is written to row ``row_index[m]``;
+    entries outside ``[0, R)`` are padding (the reference pads ``sorted_token_ids`` with ``numel``,
+    src/flag_gems/fused/moe_align_block_size.py:404-517) and store nothing, rows no entry names keep what
+    ``torch.empty`` gave them.  ``row_weights`` (fp32 [R]) multiplies the fp32 sums of sorted row m by
+    ``row_weights[row_index[m]]`` before the cast.  Both follow the epilogue of the reference's MoE kernel
+    (src/flag_gems/fused/fused_moe.py:1484-1509: ``offs_token``, ``token_mask``, ``MUL_ROUTED_WEIGHT``).
     """
     logger.debug("GEMS GROUPED_W8A8_BLOCK_FP8_MATMUL")
     assert len(block_size) == 2
@@ -58,6 +81,15 @@ def grouped_w8a8_block_fp8_matmul(
         assert row_index.ndim == 1 and row_index.dtype == torch.int32 and row_index.is_contiguous()
         assert row_index.device == A.device and index_divisor >= 1
         M = row_index.numel()
+    c_rows = 0
+    if scatter_rows is not None:
+        assert row_index is not None, "scattered results are addressed through row_index"
+        assert scatter_rows >= 1
+        c_rows = int(scatter_rows)
+    if row_weights is not None:
+        assert c_rows > 0, "row_weights are indexed like the scattered result"
+        assert row_weights.shape == (c_rows,) and row_weights.dtype == torch.float32 and row_weights.is_contiguous()
+        assert row_weights.device == A.device
     E, N, K2 = B.shape
     assert K == K2
     assert As.shape[0] == T and As.shape[1] == _cdiv(K, block_k)
@@ -73,7 +105,7 @@ def grouped_w8a8_block_fp8_matmul(
     if B.stride(2) != 1:
         B = B.contiguous()
 
-    C = A.new_empty((M, N), dtype=output_dtype)
+    C = A.new_empty((c_rows if c_rows else M, N), dtype=output_dtype)
     if M == 0 or N == 0:
         return C
     _lib.require_gpu(A, "grouped block fp8 gemm")
@@ -89,6 +121,7 @@ def grouped_w8a8_block_fp8_matmul(
             Bs.data_ptr(), Bs.stride(1), Bs.stride(2), Bs.stride(0),
             offs.data_ptr(), E,
             row_index.data_ptr() if row_index is not None else None, index_divisor, T,
+            c_rows, row_weights.data_ptr() if row_weights is not None else None,
             C.data_ptr(), C.stride(0), _lib.DTYPE_CODE[C.dtype],
             M, N, K, block_n, block_k,
             ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,

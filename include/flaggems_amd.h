@@ -292,6 +292,13 @@ int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_batch_stride
  * (entries are forced into [0, a_rows); a_rows * lda must fit 32 bits).  This is how the reference's MoE kernel
  * reads its tokens (rows = sorted_token_ids // top_k, src/flag_gems/fused/fused_moe.py:1111): the caller need not
  * materialise the activations in expert order.  NULL: A and As are already in sorted order (a_rows ignored).
+ * c_rows > 0 (needs row_index): the results are scattered as well -- C has c_rows rows, the result of sorted row m
+ * goes to row row_index[m], and entries outside [0, c_rows) are padding that stores nothing (the reference's
+ * sorted_token_ids pads every expert to a multiple of its block with the value numel,
+ * src/flag_gems/fused/moe_align_block_size.py:404-517).  row_weight (optional DEVICE fp32 [c_rows], with c_rows > 0):
+ * the fp32 sums of sorted row m are multiplied by row_weight[row_index[m]] before the cast to bf16.  This is the
+ * epilogue of the reference's MoE kernel (offs_token, token_mask, MUL_ROUTED_WEIGHT:
+ * src/flag_gems/fused/fused_moe.py:1484-1509).  c_rows = 0: C has M rows in sorted order; row_weight must be NULL.
  *
  * Stands in for the block-wise fp8 branch of fused_moe_kernel (src/flag_gems/fused/fused_moe.py:1378-1450)
  * applied to rows already gathered in expert order, with the group table of aten::_scaled_grouped_mm
@@ -305,6 +312,7 @@ int fg_grouped_block_fp8_gemm(const void* A, int64_t lda,
                               const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride, int64_t bs_group_stride,
                               const int32_t* group_ends, int64_t n_groups,
                               const int32_t* row_index, int64_t index_div, int64_t a_rows,
+                              int64_t c_rows, const float* row_weight,
                               void* C, int64_t ldc, int c_dtype,
                               int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
                               void* workspace, size_t workspace_bytes, void* stream);

@@ -155,10 +155,16 @@ def test_widened_entry_points_validate_and_refuse_the_cpu():
         return
     lib = _lib.load()
     # grouped GEMM: K that is not a multiple of 128, a non-bf16 result, a missing table
-    args = lambda k, dt, tab: (1, k, 1, k, 128 * k, 1, 2, 1, 1, 2, 1, 2, tab, 2, None, 1, 4, 1, 128, dt, 4, 128, k, 128, 128, None, 0, None)
+    args = lambda k, dt, tab: (1, k, 1, k, 128 * k, 1, 2, 1, 1, 2, 1, 2, tab, 2, None, 1, 4, 0, None, 1, 128, dt, 4, 128, k, 128, 128, None, 0, None)
     assert lib.fg_grouped_block_fp8_gemm(*args(192, _lib.FG_BF16, 1)) == _lib.FG_ERR_UNSUPPORTED
     assert lib.fg_grouped_block_fp8_gemm(*args(256, _lib.FG_F32, 1)) == _lib.FG_ERR_UNSUPPORTED
     assert lib.fg_grouped_block_fp8_gemm(*args(256, _lib.FG_BF16, None)) == _lib.FG_ERR_INVALID_ARG
+    # scattered results need the index they are addressed through; row weights need scattered results
+    bad = list(args(256, _lib.FG_BF16, 1))
+    bad[17] = 8
+    assert lib.fg_grouped_block_fp8_gemm(*bad) == _lib.FG_ERR_INVALID_ARG
+    bad[17], bad[18] = 0, 1
+    assert lib.fg_grouped_block_fp8_gemm(*bad) == _lib.FG_ERR_INVALID_ARG
     # block quantizer: only 128 x 128 blocks; empty input is accepted
     q = lambda rows, blk: lib.fg_block_quant_fp8(1, _lib.FG_BF16, rows, 256, 256, 1, _lib.FG_FP8_E4M3FN, 256, 1, 2, 1,
                                                  blk, blk, 1e-4, -448.0, 448.0, 1.0 / 448.0, 1, 0, 0, None)
@@ -181,3 +187,12 @@ def test_batched_workspace_query_is_host_only_and_never_below_the_single_problem
         for batch in (2, 8, 16, 128):
             assert lib.fg_batched_block_fp8_gemm_workspace_bytes(batch, M, N, K) >= single
     assert lib.fg_batched_block_fp8_gemm_workspace_bytes(16, 64, 1024, 7168) > lib.fg_block_fp8_gemm_workspace_bytes(64, 1024, 7168)
+
+
+def test_group_ends_from_the_per_block_expert_table():
+    """expert_ids as the reference's moe_align_block_size lays it out (one entry per block of sorted rows, experts
+    ascending, -1 past the padded end) -> cumulative row ends per expert."""
+    ids = torch.tensor([0, 0, 2, 3, 3, 3, -1, -1], dtype=torch.int32)
+    ends = flag_gems.group_ends_from_expert_ids(ids, 64, 5)
+    assert ends.dtype == torch.int32 and ends.tolist() == [128, 128, 192, 384, 384]
+    assert flag_gems.group_ends_from_expert_ids(torch.tensor([-1], dtype=torch.int32), 16, 2).tolist() == [0, 0]

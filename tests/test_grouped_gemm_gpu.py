@@ -106,7 +106,7 @@ def test_scale_layouts_and_missing_workspace_through_the_c_abi():
     c = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
     st = _lib.load().fg_grouped_block_fp8_gemm(
         a.data_ptr(), K, b.data_ptr(), K, N * K, a_s.data_ptr(), a_s.stride(0), 1,
-        b_s.data_ptr(), b_s.stride(1), 1, b_s.stride(0), e.data_ptr(), E, None, 1, M,
+        b_s.data_ptr(), b_s.stride(1), 1, b_s.stride(0), e.data_ptr(), E, None, 1, M, 0, None,
         c.data_ptr(), N, _lib.DTYPE_CODE[torch.bfloat16], M, N, K, 128, 128,
         None, 0, _lib.current_stream_ptr(torch.device(DEV)))
     _lib.check(st, "fg_grouped_block_fp8_gemm")
@@ -169,3 +169,88 @@ def test_gather_index_is_forced_into_range():
                                                   row_index=idx.to(DEV))
     src = idx.long().clamp(0, T - 1)
     _check(got, xq.view(torch.uint8)[src].view(FP8), wq, xs[src], ws, ends)
+
+
+def _aligned_layout(expert_of, E, block_m):
+    """sorted_token_ids / cumulative ends in the layout of the reference's moe_align_block_size
+    (src/flag_gems/fused/moe_align_block_size.py:404-517): slots grouped by expert, every expert padded to a multiple
+    of block_m with the value numel."""
+    numel = expert_of.numel()
+    ids, ends, total = [], [], 0
+    for e in range(E):
+        mine = torch.nonzero(expert_of == e).flatten().to(torch.int32)
+        pad = (-mine.numel()) % block_m
+        ids += [mine, torch.full((pad,), numel, dtype=torch.int32)]
+        total += mine.numel() + pad
+        ends.append(total)
+    return torch.cat(ids), torch.tensor(ends, dtype=torch.int32)
+
+
+@pytest.mark.parametrize("weighted", [False, True])
+@pytest.mark.parametrize("T,N,K,top_k,block_m", [(64, 1024, 1024, 2, 16), (700, 2144, 512, 2, 64), (333, 640, 256, 4, 64),
+                                                 (1500, 768, 2048, 1, 128)])
+def test_results_scattered_and_weighted_like_the_moe_kernel(T, N, K, top_k, block_m, weighted):
+    """The whole GEMM of the reference's MoE kernel (src/flag_gems/fused/fused_moe.py:1084-1125, 1484-1509): rows read
+    through sorted_token_ids // top_k, results written to row sorted_token_ids[m] of a [T * top_k, N] matrix, padding
+    entries (value numel) skipped, and with MUL_ROUTED_WEIGHT the fp32 sums multiplied by the slot's routing weight
+    before the cast.  Expected: the oracle's per-expert product of every slot's token, times the weight in fp32."""
+    E = 8
+    g = torch.Generator().manual_seed(T * 3 + N)
+    xq, wq, xs, ws = _inputs(T, N, K, E, seed=T + 1)
+    slots = T * top_k
+    expert_of = torch.randint(0, E, (slots,), generator=g)
+    expert_of[expert_of == 5] = 4                                   # an expert nobody is routed to
+    sorted_ids, ends = _aligned_layout(expert_of, E, block_m)
+    assert sorted_ids.numel() == int(ends[-1]) and sorted_ids.numel() % block_m == 0
+    weights = torch.rand(slots, generator=g) + 0.25 if weighted else None
+    got = flag_gems.grouped_w8a8_block_fp8_matmul(
+        xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), ends.to(DEV), [128, 128], row_index=sorted_ids.to(DEV),
+        index_divisor=top_k, scatter_rows=slots, row_weights=weights.to(DEV) if weighted else None)
+    assert got.shape == (slots, N) and got.dtype == torch.bfloat16
+    # oracle: slots in expert order without padding, then back to slot order
+    order = torch.argsort(expert_of, stable=True)
+    src = (order // top_k).long()
+    plain_ends = torch.cumsum(torch.bincount(expert_of, minlength=E), 0).to(torch.int32)
+    ref_sorted = O.grouped_block_fp8_matmul_ref(xq.view(torch.uint8)[src].view(FP8), wq, xs[src], ws, plain_ends, [128, 128])
+    want = torch.empty(slots, N)
+    want[order] = ref_sorted * (weights[order].unsqueeze(1) if weighted else 1.0)
+    torch.testing.assert_close(got.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    err = (got.cpu().double() - want.double()).abs()
+    assert float((err / (want.double().abs() / 128 + 2e-3)).max()) < 1.0
+    # the same bits as the call that leaves the rows in sorted order, row by row (no weights: nothing but the row moves)
+    if not weighted:
+        in_order = flag_gems.grouped_w8a8_block_fp8_matmul(
+            xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), ends.to(DEV), [128, 128], row_index=sorted_ids.to(DEV),
+            index_divisor=top_k)
+        real = (sorted_ids < slots).to(DEV)
+        assert torch.equal(got[sorted_ids.to(DEV)[real].long()], in_order[real])
+    again = flag_gems.grouped_w8a8_block_fp8_matmul(
+        xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), ends.to(DEV), [128, 128], row_index=sorted_ids.to(DEV),
+        index_divisor=top_k, scatter_rows=slots, row_weights=weights.to(DEV) if weighted else None)
+    assert torch.equal(again, got)
+
+
+def test_scatter_skips_padding_and_rows_out_of_range():
+    """Entries outside [0, scatter_rows) store nothing: the rows they would have hit keep their contents."""
+    T, N, K, E = 40, 256, 256, 2
+    xq, wq, xs, ws = _inputs(T, N, K, E, seed=11)
+    idx = torch.tensor([3, 40, -1, 7, 10 ** 6, 0, 39, 12], dtype=torch.int32)
+    ends = torch.tensor([4, 8], dtype=torch.int32)
+    lib = _lib.load()
+    c = torch.full((T, N), 7.0, dtype=torch.bfloat16, device=DEV)
+    a, b, a_s, b_s, e, ix = xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), ends.to(DEV), idx.to(DEV)
+    st = lib.fg_grouped_block_fp8_gemm(
+        a.data_ptr(), K, b.data_ptr(), K, N * K, a_s.data_ptr(), a_s.stride(0), 1,
+        b_s.data_ptr(), b_s.stride(1), 1, b_s.stride(0), e.data_ptr(), E, ix.data_ptr(), 1, T, T, None,
+        c.data_ptr(), N, _lib.DTYPE_CODE[torch.bfloat16], idx.numel(), N, K, 128, 128,
+        None, 0, _lib.current_stream_ptr(torch.device(DEV)))
+    _lib.check(st, "fg_grouped_block_fp8_gemm")
+    torch.cuda.synchronize()
+    written = [3, 7, 0, 39, 12]
+    untouched = sorted(set(range(T)) - set(written))
+    assert (c[untouched] == 7.0).all()
+    src = idx.long().clamp(0, T - 1)
+    ref = O.grouped_block_fp8_matmul_ref(xq.view(torch.uint8)[src].view(FP8), wq, xs[src], ws, ends, [128, 128])
+    for m, row in enumerate(idx.tolist()):
+        if 0 <= row < T:
+            torch.testing.assert_close(c[row].cpu().float(), ref[m], rtol=1e-2, atol=1e-2)
