@@ -17,7 +17,7 @@ Prints ONE JSON line with the driver's fields plus
   cpu_baseline  the CPU oracle (torch restatement of the reference's torch implementation) timed on
                 the host cores on a bounded sample of the same sweep
   detail        per-(M, N, K) time, TFLOP/s, GB/s and roofline fractions (MFMA for M >= 512, HBM below)
-  cutlass_scaled_mm_n8192_k8192_bias, llama3_8b_linears
+  block_fp8_gemm_pow2_scales_m4096, cutlass_scaled_mm_n8192_k8192_bias, llama3_8b_linears
                 the other configurations of the path (per-token x per-channel scaled GEMM with bias; Llama-3-8B
                 linears as GEMM alone and as act_quant + GEMM), graph replays of one shape at a time with ONE copy
                 of the weights (small-M figures there may be served by the 256 MB Infinity Cache), not part of `value`
@@ -353,6 +353,27 @@ def main():
     def time_eager(fn, reps):
         return time_graph(lambda r: fn(), launches=max(reps, 20))
 
+    # the M = 4096 GEMMs of the sweep once more with power-of-two scales (ue8m0 quantization: act_quant scale_fmt
+    # "ue8m0", per_block_cast_to_fp8 use_ue8m0), through the entry point that hands the scales to the matrix
+    # instruction; the same call without that promise beside it
+    pow2 = []
+    for (n, k) in DSV3_NK:
+        x = torch.randn(4096, k, device=dev, generator=gen).bfloat16()
+        xq2, xs2 = flag_gems.act_quant_triton(x, 128, "ue8m0")
+        w = (0.02 * torch.randn(n, k, device=dev, generator=gen)).bfloat16()
+        wq2, ws2 = flag_gems.per_block_cast_to_fp8(w, use_ue8m0=True)
+        del x, w
+        us_plain = time_eager(lambda: flag_gems.w8a8_block_fp8_matmul(xq2, wq2, xs2, ws2, [128, 128]), 20)
+        us_pow2 = time_eager(lambda: flag_gems.w8a8_block_fp8_matmul(xq2, wq2, xs2, ws2, [128, 128], scales_are_powers_of_two=True), 20)
+        pow2.append({"M": 4096, "N": n, "K": k, "us": round(us_pow2, 2), "tflops": round(gemm_flops(4096, n, k) / us_pow2 / 1e6, 1),
+                     "frac_mfma": round(gemm_flops(4096, n, k) / us_pow2 / 1e6 / PEAK_FP8_TFLOPS, 4),
+                     "us_without_the_promise": round(us_plain, 2)})
+        del xq2, xs2, wq2, ws2
+    pow2_total = sum(r["us"] for r in pow2)
+    pow2_summary = {"rows": pow2, "tflops": round(sum(gemm_flops(4096, n, k) for (n, k) in DSV3_NK) / pow2_total / 1e6, 1),
+                    "frac_mfma": round(sum(gemm_flops(4096, n, k) for (n, k) in DSV3_NK) / pow2_total / 1e6 / PEAK_FP8_TFLOPS, 4),
+                    "note": "not the headline configuration: scales restricted to powers of two"}
+
     # cutlass_scaled_mm semantics: per-token x per-channel scales, bf16 bias, N = K = 8192
     scaled = []
     nk = 8192
@@ -534,6 +555,7 @@ def main():
         "weight_quantizer_128x128": weight_quant,
         "silu_mul_quantizer": fused,
         "rms_norm_quantizer": norm_quant,
+        "block_fp8_gemm_pow2_scales_m4096": pow2_summary,
         "cutlass_scaled_mm_n8192_k8192_bias": scaled,
         "scaled_mm_unquantized_operands": generic,
         "fp8_einsum_bhr_hdr": einsum,

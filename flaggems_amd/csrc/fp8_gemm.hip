@@ -850,22 +850,23 @@ extern "C" size_t fg_scaled_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64
   return fg_block_fp8_gemm_workspace_bytes(M, N, K);
 }
 
-extern "C" int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
+namespace fg {
+namespace {
+int block_fp8_gemm(const char* who, int scales_pow2, const void* A, int64_t lda, const void* B, int64_t ldb,
                                  const float* As, int64_t as_row_stride, int64_t as_col_stride,
                                  const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride,
                                  void* C, int64_t ldc, int c_dtype,
                                  int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
                                  void* workspace, size_t workspace_bytes, void* stream) {
-  using namespace fg;
   if (block_n != 128 || block_k != 128)
-    FG_FAIL(FG_ERR_UNSUPPORTED, "fg_block_fp8_gemm: only 128x128 scale blocks are implemented (got %lld x %lld)",
+    FG_FAIL(FG_ERR_UNSUPPORTED, "%s: only 128x128 scale blocks are implemented (got %lld x %lld)", who,
             (long long)block_n, (long long)block_k);
   if (c_dtype != FG_BF16 && c_dtype != FG_F16 && c_dtype != FG_F32)
-    FG_FAIL(FG_ERR_INVALID_ARG, "fg_block_fp8_gemm: c_dtype %d", c_dtype);
-  int rc = check_common(A, B, C, lda, ldb, ldc, M, N, K, "fg_block_fp8_gemm");
+    FG_FAIL(FG_ERR_INVALID_ARG, "%s: c_dtype %d", who, c_dtype);
+  int rc = check_common(A, B, C, lda, ldb, ldc, M, N, K, who);
   if (rc < 0) return rc;
   if (rc == 1) return FG_OK;
-  if (K > 0 && (!As || !Bs)) FG_FAIL(FG_ERR_INVALID_ARG, "fg_block_fp8_gemm: null scale pointer");
+  if (K > 0 && (!As || !Bs)) FG_FAIL(FG_ERR_INVALID_ARG, "%s: null scale pointer", who);
   GemmArgs a = {};
   a.X = (const uint8_t*)A; a.W = (const uint8_t*)B; a.C = C;
   a.xs = As; a.ws = Bs; a.bias = nullptr;
@@ -873,7 +874,30 @@ extern "C" int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int6
   a.xs_rs = as_row_stride; a.xs_cs = as_col_stride; a.ws_rs = bs_row_stride; a.ws_cs = bs_col_stride;
   a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)ceil_div(K, 128);
   a.c_dtype = c_dtype;
+  a.scales_pow2 = scales_pow2;
   return launch_gemm<kModeBlock>(a, workspace, workspace_bytes, (hipStream_t)stream);
+}
+}  // namespace
+}  // namespace fg
+
+extern "C" int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
+                                 const float* As, int64_t as_row_stride, int64_t as_col_stride,
+                                 const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride,
+                                 void* C, int64_t ldc, int c_dtype,
+                                 int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+  return fg::block_fp8_gemm("fg_block_fp8_gemm", 0, A, lda, B, ldb, As, as_row_stride, as_col_stride, Bs, bs_row_stride, bs_col_stride,
+                            C, ldc, c_dtype, M, N, K, block_n, block_k, workspace, workspace_bytes, stream);
+}
+
+extern "C" int fg_block_fp8_gemm_pow2_scales(const void* A, int64_t lda, const void* B, int64_t ldb,
+                                             const float* As, int64_t as_row_stride, int64_t as_col_stride,
+                                             const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride,
+                                             void* C, int64_t ldc, int c_dtype,
+                                             int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
+                                             void* workspace, size_t workspace_bytes, void* stream) {
+  return fg::block_fp8_gemm("fg_block_fp8_gemm_pow2_scales", 1, A, lda, B, ldb, As, as_row_stride, as_col_stride, Bs, bs_row_stride,
+                            bs_col_stride, C, ldc, c_dtype, M, N, K, block_n, block_k, workspace, workspace_bytes, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

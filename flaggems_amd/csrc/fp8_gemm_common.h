@@ -22,6 +22,8 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int c_dtype, bias_dtype;
   int xs_per_row, ws_per_col;
+  // block mode: the caller guarantees that every scale is a power of two (only the persistent kernel makes use of it)
+  int scales_pow2;
   // tile kernel with K split over blocks (fp8_gemm.hip): block b computes K-blocks
   // [split * kb_per_split, ...) of tile b % tiles, split = b / tiles
   int splits, kb_per_split;

@@ -288,6 +288,17 @@ __device__ __forceinline__ void mfma_accumulate(v4f& c, const v8i& w, const v8i&
   asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(c) : "v"(w), "v"(x));
 }
 
+// Scales that are powers of two (POW2): the block-scaled form of the instruction multiplies the products by
+// 2^(sw - 127) * 2^(sx - 127) on their way into the sum, so the matrix pipe accumulates the scaled K-blocks itself and
+// the multiply phase has no vector-ALU work at all.  sw / sx: E8M0 exponent in the low byte of a register per lane,
+// taken for the operand row the lane holds (lane & 15); every 32-element K group of a row gets the same one here.
+__device__ __forceinline__ void mfma_scaled_accumulate(v4f& c, const v8i& w, const v8i& x, int sw, int sx) {
+  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[0,0,0] op_sel_hi:[0,0,0]"
+               : "+v"(c)
+               : "v"(w), "v"(x), "v"(sw), "v"(sx));
+}
+__device__ __forceinline__ int e8m0_of(float s) { return (int)((float_to_bits(s) >> 23) & 0xFFu); }
+
 // acc += p * s.  A wavefront issues one instruction every four cycles and the matrix pipe takes an MFMA of
 // this shape every 32, so a multiply step has eight issue slots: the MFMA, these four FMAs and three spare
 // (LDS reads, tile loads).  p is the result of the MFMA issued TWO steps earlier: at least 64 cycles have
@@ -541,8 +552,10 @@ __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (
 // ALIGNED: M and N are multiples of the tile; no tile has an edge, and the per-lane offsets of the tile loads
 // and of the scale loads never change (a tile change then touches scalar registers only).
 // GROUPED: the rows are segments with a weight matrix each (see PpArgs::groups).
-template <bool SK, int MODE, bool ALIGNED, bool GROUPED = false>
+// POW2: block scales that are powers of two, applied by the instruction (mfma_scaled_accumulate).
+template <bool SK, int MODE, bool ALIGNED, bool GROUPED = false, bool POW2 = false>
 __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
+  static_assert(!POW2 || (MODE == kModeBlock && !GROUPED), "power-of-two scales: plain block-scaled problems");
   static_assert(!GROUPED || (!SK && !ALIGNED && MODE == kModeBlock), "grouped problems: whole tiles with edges, block scales");
   using Walk = WalkT<GROUPED>;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -738,6 +751,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     // Scales of this step were requested a step ago; the only younger vector-memory operations are the eight
     // tile loads that followed them (for A those have landed as well: it waited at the end of its multiply).
     float xs[kTM], sc[kTM];
+    int se[kTM], swe = 0;  // POW2: exponents of the activation-row scales and of the weight-block scale
     const bool more = T + 1 < total;
     float ws = 1.f;
     if (MODE == kModeBlock) {
@@ -787,8 +801,14 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
       }
     }
     if (MODE == kModeBlock) {
+      if (POW2) {
+        swe = e8m0_of(ws);
 #pragma unroll
-      for (int j = 0; j < kTM; ++j) sc[j] = xs[j] * ws;
+        for (int j = 0; j < kTM; ++j) se[j] = e8m0_of(xs[j]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < kTM; ++j) sc[j] = xs[j] * ws;
+      }
     }
     const bool flushed_now = pending;
     if (pending) flush_whole_tile();  // after the waits, so that no wait of this slot covers the stores
@@ -802,6 +822,13 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
       for (int st = 0; st < kTN * kTM; ++st) {
         const int t = st / kTM, j = st % kTM;
         mfma_accumulate(acc[t][j], wr[t % 3], xf[j]);
+        if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
+      }
+    } else if (POW2) {
+#pragma unroll
+      for (int st = 0; st < kTN * kTM; ++st) {
+        const int t = st / kTM, j = st % kTM;
+        mfma_scaled_accumulate(acc[t][j], wr[t % 3], xf[j], swe, se[j]);
         if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
       }
     } else {
@@ -1005,15 +1032,19 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     // n * magic >> 40 == n / d for every n with n * d < 2^40 (the tile numbers of whole problems are below `tiles`)
     a.group4_magic = (d > 0 && (uint64_t)tiles * d < (1ull << 40)) ? ((1ull << 40) + d - 1) / d : 0;
   }
-  static PerDeviceFlags lds_limit_raised[7] = {};
-  const void* const kernels[7] = {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false>),
+  static PerDeviceFlags lds_limit_raised[11] = {};
+  const void* const kernels[11] = {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, true>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, false>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, true>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false, true>)};
-  for (int i = 0; i < 7; ++i) {
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false, true>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false, false, true>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, true, false, true>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false, false, true>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, true>)};
+  for (int i = 0; i < 11; ++i) {
     const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised[i], kLdsBytes, kernels[i]);
     if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
   }
@@ -1066,6 +1097,11 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     kern = aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true> : fp8_gemm_pingpong_kernel<true, kModeBlock, false>;
   else
     kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeBlock, true> : fp8_gemm_pingpong_kernel<false, kModeBlock, false>;
+  const bool pow2 = mode == kModeBlock && grouped == nullptr && g.scales_pow2 != 0;
+  if (pow2) {
+    if (a.sk) kern = aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, true> : fp8_gemm_pingpong_kernel<true, kModeBlock, false, false, true>;
+    else kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeBlock, true, false, true> : fp8_gemm_pingpong_kernel<false, kModeBlock, false, false, true>;
+  }
   if (tp.use && !a.sk && workspace != nullptr && workspace_bytes >= need && (size_t)tp.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
       (uintptr_t)workspace % 16 == 0) {
     PpArgs whole = a;
@@ -1081,6 +1117,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     rest.partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
     void (*shared)(PpArgs) = fp8_gemm_pingpong_kernel<true, kModeBlock, false>;
     if (aligned) shared = fp8_gemm_pingpong_kernel<true, kModeBlock, true>;
+    if (pow2) shared = aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, true> : fp8_gemm_pingpong_kernel<true, kModeBlock, false, false, true>;
     FG_LAUNCH(shared, dim3((uint32_t)tp.grid), dim3(kThreads), kLdsBytes, stream, rest);
     FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel (last tiles)");
     return FG_OK;

@@ -27,7 +27,7 @@ def _cdiv(a: int, b: int) -> int:
     return (a + b - 1) // b
 
 
-def _launch_block_gemm(a2d, b, as2d, bs, c2d, block_n: int, block_k: int) -> None:
+def _launch_block_gemm(a2d, b, as2d, bs, c2d, block_n: int, block_k: int, scales_pow2: bool = False) -> None:
     _lib.require_gpu(a2d, "block fp8 gemm")
     lib = _lib.load()
     m, k = a2d.shape
@@ -36,7 +36,8 @@ def _launch_block_gemm(a2d, b, as2d, bs, c2d, block_n: int, block_k: int) -> Non
     with torch.cuda.device(dev):
         ws_bytes = lib.fg_block_fp8_gemm_workspace_bytes(m, n, k)
         ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
-        status = lib.fg_block_fp8_gemm(
+        entry = lib.fg_block_fp8_gemm_pow2_scales if scales_pow2 else lib.fg_block_fp8_gemm
+        status = entry(
             a2d.data_ptr(), a2d.stride(0) if m > 1 else max(k, a2d.stride(0)),
             b.data_ptr(), b.stride(0) if n > 1 else max(k, b.stride(0)),
             as2d.data_ptr(), as2d.stride(0), as2d.stride(1),
@@ -56,11 +57,17 @@ def w8a8_block_fp8_matmul(
     Bs: torch.Tensor,
     block_size: List[int],
     output_dtype: torch.dtype = torch.bfloat16,
+    scales_are_powers_of_two: bool = False,
 ) -> torch.Tensor:
     """C = (A dequantised by As per 1 x block_k group) @ (B dequantised by Bs per block_n x block_k block)^T.
 
     A [..., K] contiguous e4m3fn, As [..., ceil(K/block_k)] fp32, B [N, K] e4m3fn,
     Bs [ceil(N/block_n), ceil(K/block_k)] fp32; returns [..., N] in ``output_dtype``.
+
+    ``scales_are_powers_of_two`` (not in the reference's signature): the caller's promise that every entry of As and
+    Bs is a power of two, as the ue8m0 forms of the quantizers produce them; large problems then run with the scales
+    inside the matrix instruction (``fg_block_fp8_gemm_pow2_scales``).  Scales of dtype ``float8_e8m0fnu`` carry
+    that promise by construction.
     """
     logger.debug("GEMS W8A8_BLOCK_FP8_MATMUL")
     assert len(block_size) == 2
@@ -79,6 +86,8 @@ def w8a8_block_fp8_matmul(
         raise NotImplementedError(f"w8a8_block_fp8_matmul: operands must be float8_e4m3fn, got {A.dtype}, {B.dtype}")
     if output_dtype not in _OUT_DTYPES:
         raise NotImplementedError(f"w8a8_block_fp8_matmul: unsupported output dtype {output_dtype}")
+    e8m0 = getattr(torch, "float8_e8m0fnu", None)
+    pow2 = scales_are_powers_of_two or (e8m0 is not None and As.dtype == e8m0 and Bs.dtype == e8m0)
     if As.dtype != torch.float32 or Bs.dtype != torch.float32:
         As, Bs = As.to(torch.float32), Bs.to(torch.float32)
 
@@ -90,7 +99,7 @@ def w8a8_block_fp8_matmul(
         B = B.contiguous()
     a2d = A.view(M, K)
     as2d = As if As.dim() == 2 else As.reshape(M, As.shape[-1])
-    _launch_block_gemm(a2d, B, as2d, Bs, C.view(M, N), block_n, block_k)
+    _launch_block_gemm(a2d, B, as2d, Bs, C.view(M, N), block_n, block_k, pow2)
     return C
 
 
@@ -104,7 +113,8 @@ def fp8_matmul(
     """Block-wise scaled FP8 matmul with 128-wide groups and bf16 output.
 
     a [..., K] e4m3fn contiguous, a_s [..., K/128], b [N, K] e4m3fn contiguous, b_s [N/128, K/128];
-    scales given as float8_e8m0fnu are widened to fp32 first.
+    scales given as float8_e8m0fnu are widened to fp32 first (and, being powers of two, may be applied inside the
+    matrix instruction: ``fg_block_fp8_gemm_pow2_scales``).
     """
     logger.debug("GEMS FP8_MATMUL")
     assert b.ndim == 2
@@ -114,14 +124,15 @@ def fp8_matmul(
     M = a.numel() // K
     N, K2 = b.shape
     assert K == K2
-    if scale_dtype == torch.float8_e8m0fnu:
+    pow2 = scale_dtype == torch.float8_e8m0fnu
+    if pow2:
         a_s = a_s.to(torch.float32)
         b_s = b_s.to(torch.float32)
     out_shape = (*a.size()[:-1], N)
     C = torch.empty((M, N), device=a.device, dtype=torch.bfloat16)
     if M == 0 or N == 0:
         return C.view(out_shape)
-    _launch_block_gemm(a.view(M, K), b, a_s.view(M, -1), b_s, C, GROUP_SIZE, GROUP_SIZE)
+    _launch_block_gemm(a.view(M, K), b, a_s.view(M, -1), b_s, C, GROUP_SIZE, GROUP_SIZE, pow2)
     return C.view(out_shape)
 
 

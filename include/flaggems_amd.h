@@ -230,6 +230,27 @@ int fg_block_fp8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
 size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
+ * fg_block_fp8_gemm for scales the caller knows to be powers of two (fp32 values with a zero mantissa: E8M0 scales
+ * widened to fp32, or the ue8m0 rounding of the quantizers).  Same arguments, same workspace rules, same result up
+ * to the order of fp32 roundings: where the persistent kernel takes the problem (M > 128, K a multiple of 128,
+ * 16-byte aligned rows, bf16 result) the scales go into the block-scaled form of the MFMA instruction as E8M0
+ * exponents and the matrix pipe accumulates the scaled K-blocks itself, instead of one fp32 multiply-add per
+ * result element and K-block; every other shape runs exactly the kernels of fg_block_fp8_gemm.  A scale that is not
+ * a power of two is used as if its mantissa were zero: the caller's guarantee is not checked.
+ *
+ * Stands in for fp8_matmul with scale_dtype = float8_e8m0fnu (src/flag_gems/ops/fp8_matmul.py:137-205: the scales
+ * arrive as E8M0 and are widened at :165-167) and for block-fp8 GEMMs whose operands were quantized with power-of-two
+ * scales (per_token_cast_to_fp8 / per_block_cast_to_fp8 with use_ue8m0, tests/test_fp8_einsum.py:63-103;
+ * act_quant with scale_fmt "ue8m0", src/flag_gems/fused/act_quant.py:111-174).
+ */
+int fg_block_fp8_gemm_pow2_scales(const void* A, int64_t lda, const void* B, int64_t ldb,
+                                  const float* As, int64_t as_row_stride, int64_t as_col_stride,
+                                  const float* Bs, int64_t bs_row_stride, int64_t bs_col_stride,
+                                  void* C, int64_t ldc, int c_dtype,
+                                  int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * fg_block_fp8_gemm without the workspace arguments, for callers that cannot allocate device memory: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose
  * wrappers allocate through torch).  The workspace is an array of FG_NOALLOC_SCRATCH_BYTES built into the library's
