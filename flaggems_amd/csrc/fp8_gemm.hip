@@ -807,7 +807,9 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
     // resident at a time, two on each compute unit (560 tiles: M = 1280, N = 7168, K = 2304 went from 36 to 51 us); the persistent kernel has a quarter of the tiles and spends its
     // time filling and draining.  Measured: M = 256, N = 24576, K = 1536: 27.7 -> 23.4 us; M = 768, N = 7168, K = 2304:
     // 34.8 -> 28.9; N = 6144, K = 4096: 50.0 -> 43.4; M = 1024, N = 7168, K = 2304: 35.3 -> 29.6 (N = K = 8192: 86 -> 89).
-    if (direct && a.M > 128 && a.M <= 1024 && tiles128 > 256 && ((tiles128 <= 512 && a.KB <= 32) || (tiles128 <= 448 && a.KB <= 64)))
+    // The tile count decides, whatever M: M = 2048, N = 3072, K = 2048: 34.0 -> 24.8 us; M = 3072, N = K = 2048: 34.0 -> 24.2;
+    // M = 2048, N = K = 4096: 51.0 -> 45.2; M = 2048, N = 2112, K = 7168: 66.5 -> 63.5.
+    if (direct && a.M > 128 && tiles128 > 256 && ((tiles128 <= 512 && a.KB <= 32) || (tiles128 <= 448 && a.KB <= 64)))
       return launch_cfg<128, 128, 4, 2, MODE, true>(a, stream);  // eight wavefronts: 7-13 % faster than four on these shapes
   }
   const bool big = a.M > 128;

@@ -911,13 +911,15 @@ SkPlan plan_stream_k(int64_t tiles, int KB, int cus) {
   // ranges of total / cus steps lose unless they happen to cut every tile alike.  They pay when the cuts are long
   // and nearly fill the GPU: measured M = 512, N = 7168, K = 16384 (56 tiles): 4 cuts of 32 steps on 224 units
   // 86 us against 110 us for 256 ranges of 28 steps; M = 1024, same N and K: 2 cuts of 64 steps 125 us against
-  // 174 us.  Cuts of 8 or 28 steps lose to the contiguous ranges (the partial tiles dominate either way).
+  // 174 us.  Cuts down to 16 steps on at least half of the units still win (M = 2048, N = 3072, K = 8192, 96 tiles in
+  // 2 cuts of 32: 84 -> 70 us; M = 4096, N = 1536, K = 7168, 96 tiles in 2 cuts of 28: 76 -> 65 us; M = 3072,
+  // N = 2112, K = 7168: 85 -> 73 us); cuts of 8 steps lose to the contiguous ranges.
   const bool ranges_cut_tiles_alike = total % cus == 0 && q > 0 && KB % q == 0;
   if (!ranges_cut_tiles_alike) {
     for (int64_t S = cus / tiles; S >= 2; --S) {
       if (KB % S != 0) continue;
       const int64_t cut = KB / S;
-      if (cut < 32 || tiles * S * 5 < (int64_t)cus * 4) break;  // shorter cuts or emptier grids only get worse
+      if (cut < 16 || tiles * S * 2 < (int64_t)cus) break;  // shorter cuts or emptier grids only get worse
       if ((cut + 16) >= dp_steps) break;                         // ~16 steps to publish and add the partial tiles
       p.use = true; p.grid = (int)(tiles * S); p.q = (int)cut; p.r = 0; p.split = (int)S;
       return p;
