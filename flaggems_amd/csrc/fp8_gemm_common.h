@@ -129,6 +129,8 @@ struct SmallMPlan {
   bool staged;    // weight bytes fetched in 256-byte runs (K-block pairs) and transposed through LDS
   int tmx;        // 16-row activation fragments: 1, 2 or 4
   int rg;         // 16-row weight groups per output chunk: 1, 2 or 4
+  int q;          // staged: 4-row weight groups the kernel loads per chunk (<= 4 * rg)
+  bool xlds;      // staged: the block keeps the activations of its K range in LDS
   int waves;      // wavefronts per block: 4 or 8
   int kpw;        // K-blocks (K-block pairs when staged) per wavefront
   int splits;     // blocks along K that share one 64-row output chunk

@@ -1,25 +1,29 @@
 // Small-M (decode) FP8 GEMM for gfx950: M <= 64 activation rows against an [N, K] weight that is read
-// exactly once.  The kernel is bound by HBM bandwidth, so the design is about bytes in flight, not
-// about the matrix core:
+// exactly once.  The kernels are bound by HBM bandwidth and, for launches of a few microseconds, by what a
+// compute unit does before and after its bytes arrive, so the design is about bytes in flight and about the
+// number of vector-memory instructions, not about the matrix core.  Two kernels:
 //
-//  * Work unit = (64 weight rows) x (one 128-byte K-block).  A wavefront streams its units straight
-//    from global memory into registers: lane l owns weight row (l & 15) of each of the four 16-row
-//    groups and the K bytes [16g, 16g+16) and [64+16g, 64+16g+16), g = l >> 4 -- the MFMA operand
-//    layout, so no LDS staging is needed; the tiny activation fragment is fetched the same way (it
-//    stays in L2).  The next unit's loads are issued before the current unit is multiplied.
-//  * A block of 4 or 8 wavefronts shares one 64-row output chunk; its wavefronts take interleaved
-//    K-blocks (adjacent wavefronts read adjacent 128-byte pieces of the same rows) and add their
-//    fp32 results in LDS.
-//  * When N/64 chunks do not give enough blocks to cover the GPU, several blocks split K.  Each
-//    writes an fp32 partial tile to the workspace; the block that arrives last (a counter per
-//    chunk) adds the partials in split order -- a fixed order, so results do not depend on timing --
-//    and resets the counter, so the workspace needs zeroing only once, when it is allocated.
+//  * fp8_gemm_transpose_kernel (M <= 32, K >= 1024): the weight rows are dealt out evenly over one block per
+//    compute unit; a block's wavefronts take interleaved pairs of K-blocks, fetch them in runs of 256 bytes per
+//    row and transpose them into MFMA operand layout through wavefront-private LDS slabs (see the kernel).
+//  * fp8_gemm_smallm_kernel (the rest): work unit = (64 weight rows) x (one 128-byte K-block).  A wavefront
+//    streams its units straight from global memory into registers: lane l owns weight row (l & 15) of each of
+//    the four 16-row groups and the K bytes [16g, 16g+16) and [64+16g, 64+16g+16), g = l >> 4 -- the MFMA
+//    operand layout, so no LDS staging is needed; the tiny activation fragment is fetched the same way (it stays
+//    in L2).  The next unit's loads are issued before the current unit is multiplied.
+//
+// In both, the wavefronts of a block add their fp32 results in LDS.  When the chunks of rows do not give enough
+// blocks to cover the GPU, several blocks split K.  Each writes an fp32 partial tile to the workspace; the block
+// that arrives last (a counter per chunk) adds the partials in split order -- a fixed order, so results do not
+// depend on timing -- and resets the counter, so the workspace needs zeroing only once, when it is allocated.
 //
 // Arithmetic follows the tile kernel: per K-block products accumulated by the fp8 MFMA, multiplied by
 // As[m, kb] * Bs[n / 128, kb] in fp32 (block mode) or accumulated unscaled and scaled per row and column
 // at the end (row/column mode).
 
 #include "fp8_gemm_common.h"
+
+#include <algorithm>
 
 namespace fg {
 namespace {
@@ -30,15 +34,17 @@ constexpr int kRowGroups = 4;   // 16-row MFMA groups per chunk
 struct SmallArgs {
   GemmArgs g;
   int kpw, splits, n_chunks;
+  // staged kernels: chunk c owns rows_lo + (c < rows_rem) weight rows, the chunks in ascending row order; the
+  // activations of the block's K range are kept in LDS with rows x_lds_stride bytes apart (0: not kept)
+  int rows_lo, rows_rem, x_lds_stride;
   float* partials;      // [n_chunks][splits][16 * TMX][64]
   unsigned int* counters;
   int64_t partials_per_entry;  // floats; a batch (g.batch > 1, entry = blockIdx.y) keeps one such array and n_chunks counters per entry
 };
 
-// blockIdx.y-th problem of a batch: operands, partial sums and counters of that entry
-__device__ __forceinline__ void select_batch_entry(SmallArgs& a) {
+// z-th problem of a batch: operands, partial sums and counters of that entry
+__device__ __forceinline__ void select_batch_entry(SmallArgs& a, int64_t z) {
   if (a.g.batch > 1) {  // uniform
-    const int64_t z = blockIdx.y;
     a.g.X += z * a.g.x_batch_bytes;
     a.g.W += z * a.g.w_batch_bytes;
     a.g.C = reinterpret_cast<uint8_t*>(a.g.C) + z * a.g.c_batch_bytes;
@@ -106,10 +112,10 @@ __device__ __forceinline__ void compute_unit(const Unit<TMX>& u, v4f (&acc)[kRow
 }
 
 // Adds the wavefronts' accumulators in LDS and writes the chunk (or publishes a split-K partial tile and,
-// in the block that arrives last, adds the partial tiles in split order).  `red` is [WAVES][16*TMX][64].
+// in the block that arrives last, adds the partial tiles in split order).  `red` is [WAVES][16*TMX][16*RG]; the chunk is rows n0 .. n0 + rows - 1.
 template <int TMX, int RG, int WAVES, int MODE>
 __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int* last_flag,
-                                             const v4f (&acc)[RG][TMX], int chunk, int split) {
+                                             const v4f (&acc)[RG][TMX], int chunk, int split, int n0, int rows) {
   constexpr int NT = WAVES * 64;
   constexpr int MROWS = 16 * TMX;
   constexpr int kChunkRows = 16 * RG;
@@ -118,7 +124,6 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
   const GemmArgs& g = a.g;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, lg = lane >> 4;
-  const int n0 = chunk * kChunkRows;
   // lane holds m = t*16 + l16, n = r*16 + 4*lg + [0,4)
 #pragma unroll
   for (int r = 0; r < kRowGroups; ++r)
@@ -133,7 +138,7 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
       float v = 0.f;
 #pragma unroll
       for (int w = 0; w < WAVES; ++w) v += red[w * kOut + i];
-      if (m < g.M && n0 + nn < g.N) store_output<MODE>(g, m, n0 + nn, v);
+      if (m < g.M && nn < rows) store_output<MODE>(g, m, n0 + nn, v);
     }
     return;
   }
@@ -165,7 +170,7 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
     float v = 0.f;
     for (int s = 0; s < a.splits; ++s)
       v += __hip_atomic_load(all + (int64_t)s * kOut + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (m < g.M && n0 + nn < g.N) store_output<MODE>(g, m, n0 + nn, v);
+    if (m < g.M && nn < rows) store_output<MODE>(g, m, n0 + nn, v);
   }
   if (tid == 0) __hip_atomic_store(&a.counters[chunk], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
 }
@@ -178,7 +183,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_smallm_kernel(SmallArgs a
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  select_batch_entry(a);
+  select_batch_entry(a, blockIdx.y);
   const int chunk = blockIdx.x % a.n_chunks;
   const int split = blockIdx.x / a.n_chunks;
   const int n0 = chunk * kChunkRows;
@@ -226,7 +231,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_smallm_kernel(SmallArgs a
     compute_unit<TMX, MODE>(cur, acc);
   }
 
-  finish_chunk<TMX, kRowGroups, WAVES, MODE>(a, &red[0][0][0], &last_flag, acc, chunk, split);
+  finish_chunk<TMX, kRowGroups, WAVES, MODE>(a, &red[0][0][0], &last_flag, acc, chunk, split, n0, min(kChunkRows, g.N - n0));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -241,51 +246,146 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_smallm_kernel(SmallArgs a
 // logical chunk p ^ (row & 15)) so that both the writes (4 rows x 256 B) and the operand reads (16 rows
 // 256 bytes apart) spread over all LDS banks.
 // ---------------------------------------------------------------------------------------------
-template <int TMX, int RG>
+template <int TMX, int Q>
 struct PairRegs {
-  u32x4 w[4 * RG];             // load j: rows 4j..4j+3, lane -> row 4j + (l >> 4), bytes 16*(l & 15) of the pair
-  u32x4 xlo[2][TMX], xhi[2][TMX];
+  u32x4 w[Q];                  // load j: rows 4j..4j+3, lane -> row 4j + (l >> 4), bytes 16*(l & 15) of the pair
+  u32x4 xlo[2][TMX], xhi[2][TMX];  // the last three only when the activations do not come from LDS
   float xs[2][TMX];
-  float ws[2];
+  float wsv;                   // lane & 3 -> weight scale of K-block (lane & 1) of the pair in scale block (lane >> 1) & 1 of the chunk
 };
 
-// RG = 16-row groups per chunk (1, 2 or 4), DEPTH = K-block pairs in flight per wavefront.
-template <int TMX, int RG, int DEPTH, int WAVES, int MODE>
+// Global -> LDS copies the compiler does not see: 16 (4) bytes per lane to lds_addr + 16 (4) * lane.  `base` and
+// `lds_addr` are wave-uniform; the copies count in vmcnt like loads and complete in order with them.
+__device__ __forceinline__ void dma_to_lds_16(uint32_t byte_off, const void* base, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
+}
+__device__ __forceinline__ void dma_to_lds_4(uint32_t byte_off, const void* base, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
+}
+
+// Q = 4-row groups of weights per chunk (a chunk has up to 4Q rows, the block's wavefronts take interleaved pairs
+// of K-blocks), DEPTH = K-block pairs in flight per wavefront.
+//
+// A launch of a few microseconds is bound by the number of vector-memory instructions a compute unit has to push
+// through its address unit (about 14 cycles each, whatever they carry), so nothing but weights is loaded per pair
+// of K-blocks when XLDS is set: at its start the block copies the activations of its K range (M <= 16 rows) and
+// their scales into LDS with a handful of global -> LDS copies, the weight scales come through the scalar cache,
+// and the chunk has no more 4-row groups than its rows need.  Without XLDS (activations too large for LDS) the
+// activation fragments travel in the register ring next to the weights.
+template <int TMX, int Q, int DEPTH, int WAVES, int MODE, bool XLDS>
 __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArgs a) {
+  static_assert(!XLDS || TMX == 1, "activations are kept in LDS for M <= 16 only");
+  constexpr int RG = (Q + 3) / 4;
   constexpr int kRows = 16 * RG;
   constexpr int kSlab = kRows * 256;  // one K-block pair of the chunk
-  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // WAVES slabs; later the reduction buffer
+  constexpr int NT = WAVES * 64;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // WAVES slabs (later the reduction buffer), activations, scales
   __shared__ int last_flag;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  select_batch_entry(a);
-  const int chunk = blockIdx.x % a.n_chunks;
-  const int split = blockIdx.x / a.n_chunks;
-  const int n0 = chunk * kRows;
   const int l16 = lane & 15, lg = lane >> 4;
   const GemmArgs& g = a.g;
+  const int64_t z = blockIdx.z;  // batch entry
+  const int chunk = blockIdx.x, split = blockIdx.y;
+  const int n0 = chunk * a.rows_lo + min(chunk, a.rows_rem);
+  const int rows_valid = a.rows_lo + (chunk < a.rows_rem ? 1 : 0);  // 1 .. 4Q
   uint8_t* const slab = lds + wave * kSlab;
 
-  const uint8_t* const w_base = g.W + (int64_t)n0 * g.ldw + l16 * 16;
-  const int rows_valid = g.N - n0;
-  uint32_t w_off[4 * RG];
+  const int pairs_total = (g.KB + 1) >> 1;
+  const int pair_lo = split * a.kpw * WAVES;
+  const int pair_end = min(pairs_total, pair_lo + a.kpw * WAVES);
+  const int kb_lo = pair_lo * 2;
+  const int kbc = min(g.KB, pair_end * 2) - kb_lo;  // K-blocks of this block
+
+  const uint8_t* const x_base = g.X + z * g.x_batch_bytes;
+  const float* const xs_base = (MODE == kModeBlock) ? g.xs + z * g.xs_batch_stride : nullptr;
+  const uint32_t xs_cs = (uint32_t)g.xs_cs;
+
+  // weight scales: a chunk may begin anywhere, so its rows can lie in two 128-row scale blocks; second[r][i] says
+  // that this lane's column r*16 + 4*lg + i belongs to the second (lane masks, set up once).
+  const float* const ws_base =
+      (MODE == kModeBlock) ? g.ws + z * g.ws_batch_stride + (int64_t)(n0 >> 7) * g.ws_rs : nullptr;
+  const int64_t ws_second = (((n0 + rows_valid - 1) >> 7) != (n0 >> 7)) ? g.ws_rs : 0;
+  bool second[RG][4];
 #pragma unroll
-  for (int j = 0; j < 4 * RG; ++j) {
-    int r = 4 * j + lg;
-    r = r < rows_valid ? r : rows_valid - 1;  // rows past the edge alias the last valid row; never stored
-    w_off[j] = (uint32_t)r * (uint32_t)g.ldw;
+  for (int r = 0; r < RG; ++r)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) second[r][i] = ((n0 + r * 16 + lg * 4 + i) >> 7) != (n0 >> 7);
+
+
+  // ---- activations and their scales -> LDS (issued before the first weight load: they arrive first)
+  const uint32_t lds_x = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + WAVES * kSlab;  // rows x_lds_stride apart, 16-byte pieces permuted
+  const uint32_t x_stride = (uint32_t)a.x_lds_stride;
+  const uint32_t lds_xs = lds_x + (uint32_t)g.M * x_stride;         // [M][kbc] floats
+  const uint32_t lds_ws = lds_xs + (uint32_t)(g.M * kbc) * 4u;      // [2][kbc] floats: the chunk's two weight-scale blocks
+  if (XLDS) {
+    // one copy = 64 pieces of 16 bytes of one row; piece p of a row lies at position p ^ perm(row) within its
+    // K-block (8 pieces), perm(row) = (row >> 1) & 7, and the row stride is an odd multiple of 128 bytes: the 16
+    // rows a wavefront reads together then fall into 16 different 16-byte bank groups
+    const int row_pieces = kbc * 8;
+    const int row_units = (row_pieces + 63) >> 6;
+    const int units = g.M * row_units;
+    int m = 0, ru = wave;
+    while (ru >= row_units) { ru -= row_units; ++m; }
+    for (int u = wave; u < units; u += WAVES) {
+      const int p = ru * 64 + lane;
+      if (p < row_pieces) {
+        const uint32_t src = (uint32_t)m * (uint32_t)g.ldx + (uint32_t)kb_lo * 128u +
+                             (uint32_t)(((p & ~7) | ((p & 7) ^ ((m >> 1) & 7))) << 4);
+        dma_to_lds_16(src, x_base, lds_x + (uint32_t)m * x_stride + (uint32_t)ru * 1024u);
+      }
+      ru += WAVES;
+      while (ru >= row_units) { ru -= row_units; ++m; }
+    }
+    if (MODE == kModeBlock) {
+      const int count = g.M * kbc;
+      for (int e0 = wave * 64; e0 < count; e0 += NT) {
+        const int e = e0 + lane;
+        if (e < count) {
+          const int mm = e / kbc, kk = e - mm * kbc;
+          dma_to_lds_4(((uint32_t)mm * (uint32_t)g.xs_rs + (uint32_t)(kb_lo + kk) * xs_cs) * 4u, xs_base, lds_xs + (uint32_t)e0 * 4u);
+        }
+      }
+    }
+    if (MODE == kModeBlock) {
+      const int row_units = (kbc + 63) >> 6;
+      for (int c = wave; c < 2 * row_units; c += WAVES) {
+        const int row = c & 1, k0 = (c >> 1) * 64;
+        if (k0 + lane < kbc)
+          dma_to_lds_4((uint32_t)((int64_t)(kb_lo + k0 + lane) * g.ws_cs + (row ? ws_second : 0)) * 4u, ws_base,
+                       lds_ws + (uint32_t)(row * kbc + k0) * 4u);
+      }
+    }
   }
-  const uint8_t* xrow[TMX];
-  const float* xsrow[TMX];
+
+  // ---- weights: rows 4j + lg of the chunk, 16 bytes at l16 * 16 of the pair (rows past the chunk's last alias it;
+  // never stored); a uniform 64-bit base plus 32-bit lane offsets
+  const uint8_t* const w_base = g.W + z * g.w_batch_bytes + (int64_t)n0 * g.ldw;
+  uint32_t w_off[Q];
+#pragma unroll
+  for (int j = 0; j < Q; ++j) {
+    int r = 4 * j + lg;
+    r = r < rows_valid ? r : rows_valid - 1;
+    w_off[j] = (uint32_t)r * (uint32_t)g.ldw + (uint32_t)l16 * 16u;
+  }
+  // an odd K-block count leaves a single block at the end: lanes 8..15 of a row, which own the second K-block of
+  // a pair, re-read the first
+  const uint32_t tail_adj = l16 >= 8 ? 0xFFFFFF80u : 0u;
+
+  // activation fragments of this lane: row t*16 + l16 (rows past M alias the last; never stored)
+  uint32_t x_off[TMX], xs_off[TMX], lds_xrow[TMX], lds_xsrow[TMX];
 #pragma unroll
   for (int t = 0; t < TMX; ++t) {
     int m = t * 16 + l16;
     m = m < g.M ? m : g.M - 1;
-    xrow[t] = g.X + (int64_t)m * g.ldx + lg * 16;
-    xsrow[t] = (MODE == kModeBlock) ? g.xs + (int64_t)m * g.xs_rs : nullptr;
+    x_off[t] = (uint32_t)m * (uint32_t)g.ldx + (uint32_t)lg * 16u;
+    xs_off[t] = (uint32_t)m * (uint32_t)g.xs_rs;
+    lds_xrow[t] = lds_x + (uint32_t)m * x_stride;
+    lds_xsrow[t] = lds_xs + (uint32_t)(m * kbc) * 4u;
   }
-  const float* wsrow = (MODE == kModeBlock) ? g.ws + (int64_t)(n0 >> 7) * g.ws_rs : nullptr;
+  const uint32_t perm = (uint32_t)(((l16 < g.M ? l16 : g.M - 1) >> 1) & 7);  // TMX == 1 when used
+  const uint32_t x_lo_piece = ((uint32_t)lg ^ perm) << 4, x_hi_piece = ((uint32_t)(lg + 4) ^ perm) << 4;
 
   v4f acc[RG][TMX];
 #pragma unroll
@@ -293,44 +393,74 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
 #pragma unroll
     for (int t = 0; t < TMX; ++t) acc[r][t] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  const int pairs_total = (g.KB + 1) >> 1;
-  const int per_split = a.kpw * WAVES;
-  const int pair_end = min(pairs_total, (split + 1) * per_split);
-
-  auto load_pair = [&](PairRegs<TMX, RG>& u, int pair) __attribute__((always_inline)) {
-    const int kb = pair * 2;
-    const bool two = kb + 1 < g.KB;  // an odd K-block count leaves a single block at the end
-    const int64_t k = (int64_t)kb * 128;
-    // lanes 8..15 of a row own the second K-block; when it does not exist they re-read the first
-    const int64_t kw = k - ((!two && l16 >= 8) ? 128 : 0);
+  auto load_w = [&](PairRegs<TMX, Q>& u, int pair) __attribute__((always_inline)) {
+    const bool two = pair * 2 + 1 < g.KB;
+    const uint8_t* const base = w_base + (uint32_t)pair * 256u;
+    const uint32_t adj = two ? 0u : tail_adj;
 #pragma unroll
-    for (int j = 0; j < 4 * RG; ++j)
-      u.w[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w_base + kw + w_off[j]));
+    for (int j = 0; j < Q; ++j)
+      u.w[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + (size_t)(w_off[j] + adj)));
+  };
+  auto load_x = [&](PairRegs<TMX, Q>& u, int pair) __attribute__((always_inline)) {
+    if (XLDS) return;
+    const int kb = pair * 2;
+    const bool two = kb + 1 < g.KB;
+    if (MODE == kModeBlock) u.wsv = ws_base[(int64_t)(kb + ((two && (lane & 1)) ? 1 : 0)) * g.ws_cs + ((lane & 2) ? ws_second : 0)];
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-      const int kbb = kb + ((b == 1 && two) ? 1 : 0);
+      const uint32_t kbb = (uint32_t)(kb + ((b == 1 && two) ? 1 : 0));
+      const uint8_t* const base = x_base + kbb * 128u;
 #pragma unroll
       for (int t = 0; t < TMX; ++t) {
-        u.xlo[b][t] = *reinterpret_cast<const u32x4*>(xrow[t] + (int64_t)kbb * 128);
-        u.xhi[b][t] = *reinterpret_cast<const u32x4*>(xrow[t] + (int64_t)kbb * 128 + 64);
-        if (MODE == kModeBlock) u.xs[b][t] = xsrow[t][(int64_t)kbb * g.xs_cs];
+        u.xlo[b][t] = *reinterpret_cast<const u32x4*>(base + (size_t)x_off[t]);
+        u.xhi[b][t] = *reinterpret_cast<const u32x4*>(base + (size_t)(x_off[t] + 64u));
+        if (MODE == kModeBlock) u.xs[b][t] = xs_base[(size_t)(xs_off[t] + kbb * xs_cs)];
       }
-      if (MODE == kModeBlock) u.ws[b] = wsrow[(int64_t)kbb * g.ws_cs];
     }
   };
 
-  auto multiply = [&](const PairRegs<TMX, RG>& u, int pair) __attribute__((always_inline)) {
-    const bool two = pair * 2 + 1 < g.KB;
-    // registers -> slab: row R = 4j + lg, logical chunk l16 goes to physical chunk l16 ^ (R & 15)
+  // registers -> slab: row R = 4j + lg, logical chunk l16 goes to physical chunk l16 ^ (R & 15)
+  auto stage = [&](const PairRegs<TMX, Q>& u) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 4 * RG; ++j) {
+    for (int j = 0; j < Q; ++j) {
       const int R = 4 * j + lg;
       *reinterpret_cast<u32x4*>(slab + R * 256 + ((l16 ^ (R & 15)) << 4)) = u.w[j];
     }
-    // slab -> operand fragments: lane owns row rg*16 + l16 and logical chunks b*8 + lg, b*8 + lg + 4
+  };
+  // slab -> operand fragments: lane owns row rg*16 + l16 and logical chunks b*8 + lg, b*8 + lg + 4
+  auto multiply = [&](const PairRegs<TMX, Q>& u, int pair) __attribute__((always_inline)) {
+    const int kb = pair * 2;
+    const bool two = kb + 1 < g.KB;
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       if (b == 1 && !two) break;
+      float ws1 = 1.f, ws2 = 1.f;
+      if (MODE == kModeBlock) {
+        if (XLDS) {
+          ws1 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(lds_ws + (uint32_t)(kb + b - kb_lo) * 4u);
+          ws2 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(lds_ws + (uint32_t)(kbc + kb + b - kb_lo) * 4u);
+        } else {
+          ws1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, u.wsv), b));
+          ws2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, u.wsv), 2 + b));
+        }
+      }
+      v8i xf[TMX];
+      float xsc[TMX];
+#pragma unroll
+      for (int t = 0; t < TMX; ++t) {
+        if (XLDS) {
+          const uint32_t at = lds_xrow[t] + (uint32_t)(kb + b - kb_lo) * 128u;
+          const u32x4 lo = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + x_lo_piece);
+          const u32x4 hi = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + x_hi_piece);
+          xf[t] = join(lo, hi);
+          xsc[t] = (MODE == kModeBlock)
+                       ? *reinterpret_cast<const __attribute__((address_space(3))) float*>(lds_xsrow[t] + (uint32_t)(kb + b - kb_lo) * 4u)
+                       : 1.f;
+        } else {
+          xf[t] = join(u.xlo[b][t], u.xhi[b][t]);
+          xsc[t] = (MODE == kModeBlock) ? u.xs[b][t] : 1.f;
+        }
+      }
 #pragma unroll
       for (int r = 0; r < RG; ++r) {
         const uint8_t* row = slab + (r * 16 + l16) * 256;
@@ -339,44 +469,63 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
         const v8i wf = join(lo, hi);
 #pragma unroll
         for (int t = 0; t < TMX; ++t) {
-          const v8i xf = join(u.xlo[b][t], u.xhi[b][t]);
           if (MODE == kModeBlock) {
-            const float sc = u.xs[b][t] * u.ws[b];
-            const v4f p = mfma_fp8_16x16x128(wf, xf, v4f{0.f, 0.f, 0.f, 0.f});
-            acc[r][t][0] = __builtin_fmaf(p[0], sc, acc[r][t][0]);
-            acc[r][t][1] = __builtin_fmaf(p[1], sc, acc[r][t][1]);
-            acc[r][t][2] = __builtin_fmaf(p[2], sc, acc[r][t][2]);
-            acc[r][t][3] = __builtin_fmaf(p[3], sc, acc[r][t][3]);
+            const float sc1 = xsc[t] * ws1, sc2 = xsc[t] * ws2;
+            const v4f p = mfma_fp8_16x16x128(wf, xf[t], v4f{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[r][t][i] = __builtin_fmaf(p[i], second[r][i] ? sc2 : sc1, acc[r][t][i]);
           } else {
-            acc[r][t] = mfma_fp8_16x16x128(wf, xf, acc[r][t]);
+            acc[r][t] = mfma_fp8_16x16x128(wf, xf[t], acc[r][t]);
           }
         }
       }
     }
   };
 
-  // DEPTH register sets form a ring; the loop body is written out once per set so that the ring index
-  // is static and nothing is copied between sets
-  int pair = split * per_split + wave;
-  PairRegs<TMX, RG> ring[DEPTH];
+  // DEPTH register sets form a ring; the loop body is written out once per set so that the ring index is static
+  // and nothing is copied between sets.
+  int pair = pair_lo + wave;
+  PairRegs<TMX, Q> ring[DEPTH];
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d)
-    if (pair + d * WAVES < pair_end) load_pair(ring[d], pair + d * WAVES);
+    if (pair + d * WAVES < pair_end) {
+      load_w(ring[d], pair + d * WAVES);
+      load_x(ring[d], pair + d * WAVES);
+    }
   bool done = pair >= pair_end;
+  bool staged_ahead = false;
+  if (XLDS) {
+    // The wait for the first pair of weights is also the wait for this wavefront's copies, which were issued
+    // earlier and complete in order; a wavefront without work waits for its copies alone.
+    if (!done) { stage(ring[0]); staged_ahead = true; }
+    else wait_vmem_all();
+    __syncthreads();
+  }
   while (!done) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       if (!done) {
-        multiply(ring[d], pair);
         const int refill = pair + DEPTH * WAVES;
-        if (refill < pair_end) load_pair(ring[d], refill);
+        if (d == 0 && staged_ahead) staged_ahead = false;
+        else stage(ring[d]);
+        // With the activations in LDS the ring holds weights only and its registers are free once they are in
+        // the slab: the refill goes out before the multiplication, so the slab double-buffers the ring.  With
+        // activation fragments in the ring the refill has to follow the multiplication.
+        if (XLDS && refill < pair_end) load_w(ring[d], refill);
+        multiply(ring[d], pair);
+        if (!XLDS && refill < pair_end) {
+          load_w(ring[d], refill);
+          load_x(ring[d], refill);
+        }
         pair += WAVES;
         done = pair >= pair_end;
       }
     }
   }
-  __syncthreads();  // the slabs are dead; their memory now holds the reduction buffer
-  finish_chunk<TMX, RG, WAVES, MODE>(a, reinterpret_cast<float*>(lds), &last_flag, acc, chunk, split);
+
+  select_batch_entry(a, z);  // the epilogue's view of the operands
+  __syncthreads();           // the slabs are dead; their memory now holds the reduction buffer
+  finish_chunk<TMX, RG, WAVES, MODE>(a, reinterpret_cast<float*>(lds), &last_flag, acc, chunk, split, n0, rows_valid);
 }
 
 template <int TMX, int WAVES>
@@ -388,22 +537,33 @@ int launch_t(const SmallArgs& sa, int mode, hipStream_t stream) {
   return FG_OK;
 }
 
-template <int TMX, int RG, int DEPTH, int WAVES>
+constexpr int kDecodeLdsLimit = 160 * 1024 - 1024;  // dynamic LDS a block may ask for (a little is static)
+
+// bytes between activation rows in LDS: the K-blocks of the block's range, an odd number of 128-byte units
+inline int x_lds_stride_for(int64_t kbc) { return (int)((kbc | 1) * 128); }
+// dynamic LDS of the staged kernel with the activations kept in LDS
+inline int64_t decode_lds_bytes(int q, int waves, int64_t M, int64_t kbc) {
+  return (int64_t)waves * 16 * ((q + 3) / 4) * 256 + M * x_lds_stride_for(kbc) + (M + 2) * kbc * 4;
+}
+
+template <int TMX, int Q, int DEPTH, int WAVES, bool XLDS>
 int launch_transpose(const SmallArgs& sa, int mode, hipStream_t stream) {
-  // WAVES slabs of RG * 4 KB; the reduction buffer (WAVES * 16*TMX * 16*RG floats) reuses the same memory
-  constexpr int kSlabs = WAVES * 16 * RG * 256;
-  constexpr int kRed = WAVES * 16 * TMX * 16 * RG * 4;
-  constexpr int kLds = kSlabs > kRed ? kSlabs : kRed;
-  const dim3 grid((uint32_t)(sa.n_chunks * sa.splits), (uint32_t)(sa.g.batch > 1 ? sa.g.batch : 1)), block(WAVES * 64);
-  auto kb = fp8_gemm_transpose_kernel<TMX, RG, DEPTH, WAVES, kModeBlock>;
-  auto kr = fp8_gemm_transpose_kernel<TMX, RG, DEPTH, WAVES, kModeRowCol>;
+  // WAVES slabs of 4 KB per 16 rows; the reduction buffer (WAVES * 16*TMX * rows floats) reuses the same memory
+  constexpr int kSlabs = WAVES * 16 * ((Q + 3) / 4) * 256;
+  const int64_t kbc = std::min<int64_t>(sa.g.KB, (int64_t)sa.kpw * WAVES * 2);
+  const int lds_bytes = XLDS ? (int)decode_lds_bytes(Q, WAVES, sa.g.M, kbc) : kSlabs;
+  if (lds_bytes > kDecodeLdsLimit) FG_FAIL(FG_ERR_LAUNCH, "fp8 gemm (small M): %d bytes of LDS planned", lds_bytes);
+  const dim3 grid((uint32_t)sa.n_chunks, (uint32_t)sa.splits, (uint32_t)(sa.g.batch > 1 ? sa.g.batch : 1));
+  const dim3 block(WAVES * 64);
+  auto kb = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeBlock, XLDS>;
+  auto kr = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeRowCol, XLDS>;
   static PerDeviceFlags lds_limit_raised = {};  // per instantiation
   {
-    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, kLds, reinterpret_cast<const void*>(kb), reinterpret_cast<const void*>(kr));
-    if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLds, hipGetErrorString(e));
+    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, XLDS ? kDecodeLdsLimit : kSlabs, reinterpret_cast<const void*>(kb), reinterpret_cast<const void*>(kr));
+    if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(LDS limit): %s", hipGetErrorString(e));
   }
-  if (mode == kModeBlock) FG_LAUNCH(kb, grid, block, kLds, stream, sa);
-  else FG_LAUNCH(kr, grid, block, kLds, stream, sa);
+  if (mode == kModeBlock) FG_LAUNCH(kb, grid, block, lds_bytes, stream, sa);
+  else FG_LAUNCH(kr, grid, block, lds_bytes, stream, sa);
   FG_CHECK_LAUNCH("fp8_gemm_transpose_kernel");
   return FG_OK;
 }
@@ -419,18 +579,24 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   const int64_t KB = K / 128;
   int64_t kpw, splits;
   p.rg = kRowGroups;
+  p.q = 4 * kRowGroups;
+  p.xlds = false;
   p.staged = p.tmx <= 2 && KB >= 8;
+  int64_t chunks = 0;
   if (p.staged) {
-    // Rows per chunk: the largest of 64 / 32 / 16 that still yields at least ~140 blocks, so that K is
-    // split across blocks only for very narrow weights (a split costs a round trip of partial tiles
-    // through memory: measured 6.1 us unsplit against 8.6 us split in two for N = 2112, K = 7168).
-    p.rg = 4;
-    while (p.rg > 1 && ceil_div(N, 16 * p.rg) * entries < 140) p.rg >>= 1;
+    // One block per compute unit with the rows dealt out evenly (chunks differ by at most one row): a launch
+    // takes as long as the compute unit with most bytes to fetch.  Narrow weights get chunks of at least 4 rows
+    // and K split over blocks below; weights with more than 64 rows per compute unit get whole rounds of blocks.
+    const int64_t B = std::max<int64_t>(1, cu_count() / entries);
+    chunks = N <= 64 * B ? std::min<int64_t>(B, ceil_div(N, 4)) : ceil_div(N, 64 * B) * B;
+    const int64_t rows_max = ceil_div(N, chunks);
+    p.q = (int)ceil_div(rows_max, 4);
+    p.rg = p.q <= 4 ? 1 : (p.q <= 8 ? 2 : 4);
     p.waves = (p.tmx == 2 && p.rg == 4) ? 4 : 8;
   } else {
     p.waves = p.tmx == 4 ? 4 : 8;  // LDS reduction buffer is 4 KB * tmx per wavefront
   }
-  p.n_chunks = (int)ceil_div(N, 16 * p.rg);
+  p.n_chunks = p.staged ? (int)chunks : (int)ceil_div(N, 16 * p.rg);
   if (p.n_chunks > FG_WORKSPACE_COUNTER_BYTES / 4) return p;
   // partial tiles cost 2 * splits * 16*tmx * rows * 4 bytes per chunk against rows * K weight bytes: keep
   // them under a quarter of the weight traffic
@@ -440,6 +606,14 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
     splits = 1;
     while (p.n_chunks * entries * splits < 100 && splits * 2 <= max_splits && splits * 2 * p.waves <= pairs) splits *= 2;
     kpw = ceil_div(pairs, splits * p.waves);
+    // activations in LDS when M <= 16 and they fit beside the slabs; the chunk then has exactly the 4-row groups
+    // it needs (instantiated: 1, 2, 3, 4, 6, 8, 12, 16), otherwise whole 16-row groups
+    static const int kQ[] = {1, 2, 3, 4, 6, 8, 12, 16};
+    int q = 16;
+    for (int i = 7; i >= 0; --i) if (kQ[i] >= p.q) q = kQ[i];
+    const int64_t kbc = std::min<int64_t>(KB, kpw * p.waves * 2);
+    p.xlds = p.tmx == 1 && kpw >= 3 && decode_lds_bytes(q, p.waves, M, kbc) <= kDecodeLdsLimit;
+    p.q = p.xlds ? q : 4 * p.rg;
   } else {
     // aim for ~8 wavefronts per CU on 256 CUs, each with at least one K-block
     const int64_t units = (int64_t)p.n_chunks * entries * KB;
@@ -468,6 +642,9 @@ int launch_small_m(const GemmArgs& g, int mode, const SmallMPlan& plan, void* wo
   sa.kpw = plan.kpw;
   sa.splits = plan.splits;
   sa.n_chunks = plan.n_chunks;
+  sa.rows_lo = (int)(g.N / plan.n_chunks);
+  sa.rows_rem = (int)(g.N % plan.n_chunks);
+  sa.x_lds_stride = plan.xlds ? x_lds_stride_for(std::min<int64_t>(g.KB, (int64_t)plan.kpw * plan.waves * 2)) : 0;
   sa.partials = nullptr;
   sa.counters = nullptr;
   sa.partials_per_entry = 0;
@@ -486,14 +663,34 @@ int launch_small_m(const GemmArgs& g, int mode, const SmallMPlan& plan, void* wo
     sa.partials = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
   }
   if (plan.staged) {
-    if (plan.tmx == 1) {
-      if (plan.rg == 1) return launch_transpose<1, 1, 4, 8>(sa, mode, stream);
-      if (plan.rg == 2) return launch_transpose<1, 2, 3, 8>(sa, mode, stream);
-      return launch_transpose<1, 4, 2, 8>(sa, mode, stream);
+    // the staged kernels address with 32-bit lane offsets from uniform bases
+    const uint64_t lim = 1ull << 32;
+    if (g.ldw <= 0 || g.ldx <= 0 || g.xs_rs < 0 || g.xs_cs < 0 || (uint64_t)g.ldw * 64 + (uint64_t)g.K >= lim ||
+        (uint64_t)g.ldx * 64 + (uint64_t)g.K >= lim || ((uint64_t)g.xs_rs * 64 + (uint64_t)g.xs_cs * g.KB) * 4 >= lim ||
+        g.ws_rs < 0 || g.ws_cs < 0 || ((uint64_t)g.ws_rs + (uint64_t)g.ws_cs * g.KB) * 4 >= lim)
+      FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm (small M): row strides of %lld / %lld bytes are beyond the kernel's 32-bit offsets",
+              (long long)g.ldx, (long long)g.ldw);
+    if (g.batch > 65535) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm (small M): at most 65535 batch entries per launch, got %d", g.batch);
+    if (plan.xlds) {
+      switch (plan.q) {
+        case 1: return launch_transpose<1, 1, 1, 8, true>(sa, mode, stream);
+        case 2: return launch_transpose<1, 2, 1, 8, true>(sa, mode, stream);
+        case 3: return launch_transpose<1, 3, 1, 8, true>(sa, mode, stream);
+        case 4: return launch_transpose<1, 4, 1, 8, true>(sa, mode, stream);
+        case 6: return launch_transpose<1, 6, 1, 8, true>(sa, mode, stream);
+        case 8: return launch_transpose<1, 8, 1, 8, true>(sa, mode, stream);
+        case 12: return launch_transpose<1, 12, 1, 8, true>(sa, mode, stream);
+        default: return launch_transpose<1, 16, 1, 8, true>(sa, mode, stream);
+      }
     }
-    if (plan.rg == 1) return launch_transpose<2, 1, 3, 8>(sa, mode, stream);
-    if (plan.rg == 2) return launch_transpose<2, 2, 2, 8>(sa, mode, stream);
-    return launch_transpose<2, 4, 2, 4>(sa, mode, stream);
+    if (plan.tmx == 1) {
+      if (plan.rg == 1) return launch_transpose<1, 4, 4, 8, false>(sa, mode, stream);
+      if (plan.rg == 2) return launch_transpose<1, 8, 3, 8, false>(sa, mode, stream);
+      return launch_transpose<1, 16, 2, 8, false>(sa, mode, stream);
+    }
+    if (plan.rg == 1) return launch_transpose<2, 4, 3, 8, false>(sa, mode, stream);
+    if (plan.rg == 2) return launch_transpose<2, 8, 2, 8, false>(sa, mode, stream);
+    return launch_transpose<2, 16, 2, 4, false>(sa, mode, stream);
   }
   if (plan.tmx == 1) return plan.waves == 8 ? launch_t<1, 8>(sa, mode, stream) : launch_t<1, 4>(sa, mode, stream);
   if (plan.tmx == 2) return plan.waves == 8 ? launch_t<2, 8>(sa, mode, stream) : launch_t<2, 4>(sa, mode, stream);

@@ -161,6 +161,42 @@ def test_33_to_128_rows(M, N, K, dtype):
     assert torch.equal(cm.view(torch.int8), got.view(torch.int8))
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 2112, 7168), (16, 2112, 7168), (5, 1000, 7168), (3, 200, 8192), (7, 300, 16512),
+                                   (16, 4608, 7168), (12, 7168, 16384), (2, 7168, 16384), (1, 24576, 1536),
+                                   (32, 2112, 7168), (20, 4608, 4096), (1, 9, 1024), (4, 130, 2048), (9, 4099, 7296)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_up_to_32_rows_uneven_chunks(M, N, K, dtype):
+    """M <= 32 takes the kernel that deals the weight rows out evenly over the compute units: chunks that differ by a
+    row and begin anywhere (so that a chunk's rows lie in two 128-row scale blocks), chunks of fewer than 16 rows, N
+    that is no multiple of 4, K split over blocks, an odd number of K-blocks, activations kept in LDS (long K, M <=
+    16) or fetched per K-block (short K, M = 12 with K = 16384, M > 16), column-major activation scales; against the
+    oracle and bit-identical on reruns."""
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=17)
+    want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
+    args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    got = flag_gems.w8a8_block_fp8_matmul(*args, output_dtype=dtype)
+    assert got.dtype == dtype and got.shape == (M, N)
+    tol = dict(rtol=1e-4, atol=2e-4) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(got.cpu().float(), want, **tol)
+    for _ in range(2):
+        assert torch.equal(flag_gems.w8a8_block_fp8_matmul(*args, output_dtype=dtype).view(torch.int8), got.view(torch.int8))
+    xs_cm = xs.to(DEV).t().contiguous().t()
+    cm = flag_gems.w8a8_block_fp8_matmul(args[0], args[1], xs_cm, args[3], [128, 128], output_dtype=dtype)
+    assert torch.equal(cm.view(torch.int8), got.view(torch.int8))
+
+
+def test_rows_of_a_small_batch_do_not_depend_on_its_size():
+    """Row m of the product is the same bits whether the call has 1, 8 or 16 activation rows: the kernels for M <= 16
+    differ only in where the activations are kept."""
+    N, K = 2112, 7168
+    xq, wq, xs, ws = _quantized_inputs(16, N, K, seed=23)
+    xq, wq, xs, ws = xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV)
+    full = flag_gems.w8a8_block_fp8_matmul(xq, wq, xs, ws, [128, 128], output_dtype=torch.float32)
+    for rows in (1, 8):
+        part = flag_gems.w8a8_block_fp8_matmul(xq[:rows].contiguous(), wq, xs[:rows].contiguous(), ws, [128, 128], output_dtype=torch.float32)
+        assert torch.equal(part.view(torch.int32), full[:rows].view(torch.int32))
+
+
 @pytest.mark.parametrize("M,N,K", [(1024, 7168, 8192), (300, 7000, 16384)])
 def test_tiles_cut_into_equal_ranges_along_k(M, N, K):
     """112 tiles x 64 K-blocks and 56 tiles x 128 K-blocks (ragged in M and N): the persistent kernel cuts every
