@@ -131,6 +131,7 @@ struct SmallMPlan {
   int rg;         // 16-row weight groups per output chunk: 1, 2 or 4
   int q;          // staged: 4-row weight groups the kernel loads per chunk (<= 4 * rg)
   bool xlds;      // staged: the block keeps the activations of its K range in LDS
+  bool own;       // staged: every wavefront has a chunk of its own and walks all of K
   int waves;      // wavefronts per block: 4 or 8
   int kpw;        // K-blocks (K-block pairs when staged) per wavefront
   int splits;     // blocks along K that share one 64-row output chunk

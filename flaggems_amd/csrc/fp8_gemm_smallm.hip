@@ -272,9 +272,10 @@ __device__ __forceinline__ void dma_to_lds_4(uint32_t byte_off, const void* base
 // their scales into LDS with a handful of global -> LDS copies, the weight scales come through the scalar cache,
 // and the chunk has no more 4-row groups than its rows need.  Without XLDS (activations too large for LDS) the
 // activation fragments travel in the register ring next to the weights.
-template <int TMX, int Q, int DEPTH, int WAVES, int MODE, bool XLDS>
+template <int TMX, int Q, int DEPTH, int WAVES, int MODE, bool XLDS, bool OWN = false>
 __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArgs a) {
   static_assert(!XLDS || TMX == 1, "activations are kept in LDS for M <= 16 only");
+  static_assert(!OWN || XLDS, "wavefronts with chunks of their own share the activations through LDS");
   constexpr int RG = (Q + 3) / 4;
   constexpr int kRows = 16 * RG;
   constexpr int kSlab = kRows * 256;  // one K-block pair of the chunk
@@ -287,14 +288,18 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
   const int l16 = lane & 15, lg = lane >> 4;
   const GemmArgs& g = a.g;
   const int64_t z = blockIdx.z;  // batch entry
-  const int chunk = blockIdx.x, split = blockIdx.y;
+  const int split = blockIdx.y;
+  // OWN: every wavefront has a chunk of its own and walks all of K (nothing is added across wavefronts); the last
+  // block may have wavefronts without a chunk, which still help to copy the activations
+  const int chunk = OWN ? min((int)blockIdx.x * WAVES + wave, a.n_chunks - 1) : (int)blockIdx.x;
+  const bool idle = OWN && (int)blockIdx.x * WAVES + wave >= a.n_chunks;
   const int n0 = chunk * a.rows_lo + min(chunk, a.rows_rem);
   const int rows_valid = a.rows_lo + (chunk < a.rows_rem ? 1 : 0);  // 1 .. 4Q
   uint8_t* const slab = lds + wave * kSlab;
 
   const int pairs_total = (g.KB + 1) >> 1;
-  const int pair_lo = split * a.kpw * WAVES;
-  const int pair_end = min(pairs_total, pair_lo + a.kpw * WAVES);
+  const int pair_lo = OWN ? 0 : split * a.kpw * WAVES;
+  const int pair_end = OWN ? pairs_total : min(pairs_total, pair_lo + a.kpw * WAVES);
   const int kb_lo = pair_lo * 2;
   const int kbc = min(g.KB, pair_end * 2) - kb_lo;  // K-blocks of this block
 
@@ -318,7 +323,8 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
   const uint32_t lds_x = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + WAVES * kSlab;  // rows x_lds_stride apart, 16-byte pieces permuted
   const uint32_t x_stride = (uint32_t)a.x_lds_stride;
   const uint32_t lds_xs = lds_x + (uint32_t)g.M * x_stride;         // [M][kbc] floats
-  const uint32_t lds_ws = lds_xs + (uint32_t)(g.M * kbc) * 4u;      // [2][kbc] floats: the chunk's two weight-scale blocks
+  // [2][kbc] floats: the chunk's two weight-scale blocks (per wavefront when every wavefront has its own chunk)
+  const uint32_t lds_ws = lds_xs + (uint32_t)(g.M * kbc) * 4u + (OWN ? (uint32_t)(wave * 2 * kbc) * 4u : 0u);
   if (XLDS) {
     // one copy = 64 pieces of 16 bytes of one row; piece p of a row lies at position p ^ perm(row) within its
     // K-block (8 pieces), perm(row) = (row >> 1) & 7, and the row stride is an odd multiple of 128 bytes: the 16
@@ -350,7 +356,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
     }
     if (MODE == kModeBlock) {
       const int row_units = (kbc + 63) >> 6;
-      for (int c = wave; c < 2 * row_units; c += WAVES) {
+      for (int c = OWN ? 0 : wave; c < 2 * row_units; c += OWN ? 1 : WAVES) {
         const int row = c & 1, k0 = (c >> 1) * 64;
         if (k0 + lane < kbc)
           dma_to_lds_4((uint32_t)((int64_t)(kb_lo + k0 + lane) * g.ws_cs + (row ? ws_second : 0)) * 4u, ws_base,
@@ -484,13 +490,14 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
 
   // DEPTH register sets form a ring; the loop body is written out once per set so that the ring index is static
   // and nothing is copied between sets.
-  int pair = pair_lo + wave;
+  constexpr int STEP = OWN ? 1 : WAVES;
+  int pair = OWN ? (idle ? pair_end : pair_lo) : pair_lo + wave;
   PairRegs<TMX, Q> ring[DEPTH];
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d)
-    if (pair + d * WAVES < pair_end) {
-      load_w(ring[d], pair + d * WAVES);
-      load_x(ring[d], pair + d * WAVES);
+    if (pair + d * STEP < pair_end) {
+      load_w(ring[d], pair + d * STEP);
+      load_x(ring[d], pair + d * STEP);
     }
   bool done = pair >= pair_end;
   bool staged_ahead = false;
@@ -505,7 +512,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       if (!done) {
-        const int refill = pair + DEPTH * WAVES;
+        const int refill = pair + DEPTH * STEP;
         if (d == 0 && staged_ahead) staged_ahead = false;
         else stage(ring[d]);
         // With the activations in LDS the ring holds weights only and its registers are free once they are in
@@ -517,13 +524,25 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
           load_w(ring[d], refill);
           load_x(ring[d], refill);
         }
-        pair += WAVES;
+        pair += STEP;
         done = pair >= pair_end;
       }
     }
   }
 
   select_batch_entry(a, z);  // the epilogue's view of the operands
+  if (OWN) {
+    if (idle) return;
+    // lane holds m = l16, n = n0 + r*16 + 4*lg + [0,4)
+#pragma unroll
+    for (int r = 0; r < RG; ++r)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int nn = r * 16 + lg * 4 + i;
+        if (l16 < g.M && nn < rows_valid) store_output<MODE>(g, l16, n0 + nn, acc[r][0][i]);
+      }
+    return;
+  }
   __syncthreads();           // the slabs are dead; their memory now holds the reduction buffer
   finish_chunk<TMX, RG, WAVES, MODE>(a, reinterpret_cast<float*>(lds), &last_flag, acc, chunk, split, n0, rows_valid);
 }
@@ -541,22 +560,23 @@ constexpr int kDecodeLdsLimit = 160 * 1024 - 1024;  // dynamic LDS a block may a
 
 // bytes between activation rows in LDS: the K-blocks of the block's range, an odd number of 128-byte units
 inline int x_lds_stride_for(int64_t kbc) { return (int)((kbc | 1) * 128); }
-// dynamic LDS of the staged kernel with the activations kept in LDS
+// dynamic LDS of the staged kernel with the activations kept in LDS (weight scales counted once per wavefront,
+// which only the kernel with a chunk per wavefront needs)
 inline int64_t decode_lds_bytes(int q, int waves, int64_t M, int64_t kbc) {
-  return (int64_t)waves * 16 * ((q + 3) / 4) * 256 + M * x_lds_stride_for(kbc) + (M + 2) * kbc * 4;
+  return (int64_t)waves * 16 * ((q + 3) / 4) * 256 + M * x_lds_stride_for(kbc) + (M + 2 * waves) * kbc * 4;
 }
 
-template <int TMX, int Q, int DEPTH, int WAVES, bool XLDS>
+template <int TMX, int Q, int DEPTH, int WAVES, bool XLDS, bool OWN = false>
 int launch_transpose(const SmallArgs& sa, int mode, hipStream_t stream) {
   // WAVES slabs of 4 KB per 16 rows; the reduction buffer (WAVES * 16*TMX * rows floats) reuses the same memory
   constexpr int kSlabs = WAVES * 16 * ((Q + 3) / 4) * 256;
-  const int64_t kbc = std::min<int64_t>(sa.g.KB, (int64_t)sa.kpw * WAVES * 2);
+  const int64_t kbc = OWN ? sa.g.KB : std::min<int64_t>(sa.g.KB, (int64_t)sa.kpw * WAVES * 2);
   const int lds_bytes = XLDS ? (int)decode_lds_bytes(Q, WAVES, sa.g.M, kbc) : kSlabs;
   if (lds_bytes > kDecodeLdsLimit) FG_FAIL(FG_ERR_LAUNCH, "fp8 gemm (small M): %d bytes of LDS planned", lds_bytes);
-  const dim3 grid((uint32_t)sa.n_chunks, (uint32_t)sa.splits, (uint32_t)(sa.g.batch > 1 ? sa.g.batch : 1));
+  const dim3 grid((uint32_t)(OWN ? ceil_div(sa.n_chunks, WAVES) : sa.n_chunks), (uint32_t)sa.splits, (uint32_t)(sa.g.batch > 1 ? sa.g.batch : 1));
   const dim3 block(WAVES * 64);
-  auto kb = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeBlock, XLDS>;
-  auto kr = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeRowCol, XLDS>;
+  auto kb = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeBlock, XLDS, OWN>;
+  auto kr = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeRowCol, XLDS, OWN>;
   static PerDeviceFlags lds_limit_raised = {};  // per instantiation
   {
     const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, XLDS ? kDecodeLdsLimit : kSlabs, reinterpret_cast<const void*>(kb), reinterpret_cast<const void*>(kr));
@@ -626,6 +646,16 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
     // a block with idle wavefronts wastes launch slots: fewer wavefronts when K is short
     if (splits == 1 && KB <= 4) { p.waves = 4; kpw = ceil_div(KB, 4); }
   }
+  // Wide weights (five or more 16-row groups per compute unit, M <= 16): a wavefront per 16 rows walks all of K, four
+  // wavefronts to a block that shares the activations through LDS; two or more such blocks fit a compute unit.
+  // Measured against whole chunks shared by eight wavefronts: N = 24576, K = 1536: 12.3 -> 9.2 us; N = 32768,
+  // K = 512: 6.5 -> 6.1 us; N = 28672, K = 4096: 26.5 -> 25 us; N = 16384, K = 2048 (four groups per unit): no gain.
+  p.own = p.tmx == 1 && KB >= 2 && ceil_div(N, 16) * entries >= 5 * (int64_t)cu_count() &&
+          decode_lds_bytes(4, 4, M, KB) <= kDecodeLdsLimit / 2;
+  if (p.own) {
+    p.staged = true; p.xlds = true; p.q = 4; p.rg = 1; p.waves = 4; splits = 1; kpw = (KB + 1) / 2;
+    p.n_chunks = (int)ceil_div(N, 16);
+  }
   p.kpw = (int)kpw;
   p.splits = (int)splits;
   p.workspace_bytes = splits > 1
@@ -671,6 +701,7 @@ int launch_small_m(const GemmArgs& g, int mode, const SmallMPlan& plan, void* wo
       FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm (small M): row strides of %lld / %lld bytes are beyond the kernel's 32-bit offsets",
               (long long)g.ldx, (long long)g.ldw);
     if (g.batch > 65535) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm (small M): at most 65535 batch entries per launch, got %d", g.batch);
+    if (plan.own) return launch_transpose<1, 4, 1, 4, true, true>(sa, mode, stream);
     if (plan.xlds) {
       switch (plan.q) {
         case 1: return launch_transpose<1, 1, 1, 8, true>(sa, mode, stream);

@@ -163,14 +163,16 @@ def test_33_to_128_rows(M, N, K, dtype):
 
 @pytest.mark.parametrize("M,N,K", [(1, 2112, 7168), (16, 2112, 7168), (5, 1000, 7168), (3, 200, 8192), (7, 300, 16512),
                                    (16, 4608, 7168), (12, 7168, 16384), (2, 7168, 16384), (1, 24576, 1536),
-                                   (32, 2112, 7168), (20, 4608, 4096), (1, 9, 1024), (4, 130, 2048), (9, 4099, 7296)])
+                                   (32, 2112, 7168), (20, 4608, 4096), (1, 9, 1024), (4, 130, 2048), (9, 4099, 7296),
+                                   (16, 32768, 512), (5, 24580, 384), (2, 20480, 256), (16, 28672, 4096)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_up_to_32_rows_uneven_chunks(M, N, K, dtype):
     """M <= 32 takes the kernel that deals the weight rows out evenly over the compute units: chunks that differ by a
     row and begin anywhere (so that a chunk's rows lie in two 128-row scale blocks), chunks of fewer than 16 rows, N
     that is no multiple of 4, K split over blocks, an odd number of K-blocks, activations kept in LDS (long K, M <=
-    16) or fetched per K-block (short K, M = 12 with K = 16384, M > 16), column-major activation scales; against the
-    oracle and bit-identical on reruns."""
+    16) or fetched per K-block (short K, M = 12 with K = 16384, M > 16), wide weights (a wavefront per 16 rows, the
+    last four shapes: K of 2, 3 and 4 K-blocks, N that ends inside a 16-row group, activations too large to share),
+    column-major activation scales; against the oracle and bit-identical on reruns."""
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=17)
     want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
     args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
