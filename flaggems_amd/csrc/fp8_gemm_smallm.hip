@@ -603,16 +603,19 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   p.xlds = false;
   p.staged = p.tmx <= 2 && KB >= 8;
   int64_t chunks = 0;
-  if (p.staged) {
-    // One block per compute unit with the rows dealt out evenly (chunks differ by at most one row): a launch
-    // takes as long as the compute unit with most bytes to fetch.  Narrow weights get chunks of at least 4 rows
-    // and K split over blocks below; weights with more than 64 rows per compute unit get whole rounds of blocks.
-    const int64_t B = std::max<int64_t>(1, cu_count() / entries);
-    chunks = N <= 64 * B ? std::min<int64_t>(B, ceil_div(N, 4)) : ceil_div(N, 64 * B) * B;
+  // One block per compute unit with the rows dealt out evenly (chunks differ by at most one row): a launch takes as
+  // long as the compute unit with most bytes to fetch.  Narrow weights get chunks of at least `rows_min` rows and K
+  // split over blocks below; weights with more than 64 rows per compute unit get whole rounds of blocks.
+  const int64_t B = std::max<int64_t>(1, cu_count() / entries);
+  auto deal_rows = [&](int64_t rows_min) {
+    chunks = N <= 64 * B ? std::min<int64_t>(B, ceil_div(N, rows_min)) : ceil_div(N, 64 * B) * B;
     const int64_t rows_max = ceil_div(N, chunks);
     p.q = (int)ceil_div(rows_max, 4);
     p.rg = p.q <= 4 ? 1 : (p.q <= 8 ? 2 : 4);
     p.waves = (p.tmx == 2 && p.rg == 4) ? 4 : 8;
+  };
+  if (p.staged) {
+    deal_rows(p.tmx == 1 ? 4 : 16);
   } else {
     p.waves = p.tmx == 4 ? 4 : 8;  // LDS reduction buffer is 4 KB * tmx per wavefront
   }
@@ -623,17 +626,29 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   const int64_t max_splits = K / (32 * 16 * p.tmx) > 1 ? K / (32 * 16 * p.tmx) : 1;
   if (p.staged) {
     const int64_t pairs = (KB + 1) / 2;
-    splits = 1;
-    while (p.n_chunks * entries * splits < 100 && splits * 2 <= max_splits && splits * 2 * p.waves <= pairs) splits *= 2;
-    kpw = ceil_div(pairs, splits * p.waves);
-    // activations in LDS when M <= 16 and they fit beside the slabs; the chunk then has exactly the 4-row groups
-    // it needs (instantiated: 1, 2, 3, 4, 6, 8, 12, 16), otherwise whole 16-row groups
+    auto split_k = [&]() {
+      p.n_chunks = (int)chunks;
+      splits = 1;
+      while (p.n_chunks * entries * splits < 100 && splits * 2 <= max_splits && splits * 2 * p.waves <= pairs) splits *= 2;
+      kpw = ceil_div(pairs, splits * p.waves);
+    };
+    split_k();
+    // activations in LDS when M <= 16, a wavefront has three or more pairs of K-blocks and they fit beside the
+    // slabs.  A chunk has exactly the 4-row groups it needs (instantiated: 1, 2, 3, 4, 6, 8, 12, 16) when M <= 16,
+    // whole 16-row groups otherwise.
     static const int kQ[] = {1, 2, 3, 4, 6, 8, 12, 16};
-    int q = 16;
-    for (int i = 7; i >= 0; --i) if (kQ[i] >= p.q) q = kQ[i];
-    const int64_t kbc = std::min<int64_t>(KB, kpw * p.waves * 2);
-    p.xlds = p.tmx == 1 && kpw >= 3 && decode_lds_bytes(q, p.waves, M, kbc) <= kDecodeLdsLimit;
-    p.q = p.xlds ? q : 4 * p.rg;
+    auto round_q = [&](int need) { int q = 16; for (int i = 7; i >= 0; --i) if (kQ[i] >= need) q = kQ[i]; return q; };
+    int q = round_q(p.q);
+    p.xlds = p.tmx == 1 && kpw >= 3 && decode_lds_bytes(q, p.waves, M, std::min<int64_t>(KB, kpw * p.waves * 2)) <= kDecodeLdsLimit;
+    if (!p.xlds && p.tmx == 1 && M > 4 && N <= 64 * B) {
+      // every block fetches all M activation rows of its K range per pair of K-blocks: chunks of fewer rows than
+      // that move more activation than weight bytes (N = 2048, K = 1024, M = 16: 256 chunks of 8 rows 3.8 us,
+      // 128 of 16 rows 3.5 us; N = 1024, K = 8192: 9.1 against 7.9 us)
+      deal_rows((M + 3) / 4 * 4);
+      split_k();
+      q = round_q(p.q);
+    }
+    p.q = p.tmx == 1 ? q : 4 * p.rg;
   } else {
     // aim for ~8 wavefronts per CU on 256 CUs, each with at least one K-block
     const int64_t units = (int64_t)p.n_chunks * entries * KB;
@@ -650,7 +665,9 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   // wavefronts to a block that shares the activations through LDS; two or more such blocks fit a compute unit.
   // Measured against whole chunks shared by eight wavefronts: N = 24576, K = 1536: 12.3 -> 9.2 us; N = 32768,
   // K = 512: 6.5 -> 6.1 us; N = 28672, K = 4096: 26.5 -> 25 us; N = 16384, K = 2048 (four groups per unit): no gain.
-  p.own = p.tmx == 1 && KB >= 2 && ceil_div(N, 16) * entries >= 5 * (int64_t)cu_count() &&
+  // With more than 16 pairs of K-blocks the walk of a single wavefront gets long and the shared chunks are as fast
+  // (N = 32768, K = 8192: 51 us shared, 53-56 us here), so this form stops at K = 4096.
+  p.own = p.tmx == 1 && KB >= 2 && KB <= 32 && ceil_div(N, 16) * entries >= 5 * (int64_t)cu_count() &&
           decode_lds_bytes(4, 4, M, KB) <= kDecodeLdsLimit / 2;
   if (p.own) {
     p.staged = true; p.xlds = true; p.q = 4; p.rg = 1; p.waves = 4; splits = 1; kpw = (KB + 1) / 2;
@@ -715,9 +732,16 @@ int launch_small_m(const GemmArgs& g, int mode, const SmallMPlan& plan, void* wo
       }
     }
     if (plan.tmx == 1) {
-      if (plan.rg == 1) return launch_transpose<1, 4, 4, 8, false>(sa, mode, stream);
-      if (plan.rg == 2) return launch_transpose<1, 8, 3, 8, false>(sa, mode, stream);
-      return launch_transpose<1, 16, 2, 8, false>(sa, mode, stream);
+      switch (plan.q) {
+        case 1: return launch_transpose<1, 1, 4, 8, false>(sa, mode, stream);
+        case 2: return launch_transpose<1, 2, 4, 8, false>(sa, mode, stream);
+        case 3: return launch_transpose<1, 3, 4, 8, false>(sa, mode, stream);
+        case 4: return launch_transpose<1, 4, 4, 8, false>(sa, mode, stream);
+        case 6: return launch_transpose<1, 6, 3, 8, false>(sa, mode, stream);
+        case 8: return launch_transpose<1, 8, 3, 8, false>(sa, mode, stream);
+        case 12: return launch_transpose<1, 12, 2, 8, false>(sa, mode, stream);
+        default: return launch_transpose<1, 16, 2, 8, false>(sa, mode, stream);
+      }
     }
     if (plan.rg == 1) return launch_transpose<2, 4, 3, 8, false>(sa, mode, stream);
     if (plan.rg == 2) return launch_transpose<2, 8, 2, 8, false>(sa, mode, stream);
