@@ -112,9 +112,10 @@ __device__ __forceinline__ void compute_unit(const Unit<TMX>& u, v4f (&acc)[kRow
 }
 
 // Adds the wavefronts' accumulators in LDS and writes the chunk (or publishes a split-K partial tile and,
-// in the block that arrives last, adds the partial tiles in split order).  `red` is [WAVES][16*TMX][16*RG]; the chunk is rows n0 .. n0 + rows - 1.
+// in the block that arrives last, adds the partial tiles in split order).  Wavefront w's sums go to red[w * red_stride + m * 16*RG + n]; the chunk is
+// rows n0 .. n0 + rows - 1.
 template <int TMX, int RG, int WAVES, int MODE>
-__device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int* last_flag,
+__device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int red_stride, int* last_flag,
                                              const v4f (&acc)[RG][TMX], int chunk, int split, int n0, int rows) {
   constexpr int NT = WAVES * 64;
   constexpr int MROWS = 16 * TMX;
@@ -124,12 +125,16 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
   const GemmArgs& g = a.g;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, lg = lane >> 4;
+  // bf16 results of the block-scaled product, the case these kernels meet in practice, are stored by a few
+  // instructions of their own: the general epilogue is a long chain of branches, and at the end of a launch of a few
+  // microseconds every instruction line it fetches is waited for by the whole GPU
+  const bool plain = MODE == kModeBlock && g.c_dtype == FG_BF16;
   // lane holds m = t*16 + l16, n = r*16 + 4*lg + [0,4)
 #pragma unroll
   for (int r = 0; r < kRowGroups; ++r)
 #pragma unroll
     for (int t = 0; t < TMX; ++t)
-      *reinterpret_cast<v4f*>(red + ((wave * MROWS + t * 16 + l16) * kChunkRows + r * 16 + lg * 4)) = acc[r][t];
+      *reinterpret_cast<v4f*>(red + wave * red_stride + ((t * 16 + l16) * kChunkRows + r * 16 + lg * 4)) = acc[r][t];
   __syncthreads();
 
   if (a.splits == 1) {
@@ -137,8 +142,11 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
       const int m = i / kChunkRows, nn = i % kChunkRows;
       float v = 0.f;
 #pragma unroll
-      for (int w = 0; w < WAVES; ++w) v += red[w * kOut + i];
-      if (m < g.M && nn < rows) store_output<MODE>(g, m, n0 + nn, v);
+      for (int w = 0; w < WAVES; ++w) v += red[w * red_stride + i];
+      if (m < g.M && nn < rows) {
+        if (plain) reinterpret_cast<uint16_t*>(g.C)[(int64_t)m * g.ldc + n0 + nn] = float_to_bf16_bits(v);
+        else store_output<MODE>(g, m, n0 + nn, v);
+      }
     }
     return;
   }
@@ -147,7 +155,7 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
   for (int i = tid; i < kOut; i += NT) {
     float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) v += red[w * kOut + i];
+    for (int w = 0; w < WAVES; ++w) v += red[w * red_stride + i];
     // device-scope store: written through to memory, where blocks on other XCDs (own L2 each) read it
     __hip_atomic_store(mine + i, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
@@ -170,7 +178,10 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
     float v = 0.f;
     for (int s = 0; s < a.splits; ++s)
       v += __hip_atomic_load(all + (int64_t)s * kOut + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (m < g.M && nn < rows) store_output<MODE>(g, m, n0 + nn, v);
+    if (m < g.M && nn < rows) {
+      if (plain) reinterpret_cast<uint16_t*>(g.C)[(int64_t)m * g.ldc + n0 + nn] = float_to_bf16_bits(v);
+      else store_output<MODE>(g, m, n0 + nn, v);
+    }
   }
   if (tid == 0) __hip_atomic_store(&a.counters[chunk], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
 }
@@ -231,7 +242,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_smallm_kernel(SmallArgs a
     compute_unit<TMX, MODE>(cur, acc);
   }
 
-  finish_chunk<TMX, kRowGroups, WAVES, MODE>(a, &red[0][0][0], &last_flag, acc, chunk, split, n0, min(kChunkRows, g.N - n0));
+  finish_chunk<TMX, kRowGroups, WAVES, MODE>(a, &red[0][0][0], MROWS * kChunkRows, &last_flag, acc, chunk, split, n0, min(kChunkRows, g.N - n0));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -533,18 +544,25 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
   select_batch_entry(a, z);  // the epilogue's view of the operands
   if (OWN) {
     if (idle) return;
-    // lane holds m = l16, n = n0 + r*16 + 4*lg + [0,4)
+    // lane holds m = l16, n = n0 + r*16 + 4*lg + [0,4); bf16 results of the block-scaled product take a short path
+    // of their own (see finish_chunk)
+    const bool plain = MODE == kModeBlock && g.c_dtype == FG_BF16;
+    uint16_t* const c_row = reinterpret_cast<uint16_t*>(g.C) + (int64_t)l16 * g.ldc + n0;
 #pragma unroll
     for (int r = 0; r < RG; ++r)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int nn = r * 16 + lg * 4 + i;
-        if (l16 < g.M && nn < rows_valid) store_output<MODE>(g, l16, n0 + nn, acc[r][0][i]);
+        if (l16 < g.M && nn < rows_valid) {
+          if (plain) c_row[nn] = float_to_bf16_bits(acc[r][0][i]);
+          else store_output<MODE>(g, l16, n0 + nn, acc[r][0][i]);
+        }
       }
     return;
   }
-  __syncthreads();           // the slabs are dead; their memory now holds the reduction buffer
-  finish_chunk<TMX, RG, WAVES, MODE>(a, reinterpret_cast<float*>(lds), &last_flag, acc, chunk, split, n0, rows_valid);
+  // a wavefront's sums (16*TMX x 16*RG floats) go into its own slab, which only it has used: no barrier before them
+  static_assert(16 * TMX * 4 <= 256, "a wavefront's sums fit its slab");
+  finish_chunk<TMX, RG, WAVES, MODE>(a, reinterpret_cast<float*>(lds), kSlab / 4, &last_flag, acc, chunk, split, n0, rows_valid);
 }
 
 template <int TMX, int WAVES>
