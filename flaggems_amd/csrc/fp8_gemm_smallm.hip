@@ -37,6 +37,8 @@ struct SmallArgs {
   // staged kernels: chunk c owns rows_lo + (c < rows_rem) weight rows, the chunks in ascending row order; the
   // activations of the block's K range are kept in LDS with rows x_lds_stride bytes apart (0: not kept)
   int rows_lo, rows_rem, x_lds_stride;
+  int pw_pairs;  // pairs of K-blocks of the blocks that have most (per-wavefront form of the activations in LDS)
+  int m_recip;  // 65535 / M + 1: (u * m_recip) >> 16 == u / M for the small u the kernel divides
   float* partials;      // [n_chunks][splits][16 * TMX][64]
   unsigned int* counters;
   int64_t partials_per_entry;  // floats; a batch (g.batch > 1, entry = blockIdx.y) keeps one such array and n_chunks counters per entry
@@ -277,12 +279,17 @@ __device__ __forceinline__ void dma_to_lds_4(uint32_t byte_off, const void* base
 // Q = 4-row groups of weights per chunk (a chunk has up to 4Q rows, the block's wavefronts take interleaved pairs
 // of K-blocks), DEPTH = K-block pairs in flight per wavefront.
 //
-// A launch of a few microseconds is bound by the number of vector-memory instructions a compute unit has to push
-// through its address unit (about 14 cycles each, whatever they carry), so nothing but weights is loaded per pair
-// of K-blocks when XLDS is set: at its start the block copies the activations of its K range (M <= 16 rows) and
-// their scales into LDS with a handful of global -> LDS copies, the weight scales come through the scalar cache,
-// and the chunk has no more 4-row groups than its rows need.  Without XLDS (activations too large for LDS) the
-// activation fragments travel in the register ring next to the weights.
+// A launch of a few microseconds is bound by what a compute unit does around its bytes: every vector-memory
+// instruction occupies the address unit (about 14 cycles each, whatever it carries), and a wavefront that issues a
+// load while the memory pipeline is full blocks at the issue.  So, when XLDS is set (M <= 16), nothing but weights is
+// loaded per pair of K-blocks: at its start every wavefront copies the activations its own pairs need, their scales
+// and the weight scales into LDS with a handful of global -> LDS copies (no barrier: a pair is multiplied by the
+// wavefront that copied for it, and the wait for its first weights is also the wait for its copies, which were
+// issued earlier and complete in order); the ring holds one pair, whose refill goes out as soon as it is in the slab,
+// and the chunk has no more 4-row groups than its rows need.  OWN (wide weights): every wavefront has a chunk of
+// its own and walks all of K, so the block shares the activations (one barrier) and nothing is added across
+// wavefronts.  Without XLDS (activations too large for LDS, or too few pairs per wavefront to pay for the copies)
+// the activation fragments travel in the register ring next to the weights.
 template <int TMX, int Q, int DEPTH, int WAVES, int MODE, bool XLDS, bool OWN = false>
 __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArgs a) {
   static_assert(!XLDS || TMX == 1, "activations are kept in LDS for M <= 16 only");
@@ -331,12 +338,63 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
 
 
   // ---- activations and their scales -> LDS (issued before the first weight load: they arrive first)
-  const uint32_t lds_x = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + WAVES * kSlab;  // rows x_lds_stride apart, 16-byte pieces permuted
+  constexpr bool PW = XLDS && !OWN;  // every wavefront copies what its own pairs of K-blocks need: no barrier
+  const uint32_t lds_x = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + WAVES * kSlab;
+  // shared form (OWN): rows x_lds_stride apart, 16-byte pieces permuted; [M][kbc] activation scales; [2][kbc] weight
+  // scales per wavefront
   const uint32_t x_stride = (uint32_t)a.x_lds_stride;
-  const uint32_t lds_xs = lds_x + (uint32_t)g.M * x_stride;         // [M][kbc] floats
-  // [2][kbc] floats: the chunk's two weight-scale blocks (per wavefront when every wavefront has its own chunk)
-  const uint32_t lds_ws = lds_xs + (uint32_t)(g.M * kbc) * 4u + (OWN ? (uint32_t)(wave * 2 * kbc) * 4u : 0u);
-  if (XLDS) {
+  const uint32_t lds_xs = lds_x + (uint32_t)g.M * x_stride;
+  const uint32_t lds_ws = lds_xs + (uint32_t)(g.M * kbc) * 4u + (uint32_t)(wave * 2 * kbc) * 4u;
+  // per-wavefront form (PW): slot i of a wavefront is its i-th pair; [slot][row][256 B] activations with the 16
+  // pieces of a row's pair permuted by the row, [slot][K-block][row] activation scales, [slot][scale block][K-block]
+  // weight scales
+  // (the block's pairs are dealt round-robin, so wavefront w's slots begin after those of the wavefronts before it)
+  const int blk_pairs = pair_end - pair_lo;
+  const uint32_t slot0 = (uint32_t)(wave * (blk_pairs / WAVES) + min(wave, blk_pairs % WAVES));
+  const uint32_t pw_x = lds_x + slot0 * (uint32_t)g.M * 256u;
+  const uint32_t pw_xs = lds_x + (uint32_t)(a.pw_pairs * g.M) * 256u + slot0 * (uint32_t)(2 * g.M) * 4u;
+  const uint32_t pw_ws = lds_x + (uint32_t)(a.pw_pairs * g.M) * (256u + 8u) + slot0 * 16u;
+  if (PW) {
+    const int first = pair_lo + wave;
+    const int my_pairs = first < pair_end ? (pair_end - first + WAVES - 1) / WAVES : 0;
+    const int recip = a.m_recip;
+    // one copy = 4 (slot, row) units of 256 bytes; physical piece l16 of a unit holds logical piece l16 ^ (row & 15),
+    // so that the 16 rows a wavefront reads together fall into 16 different 16-byte bank groups.  Where the pair's
+    // second K-block does not exist its pieces repeat the first's.
+    const int units = my_pairs * g.M;
+    for (int j = 0; j * 4 < units; ++j) {
+      const int u = j * 4 + lg;
+      if (u < units) {
+        const int i = (u * recip) >> 16, m = u - i * g.M;
+        const int p = first + i * WAVES;
+        int piece = l16 ^ (m & 15);
+        if (p * 2 + 1 >= g.KB && piece >= 8) piece -= 8;
+        dma_to_lds_16((uint32_t)m * (uint32_t)g.ldx + (uint32_t)p * 256u + (uint32_t)piece * 16u, x_base, pw_x + (uint32_t)j * 1024u);
+      }
+    }
+    if (MODE == kModeBlock) {
+      const int count = my_pairs * 2 * g.M;  // e = (slot * 2 + b) * M + row
+      for (int j = 0; j * 64 < count; ++j) {
+        const int e = j * 64 + lane;
+        if (e < count) {
+          const int q = (e * recip) >> 16, m = e - q * g.M;
+          const int p = first + (q >> 1) * WAVES;
+          const int kb = p * 2 + (((q & 1) && p * 2 + 1 < g.KB) ? 1 : 0);
+          dma_to_lds_4(((uint32_t)m * (uint32_t)g.xs_rs + (uint32_t)kb * xs_cs) * 4u, xs_base, pw_xs + (uint32_t)j * 256u);
+        }
+      }
+      const int wcount = my_pairs * 4;  // e = slot * 4 + scale block * 2 + b
+      for (int j = 0; j * 64 < wcount; ++j) {
+        const int e = j * 64 + lane;
+        if (e < wcount) {
+          const int p = first + (e >> 2) * WAVES;
+          const int kb = p * 2 + (((e & 1) && p * 2 + 1 < g.KB) ? 1 : 0);
+          dma_to_lds_4((uint32_t)((int64_t)kb * g.ws_cs + ((e & 2) ? ws_second : 0)) * 4u, ws_base, pw_ws + (uint32_t)j * 256u);
+        }
+      }
+    }
+  }
+  if (XLDS && OWN) {
     // one copy = 64 pieces of 16 bytes of one row; piece p of a row lies at position p ^ perm(row) within its
     // K-block (8 pieces), perm(row) = (row >> 1) & 7, and the row stride is an odd multiple of 128 bytes: the 16
     // rows a wavefront reads together then fall into 16 different 16-byte bank groups
@@ -367,7 +425,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
     }
     if (MODE == kModeBlock) {
       const int row_units = (kbc + 63) >> 6;
-      for (int c = OWN ? 0 : wave; c < 2 * row_units; c += OWN ? 1 : WAVES) {
+      for (int c = 0; c < 2 * row_units; ++c) {
         const int row = c & 1, k0 = (c >> 1) * 64;
         if (k0 + lane < kbc)
           dma_to_lds_4((uint32_t)((int64_t)(kb_lo + k0 + lane) * g.ws_cs + (row ? ws_second : 0)) * 4u, ws_base,
@@ -401,8 +459,10 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
     lds_xrow[t] = lds_x + (uint32_t)m * x_stride;
     lds_xsrow[t] = lds_xs + (uint32_t)(m * kbc) * 4u;
   }
-  const uint32_t perm = (uint32_t)(((l16 < g.M ? l16 : g.M - 1) >> 1) & 7);  // TMX == 1 when used
+  const uint32_t mrow = (uint32_t)(l16 < g.M ? l16 : g.M - 1);  // TMX == 1 when used
+  const uint32_t perm = PW ? (mrow & 15u) : ((mrow >> 1) & 7u);
   const uint32_t x_lo_piece = ((uint32_t)lg ^ perm) << 4, x_hi_piece = ((uint32_t)(lg + 4) ^ perm) << 4;
+  int slot = 0;  // PW: index of the pair among this wavefront's
 
   v4f acc[RG][TMX];
 #pragma unroll
@@ -453,7 +513,10 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
       if (b == 1 && !two) break;
       float ws1 = 1.f, ws2 = 1.f;
       if (MODE == kModeBlock) {
-        if (XLDS) {
+        if (PW) {
+          ws1 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(pw_ws + (uint32_t)(slot * 4 + b) * 4u);
+          ws2 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(pw_ws + (uint32_t)(slot * 4 + 2 + b) * 4u);
+        } else if (XLDS) {
           ws1 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(lds_ws + (uint32_t)(kb + b - kb_lo) * 4u);
           ws2 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(lds_ws + (uint32_t)(kbc + kb + b - kb_lo) * 4u);
         } else {
@@ -465,7 +528,16 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
       float xsc[TMX];
 #pragma unroll
       for (int t = 0; t < TMX; ++t) {
-        if (XLDS) {
+        if (PW) {
+          // the pair's 16 pieces are permuted as a whole: logical piece b*8 + lg (+4) sits at that number ^ perm
+          const uint32_t at = pw_x + ((uint32_t)(slot * g.M) + mrow) * 256u;
+          const u32x4 lo = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + (((uint32_t)(b * 8 + lg) ^ perm) << 4));
+          const u32x4 hi = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + (((uint32_t)(b * 8 + lg + 4) ^ perm) << 4));
+          xf[t] = join(lo, hi);
+          xsc[t] = (MODE == kModeBlock)
+                       ? *reinterpret_cast<const __attribute__((address_space(3))) float*>(pw_xs + ((uint32_t)((slot * 2 + b) * g.M) + mrow) * 4u)
+                       : 1.f;
+        } else if (XLDS) {
           const uint32_t at = lds_xrow[t] + (uint32_t)(kb + b - kb_lo) * 128u;
           const u32x4 lo = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + x_lo_piece);
           const u32x4 hi = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + x_hi_piece);
@@ -517,7 +589,8 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
     // earlier and complete in order; a wavefront without work waits for its copies alone.
     if (!done) { stage(ring[0]); staged_ahead = true; }
     else wait_vmem_all();
-    __syncthreads();
+    if (OWN) __syncthreads();
+    else asm volatile("" ::: "memory");  // the reads of what the copies brought stay behind that wait
   }
   while (!done) {
 #pragma unroll
@@ -536,6 +609,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
           load_x(ring[d], refill);
         }
         pair += STEP;
+        ++slot;
         done = pair >= pair_end;
       }
     }
@@ -583,13 +657,17 @@ inline int x_lds_stride_for(int64_t kbc) { return (int)((kbc | 1) * 128); }
 inline int64_t decode_lds_bytes(int q, int waves, int64_t M, int64_t kbc) {
   return (int64_t)waves * 16 * ((q + 3) / 4) * 256 + M * x_lds_stride_for(kbc) + (M + 2 * waves) * kbc * 4;
 }
+// the same with every wavefront keeping what its own pairs of K-blocks need; `pairs` = pairs of K-blocks per block
+inline int64_t decode_lds_bytes_per_wave(int q, int waves, int64_t M, int64_t pairs) {
+  return (int64_t)waves * 16 * ((q + 3) / 4) * 256 + pairs * (M * 256 + 2 * M * 4 + 16);
+}
 
 template <int TMX, int Q, int DEPTH, int WAVES, bool XLDS, bool OWN = false>
 int launch_transpose(const SmallArgs& sa, int mode, hipStream_t stream) {
   // WAVES slabs of 4 KB per 16 rows; the reduction buffer (WAVES * 16*TMX * rows floats) reuses the same memory
   constexpr int kSlabs = WAVES * 16 * ((Q + 3) / 4) * 256;
   const int64_t kbc = OWN ? sa.g.KB : std::min<int64_t>(sa.g.KB, (int64_t)sa.kpw * WAVES * 2);
-  const int lds_bytes = XLDS ? (int)decode_lds_bytes(Q, WAVES, sa.g.M, kbc) : kSlabs;
+  const int lds_bytes = !XLDS ? kSlabs : OWN ? (int)decode_lds_bytes(Q, WAVES, sa.g.M, kbc) : (int)decode_lds_bytes_per_wave(Q, WAVES, sa.g.M, sa.pw_pairs);
   if (lds_bytes > kDecodeLdsLimit) FG_FAIL(FG_ERR_LAUNCH, "fp8 gemm (small M): %d bytes of LDS planned", lds_bytes);
   const dim3 grid((uint32_t)(OWN ? ceil_div(sa.n_chunks, WAVES) : sa.n_chunks), (uint32_t)sa.splits, (uint32_t)(sa.g.batch > 1 ? sa.g.batch : 1));
   const dim3 block(WAVES * 64);
@@ -651,13 +729,13 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
       kpw = ceil_div(pairs, splits * p.waves);
     };
     split_k();
-    // activations in LDS when M <= 16, a wavefront has three or more pairs of K-blocks and they fit beside the
-    // slabs.  A chunk has exactly the 4-row groups it needs (instantiated: 1, 2, 3, 4, 6, 8, 12, 16) when M <= 16,
+    // activations in LDS when M <= 16, a wavefront has three or more pairs of K-blocks (two with more than 8
+    // activation rows: N = K = 4096, M = 16: 7.2 -> 6.5 us, M = 1: 5.8 -> 5.9 us) and they fit beside the slabs.  A chunk has exactly the 4-row groups it needs (instantiated: 1, 2, 3, 4, 6, 8, 12, 16) when M <= 16,
     // whole 16-row groups otherwise.
     static const int kQ[] = {1, 2, 3, 4, 6, 8, 12, 16};
     auto round_q = [&](int need) { int q = 16; for (int i = 7; i >= 0; --i) if (kQ[i] >= need) q = kQ[i]; return q; };
     int q = round_q(p.q);
-    p.xlds = p.tmx == 1 && kpw >= 3 && decode_lds_bytes(q, p.waves, M, std::min<int64_t>(KB, kpw * p.waves * 2)) <= kDecodeLdsLimit;
+    p.xlds = p.tmx == 1 && kpw >= (M > 8 ? 2 : 3) && decode_lds_bytes_per_wave(q, p.waves, M, std::min<int64_t>(pairs, kpw * p.waves)) <= kDecodeLdsLimit;
     if (!p.xlds && p.tmx == 1 && M > 4 && N <= 64 * B) {
       // every block fetches all M activation rows of its K range per pair of K-blocks: chunks of fewer rows than
       // that move more activation than weight bytes (N = 2048, K = 1024, M = 16: 256 chunks of 8 rows 3.8 us,
@@ -710,6 +788,8 @@ int launch_small_m(const GemmArgs& g, int mode, const SmallMPlan& plan, void* wo
   sa.rows_lo = (int)(g.N / plan.n_chunks);
   sa.rows_rem = (int)(g.N % plan.n_chunks);
   sa.x_lds_stride = plan.xlds ? x_lds_stride_for(std::min<int64_t>(g.KB, (int64_t)plan.kpw * plan.waves * 2)) : 0;
+  sa.m_recip = (int)(65535 / g.M + 1);
+  sa.pw_pairs = (int)std::min<int64_t>((g.KB + 1) / 2, (int64_t)plan.kpw * plan.waves);
   sa.partials = nullptr;
   sa.counters = nullptr;
   sa.partials_per_entry = 0;
