@@ -153,3 +153,25 @@ def test_workspace_outlives_the_graphs_that_captured_it():
         stream.synchronize()
         assert torch.equal(again, out_big)
         del junk, graph
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 2112, 7168), (16, 24576, 1536), (8, 7168, 2304), (16, 4096, 4096)])
+def test_decode_kernels_replayed_from_a_graph(M, N, K):
+    """The decode kernels in their three forms (activations copied into LDS per wavefront, a wavefront per 16 rows of
+    wide weights, activation fragments in registers) give, replayed from a HIP graph several times with eager work
+    between the replays, the bits of the eager call."""
+    args, want = _quantized(M, N, K, 5)
+    eager = flag_gems.w8a8_block_fp8_matmul(*args, [128, 128])
+    torch.testing.assert_close(eager.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        out = flag_gems.w8a8_block_fp8_matmul(*args, [128, 128])
+    for _ in range(3):
+        out.zero_()
+        other = flag_gems.w8a8_block_fp8_matmul(args[0], args[1], args[2] * 2, args[3], [128, 128])  # eager work in between
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        assert not torch.equal(other, eager)
