@@ -53,11 +53,11 @@ REPEATS = 6               # timed replays per shape; the first is dropped, the m
 # half of the copied bytes, factor 2.0; WRITE_SIZE read all of them, factor 1.0).  (N, K) -> (fetch, write) KiB.
 TRAFFIC_M4096_KIB = {
     (2112, 7168): (2.0 * 63362.8, 17792.0),
-    (24576, 1536): (2.0 * 111956.0, 196800.0),
-    (32768, 512): (2.0 * 48180.8, 262148.5),
-    (7168, 16384): (2.0 * 365837.2, 59392.1),
-    (4608, 7168): (2.0 * 123754.7, 70568.2),
-    (7168, 2304): (2.0 * 51571.5, 57632.0),
+    (24576, 1536): (2.0 * 111957.9, 196800.0),
+    (32768, 512): (2.0 * 48283.8, 262144.0),
+    (7168, 16384): (2.0 * 365833.0, 59392.0),
+    (4608, 7168): (2.0 * 123754.8, 70568.0),
+    (7168, 2304): (2.0 * 51571.1, 57632.0),
 }
 
 
