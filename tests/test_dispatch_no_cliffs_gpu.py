@@ -1,5 +1,5 @@
 """The launch planner picks a kernel from (M, N, K) by thresholds that were fitted on the benchmark shapes.  This test
-walks shapes off that grid and checks that none falls into a slow corner: every call must finish within twice a
+walks shapes off that grid (decode-sized M and wide weights included) and checks that none falls into a slow corner: every call must finish within twice a
 deliberately loose cost model (the slower of 1.2 PFLOP/s and 2.5 TB/s, plus 15 us of fixed cost -- about half of what
 the tuned shapes reach), so a rule that sends a shape to a kernel three times too slow for it fails here.  Results
 are checked elsewhere; this file only times."""
@@ -13,8 +13,8 @@ DEV = "cuda"
 FP8 = torch.float8_e4m3fn
 
 NK = [(1000, 1024), (2112, 7168), (3000, 3072), (5120, 2048), (7168, 2304), (12288, 1536), (4096, 8192), (1536, 16384),
-      (28672, 4096), (512, 4096), (512, 7168), (2048, 16384)]
-MS = [3, 17, 33, 48, 65, 100, 130, 200, 300, 400, 600, 777, 1000, 1100, 1500, 2048, 3000, 5000]
+      (28672, 4096), (512, 4096), (512, 7168), (2048, 16384), (32768, 1024), (65536, 2048), (20480, 8192)]
+MS = [1, 3, 9, 17, 33, 48, 65, 100, 130, 200, 300, 400, 600, 777, 1000, 1100, 1500, 2048, 3000, 5000]
 
 
 def _model_us(M, N, K):
