@@ -248,13 +248,13 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_smallm_kernel(SmallArgs a
 }
 
 // ---------------------------------------------------------------------------------------------
-// Transposing variant (M <= 32, K >= 1024).  Same decomposition, but the weight bytes are fetched in
+// Transposing variant (M <= 32, K >= 1024, and wide weights from K = 256 on).  The weight bytes are fetched in
 // runs of 256 contiguous bytes per row (two K-blocks; 4 rows per wavefront load instruction) instead
 // of the 64-byte pieces the MFMA operand layout dictates: measured on MI355X a pure load of a
-// [7168, 16384] matrix reaches 5.8 TB/s with 256-byte runs against 5.0 TB/s with 64-byte pieces.  The
-// loads land in registers (the register file holds far more bytes in flight than LDS could); when a
-// pair of K-blocks has arrived the wavefront writes it to its private 16 KB LDS slab and reads it back
-// in operand layout.  No barrier is involved before the final reduction: a wavefront's LDS operations
+// [7168, 16384] matrix reaches 5.8 TB/s with 256-byte runs against 5.0 TB/s with 64-byte pieces, and of a
+// [2112, 7168] matrix with this kernel's ownership 3.6 against 2.5 TB/s.  The loads land in registers; when a
+// pair of K-blocks has arrived the wavefront writes it to its private LDS slab (4 KB per 16 rows) and reads it
+// back in operand layout.  No barrier is involved before the final reduction: a wavefront's LDS operations
 // execute in order.  Within a row the sixteen 16-byte chunks are permuted (physical chunk p holds
 // logical chunk p ^ (row & 15)) so that both the writes (4 rows x 256 B) and the operand reads (16 rows
 // 256 bytes apart) spread over all LDS banks.
