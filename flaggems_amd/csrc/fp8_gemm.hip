@@ -1171,6 +1171,8 @@ extern "C" int fg_scaled_int8_gemm(const void* A, int64_t lda, const void* B, in
   const bool direct = (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) && (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
                       ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
   hipStream_t st = (hipStream_t)stream;
+  // bf16 results with M > 128: the persistent kernel, as for fp8 operands with row and column scales
+  if (direct && M > 128 && pingpong_takes(a, kModeRowColI8, nullptr, 0)) return launch_pingpong(a, kModeRowColI8, nullptr, 0, st);
   if (M > 128)
     return direct ? launch_cfg<256, 256, 4, 2, kModeRowColI8, true>(a, st) : launch_cfg<256, 256, 4, 2, kModeRowColI8, false>(a, st);
   return direct ? launch_cfg<128, 128, 2, 2, kModeRowColI8, true>(a, st) : launch_cfg<128, 128, 2, 2, kModeRowColI8, false>(a, st);

@@ -288,6 +288,17 @@ __device__ __forceinline__ void mfma_accumulate(v4f& c, const v8i& w, const v8i&
   asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(c) : "v"(w), "v"(x));
 }
 
+// int8 operands (kModeRowColI8): the same fragment as two 16x16x64 products (`half` = 0: the lane's first 16 bytes of
+// the K-block, 1: its second 16), int32 sums kept as bit patterns in the accumulator registers; the two instructions
+// take as long as the one fp8 instruction.  The multiply phase issues the two halves of one accumulator kTM
+// instructions apart, so that the matrix pipe never waits for the sum it has just started.
+__device__ __forceinline__ void mfma_accumulate_i8_half(v4f& c, const v8i& w, const v8i& x, int half) {
+  typedef int v4i_ __attribute__((ext_vector_type(4)));
+  const v4i_ wh = half ? v4i_{w[4], w[5], w[6], w[7]} : v4i_{w[0], w[1], w[2], w[3]};
+  const v4i_ xh = half ? v4i_{x[4], x[5], x[6], x[7]} : v4i_{x[0], x[1], x[2], x[3]};
+  asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(c) : "v"(wh), "v"(xh));
+}
+
 // Scales that are powers of two (POW2): the block-scaled form of the instruction multiplies the products by
 // 2^(sw - 127) * 2^(sx - 127) on their way into the sum, so the matrix pipe accumulates the scaled K-blocks itself and
 // the multiply phase has no vector-ALU work at all.  sw / sx: E8M0 exponent in the low byte of a register per lane,
@@ -377,7 +388,7 @@ template <int MODE, bool ALIGNED, bool SCATTER = false>
 __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[kTN][kTM], int m_base, int n_base,
                                            int l16, int lg, int m_end, const int* out_index = nullptr, int c_rows = 0,
                                            const float* row_weight = nullptr) {
-  if (MODE == kModeRowCol) {
+  if (MODE != kModeBlock) {
     // eight columns at a time, so that only eight column scales and bias values are live
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
@@ -399,8 +410,13 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
 #pragma unroll
         for (int h = 0; h < 4; ++h) {  // two columns per word
           const int t = 2 * q + (h >> 1), e0 = (h & 1) * 2;
-          const float v0 = (acc[t][j][e0] * sa) * sb[4 * (h >> 1) + e0];
-          const float v1 = (acc[t][j][e0 + 1] * sa) * sb[4 * (h >> 1) + e0 + 1];
+          // (int8 operands: the registers hold int32 sums.  The element is copied to a scalar before the bit cast:
+          // a bit cast applied to the vector element itself reads element 0 whatever the index.)
+          const float r0 = acc[t][j][e0], r1 = acc[t][j][e0 + 1];
+          const float s0 = MODE == kModeRowColI8 ? (float)__float_as_int(r0) : r0;
+          const float s1 = MODE == kModeRowColI8 ? (float)__float_as_int(r1) : r1;
+          const float v0 = (s0 * sa) * sb[4 * (h >> 1) + e0];
+          const float v1 = (s1 * sa) * sb[4 * (h >> 1) + e0 + 1];
           w[h] = pack_bf16(v0, v1);
           if (a.bias)
             w[h] = pack_bf16(bits_to_float(w[h] << 16) + bias[4 * (h >> 1) + e0],
@@ -816,7 +832,19 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
 
     // ================= multiply(T)
     __builtin_amdgcn_s_setprio(kMultiplyPrio);
-    if (MODE != kModeBlock) {
+    if (MODE == kModeRowColI8) {
+      // int8: per row of tiles first the kTM products of the lower K half, then those of the upper
+#pragma unroll
+      for (int t = 0; t < kTN; ++t) {
+#pragma unroll
+        for (int j = 0; j < kTM; ++j) {
+          mfma_accumulate_i8_half(acc[t][j], wr[t % 3], xf[j], 0);
+          if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
+        }
+#pragma unroll
+        for (int j = 0; j < kTM; ++j) mfma_accumulate_i8_half(acc[t][j], wr[t % 3], xf[j], 1);
+      }
+    } else if (MODE != kModeBlock) {
       // row/column mode: the matrix pipe accumulates; scales and bias wait for the epilogue
 #pragma unroll
       for (int st = 0; st < kTN * kTM; ++st) {
@@ -1034,8 +1062,8 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     // n * magic >> 40 == n / d for every n with n * d < 2^40 (the tile numbers of whole problems are below `tiles`)
     a.group4_magic = (d > 0 && (uint64_t)tiles * d < (1ull << 40)) ? ((1ull << 40) + d - 1) / d : 0;
   }
-  static PerDeviceFlags lds_limit_raised[11] = {};
-  const void* const kernels[11] = {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false>),
+  static PerDeviceFlags lds_limit_raised[13] = {};
+  const void* const kernels[13] = {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, true>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true>),
@@ -1045,8 +1073,10 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false, false, true>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, true, false, true>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false, false, true>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, true>)};
-  for (int i = 0; i < 11; ++i) {
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, true>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowColI8, false>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowColI8, true>)};
+  for (int i = 0; i < 13; ++i) {
     const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised[i], kLdsBytes, kernels[i]);
     if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
   }
@@ -1093,6 +1123,8 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   void (*kern)(PpArgs);
   if (grouped != nullptr)
     kern = fp8_gemm_pingpong_kernel<false, kModeBlock, false, true>;
+  else if (mode == kModeRowColI8)
+    kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeRowColI8, true> : fp8_gemm_pingpong_kernel<false, kModeRowColI8, false>;
   else if (mode != kModeBlock)
     kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeRowCol, true> : fp8_gemm_pingpong_kernel<false, kModeRowCol, false>;
   else if (a.sk)

@@ -36,7 +36,8 @@ def _exact(a, b, sa, sb):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 256, 128), (16, 512, 512), (33, 1024, 1024), (100, 640, 4096), (256, 4096, 4096),
-                                   (512, 8192, 1024), (1100, 1300, 2048), (64, 200, 192), (7, 24, 40)])
+                                   (512, 8192, 1024), (1100, 1300, 2048), (64, 200, 192), (7, 24, 40), (1024, 2304, 512),
+                                   (129, 264, 128), (700, 8, 384)])
 @pytest.mark.parametrize("kinds", [("scalar", "scalar"), ("vector", "vector"), ("vector", "scalar")])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16])
 def test_int8_cutlass_scaled_mm(M, N, K, kinds, out_dtype):
@@ -78,6 +79,34 @@ def test_int8_sums_are_exact():
     assert want.abs().max() <= 2 ** 24  # exactly representable in fp32
     assert torch.equal(c.cpu().double(), want)
     assert c[0, 0].item() == 128 * 128 * K and c[1, 0].item() == -127 * 128 * K
+
+
+def test_int8_sums_are_exact_in_bf16_above_128_rows():
+    """bf16 output and M > 128 (the kernel that serves the large fp8 problems): sums that bf16 holds exactly come back
+    exactly, on tiles inside the matrix and on ragged ones, and so do the extremes of int8."""
+    g = torch.Generator().manual_seed(5)
+    one = torch.ones(1, device=DEV)
+    for (M, N, K) in ((512, 768, 256), (300, 520, 256), (257, 8, 128)):
+        a = torch.randint(-1, 2, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+        b = torch.randint(-1, 2, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+        c = torch.empty(M, -(-N // 16) * 16, dtype=torch.bfloat16, device=DEV)[:, :N]
+        flag_gems.cutlass_scaled_mm(c, a.to(DEV), b.to(DEV).t(), one, one, None)
+        want = a.double() @ b.double().t()
+        assert want.abs().max() <= 256
+        assert torch.equal(c.cpu().double(), want), (M, N, K)
+    M, N, K = 256, 256, 4096
+    a = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+    b = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+    a[0, :] = -128
+    a[1, :] = 127
+    b[0, :] = -128
+    b[1, :] = 64
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    flag_gems.cutlass_scaled_mm(c, a.to(DEV), b.to(DEV).t(), one, one, None)
+    assert c[0, 0].item() == 128 * 128 * K and c[1, 0].item() == -127 * 128 * K  # 2^26 and -127 * 2^19
+    assert c[0, 1].item() == -128 * 64 * K and c[1, 1].item() == 127 * 64 * K
+    want = (a.double() @ b.double().t()).float().to(torch.bfloat16)  # one rounding of the exact sum
+    assert torch.equal(c.cpu(), want)
 
 
 def test_int8_through_aten_scaled_mm():
