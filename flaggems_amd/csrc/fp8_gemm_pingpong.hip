@@ -41,6 +41,11 @@
 // Registers.  Two wavefronts per SIMD leave 256 registers each: 128 fp32 accumulators, the four activation
 // fragments of the K-block (32) and a ring of three weight fragments (24) that the multiply phase refills two
 // MFMA rows ahead of use.
+//
+// Short tiles (JN = 1, grouped problems with few rows per segment).  The same program on tiles of 64 rows: each
+// wavefront of a group takes one 16-row fragment, 32 accumulators.  The step is then set by how fast a compute unit
+// can stream its 32 KB of weights, not by MFMAs on rows that do not exist; the tiles of the last, partly filled
+// round of the grid are cut along K so that every compute unit streams to the end (finish_cut_tile).
 
 #include "fp8_gemm_common.h"
 
@@ -100,6 +105,13 @@ struct PpArgs {
   // writes (offs_token, token_mask, MUL_ROUTED_WEIGHT: src/flag_gems/fused/fused_moe.py:1484-1509).
   int c_rows;
   const float* row_weight;
+  // Short tiles of a grouped problem, the last round cut along K (cut_shift > 0): the first cut_full tiles, whole
+  // rounds of the grid, are work items of their own; each of the rest is 2^cut_shift work items of cut_steps
+  // K-blocks, item cut_full + r = tile cut_full + (r >> cut_shift), cut (r & mask), and the items of a tile add
+  // their sums through `partials` and `counters` (finish_cut_tile).  The host passes the largest shift the shape
+  // and the workspace allow in cut_shift; the kernel, which knows the real tile count, replaces it by the one it
+  // takes and sets cut_full and cut_steps.
+  int cut_shift, cut_steps, cut_full;
   uint64_t group4_magic;  // ceil(2^40 / (4 * tiles_n)) when that divides every tile number exactly, else 0 (see tile_of_sid)
 };
 
@@ -161,31 +173,47 @@ __device__ __forceinline__ int segment_end(const PpArgs& a, int e, int begin) {
   return end > begin ? end : begin;
 }
 
-template <bool GROUPED>
+// TILE_ROWS: activation rows per tile (kBM; less for the grouped kernel that serves short segments)
+// CUTS: the ids are work items of a grouped problem whose tiles are cut along K (PpArgs::cut_shift).
+template <bool GROUPED, int TILE_ROWS = kBM, bool CUTS = false>
 struct WalkT {
   int idx, kb, m0, n0;  // idx: virtual id (data-parallel rounds) or tile number (stream-K)
+  int kb_end;           // the walk leaves the tile (the work item) before this K-block
   int m_end, group;     // first row past the tile's segment (M when the problem is not grouped); its weight matrix
   int n_tiles, tiles_m; // of the whole problem (a grouped problem's are counted by the kernel)
+  __device__ __forceinline__ bool inside(const PpArgs& a) const {
+    return (CUTS && idx >= a.cut_full ? a.cut_full + ((idx - a.cut_full) >> a.cut_shift) : idx) < n_tiles;
+  }
   __device__ __forceinline__ void locate(const PpArgs& a) {
     int tm = 0, tn = 0;
-    if (idx < n_tiles) {
+    kb_end = a.g.KB;
+    if (CUTS) {
+      int tile = idx;
+      if (idx >= a.cut_full) {
+        const int r = idx - a.cut_full;
+        tile = a.cut_full + (r >> a.cut_shift);
+        kb = (r - ((r >> a.cut_shift) << a.cut_shift)) * a.cut_steps;
+        kb_end = kb + a.cut_steps;
+      }
+      if (tile < n_tiles) tile_of_index(tile, tiles_m, a.g.tiles_n, a.group4_magic, tm, tn);
+    } else if (idx < n_tiles) {
       if (a.sk && a.tile_base == 0) tile_of_sid(idx, tiles_m, a.g.tiles_n, a.group4_magic, tm, tn);
       else if (a.sk) tile_of_index(idx + a.tile_base, tiles_m, a.g.tiles_n, a.group4_magic, tm, tn);
       else tile_of_index(idx, tiles_m, a.g.tiles_n, a.group4_magic, tm, tn);
     }
-    m0 = tm * kBM; n0 = tn * kBN;
+    m0 = tm * TILE_ROWS; n0 = tn * kBN;
     m_end = a.g.M; group = 0;
     if (GROUPED) {
       // tile row tm of the whole problem -> segment and tile row inside it
       int begin = 0, t = tm, e = 0, end = 0;
       for (; e < a.n_groups; ++e) {
         end = segment_end(a, e, begin);
-        const int nt = (end - begin + kBM - 1) / kBM;
+        const int nt = (end - begin + TILE_ROWS - 1) / TILE_ROWS;
         if (t < nt) break;
         t -= nt;
         begin = end;
       }
-      m0 = begin + t * kBM; m_end = end; group = e < a.n_groups ? e : 0;
+      m0 = begin + t * TILE_ROWS; m_end = end; group = e < a.n_groups ? e : 0;
     }
   }
   __device__ __forceinline__ void start(const PpArgs& a, int first_idx, int first_kb, int n_tiles_, int tiles_m_) {
@@ -194,7 +222,7 @@ struct WalkT {
   }
   // true when the walk entered a new tile
   __device__ __forceinline__ bool next(const PpArgs& a) {
-    if (++kb < a.g.KB) return false;
+    if (++kb < kb_end) return false;
     kb = 0; idx += a.sk ? 1 : (int)gridDim.x;
     locate(a);
     return true;
@@ -244,10 +272,12 @@ struct LoadShare {
     ptr = wave >= 4 ? a.W + w_group_off + (int64_t)n0 * a.ldw : a.X + (int64_t)m0 * a.ldx;
   }
   // m_end: first row past the segment the tile belongs to (M when the problem is not grouped)
+  template <int TILE_ROWS = kBM>
   __device__ __forceinline__ void set_tile(const GemmArgs& a, int m0, int n0, int wave, int lane, int m_end, int64_t w_group_off = 0) {
     set_ptr(a, m0, n0, wave, w_group_off);
     const int valid = wave >= 4 ? a.N - n0 : m_end - m0;
-    set_offsets(a, valid < 256 ? valid : 256, wave, lane);
+    const int most = wave >= 4 ? kBN : TILE_ROWS;
+    set_offsets(a, valid < most ? valid : most, wave, lane);
   }
   // The load is written out instead of using the compiler's builtin: the compiler books a global->LDS
   // load as an access that may return through either counter, and from then on turns every wait for an LDS
@@ -384,8 +414,9 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 // ALIGNED: the tile lies inside the matrix; a wavefront then issues exactly kStoresPerTile store instructions.
 constexpr int kStoresPerTile = 16;
 // SCATTER (grouped problems): rows go where out_index says (see PpArgs::c_rows).
-template <int MODE, bool ALIGNED, bool SCATTER = false>
-__device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[kTN][kTM], int m_base, int n_base,
+// JN: activation fragments per wavefront (rows m_base .. m_base + 16 JN).
+template <int MODE, bool ALIGNED, bool SCATTER = false, int JN = kTM>
+__device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[kTN][JN], int m_base, int n_base,
                                            int l16, int lg, int m_end, const int* out_index = nullptr, int c_rows = 0,
                                            const float* row_weight = nullptr) {
   if (MODE != kModeBlock) {
@@ -402,7 +433,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
         bias[e] = a.bias ? load_as_float(a.bias, ne, a.bias_dtype) : 0.f;
       }
 #pragma unroll
-      for (int j = 0; j < kTM; ++j) {
+      for (int j = 0; j < JN; ++j) {
         const int m = m_base + j * 16 + l16;
         if (!ALIGNED && m >= m_end) continue;
         const float sa = a.xs[a.xs_per_row ? m : 0];
@@ -435,7 +466,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
     return;
   }
 #pragma unroll
-  for (int j = 0; j < kTM; ++j) {
+  for (int j = 0; j < JN; ++j) {
     const int m = m_base + j * 16 + l16;
     if (!ALIGNED && m >= m_end) continue;
     int64_t out_row = m;
@@ -565,23 +596,86 @@ __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the counted waits of the main loop start from zero
 }
 
+// Finishes a short tile of a grouped problem that is cut along K (PpArgs::cut_shift): the same protocol as
+// finish_partial_tile -- publish, count in, the last of the tile's work items to arrive adds all partial sums in cut
+// order and stores -- on the wavefront's 16 JN x 128 piece, which is small enough to be summed whole and handed to
+// store_tile, so gathered, scattered and weighted results take the one store path.  A slot per (work item, wavefront).
+template <bool SCATTER, int JN>
+__device__ __forceinline__ void finish_cut_tile(const PpArgs& a, const v4f (&acc)[kTN][JN], int item, int m_base, int n_base,
+                                                int m_end, int wave, int lane, int l16, int lg) {
+  constexpr int kFloats = kTN * JN * 256;  // per wavefront
+  // item, tile: counted from the first cut one
+  const int tile = item >> a.cut_shift, cuts = 1 << a.cut_shift;
+  const uint32_t lane_off = (uint32_t)lane * 16u;
+  float* const mine = uniform_ptr(a.partials + ((size_t)item * 8 + wave) * kFloats);
+#pragma unroll
+  for (int t = 0; t < kTN; ++t)
+#pragma unroll
+    for (int j = 0; j < JN; ++j) store_x4_agent(mine + (t * JN + j) * 256, lane_off, acc[t][j]);
+  wait_vmem<0>();
+  unsigned int* const cnt = a.counters + tile * 8 + wave;
+  unsigned int prev = 0;
+  if (lane == 0) prev = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  prev = (unsigned int)__builtin_amdgcn_readfirstlane((int)prev);
+  if (prev != (unsigned int)(cuts - 1)) return;
+  v4f r[kTN][JN];
+  for (int q = 0; q < cuts; ++q) {
+    const float* const src = uniform_ptr(a.partials + ((size_t)((tile << a.cut_shift) + q) * 8 + wave) * kFloats);
+    v4f tmp[kTN][JN];
+#pragma unroll
+    for (int t = 0; t < kTN; ++t)
+#pragma unroll
+      for (int j = 0; j < JN; ++j) load_x4_agent(tmp[t][j], src + (t * JN + j) * 256, lane_off);
+#pragma unroll
+    for (int t = 0; t < kTN; ++t)
+#pragma unroll
+      for (int j = 0; j < JN; ++j)  // the values are operands of the wait, so no use can move above it
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[t][j]) : : "memory");
+#pragma unroll
+    for (int t = 0; t < kTN; ++t)
+#pragma unroll
+      for (int j = 0; j < JN; ++j) {
+        if (q == 0) r[t][j] = tmp[t][j]; else r[t][j] += tmp[t][j];  // (no "0 + x" in the sum)
+      }
+  }
+  store_tile<kModeBlock, false, SCATTER, JN>(a.g, r, m_base, n_base, l16, lg, m_end, SCATTER && a.c_rows > 0 ? a.row_index : nullptr,
+                                             a.c_rows, a.row_weight);
+  if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the counted waits of the main loop start from zero
+}
+
 // ALIGNED: M and N are multiples of the tile; no tile has an edge, and the per-lane offsets of the tile loads
 // and of the scale loads never change (a tile change then touches scalar registers only).
 // GROUPED: the rows are segments with a weight matrix each (see PpArgs::groups).
 // POW2: block scales that are powers of two, applied by the instruction (mfma_scaled_accumulate).
-template <bool SK, int MODE, bool ALIGNED, bool GROUPED = false, bool POW2 = false>
+// JN: activation fragments (16 rows) per wavefront; the tile has 64 JN rows.  Less than kTM only for grouped problems
+// whose segments are short: a 256-row tile costs its 256 rows of MFMAs however few of them belong to the segment, and
+// that, not the weight stream, sets the time of a step when a tile holds a few dozen rows.  With JN = 1 the four
+// wavefronts of a group take 16 rows each, the activation image in LDS keeps its 256-row layout (the rows past the
+// 64th are loaded like rows past an edge and never read), and everything else runs unchanged.
+template <bool SK, int MODE, bool ALIGNED, bool GROUPED = false, bool POW2 = false, int JN = kTM>
 __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
+  static_assert(JN == kTM || (GROUPED && JN >= 1 && JN < kTM), "short tiles: grouped problems only");
+  constexpr int kTileRows = 64 * JN;
+  constexpr bool kCuts = GROUPED && JN < kTM;  // tiles may be cut along K (cut_shift = 0: they are not)
+  // Short tiles stream weights for next to no arithmetic, and what sets their pace is how many weight bytes a compute
+  // unit has in flight: the activation stages shrink to the tile's rows and the LDS they leave holds a fourth weight
+  // stage, so that group B loads three steps ahead instead of two.
+  constexpr int kWSt = JN < kTM ? kWStages + 1 : kWStages;
+  constexpr int kXStBytes = JN < kTM ? kTileRows * 128 : kXStageBytes;
+  constexpr int kXReg = kWSt * kWStageBytes;
+  static_assert(kXReg + kXStages * kXStBytes <= kLdsBytes, "LDS");
   static_assert(!POW2 || (MODE == kModeBlock && !GROUPED), "power-of-two scales: plain block-scaled problems");
   static_assert(!GROUPED || (!SK && !ALIGNED && MODE == kModeBlock), "grouped problems: whole tiles with edges, block scales");
-  using Walk = WalkT<GROUPED>;
+  using Walk = WalkT<GROUPED, kTileRows, kCuts>;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const GemmArgs& g = a.g;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = wave >> 2;       // 0: group A, 1: group B
-  const int wave_m = wave & 3;     // 64-row quarter of the activation tile
-  const int wm0 = wave_m * 64, wn0 = grp * 128;
+  const int wave_m = wave & 3;     // quarter of the activation tile (64 rows of 256)
+  const int wm0 = wave_m * 16 * JN, wn0 = grp * 128;
   const int l16 = lane & 15, lg = lane >> 4;
   const int frag_off = fragment_offset(lane);
 
@@ -590,10 +684,24 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     tiles_m = 0;
     for (int e = 0, begin = 0; e < a.n_groups; ++e) {
       const int end = segment_end(a, e, begin);
-      tiles_m += (end - begin + kBM - 1) / kBM;
+      tiles_m += (end - begin + kTileRows - 1) / kTileRows;
       begin = end;
     }
     n_tiles = tiles_m * g.tiles_n;
+    if (kCuts) {
+      // The tiles past the last whole round of the grid: rounds of work items, each as long as its K-blocks plus
+      // about 8 for the start of a tile and the exchange (uniform: every block arrives at the same shift).
+      const int grid = (int)gridDim.x;
+      const int full = n_tiles / grid * grid, rest = n_tiles - full;
+      int best = 0, best_cost = g.KB;
+      for (int sh = 1; sh <= a.cut_shift; ++sh) {
+        const int cost = ((rest << sh) + grid - 1) / grid * ((g.KB >> sh) + 8);
+        if (cost < best_cost) { best_cost = cost; best = sh; }
+      }
+      a.cut_shift = best;
+      a.cut_steps = g.KB >> best;
+      a.cut_full = best != 0 ? full : n_tiles;
+    }
   }
   // steps of this block: whole tiles blockIdx.x, blockIdx.x + gridDim.x, ... or one contiguous range
   int pos = (int)blockIdx.x, first_idx = (int)blockIdx.x, first_kb = 0, total;
@@ -614,8 +722,14 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     first_kb = s0 - first_idx * g.KB;
   } else {
     // (a grouped launch sizes its grid for an upper bound of the tile count: the blocks past the real one leave)
-    const int my_tiles = (n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-    total = my_tiles > 0 ? my_tiles * g.KB : 0;
+    if (kCuts && a.cut_shift != 0) {
+      const int cut_items = (n_tiles - a.cut_full) << a.cut_shift;
+      const int mine = (cut_items - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+      total = a.cut_full / (int)gridDim.x * g.KB + (mine > 0 ? mine * a.cut_steps : 0);
+    } else {
+      const int my_tiles = (n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+      total = my_tiles > 0 ? my_tiles * g.KB : 0;
+    }
   }
   if (total <= 0) return;  // uniform over the block
   for (int i = (int)(blockIdx.x & 15) * a.stagger; i > 0; --i) __builtin_amdgcn_s_sleep(15);
@@ -627,27 +741,31 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   auto set_load_tile = [&]() __attribute__((always_inline)) {
     if (GROUPED && a.row_index != nullptr && wave < 4) {
       const int valid = lw.m_end - lw.m0;
-      share.set_gathered(g, a.row_index, a.index_div, a.x_rows, lw.m0, valid < 256 ? valid : 256, lane, wave);
+      share.set_gathered(g, a.row_index, a.index_div, a.x_rows, lw.m0, valid < kTileRows ? valid : kTileRows, lane, wave);
     } else {
-      share.set_tile(g, lw.m0, lw.n0, wave, lane, lw.m_end, GROUPED ? (int64_t)lw.group * a.w_group_stride : 0);
+      share.template set_tile<kTileRows>(g, lw.m0, lw.n0, wave, lane, lw.m_end, GROUPED ? (int64_t)lw.group * a.w_group_stride : 0);
     }
   };
   set_load_tile();
-  share.ptr += (int64_t)first_kb * 128;
+  share.ptr += (int64_t)(kCuts ? lw.kb : first_kb) * 128;
   int loaded = 0, w_slot = 0, x_slot = 0;  // stages issued by this wavefront; LDS slots of the next stage
+  // (short tiles: the activation rows past the tile's 64 JN are never read, and group A leaves their loads out)
+  constexpr int kXLoadsPerWave = JN < kTM ? 2 * JN : kSlabsPerWave;
   auto issue_stage_part = [&](int q) __attribute__((always_inline)) {
+    if (JN < kTM && grp == 0 && q >= kXLoadsPerWave) return;
     const uint32_t region = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
-    const uint32_t stage = grp ? (uint32_t)(w_slot * kWStageBytes) : (uint32_t)(kXRegion + x_slot * kXStageBytes);
+    const uint32_t stage = grp ? (uint32_t)(w_slot * kWStageBytes) : (uint32_t)(kXReg + x_slot * kXStBytes);
     share.issue_one(region + stage + (uint32_t)(wave & 3) * 1024u, q);
   };
   auto finish_stage = [&]() __attribute__((always_inline)) {
     ++loaded;
-    w_slot = (w_slot + 1 == kWStages) ? 0 : w_slot + 1;
+    w_slot = (w_slot + 1 == kWSt) ? 0 : w_slot + 1;
     x_slot ^= 1;
     if (__builtin_expect(lw.next(a), 0)) {
-      if (lw.idx < n_tiles) {
+      if (lw.inside(a)) {
         if (ALIGNED) share.set_ptr(g, lw.m0, lw.n0, wave);
         else set_load_tile();
+        if (kCuts) share.ptr += (int64_t)lw.kb * 128;
       }
     } else {
       share.ptr += 128;
@@ -683,11 +801,12 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   auto set_scale_tile = [&]() __attribute__((always_inline)) {
     if (!ALIGNED) set_scale_offsets();
     xs_ptr = gathered ? g.xs : g.xs + (int64_t)sw.m0 * g.xs_rs;
+    if (kCuts) xs_ptr += (int64_t)sw.kb * g.xs_cs;
   };
   if (MODE == kModeBlock) {
     set_scale_offsets();
     set_scale_tile();
-    xs_ptr += (int64_t)first_kb * g.xs_cs;
+    if (!kCuts) xs_ptr += (int64_t)first_kb * g.xs_cs;
   }
   auto advance_scales = [&]() __attribute__((always_inline)) {
     if (__builtin_expect(sw.next(a), 0)) set_scale_tile(); else xs_ptr += g.xs_cs;
@@ -707,13 +826,14 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   auto ws_row = [&]() __attribute__((always_inline)) -> const float* {
     int nb = (cw.n0 + wn0) >> 7;
     nb = nb < nb_last ? nb : nb_last;
-    return g.ws + (GROUPED ? (int64_t)cw.group * a.ws_group_stride : 0) + (int64_t)nb * g.ws_rs;
+    return g.ws + (GROUPED ? (int64_t)cw.group * a.ws_group_stride : 0) + (int64_t)nb * g.ws_rs + (kCuts ? (int64_t)cw.kb * g.ws_cs : 0);
   };
-  const float* ws_ptr = MODE == kModeBlock ? ws_row() + (int64_t)first_kb * g.ws_cs : nullptr;
+  const float* ws_ptr = MODE == kModeBlock ? ws_row() + (kCuts ? 0 : (int64_t)first_kb * g.ws_cs) : nullptr;
 
   // ---- prologue: A has stage 0 in flight, B stages 0 and 1; scales of step 0
   issue_stage_all();
   if (grp == 1 && total > 1) issue_stage_all();
+  if (kWSt > kWStages && grp == 1 && total > 2) issue_stage_all();
   request_scales();
   if (MODE == kModeBlock && total > 1) advance_scales();  // fetch(T) asks for the scales of step T+1
   wait_vmem_all();
@@ -721,11 +841,11 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   if (grp == 1) __builtin_amdgcn_s_barrier();  // B runs one slot behind A
   __builtin_amdgcn_s_setprio(kFetchPrio);
 
-  v4f acc[kTN][kTM];
+  v4f acc[kTN][JN];
 #pragma unroll
   for (int t = 0; t < kTN; ++t)
 #pragma unroll
-    for (int j = 0; j < kTM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < JN; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
   // A finished tile is stored at the end of its wavefront's next fetch slot, under the partner's MFMAs.
   // A tile of which this block computed only some K-blocks (stream-K) goes through finish_partial_tile at
@@ -738,17 +858,25 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
 #pragma unroll
     for (int t = 0; t < kTN; ++t)
 #pragma unroll
-      for (int j = 0; j < kTM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < JN; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
     pending = false;
   };
   auto flush_whole_tile = [&]() __attribute__((always_inline)) {
-    store_tile<MODE, ALIGNED, GROUPED>(g, acc, pend_m, pend_n, l16, lg, pend_m_end, GROUPED && a.c_rows > 0 ? a.row_index : nullptr,
+    if constexpr (kCuts) {
+      if (pend_idx >= a.cut_full) {
+        wait_vmem<0>();
+        finish_cut_tile<GROUPED, JN>(a, acc, pend_idx - a.cut_full, pend_m, pend_n, pend_m_end, wave, lane, l16, lg);
+        clear_acc();
+        return;
+      }
+    }
+    store_tile<MODE, ALIGNED, GROUPED, JN>(g, acc, pend_m, pend_n, l16, lg, pend_m_end, GROUPED && a.c_rows > 0 ? a.row_index : nullptr,
                                        a.c_rows, a.row_weight);
     clear_acc();
   };
   auto flush_partial_tile = [&]() __attribute__((always_inline)) {
     wait_vmem<0>();
-    finish_partial_tile(a, acc, pend_idx, pos, pend_m, pend_n, wave, lane, l16, lg);
+    if constexpr (SK) finish_partial_tile(a, acc, pend_idx, pos, pend_m, pend_n, wave, lane, l16, lg);
     clear_acc();
   };
 
@@ -772,12 +900,13 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     float ws = 1.f;
     if (MODE == kModeBlock) {
       if (kRelaxedStoreWaits && flushed_prev) wait_and_take<8 + kStoresPerTile>(xs, xs_nxt);
+      else if (JN < kTM && grp == 0) wait_and_take<kXLoadsPerWave>(xs, xs_nxt);
       else wait_and_take<8>(xs, xs_nxt);
       if (more) request_scales();  // of step T+1; the pointer was moved there a step ago
       ws = *(const __attribute__((address_space(4))) float*)ws_ptr;
     }
     const uint8_t* const tw = lds + rw_slot * kWStageBytes + (wn0 >> 4) * 2048;
-    const uint8_t* const tx = lds + kXRegion + rx_slot * kXStageBytes + (wm0 >> 4) * 2048;
+    const uint8_t* const tx = lds + kXReg + rx_slot * kXStBytes + (wm0 >> 4) * 2048;
     // All activation fragments and the first two weight fragments (the other six follow during the multiply,
     // each two MFMA rows before its use), interleaved with this wavefront's eight tile loads: the address
     // unit takes ~45 cycles per 1 KB load and the LDS ~25 per fragment half, and a wavefront that issues
@@ -786,15 +915,15 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     //   B the weights of stage T+2 into the slot that multiply(T-1) left a slot ago.
     // Past the last stage the loads are repeated from the last address into a slot nobody reads any more:
     // cheaper than a branch per load, and the wait counts below stay the same on every step.
-    v8i xf[kTM], wr[3];
+    v8i xf[JN], wr[3];
     issue_stage_part(0);
     xf[0] = read_frag(tx, 0, frag_off);
     issue_stage_part(1);
-    xf[1] = read_frag(tx, 1, frag_off);
+    if (JN > 1) xf[1 % JN] = read_frag(tx, 1, frag_off);
     issue_stage_part(2);
-    xf[2] = read_frag(tx, 2, frag_off);
+    if (JN > 2) xf[2 % JN] = read_frag(tx, 2, frag_off);
     issue_stage_part(3);
-    xf[3] = read_frag(tx, 3, frag_off);
+    if (JN > 3) xf[3 % JN] = read_frag(tx, 3, frag_off);
     issue_stage_part(4);
     wr[0] = read_frag(tw, 0, frag_off);
     issue_stage_part(5);
@@ -812,6 +941,9 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     if (grp == 1) {
       if (kRelaxedStoreWaits && flushed_prev) {
         if (more) wait_vmem<12 + kStoresPerTile>(); else wait_vmem<8 + kStoresPerTile>();
+      } else if (kWSt > kWStages) {
+        // (one more stage is younger; the in-order wait for the scales at the start of the slot has covered stage T+1)
+        if (more && MODE == kModeBlock) wait_vmem<20>(); else wait_vmem<16>();
       } else {
         if (more && MODE == kModeBlock) wait_vmem<12>(); else wait_vmem<8>();
       }
@@ -820,10 +952,10 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
       if (POW2) {
         swe = e8m0_of(ws);
 #pragma unroll
-        for (int j = 0; j < kTM; ++j) se[j] = e8m0_of(xs[j]);
+        for (int j = 0; j < JN; ++j) se[j] = e8m0_of(xs[j]);
       } else {
 #pragma unroll
-        for (int j = 0; j < kTM; ++j) sc[j] = xs[j] * ws;
+        for (int j = 0; j < JN; ++j) sc[j] = xs[j] * ws;
       }
     }
     const bool flushed_now = pending;
@@ -833,46 +965,46 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     // ================= multiply(T)
     __builtin_amdgcn_s_setprio(kMultiplyPrio);
     if (MODE == kModeRowColI8) {
-      // int8: per row of tiles first the kTM products of the lower K half, then those of the upper
+      // int8: per row of tiles first the JN products of the lower K half, then those of the upper
 #pragma unroll
       for (int t = 0; t < kTN; ++t) {
 #pragma unroll
-        for (int j = 0; j < kTM; ++j) {
+        for (int j = 0; j < JN; ++j) {
           mfma_accumulate_i8_half(acc[t][j], wr[t % 3], xf[j], 0);
           if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
         }
 #pragma unroll
-        for (int j = 0; j < kTM; ++j) mfma_accumulate_i8_half(acc[t][j], wr[t % 3], xf[j], 1);
+        for (int j = 0; j < JN; ++j) mfma_accumulate_i8_half(acc[t][j], wr[t % 3], xf[j], 1);
       }
     } else if (MODE != kModeBlock) {
       // row/column mode: the matrix pipe accumulates; scales and bias wait for the epilogue
 #pragma unroll
-      for (int st = 0; st < kTN * kTM; ++st) {
-        const int t = st / kTM, j = st % kTM;
+      for (int st = 0; st < kTN * JN; ++st) {
+        const int t = st / JN, j = st % JN;
         mfma_accumulate(acc[t][j], wr[t % 3], xf[j]);
         if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
       }
     } else if (POW2) {
 #pragma unroll
-      for (int st = 0; st < kTN * kTM; ++st) {
-        const int t = st / kTM, j = st % kTM;
+      for (int st = 0; st < kTN * JN; ++st) {
+        const int t = st / JN, j = st % JN;
         mfma_scaled_accumulate(acc[t][j], wr[t % 3], xf[j], swe, se[j]);
         if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
       }
     } else {
       v4f p[3];
 #pragma unroll
-      for (int st = 0; st < kTN * kTM; ++st) {
-        const int t = st / kTM, j = st % kTM;
+      for (int st = 0; st < kTN * JN; ++st) {
+        const int t = st / JN, j = st % JN;
         p[st % 3] = mfma_partial(wr[t % 3], xf[j]);
         // refill the ring after the row's first MFMA: the wait the compiler puts before that MFMA then
         // covers only reads issued a whole row earlier
         if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
-        if (st >= 2) scale_into<0>(acc[(st - 2) / kTM][(st - 2) % kTM], p[(st - 2) % 3], sc[(st - 2) % kTM]);
+        if (st >= 2) scale_into<0>(acc[(st - 2) / JN][(st - 2) % JN], p[(st - 2) % 3], sc[(st - 2) % JN]);
       }
-      constexpr int L = kTN * kTM;
-      scale_into<0>(acc[(L - 2) / kTM][(L - 2) % kTM], p[(L - 2) % 3], sc[(L - 2) % kTM]);
-      scale_into<4>(acc[(L - 1) / kTM][(L - 1) % kTM], p[(L - 1) % 3], sc[(L - 1) % kTM]);
+      constexpr int L = kTN * JN;
+      scale_into<0>(acc[(L - 2) / JN][(L - 2) % JN], p[(L - 2) % 3], sc[(L - 2) % JN]);
+      scale_into<4>(acc[(L - 1) / JN][(L - 1) % JN], p[(L - 1) % 3], sc[(L - 1) % JN]);
     }
     __builtin_amdgcn_s_setprio(kFetchPrio);
     if (grp == 0) {  // A's share of stage T+1 has landed
@@ -882,7 +1014,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     __builtin_amdgcn_s_barrier();
 
     // ================= next step; a finished tile is stored in this wavefront's next fetch slot
-    rw_slot = (rw_slot + 1 == kWStages) ? 0 : rw_slot + 1;
+    rw_slot = (rw_slot + 1 == kWSt) ? 0 : rw_slot + 1;
     rx_slot ^= 1;
     pend_m = cw.m0 + wm0; pend_n = cw.n0 + wn0; pend_idx = cw.idx; pend_m_end = cw.m_end;
     pending = __builtin_expect(cw.next(a), 0);
@@ -1039,14 +1171,33 @@ bool transposition_pays(int64_t tiles, int64_t KB, int cus) {
 }
 size_t transposed_scales_bytes(int64_t M, int64_t KB) { return (size_t)((M * KB * 4 + 255) / 256 * 256); }
 
+// Short tiles of grouped problems (the JN = 1 instantiation) and their cuts along K.
+constexpr int kShortTileRows = 64;
+constexpr size_t kCutSlotBytes = (size_t)8 * kTN * 256 * 4;  // a work item's partial sums: 8 wavefronts x 16 x 128 floats
+constexpr int kMaxCutItems = 1024;                           // work items of a cut problem (64 MB of partial sums)
+// Largest number of cuts per tile of the last round, as a shift (the kernel picks among 0..this from the real tile
+// count): whole K-blocks, at least 8 per cut, and slots for a round short of one tile.
+int max_cut_shift(int grid, int KB) {
+  int sh = 0;
+  while (sh < 2 && KB % (2 << sh) == 0 && (KB >> (sh + 1)) >= 8 && ((int64_t)(grid - 1) << (sh + 1)) <= kMaxCutItems) ++sh;
+  return sh;
+}
+
 int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream,
                  const GroupedGemm* grouped = nullptr) {
   PpArgs a = {};
   a.g = g;
   a.g.tiles_m = (int)ceil_div(g.M, kBM);
+  // Grouped problems whose segments average at most a short tile's rows take 64-row tiles (the JN = 1
+  // instantiation); the host sees only the total, and a segment longer than a tile then reads its weights once per
+  // 64 rows.  Measured on 8 segments, [28672, 4096] | [4096, 14336] weights each, 256-row -> 64-row tiles:
+  // 16 rows a segment on average 292 -> 202 | 200 -> 114 us, 32: 292 -> 214 | 206 -> 171, 64: 296 -> 291 | 221 -> 177,
+  // 128: 300 -> 415 | 204 -> 216.
+  const bool short_tiles = grouped != nullptr && g.M <= (int64_t)kShortTileRows * grouped->n_groups;
   if (grouped != nullptr) {
     // every segment ends with at most one tile that is not full; the kernel counts the real tiles
-    const int64_t bound = g.M / kBM + grouped->n_groups;
+    const int tile_rows = short_tiles ? kShortTileRows : kBM;
+    const int64_t bound = g.M / tile_rows + grouped->n_groups;
     a.g.tiles_m = (int)(bound < g.M ? bound : g.M);
     a.groups = grouped->ends; a.n_groups = (int)grouped->n_groups;
     a.w_group_stride = grouped->w_group_stride; a.ws_group_stride = grouped->ws_group_stride;
@@ -1062,8 +1213,8 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     // n * magic >> 40 == n / d for every n with n * d < 2^40 (the tile numbers of whole problems are below `tiles`)
     a.group4_magic = (d > 0 && (uint64_t)tiles * d < (1ull << 40)) ? ((1ull << 40) + d - 1) / d : 0;
   }
-  static PerDeviceFlags lds_limit_raised[13] = {};
-  const void* const kernels[13] = {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false>),
+  static PerDeviceFlags lds_limit_raised[14] = {};
+  const void* const kernels[14] = {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, true>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true>),
@@ -1075,8 +1226,9 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false, false, true>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, true>),
                                   reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowColI8, false>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowColI8, true>)};
-  for (int i = 0; i < 13; ++i) {
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowColI8, true>),
+                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, 1>)};
+  for (int i = 0; i < 14; ++i) {
     const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised[i], kLdsBytes, kernels[i]);
     if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
   }
@@ -1087,7 +1239,21 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   if (grouped != nullptr) sk.use = false;  // ranges of steps would need the tile count on the host
   TailPlan tp = plan_tail(tiles, g.KB, cus);
   if (sk.use || grouped != nullptr || mode != kModeBlock) tp.use = false;
-  const size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : (tp.use ? (size_t)tp.grid * 2 * kPartialSlotBytes : 0);
+  size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : (tp.use ? (size_t)tp.grid * 2 * kPartialSlotBytes : 0);
+  a.cut_steps = g.KB;
+  if (short_tiles) {
+    // (the grid is the compute units, also where the bound of the tile count is lower: cuts may fill them)
+    const int sh = max_cut_shift(cus, g.KB);
+    const size_t bytes = (size_t)kMaxCutItems * kCutSlotBytes;
+    if (sh > 0 && workspace != nullptr && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= FG_WORKSPACE_COUNTER_BYTES + bytes &&
+        (size_t)cus * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES) {
+      a.cut_shift = sh;
+      a.counters = reinterpret_cast<unsigned int*>(workspace);
+      a.partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
+      sk_bytes = bytes;
+      grid = (tiles << sh) < cus ? (int)(tiles << sh) : cus;
+    }
+  }
   const size_t need = FG_WORKSPACE_COUNTER_BYTES + sk_bytes;
   // rows of the activation-scale matrix: the rows of X, which a gathered problem reads through its index
   const int64_t scale_rows = (grouped != nullptr && grouped->row_index != nullptr) ? grouped->x_rows : (int64_t)g.M;
@@ -1122,7 +1288,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   const bool aligned = g.M % kBM == 0 && g.N % kBN == 0;
   void (*kern)(PpArgs);
   if (grouped != nullptr)
-    kern = fp8_gemm_pingpong_kernel<false, kModeBlock, false, true>;
+    kern = short_tiles ? fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, 1> : fp8_gemm_pingpong_kernel<false, kModeBlock, false, true>;
   else if (mode == kModeRowColI8)
     kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeRowColI8, true> : fp8_gemm_pingpong_kernel<false, kModeRowColI8, false>;
   else if (mode != kModeBlock)
@@ -1202,7 +1368,8 @@ size_t pingpong_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 
 size_t grouped_workspace_bytes(int64_t M, int64_t K) {
   if (M <= 0 || K <= 0 || K % 128 != 0) return 0;
-  return FG_WORKSPACE_COUNTER_BYTES + transposed_scales_bytes(M, K / 128);
+  // (the partial sums of cut short tiles: the number of segments is not known here, the bound of the plan is)
+  return FG_WORKSPACE_COUNTER_BYTES + (size_t)kMaxCutItems * kCutSlotBytes + transposed_scales_bytes(M, K / 128);
 }
 
 int launch_grouped(const GemmArgs& g, const GroupedGemm& grouped, void* workspace, size_t workspace_bytes, hipStream_t stream) {

@@ -52,6 +52,11 @@ CASES = [
     (3000, 6144, 256, [1000, 1900, 3000]),             # more tiles than compute units: blocks walk several
     (700, 384, 2048, [0, 0, 0, 0, 0, 0, 0, 700]),      # all rows in the last group
     (513, 256, 128, [256, 512, 513]),                  # segments that end on tile boundaries, one K-block
+    # few rows per segment (64-row tiles), few tiles, deep K: the tiles are cut along K
+    (128, 512, 4096, None),
+    (96, 264, 2048, [0, 1, 1, 40, 40, 41, 90, 96]),    # N ends inside a tile; empty and one-row segments
+    (300, 256, 3072, [0, 200, 200, 230, 299, 300, 300, 300]),  # a segment of several short tiles
+    (16, 1024, 7168, None),                            # more segments than rows have tokens
 ]
 
 
