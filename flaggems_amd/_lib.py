@@ -104,8 +104,9 @@ SIGNATURES = {
     "fg_scaled_int8_gemm": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
-         c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p],
+         c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p],
     ),
+    "fg_scaled_int8_gemm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "fg_scaled_fp8_gemm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "fg_batched_block_fp8_gemm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
 }

@@ -57,7 +57,8 @@ inline void launch(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds_byt
 // the device's copy of the kernel).  `done` is one flag array per kernel set; a race sets the attribute twice.
 constexpr int kMaxDevices = 64;
 struct PerDeviceFlags { bool done[kMaxDevices]; };
-inline hipError_t raise_dynamic_lds_limit(PerDeviceFlags& flags, int bytes, const void* k0, const void* k1 = nullptr) {
+inline hipError_t raise_dynamic_lds_limit(PerDeviceFlags& flags, int bytes, const void* k0, const void* k1 = nullptr,
+                                          const void* k2 = nullptr) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
@@ -65,6 +66,7 @@ inline hipError_t raise_dynamic_lds_limit(PerDeviceFlags& flags, int bytes, cons
   if (tracked && flags.done[dev]) return hipSuccess;
   e = hipFuncSetAttribute(k0, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
   if (e == hipSuccess && k1) e = hipFuncSetAttribute(k1, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && k2) e = hipFuncSetAttribute(k2, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
   if (e == hipSuccess && tracked) flags.done[dev] = true;
   return e;
 }

@@ -212,7 +212,7 @@ struct TileCfg {
 template <int BM, int BN, int WM, int WN, int MODE, bool DIRECT, bool SPLIT = false, int NST = 2>
 __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
   using Cfg = TileCfg<BM, BN, WM, WN, NST>;
-  static_assert(NST == 2 || (DIRECT && MODE != kModeRowColI8 && NST >= 3 && NST <= 5), "deep pipeline: direct fp8 loads, 3..5 stages");
+  static_assert(NST == 2 || (DIRECT && NST >= 3 && NST <= 5), "deep pipeline: direct loads, 3..5 stages");
   if (!SPLIT && a.batch > 1) {  // uniform: this workgroup's entry of the batch
     const int64_t z = blockIdx.y;
     a.X += z * a.x_batch_bytes;
@@ -380,7 +380,7 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
           if (i + 1 < TN) wf_next = read_fragment(tw, i + 1, frag_off);
 #pragma unroll
           for (int j = 0; j < TM; ++j) {
-            acc[i][j] = mfma_fp8_16x16x128(wf, xf[j], acc[i][j]);
+            acc[i][j] = MODE == kModeRowColI8 ? mfma_i8_16x16x128(wf, xf[j], acc[i][j]) : mfma_fp8_16x16x128(wf, xf[j], acc[i][j]);
             const int t = i * TM + j;
             if (t % kLoadEvery == 0 && t / kLoadEvery < kLoadsW + kLoadsX && more) issue_tile_part(kb_load, load_slot, t / kLoadEvery);
           }
@@ -547,8 +547,10 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
       for (int i = 0; i < TN; ++i)
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
-          // plain assignment for the first split keeps "0 + x" out of the sum
-          if (s == 0) acc[i][j] = tmp[i][j]; else acc[i][j] += tmp[i][j];
+          // plain assignment for the first split keeps "0 + x" out of the sum; int8 operands: int32 sums, added as such
+          if (s == 0) acc[i][j] = tmp[i][j];
+          else if (MODE == kModeRowColI8) acc[i][j] = __builtin_bit_cast(v4f, __builtin_bit_cast(v4i, acc[i][j]) + __builtin_bit_cast(v4i, tmp[i][j]));
+          else acc[i][j] += tmp[i][j];
         }
     }
     if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -790,7 +792,7 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
     if (mid_takes && (mid.splits == 1 || (workspace != nullptr && workspace_bytes >= mid.workspace_bytes &&
                                           (uintptr_t)workspace % 16 == 0)))
       return launch_mid_m(a, MODE, mid, workspace, workspace_bytes, stream);
-    if (MODE != kModeRowColI8) {
+    {
       const PipePlan pp = plan_pipe(a.M, a.N, a.K, MODE == kModeBlock ? a.xs_rs : 0);
       const bool ws_ok = pp.splits == 1 || (workspace != nullptr && workspace_bytes >= pp.workspace_bytes && (uintptr_t)workspace % 16 == 0);
       if (pp.use && ws_ok && !mid_takes) return launch_pipe<MODE>(a, pp, workspace, stream);
@@ -1146,12 +1148,17 @@ extern "C" int fg_scaled_fp8_gemm(const void* A, int64_t lda, const void* B, int
   return launch_gemm<kModeRowCol>(a, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
+extern "C" size_t fg_scaled_int8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  return fg_block_fp8_gemm_workspace_bytes(M, N, K);
+}
+
 extern "C" int fg_scaled_int8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
                                    const float* a_scale, int a_scale_per_row,
                                    const float* b_scale, int b_scale_per_col,
                                    const void* bias, int bias_dtype,
                                    void* C, int64_t ldc, int c_dtype,
-                                   int64_t M, int64_t N, int64_t K, void* stream) {
+                                   int64_t M, int64_t N, int64_t K,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
   using namespace fg;
   if (c_dtype != FG_BF16 && c_dtype != FG_F16 && c_dtype != FG_F32)
     FG_FAIL(FG_ERR_INVALID_ARG, "fg_scaled_int8_gemm: c_dtype %d", c_dtype);
@@ -1168,12 +1175,7 @@ extern "C" int fg_scaled_int8_gemm(const void* A, int64_t lda, const void* B, in
   a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)ceil_div(K, 128);
   a.c_dtype = c_dtype; a.bias_dtype = bias_dtype;
   a.xs_per_row = a_scale_per_row; a.ws_per_col = b_scale_per_col;
-  const bool direct = (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) && (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
-                      ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
-  hipStream_t st = (hipStream_t)stream;
-  // bf16 results with M > 128: the persistent kernel, as for fp8 operands with row and column scales
-  if (direct && M > 128 && pingpong_takes(a, kModeRowColI8, nullptr, 0)) return launch_pingpong(a, kModeRowColI8, nullptr, 0, st);
-  if (M > 128)
-    return direct ? launch_cfg<256, 256, 4, 2, kModeRowColI8, true>(a, st) : launch_cfg<256, 256, 4, 2, kModeRowColI8, false>(a, st);
-  return direct ? launch_cfg<128, 128, 2, 2, kModeRowColI8, true>(a, st) : launch_cfg<128, 128, 2, 2, kModeRowColI8, false>(a, st);
+  // the dispatch of the fp8 operands with row and column scales: the kernels take the operand type as a mode, and
+  // every exchange of partial sums adds int32 as int32
+  return launch_gemm<kModeRowColI8>(a, workspace, workspace_bytes, (hipStream_t)stream);
 }

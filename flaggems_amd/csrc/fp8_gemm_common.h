@@ -59,8 +59,9 @@ __device__ __forceinline__ float load_as_float(const void* p, int64_t i, int dty
 // does (src/flag_gems/fused/cutlass_scaled_mm.py:288-305).
 template <int MODE>
 __device__ __forceinline__ void store_output(const GemmArgs& a, int m, int n, float v) {
-  if (MODE == kModeRowCol) v = (v * a.xs[a.xs_per_row ? m : 0]) * a.ws[a.ws_per_col ? n : 0];
-  const bool has_bias = (MODE == kModeRowCol) && a.bias != nullptr;
+  if (MODE == kModeRowColI8) v = (float)__float_as_int(v);  // int8 operands: v carries the bits of an int32 sum
+  if (MODE != kModeBlock) v = (v * a.xs[a.xs_per_row ? m : 0]) * a.ws[a.ws_per_col ? n : 0];
+  const bool has_bias = (MODE != kModeBlock) && a.bias != nullptr;
   const int64_t off = (int64_t)m * a.ldc + n;
   if (a.c_dtype == FG_BF16) {
     uint16_t h = float_to_bf16_bits(v);

@@ -181,7 +181,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
               acc[r][t][2] = __builtin_fmaf(p[2], sc[t], acc[r][t][2]);
               acc[r][t][3] = __builtin_fmaf(p[3], sc[t], acc[r][t][3]);
             } else {
-              acc[r][t] = mfma_fp8_16x16x128(wf, xf[t], acc[r][t]);
+              acc[r][t] = MODE == kModeRowColI8 ? mfma_i8_16x16x128(wf, xf[t], acc[r][t]) : mfma_fp8_16x16x128(wf, xf[t], acc[r][t]);
             }
           }
         }
@@ -235,7 +235,10 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
           for (int r = 0; r < RG; ++r)
 #pragma unroll
             for (int t = 0; t < TMX; ++t) {
-              if (s0 + b == 0) acc[r][t] = tmp[b][r][t]; else acc[r][t] += tmp[b][r][t];  // no "0 + x" in the sum
+              // (no "0 + x" in the sum; int8 operands: the registers hold int32 sums, added as such)
+              if (s0 + b == 0) acc[r][t] = tmp[b][r][t];
+              else if (MODE == kModeRowColI8) acc[r][t] = __builtin_bit_cast(v4f, __builtin_bit_cast(v4i, acc[r][t]) + __builtin_bit_cast(v4i, tmp[b][r][t]));
+              else acc[r][t] += tmp[b][r][t];
             }
         }
       }
@@ -271,14 +274,17 @@ int launch_mid(const MidArgs& ma, int mode, hipStream_t stream) {
   const int lds_bytes = ma.kb_per_split * kPerKb;
   auto kb = fp8_gemm_midm_kernel<TMX, RG, WAVES, DEPTH, kModeBlock>;
   auto kr = fp8_gemm_midm_kernel<TMX, RG, WAVES, DEPTH, kModeRowCol>;
+  auto ki = fp8_gemm_midm_kernel<TMX, RG, WAVES, DEPTH, kModeRowColI8>;
   static PerDeviceFlags lds_limit_raised = {};  // per instantiation
   {
     constexpr int kMax = mid_kb_max(TMX) * kPerKb;
-    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, kMax, reinterpret_cast<const void*>(kb), reinterpret_cast<const void*>(kr));
+    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, kMax, reinterpret_cast<const void*>(kb), reinterpret_cast<const void*>(kr),
+                                                  reinterpret_cast<const void*>(ki));
     if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kMax, hipGetErrorString(e));
   }
   const dim3 grid((uint32_t)ceil_div(ma.n_chunks, WAVES), (uint32_t)ma.splits, (uint32_t)(ma.g.batch > 1 ? ma.g.batch : 1)), block(WAVES * 64);
   if (mode == kModeBlock) FG_LAUNCH(kb, grid, block, lds_bytes, stream, ma);
+  else if (mode == kModeRowColI8) FG_LAUNCH(ki, grid, block, lds_bytes, stream, ma);
   else FG_LAUNCH(kr, grid, block, lds_bytes, stream, ma);
   FG_CHECK_LAUNCH("fp8_gemm_midm_kernel");
   return FG_OK;

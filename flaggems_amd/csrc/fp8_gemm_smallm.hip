@@ -107,10 +107,15 @@ __device__ __forceinline__ void compute_unit(const Unit<TMX>& u, v4f (&acc)[kRow
         acc[r][t][2] = __builtin_fmaf(p[2], sc, acc[r][t][2]);
         acc[r][t][3] = __builtin_fmaf(p[3], sc, acc[r][t][3]);
       } else {
-        acc[r][t] = mfma_fp8_16x16x128(wf, xf, acc[r][t]);
+        acc[r][t] = MODE == kModeRowColI8 ? mfma_i8_16x16x128(wf, xf, acc[r][t]) : mfma_fp8_16x16x128(wf, xf, acc[r][t]);
       }
     }
   }
+}
+
+// Sum of two partial results: fp32, or int32 bit patterns (int8 operands, whose sums stay exact).
+__device__ __forceinline__ float add_partial(float a, float b, bool as_int) {
+  return as_int ? __int_as_float(__float_as_int(a) + __float_as_int(b)) : a + b;
 }
 
 // Adds the wavefronts' accumulators in LDS and writes the chunk (or publishes a split-K partial tile and,
@@ -131,6 +136,7 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
   // instructions of their own: the general epilogue is a long chain of branches, and at the end of a launch of a few
   // microseconds every instruction line it fetches is waited for by the whole GPU
   const bool plain = MODE == kModeBlock && g.c_dtype == FG_BF16;
+  constexpr bool as_int = MODE == kModeRowColI8;
   // lane holds m = t*16 + l16, n = r*16 + 4*lg + [0,4)
 #pragma unroll
   for (int r = 0; r < kRowGroups; ++r)
@@ -144,7 +150,7 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
       const int m = i / kChunkRows, nn = i % kChunkRows;
       float v = 0.f;
 #pragma unroll
-      for (int w = 0; w < WAVES; ++w) v += red[w * red_stride + i];
+      for (int w = 0; w < WAVES; ++w) v = add_partial(v, red[w * red_stride + i], as_int);
       if (m < g.M && nn < rows) {
         if (plain) reinterpret_cast<uint16_t*>(g.C)[(int64_t)m * g.ldc + n0 + nn] = float_to_bf16_bits(v);
         else store_output<MODE>(g, m, n0 + nn, v);
@@ -157,7 +163,7 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
   for (int i = tid; i < kOut; i += NT) {
     float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) v += red[w * red_stride + i];
+    for (int w = 0; w < WAVES; ++w) v = add_partial(v, red[w * red_stride + i], as_int);
     // device-scope store: written through to memory, where blocks on other XCDs (own L2 each) read it
     __hip_atomic_store(mine + i, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
@@ -179,7 +185,7 @@ __device__ __forceinline__ void finish_chunk(const SmallArgs& a, float* red, int
     const int m = i / kChunkRows, nn = i % kChunkRows;
     float v = 0.f;
     for (int s = 0; s < a.splits; ++s)
-      v += __hip_atomic_load(all + (int64_t)s * kOut + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v = add_partial(v, __hip_atomic_load(all + (int64_t)s * kOut + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), as_int);
     if (m < g.M && nn < rows) {
       if (plain) reinterpret_cast<uint16_t*>(g.C)[(int64_t)m * g.ldc + n0 + nn] = float_to_bf16_bits(v);
       else store_output<MODE>(g, m, n0 + nn, v);
@@ -564,7 +570,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[r][t][i] = __builtin_fmaf(p[i], second[r][i] ? sc2 : sc1, acc[r][t][i]);
           } else {
-            acc[r][t] = mfma_fp8_16x16x128(wf, xf[t], acc[r][t]);
+            acc[r][t] = MODE == kModeRowColI8 ? mfma_i8_16x16x128(wf, xf[t], acc[r][t]) : mfma_fp8_16x16x128(wf, xf[t], acc[r][t]);
           }
         }
       }
@@ -643,6 +649,7 @@ template <int TMX, int WAVES>
 int launch_t(const SmallArgs& sa, int mode, hipStream_t stream) {
   const dim3 grid((uint32_t)(sa.n_chunks * sa.splits), (uint32_t)(sa.g.batch > 1 ? sa.g.batch : 1)), block(WAVES * 64);
   if (mode == kModeBlock) FG_LAUNCH((fp8_gemm_smallm_kernel<TMX, WAVES, kModeBlock>), grid, block, 0, stream, sa);
+  else if (mode == kModeRowColI8) FG_LAUNCH((fp8_gemm_smallm_kernel<TMX, WAVES, kModeRowColI8>), grid, block, 0, stream, sa);
   else FG_LAUNCH((fp8_gemm_smallm_kernel<TMX, WAVES, kModeRowCol>), grid, block, 0, stream, sa);
   FG_CHECK_LAUNCH("fp8_gemm_smallm_kernel");
   return FG_OK;
@@ -673,12 +680,15 @@ int launch_transpose(const SmallArgs& sa, int mode, hipStream_t stream) {
   const dim3 block(WAVES * 64);
   auto kb = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeBlock, XLDS, OWN>;
   auto kr = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeRowCol, XLDS, OWN>;
+  auto ki = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeRowColI8, XLDS, OWN>;
   static PerDeviceFlags lds_limit_raised = {};  // per instantiation
   {
-    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, XLDS ? kDecodeLdsLimit : kSlabs, reinterpret_cast<const void*>(kb), reinterpret_cast<const void*>(kr));
+    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, XLDS ? kDecodeLdsLimit : kSlabs, reinterpret_cast<const void*>(kb), reinterpret_cast<const void*>(kr),
+                                                  reinterpret_cast<const void*>(ki));
     if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(LDS limit): %s", hipGetErrorString(e));
   }
   if (mode == kModeBlock) FG_LAUNCH(kb, grid, block, lds_bytes, stream, sa);
+  else if (mode == kModeRowColI8) FG_LAUNCH(ki, grid, block, lds_bytes, stream, sa);
   else FG_LAUNCH(kr, grid, block, lds_bytes, stream, sa);
   FG_CHECK_LAUNCH("fp8_gemm_transpose_kernel");
   return FG_OK;

@@ -60,6 +60,8 @@ def _launch_scaled_int8_gemm(c, a, b, a_scale, b_scale, bias) -> None:
     n = b.shape[1]
     dev = a.device
     with torch.cuda.device(dev):
+        ws_bytes = lib.fg_scaled_int8_gemm_workspace_bytes(m, n, k)
+        ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
         status = lib.fg_scaled_int8_gemm(
             a.data_ptr(), a.stride(0) if m > 1 else max(k, a.stride(0)),
             b.data_ptr(), b.stride(1) if n > 1 else max(k, b.stride(1)),
@@ -68,7 +70,9 @@ def _launch_scaled_int8_gemm(c, a, b, a_scale, b_scale, bias) -> None:
             bias.data_ptr() if bias is not None else None,
             _lib.DTYPE_CODE[bias.dtype] if bias is not None else _lib.FG_BF16,
             c.data_ptr(), c.stride(0) if m > 1 else max(n, c.stride(0)), _lib.DTYPE_CODE[c.dtype],
-            m, n, k, _lib.current_stream_ptr(dev),
+            m, n, k,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+            _lib.current_stream_ptr(dev),
         )
     _lib.check(status, "fg_scaled_int8_gemm")
 

@@ -386,8 +386,11 @@ int fg_scaled_gemm(const void* A, int64_t lda, const void* B, int64_t ldb, int a
 /*
  * The same with int8 operands: C[m, n] = float(sum_k A[m,k] * B[n,k] in int32) * a_scale[m or 0] * b_scale[n or 0],
  * rounded to c_dtype (FG_BF16, FG_F16 or FG_F32), then + bias[n] in c_dtype.  A: int8 [M, K] rows lda apart,
- * B: int8 [N, K] rows ldb apart (the column-major [K, N] operand of the reference).  Served by the tile kernel at
- * every M (no workspace, no K split): correct at decode sizes, not tuned for them.
+ * B: int8 [N, K] rows ldb apart (the column-major [K, N] operand of the reference).  The same kernels and dispatch
+ * as fg_scaled_fp8_gemm, with the int8 matrix instruction; `workspace` as for fg_block_fp8_gemm
+ * (fg_scaled_int8_gemm_workspace_bytes(M, N, K); required for M <= 64 when that is not 0).  Where K is split between
+ * wavefronts or blocks the int32 partial sums are added as integers: the result is float(exact sum) * scales
+ * whatever the split.
  * Stands in for the int8 branch of cutlass_scaled_mm (src/flag_gems/fused/cutlass_scaled_mm.py:198-344 with an
  * int32 accumulator, dispatch :394-402).
  */
@@ -396,7 +399,9 @@ int fg_scaled_int8_gemm(const void* A, int64_t lda, const void* B, int64_t ldb,
                         const float* b_scale, int b_scale_per_col,
                         const void* bias, int bias_dtype,
                         void* C, int64_t ldc, int c_dtype,
-                        int64_t M, int64_t N, int64_t K, void* stream);
+                        int64_t M, int64_t N, int64_t K,
+                        void* workspace, size_t workspace_bytes, void* stream);
+size_t fg_scaled_int8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 #ifdef __cplusplus
 }

@@ -37,7 +37,12 @@ def _exact(a, b, sa, sb):
 
 @pytest.mark.parametrize("M,N,K", [(1, 256, 128), (16, 512, 512), (33, 1024, 1024), (100, 640, 4096), (256, 4096, 4096),
                                    (512, 8192, 1024), (1100, 1300, 2048), (64, 200, 192), (7, 24, 40), (1024, 2304, 512),
-                                   (129, 264, 128), (700, 8, 384)])
+                                   (129, 264, 128), (700, 8, 384),
+                                   # up to 32 rows: the weight-streaming kernels (K split over blocks for the first)
+                                   (1, 4096, 4096), (8, 2112, 7168), (16, 7168, 2304), (32, 1024, 8192), (5, 24592, 384),
+                                   (12, 32768, 512), (20, 520, 1024),
+                                   # 33..64 rows: the kernel with the activations of a K range in LDS
+                                   (33, 2112, 7168), (64, 4096, 4096), (48, 24576, 1536), (40, 264, 512)])
 @pytest.mark.parametrize("kinds", [("scalar", "scalar"), ("vector", "vector"), ("vector", "scalar")])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16])
 def test_int8_cutlass_scaled_mm(M, N, K, kinds, out_dtype):
@@ -107,6 +112,46 @@ def test_int8_sums_are_exact_in_bf16_above_128_rows():
     assert c[0, 1].item() == -128 * 64 * K and c[1, 1].item() == 127 * 64 * K
     want = (a.double() @ b.double().t()).float().to(torch.bfloat16)  # one rounding of the exact sum
     assert torch.equal(c.cpu(), want)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 512, 8192), (4, 2112, 7168), (16, 4096, 4096), (9, 24576, 1536), (32, 768, 2048),
+                                   (33, 512, 8192), (64, 2112, 7168)])
+def test_int8_sums_are_exact_up_to_64_rows(M, N, K):
+    """The kernels for few rows split K over wavefronts and blocks: the int32 partial sums are added as integers, so
+    the fp32 result is the one rounding of the exact sum, also where the sum needs more than 24 bits."""
+    g = torch.Generator().manual_seed(7)
+    a = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+    b = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+    a[0, :] = -128
+    b[0, :] = -128
+    b[1, :] = 127
+    b[2, :] = (torch.arange(K) % 2 * 2 - 1).to(torch.int8) * 127  # sums that cancel
+    one = torch.ones(1, device=DEV)
+    c = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    flag_gems.cutlass_scaled_mm(c, a.to(DEV), b.to(DEV).t(), one, one, None)
+    want = (a.double() @ b.double().t())
+    assert want.abs().max() > 2 ** 24
+    assert torch.equal(c.cpu(), want.float())
+    assert c[0, 0].item() == 128 * 128 * K and c[0, 1].item() == -128 * 127 * K
+    # through the C ABI: a missing workspace is refused where the kernels for few rows need one
+    from flaggems_amd import _lib
+    lib = _lib.load()
+    a_d, b_d = a.to(DEV), b.to(DEV)
+    c2 = torch.empty_like(c)
+    need = lib.fg_scaled_int8_gemm_workspace_bytes(M, N, K)
+    ws = _lib.workspace(torch.device(DEV), need) if need else None
+
+    def call(ws_ptr, ws_bytes):
+        return lib.fg_scaled_int8_gemm(
+            a_d.data_ptr(), K, b_d.data_ptr(), K, one.data_ptr(), 0, one.data_ptr(), 0, None, _lib.FG_BF16,
+            c2.data_ptr(), N, _lib.DTYPE_CODE[torch.float32], M, N, K, ws_ptr, ws_bytes,
+            _lib.current_stream_ptr(torch.device(DEV)))
+
+    _lib.check(call(ws.data_ptr() if need else None, ws.numel() if need else 0), "fg_scaled_int8_gemm")
+    torch.cuda.synchronize()
+    assert torch.equal(c2, c)
+    if need:
+        assert call(None, 0) == -3  # FG_ERR_WORKSPACE
 
 
 def test_int8_through_aten_scaled_mm():
