@@ -17,8 +17,10 @@ Prints ONE JSON line with the driver's fields plus
   cpu_baseline  the CPU oracle (torch restatement of the reference's torch implementation) timed on
                 the host cores on a bounded sample of the same sweep
   detail        per-(M, N, K) time, TFLOP/s, GB/s and roofline fractions (MFMA for M >= 512, HBM below)
-  block_fp8_gemm_pow2_scales_m4096, cutlass_scaled_mm_n8192_k8192_bias, llama3_8b_linears
-                the other configurations of the path (per-token x per-channel scaled GEMM with bias; Llama-3-8B
+  block_fp8_gemm_pow2_scales_m4096, cutlass_scaled_mm_n8192_k8192_bias, cutlass_scaled_mm_int8_n8192_k8192_bias,
+  llama3_8b_linears
+                the other configurations of the path (per-token x per-channel scaled GEMM with bias, fp8 and int8
+                operands; Llama-3-8B
                 linears as GEMM alone and as act_quant + GEMM), graph replays of one shape at a time with ONE copy
                 of the weights (small-M figures there may be served by the 256 MB Infinity Cache), not part of `value`
   mixtral_moe_grouped_gemm
@@ -393,6 +395,20 @@ def main():
                        "gbps": round(nbytes / us / 1e3, 1)})
     del b_q, a_q, c
 
+    # the int8 branch of cutlass_scaled_mm on the same shapes (the reference's int8 inputs: round(clamp(randn * 5)))
+    scaled_i8 = []
+    b_i8 = torch.round((torch.randn(nk, nk, device=dev, generator=gen) * 5).clamp(-128, 127)).to(torch.int8)
+    b_si = torch.rand(nk, device=dev, generator=gen) * 0.02 + 0.001
+    for m in (1, 32, 256, 2048, 8192):
+        a_i8 = torch.round((torch.randn(m, nk, device=dev, generator=gen) * 5).clamp(-128, 127)).to(torch.int8)
+        a_si = torch.rand(m, 1, device=dev, generator=gen) * 0.02 + 0.001
+        c = torch.empty(m, nk, dtype=torch.bfloat16, device=dev)
+        us = time_eager(lambda: flag_gems.cutlass_scaled_mm(c, a_i8, b_i8.t(), a_si, b_si.view(1, nk), bias), 10 if m >= 2048 else 30)
+        nbytes = m * nk + nk * nk + 4 * m + 4 * nk + 2 * m * nk + 2 * nk
+        scaled_i8.append({"M": m, "N": nk, "K": nk, "us": round(us, 2), "tops": round(gemm_flops(m, nk, nk) / us / 1e6, 1),
+                          "gbps": round(nbytes / us / 1e3, 1)})
+    del b_i8, a_i8, c
+
     # aten::_scaled_mm on operands that are not quantized (the generic kernel): per-row x per-column scales, N = K = 4096
     generic = []
     for dt, peak in ((torch.bfloat16, 2500.0), (torch.float16, 2500.0), (torch.float32, 157.3)):
@@ -557,6 +573,7 @@ def main():
         "rms_norm_quantizer": norm_quant,
         "block_fp8_gemm_pow2_scales_m4096": pow2_summary,
         "cutlass_scaled_mm_n8192_k8192_bias": scaled,
+        "cutlass_scaled_mm_int8_n8192_k8192_bias": scaled_i8,
         "scaled_mm_unquantized_operands": generic,
         "fp8_einsum_bhr_hdr": einsum,
         "llama3_8b_linears": llama,
