@@ -48,6 +48,7 @@
 // round of the grid are cut along K so that every compute unit streams to the end (finish_cut_tile).
 
 #include "fp8_gemm_common.h"
+#include <mutex>
 
 namespace fg {
 namespace {
@@ -403,6 +404,26 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   const bf16x2_t h = __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t);
   return __builtin_bit_cast(uint32_t, h);
 }
+// Two results as the 16-bit output type, F16: fp16, else bf16 (round to nearest even both).  The empty statement
+// keeps the compiler from folding a multiplication that produced the value into the conversion (one rounding
+// instead of the two that the tile kernels and the reference perform).
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+template <bool F16>
+__device__ __forceinline__ uint32_t pack_out(float lo, float hi) {
+  if (!F16) return pack_bf16(lo, hi);
+  asm volatile("" : "+v"(lo), "+v"(hi));
+  const f16x2_t h = {(_Float16)lo, (_Float16)hi};
+  return __builtin_bit_cast(uint32_t, h);
+}
+// the two halves of such a word as fp32
+template <bool F16>
+__device__ __forceinline__ float unpack_lo(uint32_t w) {
+  return F16 ? (float)__builtin_bit_cast(f16x2_t, w)[0] : bits_to_float(w << 16);
+}
+template <bool F16>
+__device__ __forceinline__ float unpack_hi(uint32_t w) {
+  return F16 ? (float)__builtin_bit_cast(f16x2_t, w)[1] : bits_to_float(w & 0xFFFF0000u);
+}
 
 // Stores the wavefront's 64 x 128 results as bf16.  Lane (l16, lg) holds, for every activation tile j, four
 // pieces of eight consecutive columns of row m_base + 16 j + l16: piece q starts at column
@@ -415,7 +436,8 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 constexpr int kStoresPerTile = 16;
 // SCATTER (grouped problems): rows go where out_index says (see PpArgs::c_rows).
 // JN: activation fragments per wavefront (rows m_base .. m_base + 16 JN).
-template <int MODE, bool ALIGNED, bool SCATTER = false, int JN = kTM>
+// F16: the results are fp16 (else bf16).
+template <int MODE, bool ALIGNED, bool SCATTER = false, int JN = kTM, bool F16 = false>
 __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[kTN][JN], int m_base, int n_base,
                                            int l16, int lg, int m_end, const int* out_index = nullptr, int c_rows = 0,
                                            const float* row_weight = nullptr) {
@@ -448,10 +470,10 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
           const float s1 = MODE == kModeRowColI8 ? (float)__float_as_int(r1) : r1;
           const float v0 = (s0 * sa) * sb[4 * (h >> 1) + e0];
           const float v1 = (s1 * sa) * sb[4 * (h >> 1) + e0 + 1];
-          w[h] = pack_bf16(v0, v1);
+          w[h] = pack_out<F16>(v0, v1);
           if (a.bias)
-            w[h] = pack_bf16(bits_to_float(w[h] << 16) + bias[4 * (h >> 1) + e0],
-                             bits_to_float(w[h] & 0xFFFF0000u) + bias[4 * (h >> 1) + e0 + 1]);
+            w[h] = pack_out<F16>(unpack_lo<F16>(w[h]) + bias[4 * (h >> 1) + e0],
+                                 unpack_hi<F16>(w[h]) + bias[4 * (h >> 1) + e0 + 1]);
         }
         uint16_t* const cp = reinterpret_cast<uint16_t*>(a.C) + (int64_t)m * a.ldc + n;
         if (full) {
@@ -482,14 +504,14 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
     if (SCATTER && row_weight != nullptr) {
 #pragma unroll
       for (int t = 0; t < kTN; ++t) {
-        w[2 * t] = pack_bf16(acc[t][j][0] * wgt, acc[t][j][1] * wgt);
-        w[2 * t + 1] = pack_bf16(acc[t][j][2] * wgt, acc[t][j][3] * wgt);
+        w[2 * t] = pack_out<F16>(acc[t][j][0] * wgt, acc[t][j][1] * wgt);
+        w[2 * t + 1] = pack_out<F16>(acc[t][j][2] * wgt, acc[t][j][3] * wgt);
       }
     } else {
 #pragma unroll
       for (int t = 0; t < kTN; ++t) {
-        w[2 * t] = pack_bf16(acc[t][j][0], acc[t][j][1]);
-        w[2 * t + 1] = pack_bf16(acc[t][j][2], acc[t][j][3]);
+        w[2 * t] = pack_out<F16>(acc[t][j][0], acc[t][j][1]);
+        w[2 * t + 1] = pack_out<F16>(acc[t][j][2], acc[t][j][3]);
       }
     }
 #pragma unroll
@@ -520,6 +542,7 @@ __device__ __forceinline__ int sk_range_of_step(const PpArgs& a, int step) {
 // share the tile) adds all partial sums in range order -- the same order whoever comes last, so the
 // result does not depend on timing -- stores the piece, and resets the counter for the next launch.
 // Nobody waits for anybody.  On entry and exit no vector-memory operation of this wavefront is pending.
+template <bool F16>
 __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (&acc)[kTN][kTM], int tile, int pos,
                                                     int m_base, int n_base, int wave, int lane, int l16, int lg) {
   const int s_lo = tile * a.g.KB;
@@ -576,8 +599,8 @@ __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (
       uint32_t w[8];
 #pragma unroll
       for (int t = 0; t < kTN / 2; ++t) {
-        w[2 * t] = pack_bf16(r[t][j][0], r[t][j][1]);
-        w[2 * t + 1] = pack_bf16(r[t][j][2], r[t][j][3]);
+        w[2 * t] = pack_out<F16>(r[t][j][0], r[t][j][1]);
+        w[2 * t + 1] = pack_out<F16>(r[t][j][2], r[t][j][3]);
       }
 #pragma unroll
       for (int qq = 0; qq < 2; ++qq) {
@@ -600,7 +623,7 @@ __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (
 // finish_partial_tile -- publish, count in, the last of the tile's work items to arrive adds all partial sums in cut
 // order and stores -- on the wavefront's 16 JN x 128 piece, which is small enough to be summed whole and handed to
 // store_tile, so gathered, scattered and weighted results take the one store path.  A slot per (work item, wavefront).
-template <bool SCATTER, int JN>
+template <bool SCATTER, int JN, bool F16>
 __device__ __forceinline__ void finish_cut_tile(const PpArgs& a, const v4f (&acc)[kTN][JN], int item, int m_base, int n_base,
                                                 int m_end, int wave, int lane, int l16, int lg) {
   constexpr int kFloats = kTN * JN * 256;  // per wavefront
@@ -638,8 +661,8 @@ __device__ __forceinline__ void finish_cut_tile(const PpArgs& a, const v4f (&acc
         if (q == 0) r[t][j] = tmp[t][j]; else r[t][j] += tmp[t][j];  // (no "0 + x" in the sum)
       }
   }
-  store_tile<kModeBlock, false, SCATTER, JN>(a.g, r, m_base, n_base, l16, lg, m_end, SCATTER && a.c_rows > 0 ? a.row_index : nullptr,
-                                             a.c_rows, a.row_weight);
+  store_tile<kModeBlock, false, SCATTER, JN, F16>(a.g, r, m_base, n_base, l16, lg, m_end, SCATTER && a.c_rows > 0 ? a.row_index : nullptr,
+                                                  a.c_rows, a.row_weight);
   if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the counted waits of the main loop start from zero
 }
@@ -653,7 +676,9 @@ __device__ __forceinline__ void finish_cut_tile(const PpArgs& a, const v4f (&acc
 // that, not the weight stream, sets the time of a step when a tile holds a few dozen rows.  With JN = 1 the four
 // wavefronts of a group take 16 rows each, the activation image in LDS keeps its 256-row layout (the rows past the
 // 64th are loaded like rows past an edge and never read), and everything else runs unchanged.
-template <bool SK, int MODE, bool ALIGNED, bool GROUPED = false, bool POW2 = false, int JN = kTM>
+// F16: the results are fp16 (else bf16).  A template parameter and not a test of c_dtype in the flush: with both
+// forms of the stores in one kernel the bf16 flush of short-K problems got 5 % slower.
+template <bool SK, int MODE, bool ALIGNED, bool GROUPED = false, bool POW2 = false, int JN = kTM, bool F16 = false>
 __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   static_assert(JN == kTM || (GROUPED && JN >= 1 && JN < kTM), "short tiles: grouped problems only");
   constexpr int kTileRows = 64 * JN;
@@ -865,18 +890,18 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     if constexpr (kCuts) {
       if (pend_idx >= a.cut_full) {
         wait_vmem<0>();
-        finish_cut_tile<GROUPED, JN>(a, acc, pend_idx - a.cut_full, pend_m, pend_n, pend_m_end, wave, lane, l16, lg);
+        finish_cut_tile<GROUPED, JN, F16>(a, acc, pend_idx - a.cut_full, pend_m, pend_n, pend_m_end, wave, lane, l16, lg);
         clear_acc();
         return;
       }
     }
-    store_tile<MODE, ALIGNED, GROUPED, JN>(g, acc, pend_m, pend_n, l16, lg, pend_m_end, GROUPED && a.c_rows > 0 ? a.row_index : nullptr,
-                                       a.c_rows, a.row_weight);
+    store_tile<MODE, ALIGNED, GROUPED, JN, F16>(g, acc, pend_m, pend_n, l16, lg, pend_m_end, GROUPED && a.c_rows > 0 ? a.row_index : nullptr,
+                                                a.c_rows, a.row_weight);
     clear_acc();
   };
   auto flush_partial_tile = [&]() __attribute__((always_inline)) {
     wait_vmem<0>();
-    if constexpr (SK) finish_partial_tile(a, acc, pend_idx, pos, pend_m, pend_n, wave, lane, l16, lg);
+    if constexpr (SK) finish_partial_tile<F16>(a, acc, pend_idx, pos, pend_m, pend_n, wave, lane, l16, lg);
     clear_acc();
   };
 
@@ -1183,6 +1208,58 @@ int max_cut_shift(int grid, int KB) {
   return sh;
 }
 
+// The instantiation that serves a launch.
+struct KernelChoice {
+  bool grouped, short_tiles;
+  int mode;
+  bool sk, aligned, pow2;
+};
+template <bool F16>
+void (*pick_kernel(const KernelChoice& c))(PpArgs) {
+  if (c.grouped)
+    return c.short_tiles ? fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, 1, F16>
+                         : fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, kTM, F16>;
+  if (c.mode == kModeRowColI8)
+    return c.aligned ? fp8_gemm_pingpong_kernel<false, kModeRowColI8, true, false, false, kTM, F16>
+                     : fp8_gemm_pingpong_kernel<false, kModeRowColI8, false, false, false, kTM, F16>;
+  if (c.mode != kModeBlock)
+    return c.aligned ? fp8_gemm_pingpong_kernel<false, kModeRowCol, true, false, false, kTM, F16>
+                     : fp8_gemm_pingpong_kernel<false, kModeRowCol, false, false, false, kTM, F16>;
+  if (c.pow2) {
+    if (c.sk)
+      return c.aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, true, kTM, F16>
+                       : fp8_gemm_pingpong_kernel<true, kModeBlock, false, false, true, kTM, F16>;
+    return c.aligned ? fp8_gemm_pingpong_kernel<false, kModeBlock, true, false, true, kTM, F16>
+                     : fp8_gemm_pingpong_kernel<false, kModeBlock, false, false, true, kTM, F16>;
+  }
+  if (c.sk)
+    return c.aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, false, kTM, F16>
+                     : fp8_gemm_pingpong_kernel<true, kModeBlock, false, false, false, kTM, F16>;
+  return c.aligned ? fp8_gemm_pingpong_kernel<false, kModeBlock, true, false, false, kTM, F16>
+                   : fp8_gemm_pingpong_kernel<false, kModeBlock, false, false, false, kTM, F16>;
+}
+
+// Every instantiation uses all of a compute unit's LDS, which a kernel has to be allowed once per device.  The
+// kernels are few: a short table of the ones seen so far, under a lock.
+int allow_full_lds(void (*kern)(PpArgs)) {
+  constexpr int kMaxKernels = 64;
+  static std::mutex lock;
+  static const void* seen[kMaxKernels];
+  static PerDeviceFlags raised[kMaxKernels];
+  static int n_seen = 0;
+  const void* const k = reinterpret_cast<const void*>(kern);
+  std::lock_guard<std::mutex> guard(lock);
+  int i = 0;
+  while (i < n_seen && seen[i] != k) ++i;
+  if (i == n_seen) {
+    if (n_seen == kMaxKernels) FG_FAIL(FG_ERR_LAUNCH, "fp8 gemm: kernel table full");
+    seen[n_seen++] = k;
+  }
+  const hipError_t e = raise_dynamic_lds_limit(raised[i], kLdsBytes, k);
+  if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
+  return FG_OK;
+}
+
 int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream,
                  const GroupedGemm* grouped = nullptr) {
   PpArgs a = {};
@@ -1212,25 +1289,6 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     const uint64_t d = 4ull * (uint64_t)a.g.tiles_n;
     // n * magic >> 40 == n / d for every n with n * d < 2^40 (the tile numbers of whole problems are below `tiles`)
     a.group4_magic = (d > 0 && (uint64_t)tiles * d < (1ull << 40)) ? ((1ull << 40) + d - 1) / d : 0;
-  }
-  static PerDeviceFlags lds_limit_raised[14] = {};
-  const void* const kernels[14] = {reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, true>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, false>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowCol, true>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false, true>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false, false, true>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, true, false, true>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, false, false, true>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, true>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowColI8, false>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeRowColI8, true>),
-                                  reinterpret_cast<const void*>(fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, 1>)};
-  for (int i = 0; i < 14; ++i) {
-    const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised[i], kLdsBytes, kernels[i]);
-    if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", kLdsBytes, hipGetErrorString(e));
   }
   const int cus = cu_count();
   int grid = tiles < cus ? (int)tiles : cus;
@@ -1286,22 +1344,11 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     if (tile_us < batch_us) a.stagger = (int)(tile_us * 1.6e3 / 1000.0 / 16 + 0.5);  // 1.6 GHz, ~1000 cycles a sleep, 16 start slots
   }
   const bool aligned = g.M % kBM == 0 && g.N % kBN == 0;
-  void (*kern)(PpArgs);
-  if (grouped != nullptr)
-    kern = short_tiles ? fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, 1> : fp8_gemm_pingpong_kernel<false, kModeBlock, false, true>;
-  else if (mode == kModeRowColI8)
-    kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeRowColI8, true> : fp8_gemm_pingpong_kernel<false, kModeRowColI8, false>;
-  else if (mode != kModeBlock)
-    kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeRowCol, true> : fp8_gemm_pingpong_kernel<false, kModeRowCol, false>;
-  else if (a.sk)
-    kern = aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true> : fp8_gemm_pingpong_kernel<true, kModeBlock, false>;
-  else
-    kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeBlock, true> : fp8_gemm_pingpong_kernel<false, kModeBlock, false>;
   const bool pow2 = mode == kModeBlock && grouped == nullptr && g.scales_pow2 != 0;
-  if (pow2) {
-    if (a.sk) kern = aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, true> : fp8_gemm_pingpong_kernel<true, kModeBlock, false, false, true>;
-    else kern = aligned ? fp8_gemm_pingpong_kernel<false, kModeBlock, true, false, true> : fp8_gemm_pingpong_kernel<false, kModeBlock, false, false, true>;
-  }
+  const bool f16 = g.c_dtype == FG_F16;
+  const KernelChoice which = {grouped != nullptr, short_tiles, mode, a.sk != 0, aligned, pow2};
+  void (*const kern)(PpArgs) = f16 ? pick_kernel<true>(which) : pick_kernel<false>(which);
+  if (const int rc = allow_full_lds(kern)) return rc;
   if (tp.use && !a.sk && workspace != nullptr && workspace_bytes >= need && (size_t)tp.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
       (uintptr_t)workspace % 16 == 0) {
     PpArgs whole = a;
@@ -1315,9 +1362,10 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     rest.sk = 1; rest.sk_q = tp.cut; rest.sk_r = 0; rest.sk_split = tp.split;
     rest.counters = reinterpret_cast<unsigned int*>(workspace);
     rest.partials = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES);
-    void (*shared)(PpArgs) = fp8_gemm_pingpong_kernel<true, kModeBlock, false>;
-    if (aligned) shared = fp8_gemm_pingpong_kernel<true, kModeBlock, true>;
-    if (pow2) shared = aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, true> : fp8_gemm_pingpong_kernel<true, kModeBlock, false, false, true>;
+    KernelChoice tail_choice = which;
+    tail_choice.sk = true;
+    void (*const shared)(PpArgs) = f16 ? pick_kernel<true>(tail_choice) : pick_kernel<false>(tail_choice);
+    if (const int rc = allow_full_lds(shared)) return rc;
     FG_LAUNCH(shared, dim3((uint32_t)tp.grid), dim3(kThreads), kLdsBytes, stream, rest);
     FG_CHECK_LAUNCH("fp8_gemm_pingpong_kernel (last tiles)");
     return FG_OK;
@@ -1343,7 +1391,7 @@ int cu_count() {
 
 bool pingpong_takes(const GemmArgs& g, int mode, const void* workspace, size_t workspace_bytes) {
   // bf16 rows that take 16-byte stores; activation-scale offsets (bytes from the first row) that fit 32 bits
-  if (!(g.M > 64 && g.c_dtype == FG_BF16 && g.ldc % 8 == 0 && (uintptr_t)g.C % 16 == 0)) return false;
+  if (!(g.M > 64 && (g.c_dtype == FG_BF16 || g.c_dtype == FG_F16) && g.ldc % 8 == 0 && (uintptr_t)g.C % 16 == 0)) return false;
   // 64 < M <= 128 wastes half of every 256-row tile: worth it only where tiles get shared along K (few, deep tiles)
   if (g.M <= 128) {
     const SkPlan sk = plan_stream_k(ceil_div(g.N, kBN), g.KB, cu_count());
@@ -1373,8 +1421,8 @@ size_t grouped_workspace_bytes(int64_t M, int64_t K) {
 }
 
 int launch_grouped(const GemmArgs& g, const GroupedGemm& grouped, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-  if (!(g.c_dtype == FG_BF16 && g.ldc % 8 == 0 && (uintptr_t)g.C % 16 == 0))
-    FG_FAIL(FG_ERR_UNSUPPORTED, "grouped fp8 gemm: the result must be bf16 with rows that take 16-byte stores");
+  if (!((g.c_dtype == FG_BF16 || g.c_dtype == FG_F16) && g.ldc % 8 == 0 && (uintptr_t)g.C % 16 == 0))
+    FG_FAIL(FG_ERR_UNSUPPORTED, "grouped fp8 gemm: the result must be bf16 or fp16 with rows that take 16-byte stores");
   if (!(g.xs_rs >= 0 && g.xs_cs >= 0 && g.ws_rs >= 0 && g.ws_cs >= 0 && (int64_t)g.M * g.xs_rs < (1ll << 29)))
     FG_FAIL(FG_ERR_UNSUPPORTED, "grouped fp8 gemm: scale strides must be non-negative and M * row stride below 2^29");
   if (grouped.n_groups <= 0 || grouped.n_groups > 65536) FG_FAIL(FG_ERR_INVALID_ARG, "grouped fp8 gemm: 1..65536 groups");

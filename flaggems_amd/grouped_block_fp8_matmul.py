@@ -98,8 +98,8 @@ def grouped_w8a8_block_fp8_matmul(
     assert offs.device == A.device and offs.is_contiguous()
     if A.dtype != torch.float8_e4m3fn or B.dtype != torch.float8_e4m3fn:
         raise NotImplementedError(f"grouped_w8a8_block_fp8_matmul: operands must be float8_e4m3fn, got {A.dtype}, {B.dtype}")
-    if output_dtype != torch.bfloat16:
-        raise NotImplementedError(f"grouped_w8a8_block_fp8_matmul: output dtype {output_dtype} (only bfloat16)")
+    if output_dtype not in (torch.bfloat16, torch.float16):
+        raise NotImplementedError(f"grouped_w8a8_block_fp8_matmul: output dtype {output_dtype} (bfloat16 or float16)")
     if As.dtype != torch.float32 or Bs.dtype != torch.float32:
         As, Bs = As.to(torch.float32), Bs.to(torch.float32)
     if B.stride(2) != 1:

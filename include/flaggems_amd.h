@@ -304,7 +304,7 @@ int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_batch_stride
  * B: e4m3fn [n_groups, N, K]: matrix e starts b_group_stride bytes after matrix e-1, rows ldb apart.
  * Bs: fp32 [n_groups, ceil(N/block_n), K/block_k]: matrix e starts bs_group_stride floats after matrix e-1.
  * K must be a positive multiple of 128; A, B 16-byte aligned with lda, ldb, b_group_stride multiples of 16;
- * C 16-byte aligned with ldc a multiple of 8; c_dtype FG_BF16 (FG_ERR_UNSUPPORTED otherwise: there is no
+ * C 16-byte aligned with ldc a multiple of 8; c_dtype FG_BF16 or FG_F16 (FG_ERR_UNSUPPORTED otherwise: there is no
  * slower general path behind this entry point).
  * `workspace` (optional, 16-byte aligned, fg_grouped_block_fp8_gemm_workspace_bytes(M, N, K) bytes, first
  * FG_WORKSPACE_COUNTER_BYTES zero-filled once) lets row-major As be read from a transposed copy and, when the
