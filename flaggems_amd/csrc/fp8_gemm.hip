@@ -556,79 +556,13 @@ __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
     if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
-  // ---- epilogue
+  // ---- epilogue: the lane holds m = ... + l16, n = ... + 4 * lg + [0, 4) of every MFMA tile
 #pragma unroll
   for (int j = 0; j < TM; ++j) {
     const int m = m0 + wm0 + j * 16 + l16;
     if (m >= a.M) continue;
-    float sa = 1.f;
-    constexpr bool kRowCol = MODE != kModeBlock;
-    if (kRowCol) sa = a.xs[a.xs_per_row ? m : 0];
 #pragma unroll
-    for (int i = 0; i < TN; ++i) {
-      const int n = n0 + wn0 + i * 16 + lg * 4;
-      if (n >= a.N) continue;
-      float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
-      if (MODE == kModeRowColI8) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = (float)__builtin_bit_cast(int, v[e]);  // int32 sums -> fp32, then as fp8
-      }
-      const int nv = (a.N - n < 4) ? a.N - n : 4;
-      if (kRowCol) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int ne = (e < nv) ? n + e : n;
-          const float sb = a.ws[a.ws_per_col ? ne : 0];
-          v[e] = (v[e] * sa) * sb;
-        }
-      }
-      const int64_t off = (int64_t)m * a.ldc + n;
-      if (a.c_dtype == FG_BF16) {
-        uint16_t h[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          h[e] = float_to_bf16_bits(v[e]);
-          if (kRowCol && a.bias) {
-            const int ne = (e < nv) ? n + e : n;
-            h[e] = float_to_bf16_bits(bf16_bits_to_float(h[e]) + load_as_float(a.bias, ne, a.bias_dtype));
-          }
-        }
-        uint16_t* cp = reinterpret_cast<uint16_t*>(a.C) + off;
-        if (nv == 4 && ((uintptr_t)cp % 8 == 0)) {
-          u32x2 o = {(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
-          *reinterpret_cast<u32x2*>(cp) = o;
-        } else {
-          for (int e = 0; e < nv; ++e) cp[e] = h[e];
-        }
-      } else if (a.c_dtype == FG_F16) {
-        _Float16* cp = reinterpret_cast<_Float16*>(a.C) + off;
-        for (int e = 0; e < nv; ++e) {
-          _Float16 h = (_Float16)v[e];
-          if (kRowCol && a.bias) h = (_Float16)((float)h + load_as_float(a.bias, n + e, a.bias_dtype));
-          cp[e] = h;
-        }
-      } else if (a.c_dtype == FG_F32) {
-        float* cp = reinterpret_cast<float*>(a.C) + off;
-        for (int e = 0; e < nv; ++e) {
-          float h = v[e];
-          if (kRowCol && a.bias) h = h + load_as_float(a.bias, n + e, a.bias_dtype);
-          cp[e] = h;
-        }
-      } else {  // FG_FP8_E4M3FN
-        uint8_t* cp = reinterpret_cast<uint8_t*>(a.C) + off;
-        for (int e = 0; e < nv; ++e) {
-          float h = v[e];
-          uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(h, 0.f, 0, false) & 0xFFu;
-          if (kRowCol && a.bias) {
-            // the reference adds the bias to the already rounded output, in the output type
-            const float back = __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
-            h = back + load_as_float(a.bias, n + e, a.bias_dtype);
-            code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(h, 0.f, 0, false) & 0xFFu;
-          }
-          cp[e] = (uint8_t)code;
-        }
-      }
-    }
+    for (int i = 0; i < TN; ++i) store_output4<MODE>(a, m, n0 + wn0 + i * 16 + lg * 4, acc[i][j]);
   }
 }
 

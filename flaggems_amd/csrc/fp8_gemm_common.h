@@ -84,6 +84,81 @@ __device__ __forceinline__ void store_output(const GemmArgs& a, int m, int n, fl
   }
 }
 
+// Four consecutive columns n .. n + 3 of row m (the four results a lane holds of a 16 x 16 MFMA tile): the same
+// arithmetic as store_output, element by element, with the scales of the row/column modes loaded once and one
+// 8- or 16-byte store where the four columns exist and the address allows it.
+template <int MODE>
+__device__ __forceinline__ void store_output4(const GemmArgs& a, int m, int n, v4f acc4) {
+  if (n >= a.N) return;
+  constexpr bool kRowCol = MODE != kModeBlock;
+  float v[4] = {acc4[0], acc4[1], acc4[2], acc4[3]};
+  if (MODE == kModeRowColI8) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = (float)__float_as_int(v[e]);  // int32 sums
+  }
+  const int nv = (a.N - n < 4) ? a.N - n : 4;
+  float bias[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool has_bias = kRowCol && a.bias != nullptr;
+  if (kRowCol) {
+    const float sa = a.xs[a.xs_per_row ? m : 0];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int ne = (e < nv) ? n + e : n;
+      v[e] = (v[e] * sa) * a.ws[a.ws_per_col ? ne : 0];
+      if (has_bias) bias[e] = load_as_float(a.bias, ne, a.bias_dtype);
+    }
+  }
+  const int64_t off = (int64_t)m * a.ldc + n;
+  if (a.c_dtype == FG_BF16) {
+    uint16_t h[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      h[e] = float_to_bf16_bits(v[e]);
+      if (has_bias) h[e] = float_to_bf16_bits(bf16_bits_to_float(h[e]) + bias[e]);
+    }
+    uint16_t* const cp = reinterpret_cast<uint16_t*>(a.C) + off;
+    if (nv == 4 && ((uintptr_t)cp % 8 == 0)) {
+      *reinterpret_cast<u32x2*>(cp) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+    } else {
+      for (int e = 0; e < nv; ++e) cp[e] = h[e];
+    }
+  } else if (a.c_dtype == FG_F16) {
+    uint16_t h[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      _Float16 f = (_Float16)v[e];
+      if (has_bias) f = (_Float16)((float)f + bias[e]);
+      h[e] = __builtin_bit_cast(uint16_t, f);
+    }
+    uint16_t* const cp = reinterpret_cast<uint16_t*>(a.C) + off;
+    if (nv == 4 && ((uintptr_t)cp % 8 == 0)) {
+      *reinterpret_cast<u32x2*>(cp) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+    } else {
+      for (int e = 0; e < nv; ++e) cp[e] = h[e];
+    }
+  } else if (a.c_dtype == FG_F32) {
+    float* const cp = reinterpret_cast<float*>(a.C) + off;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = has_bias ? v[e] + bias[e] : v[e];
+    if (nv == 4 && ((uintptr_t)cp % 16 == 0)) {
+      *reinterpret_cast<v4f*>(cp) = v4f{v[0], v[1], v[2], v[3]};
+    } else {
+      for (int e = 0; e < nv; ++e) cp[e] = v[e];
+    }
+  } else {  // FG_FP8_E4M3FN
+    uint8_t* const cp = reinterpret_cast<uint8_t*>(a.C) + off;
+    for (int e = 0; e < nv; ++e) {
+      uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(v[e], 0.f, 0, false) & 0xFFu;
+      if (has_bias) {
+        // the reference adds the bias to the already rounded output, in the output type
+        const float back = __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
+        code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(back + bias[e], 0.f, 0, false) & 0xFFu;
+      }
+      cp[e] = (uint8_t)code;
+    }
+  }
+}
+
 __device__ __forceinline__ v4f mfma_fp8_16x16x128(v8i a, v8i b, v4f c) {
   // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled instruction
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);

@@ -247,24 +247,12 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
   }
 
   // ---- results: the lane holds m = t * 16 + l16, n = n0 + r * 16 + 4 * lg + [0, 4)
-  const bool pack_ok = MODE == kModeBlock && g.c_dtype == FG_BF16 && (g.ldc & 3) == 0 && ((uintptr_t)g.C & 7) == 0;
 #pragma unroll
   for (int t = 0; t < TMX; ++t) {
     const int m = t * 16 + l16;
     if (m >= g.M) continue;
 #pragma unroll
-    for (int r = 0; r < RG; ++r) {
-      const int n = n0 + r * 16 + lg * 4;
-      if (pack_ok && n + 4 <= g.N) {
-        const u32x2 o = {(uint32_t)float_to_bf16_bits(acc[r][t][0]) | ((uint32_t)float_to_bf16_bits(acc[r][t][1]) << 16),
-                         (uint32_t)float_to_bf16_bits(acc[r][t][2]) | ((uint32_t)float_to_bf16_bits(acc[r][t][3]) << 16)};
-        *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(g.C) + (int64_t)m * g.ldc + n) = o;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (n + e < g.N) store_output<MODE>(g, m, n + e, acc[r][t][e]);
-      }
-    }
+    for (int r = 0; r < RG; ++r) store_output4<MODE>(g, m, n0 + r * 16 + lg * 4, acc[r][t]);
   }
 }
 
