@@ -53,3 +53,34 @@ def test_no_shape_is_far_off_the_cost_model(N, K):
         if us > limit:
             slow.append((M, N, K, round(us, 1), round(limit, 1)))
     assert not slow, f"(M, N, K, measured us, limit us): {slow}"
+
+
+@pytest.mark.parametrize("N,K", [(7168, 2304), (4096, 8192), (2112, 7168)])
+def test_output_types_and_scale_modes_stay_within_the_same_model(N, K):
+    """The same walk for fp16 and fp32 results and for the row/column scaled entry point (fp8 and int8 operands): a
+    result type or a scale mode that only a slower kernel serves shows up here (the persistent kernel used to write
+    bf16 only, and fp16 results above 128 rows took six times as long in the row/column mode)."""
+    g = torch.Generator(device=DEV).manual_seed(N * K)
+    w = torch.randn(N, K, device=DEV, generator=g).to(FP8)
+    ws = torch.rand((N + 127) // 128, K // 128, device=DEV, generator=g) + 0.5
+    wi = torch.randint(-128, 128, (N, K), device=DEV, generator=g, dtype=torch.int32).to(torch.int8)
+    sb = torch.rand(1, N, device=DEV, generator=g) + 0.5
+    slow = []
+    for M in (1, 17, 48, 100, 200, 600, 1500, 4096):
+        x = torch.randn(M, K, device=DEV, generator=g).to(FP8)
+        xi = torch.randint(-128, 128, (M, K), device=DEV, generator=g, dtype=torch.int32).to(torch.int8)
+        xs = torch.rand(M, K // 128, device=DEV, generator=g) + 0.5
+        sa = torch.rand(M, 1, device=DEV, generator=g) + 0.5
+        for dt in (torch.float16, torch.float32, torch.bfloat16):
+            c = torch.empty(M, N, dtype=dt, device=DEV)
+            calls = {"row/column fp8": lambda: flag_gems.cutlass_scaled_mm(c, x, w.t(), sa, sb, None),
+                     "row/column int8": lambda: flag_gems.cutlass_scaled_mm(c, xi, wi.t(), sa, sb, None)}
+            if dt != torch.bfloat16:  # (bf16 block-scaled: the test above)
+                calls["block"] = lambda: flag_gems.w8a8_block_fp8_matmul(x, w, xs, ws, [128, 128], output_dtype=dt)
+            for name, fn in calls.items():
+                us = _time_us(fn)
+                # fp32 results are twice the bytes; the model counts two per element
+                limit = 2.0 * _model_us(M, N, K) + 20.0 + (2.0 * M * N / 2.5e12 * 1e6 if dt == torch.float32 else 0.0)
+                if us > limit:
+                    slow.append((name, str(dt), M, N, K, round(us, 1), round(limit, 1)))
+    assert not slow, f"(call, type, M, N, K, measured us, limit us): {slow}"
