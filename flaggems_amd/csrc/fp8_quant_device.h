@@ -116,9 +116,25 @@ __device__ __forceinline__ float derive_scale(float amax, const QuantArgs& a) {
     if (s != s) {
       // NaN stays NaN
     } else if (t < __builtin_huge_valf()) {
-      float l = (float)log2((double)t);
-      int k = (int)ceilf(l);
-      s = (k >= -126) ? bits_to_float((uint32_t)(k + 127) << 23) : ldexpf(1.0f, k);
+      // t = 2^n (1 + m 2^-23), n >= -34.  The fp32 logarithm of a t just above 2^n rounds to n itself, and the
+      // ceiling then stays at n: that happens while log2(1 + m 2^-23) is below half the distance from n to the
+      // next fp32 above it, 2^(j - 24) with j = floor(log2 |n|) (one less where n is minus a power of two: the
+      // floats get denser on that side), i.e. for m <= floor(ln 2 * 2^(j - 1)) = 0, 0, 1, 2, 5, 11, 22 for
+      // j = 0 .. 6 (the quotients are 0.35, 0.69, 1.39, 2.77, 5.55, 11.09, 22.18: none is near an integer, and the
+      // second-order term of the logarithm is a millionth of them).  No logarithm is evaluated: the double
+      // precision routine that was here cost as much as the rest of the quantizer together.
+      const uint32_t b = float_to_bits(t);
+      const int n = (int)(b >> 23) - 127;
+      const uint32_t m = b & 0x7FFFFFu;
+      uint32_t keep = 0;  // largest m whose logarithm still rounds to n
+      if (n != 0) {
+        const uint32_t an = (uint32_t)(n < 0 ? -n : n);
+        int j = 31 - __builtin_clz(an);
+        if (n < 0 && (an & (an - 1u)) == 0u) --j;
+        keep = j < 2 ? 0u : (uint32_t)(0.69314718f * (float)(1u << (j - 1)));
+      }
+      const int k = n + (m > keep ? 1 : 0);
+      s = bits_to_float((uint32_t)(k + 127) << 23);
     } else {
       s = t;
     }

@@ -198,3 +198,27 @@ def test_empty_inputs():
     assert y.shape == (0, 256) and s.shape == (0, 2)
     q, s = flag_gems.per_token_group_quant_fp8(torch.empty(0, 256, dtype=torch.bfloat16, device=DEV), 128)
     assert q.shape == (0, 256) and s.shape == (0, 2)
+
+
+def test_power_of_two_scales_next_to_the_powers_of_two():
+    """scale_ue8m0 rounds the scale up to a power of two through ceil(log2(s)) with an fp32 logarithm, which rounds
+    the logarithm of a scale a few steps above 2^n down to n: the kernel decides that case from the bits of the scale.
+    Rows whose maximum walks step by step across 448 * 2^n, for every n the rule distinguishes, against the oracle."""
+    import numpy as np
+    rows = []
+    for n in list(range(-33, 40)) + [60, 64, 65, 100, 119]:
+        base = np.array([448.0 * 2.0 ** n], dtype=np.float32).view(np.uint32)[0]
+        for step in range(-6, 60):
+            rows.append(np.uint32(int(base) + step))
+    amax = torch.from_numpy(np.array(rows, dtype=np.uint32).view(np.float32).copy())
+    assert torch.isfinite(amax).all()
+    g = torch.Generator().manual_seed(0)
+    x = (torch.rand(amax.numel(), 128, generator=g) * 2 - 1) * amax[:, None] * 0.5
+    x[:, 17] = -amax
+    for gs, xx in ((128, x), (64, x[:, 8:72].contiguous())):
+        want_q, want_s = O.per_token_group_quant_fp8_ref(xx, gs, scale_ue8m0=True)
+        q, s = flag_gems.per_token_group_quant_fp8(xx.to(DEV), gs, scale_ue8m0=True)
+        assert torch.equal(s.cpu().view(torch.int32), want_s.view(torch.int32))
+        assert torch.equal(q.cpu().view(torch.uint8), want_q.view(torch.uint8))
+    # the scales are powers of two, and both sides of every boundary were visited
+    assert (want_s.view(torch.int32) & 0x7FFFFF).eq(0).all()
