@@ -361,3 +361,33 @@ def test_per_block_cast_ue8m0_vs_brute_force():
             codes = e4m3.encode((blk * (F32(1.0) / s)).astype(np.float32))
             got = wq.view(torch.uint8).numpy()[bi * 128 : (bi + 1) * 128, bj * 128 : (bj + 1) * 128]
             assert np.array_equal(codes, got)
+
+
+def test_ceil_log2_in_fp32_is_decided_by_the_bits_of_the_scale():
+    """The device code of scale_ue8m0 evaluates no logarithm: for s = 2^n (1 + m 2^-23) it takes n + 1 unless
+    m <= floor(ln 2 * 2^(j - 1)), j = floor(log2 |n|) (one less where n is minus a power of two; 0 for j < 2).  That
+    closed form against the fp32 logarithm the oracle uses (torch) and against a float64 logarithm rounded to fp32, for
+    every exponent the rule can meet and every mantissa near the thresholds, plus a random sample."""
+    import numpy as np
+
+    def closed_form(bits):
+        n = (bits >> 23) - 127
+        m = bits & 0x7FFFFF
+        an = np.abs(n)
+        j = np.where(an > 0, np.floor(np.log2(np.maximum(an, 1))).astype(np.int64), 0)
+        j = j - ((n < 0) & ((an & (an - 1)) == 0)).astype(np.int64)
+        keep = np.where((n != 0) & (j >= 2), np.floor(np.float32(0.69314718) * 2.0 ** (j - 1)).astype(np.int64), 0)
+        return n + (m > keep)
+
+    ns = np.arange(-34, 128)
+    ms = np.concatenate([np.arange(0, 64), 2 ** np.arange(6, 23), np.array([0x7FFFFF, 0x7FFFFE, 0x400000])])
+    bits = (((ns[:, None] + 127) << 23) | ms[None, :]).astype(np.int64).ravel()
+    rng = np.random.default_rng(0)
+    bits = np.concatenate([bits, ((rng.integers(93, 255, 200000) << 23) | rng.integers(0, 1 << 23, 200000)).astype(np.int64)])
+    t = bits.astype(np.uint32).view(np.float32)
+    via_f64 = np.ceil(np.log2(t.astype(np.float64)).astype(np.float32)).astype(np.int64)
+    via_torch = torch.ceil(torch.log2(torch.from_numpy(t.copy()))).numpy().astype(np.int64)
+    got = closed_form(bits)
+    assert (got == via_f64).all() and (got == via_torch).all()
+    # the rounding the rule is about does happen: some scales above 2^n keep n
+    assert ((bits & 0x7FFFFF != 0) & (got == (bits >> 23) - 127)).any()
