@@ -437,15 +437,17 @@ constexpr int kStoresPerTile = 16;
 // SCATTER (grouped problems): rows go where out_index says (see PpArgs::c_rows).
 // JN: activation fragments per wavefront (rows m_base .. m_base + 16 JN).
 // F16: the results are fp16 (else bf16).
-template <int MODE, bool ALIGNED, bool SCATTER = false, int JN = kTM, bool F16 = false>
-__device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[kTN][JN], int m_base, int n_base,
+// NT, q0: `acc` holds the NT MFMA tiles of pieces q0 .. q0 + NT / 2 - 1 (all eight, or the half that the finish of a
+// shared tile sums at a time).
+template <int MODE, bool ALIGNED, bool SCATTER = false, int JN = kTM, bool F16 = false, int NT = kTN>
+__device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[NT][JN], int m_base, int n_base,
                                            int l16, int lg, int m_end, const int* out_index = nullptr, int c_rows = 0,
-                                           const float* row_weight = nullptr) {
+                                           const float* row_weight = nullptr, int q0 = 0) {
   if (MODE != kModeBlock) {
     // eight columns at a time, so that only eight column scales and bias values are live
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int n = piece_column(n_base, q, lg);
+    for (int q = 0; q < NT / 2; ++q) {
+      const int n = piece_column(n_base, q0 + q, lg);
       const bool full = ALIGNED || n + 8 <= a.N;
       float sb[8], bias[8];
 #pragma unroll
@@ -500,23 +502,23 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[k
       if (row_weight != nullptr) wgt = row_weight[idx];
     }
     uint16_t* const row = reinterpret_cast<uint16_t*>(a.C) + out_row * a.ldc;
-    uint32_t w[16];
+    uint32_t w[2 * NT];
     if (SCATTER && row_weight != nullptr) {
 #pragma unroll
-      for (int t = 0; t < kTN; ++t) {
+      for (int t = 0; t < NT; ++t) {
         w[2 * t] = pack_out<F16>(acc[t][j][0] * wgt, acc[t][j][1] * wgt);
         w[2 * t + 1] = pack_out<F16>(acc[t][j][2] * wgt, acc[t][j][3] * wgt);
       }
     } else {
 #pragma unroll
-      for (int t = 0; t < kTN; ++t) {
+      for (int t = 0; t < NT; ++t) {
         w[2 * t] = pack_out<F16>(acc[t][j][0], acc[t][j][1]);
         w[2 * t + 1] = pack_out<F16>(acc[t][j][2], acc[t][j][3]);
       }
     }
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int n = piece_column(n_base, q, lg);
+    for (int q = 0; q < NT / 2; ++q) {
+      const int n = piece_column(n_base, q0 + q, lg);
       if (ALIGNED || n + 8 <= a.N) {
         store_result_16(row + n, u32x4{w[4 * q], w[4 * q + 1], w[4 * q + 2], w[4 * q + 3]});
       } else {
@@ -542,7 +544,7 @@ __device__ __forceinline__ int sk_range_of_step(const PpArgs& a, int step) {
 // share the tile) adds all partial sums in range order -- the same order whoever comes last, so the
 // result does not depend on timing -- stores the piece, and resets the counter for the next launch.
 // Nobody waits for anybody.  On entry and exit no vector-memory operation of this wavefront is pending.
-template <bool F16>
+template <int MODE, bool F16>
 __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (&acc)[kTN][kTM], int tile, int pos,
                                                     int m_base, int n_base, int wave, int lane, int l16, int lg) {
   const int s_lo = tile * a.g.KB;
@@ -586,34 +588,14 @@ __device__ __forceinline__ void finish_partial_tile(const PpArgs& a, const v4f (
       for (int t = 0; t < kTN / 2; ++t)
 #pragma unroll
         for (int j = 0; j < kTM; ++j) {
-          // plain assignment for the first range keeps "0 + x" out of the sum
-          if (q == first) r[t][j] = tmp[t][j]; else r[t][j] += tmp[t][j];
+          // plain assignment for the first range keeps "0 + x" out of the sum; int8 operands: int32 sums, added as such
+          if (q == first) r[t][j] = tmp[t][j];
+          else if (MODE == kModeRowColI8) r[t][j] = __builtin_bit_cast(v4f, __builtin_bit_cast(v4i, r[t][j]) + __builtin_bit_cast(v4i, tmp[t][j]));
+          else r[t][j] += tmp[t][j];
         }
     }
-    // two pieces of eight columns per lane and row: 16-byte stores, or single elements at the ragged edge
-#pragma unroll
-    for (int j = 0; j < kTM; ++j) {
-      const int m = m_base + j * 16 + l16;
-      if (m >= a.g.M) continue;
-      uint16_t* const row = reinterpret_cast<uint16_t*>(a.g.C) + (int64_t)m * a.g.ldc;
-      uint32_t w[8];
-#pragma unroll
-      for (int t = 0; t < kTN / 2; ++t) {
-        w[2 * t] = pack_out<F16>(r[t][j][0], r[t][j][1]);
-        w[2 * t + 1] = pack_out<F16>(r[t][j][2], r[t][j][3]);
-      }
-#pragma unroll
-      for (int qq = 0; qq < 2; ++qq) {
-        const int n = piece_column(n_base, half * 2 + qq, lg);
-        if (n + 8 <= a.g.N) {
-          *reinterpret_cast<u32x4*>(row + n) = u32x4{w[4 * qq], w[4 * qq + 1], w[4 * qq + 2], w[4 * qq + 3]};
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (n + e < a.g.N) row[n + e] = (uint16_t)(w[4 * qq + (e >> 1)] >> (16 * (e & 1)));
-        }
-      }
-    }
+    // (scales and bias of the row/column modes, conversion, 16-byte stores or single elements at the ragged edge)
+    store_tile<MODE, false, false, kTM, F16, kTN / 2>(a.g, r, m_base, n_base, l16, lg, a.g.M, nullptr, 0, nullptr, half * 2);
   }
   if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the counted waits of the main loop start from zero
@@ -901,7 +883,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   };
   auto flush_partial_tile = [&]() __attribute__((always_inline)) {
     wait_vmem<0>();
-    if constexpr (SK) finish_partial_tile<F16>(a, acc, pend_idx, pos, pend_m, pend_n, wave, lane, l16, lg);
+    if constexpr (SK) finish_partial_tile<MODE, F16>(a, acc, pend_idx, pos, pend_m, pend_n, wave, lane, l16, lg);
     clear_acc();
   };
 
@@ -1219,12 +1201,20 @@ void (*pick_kernel(const KernelChoice& c))(PpArgs) {
   if (c.grouped)
     return c.short_tiles ? fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, 1, F16>
                          : fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, kTM, F16>;
-  if (c.mode == kModeRowColI8)
+  if (c.mode == kModeRowColI8) {
+    if (c.sk)
+      return c.aligned ? fp8_gemm_pingpong_kernel<true, kModeRowColI8, true, false, false, kTM, F16>
+                       : fp8_gemm_pingpong_kernel<true, kModeRowColI8, false, false, false, kTM, F16>;
     return c.aligned ? fp8_gemm_pingpong_kernel<false, kModeRowColI8, true, false, false, kTM, F16>
                      : fp8_gemm_pingpong_kernel<false, kModeRowColI8, false, false, false, kTM, F16>;
-  if (c.mode != kModeBlock)
+  }
+  if (c.mode != kModeBlock) {
+    if (c.sk)
+      return c.aligned ? fp8_gemm_pingpong_kernel<true, kModeRowCol, true, false, false, kTM, F16>
+                       : fp8_gemm_pingpong_kernel<true, kModeRowCol, false, false, false, kTM, F16>;
     return c.aligned ? fp8_gemm_pingpong_kernel<false, kModeRowCol, true, false, false, kTM, F16>
                      : fp8_gemm_pingpong_kernel<false, kModeRowCol, false, false, false, kTM, F16>;
+  }
   if (c.pow2) {
     if (c.sk)
       return c.aligned ? fp8_gemm_pingpong_kernel<true, kModeBlock, true, false, true, kTM, F16>
@@ -1328,7 +1318,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     FG_CHECK_LAUNCH("transpose_scales_kernel");
     a.g.xs = xs_t; a.g.xs_rs = 1; a.g.xs_cs = scale_rows;
   }
-  if (mode == kModeBlock && sk.use && workspace != nullptr && workspace_bytes >= need && (size_t)sk.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
+  if (sk.use && workspace != nullptr && workspace_bytes >= need && (size_t)sk.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
       (uintptr_t)workspace % 16 == 0) {
     a.sk = 1; a.sk_q = sk.q; a.sk_r = sk.r; a.sk_split = sk.split;
     a.counters = reinterpret_cast<unsigned int*>(workspace);

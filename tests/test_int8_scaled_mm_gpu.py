@@ -154,6 +154,28 @@ def test_int8_sums_are_exact_up_to_64_rows(M, N, K):
         assert call(None, 0) == -3  # FG_ERR_WORKSPACE
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_int8_tiles_shared_between_compute_units_are_exact(out_dtype):
+    """Few 256 x 256 tiles with a long K: compute units take ranges of K-blocks and add their int32 sums through the
+    workspace.  Sparse operands keep every sum small enough for the 16-bit result to hold it exactly; the bias is
+    added in the result type."""
+    M, N, K = 384, 5632, 8320
+    g = torch.Generator().manual_seed(9)
+    a = (torch.randint(-1, 2, (M, K), generator=g) * (torch.rand(M, K, generator=g) < 0.1)).to(torch.int8)
+    b = (torch.randint(-1, 2, (N, K), generator=g) * (torch.rand(N, K, generator=g) < 0.1)).to(torch.int8)
+    a[0, :] = 1
+    b[0, :256] = 1
+    b[0, 256:] = 0
+    one = torch.ones(1, device=DEV)
+    bias = torch.randint(-8, 9, (N,), generator=g).to(out_dtype)
+    want = a.float() @ b.float().t()  # integers far below 2^24: exact
+    assert want.abs().max() <= 256 and want[0, 0] == 256
+    for use_bias in (False, True):
+        c = torch.empty(M, N, dtype=out_dtype, device=DEV)
+        flag_gems.cutlass_scaled_mm(c, a.to(DEV), b.to(DEV).t(), one, one, bias.to(DEV) if use_bias else None)
+        assert torch.equal(c.cpu().float(), want + (bias.float() if use_bias else 0.0))
+
+
 def test_int8_through_aten_scaled_mm():
     a, b, sa, sb = _inputs(64, 128, 256, 4, "vector", "vector")
     want = O.scaled_mm_ref(a, b, sa, sb, torch.bfloat16)
