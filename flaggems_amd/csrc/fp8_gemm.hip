@@ -751,10 +751,15 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
   const bool big = a.M > 128;
   if (direct && pingpong_takes(a, MODE, workspace, workspace_bytes)) return launch_pingpong(a, MODE, workspace, workspace_bytes, stream);
   if (big) {
-    // Row/column modes whose result the persistent kernel does not write (fp32, fp8, rows that take no 16-byte
-    // stores): 128 x 128 tiles.  The 256 x 256 instantiation of these modes does not fit the registers (40 spilled):
-    // fp32 results, M = 4096, N = 7168: K = 2304 438 -> 124 us, K = 16384 3129 -> 467 us; M = 2048, N = K = 8192: 728 -> 148 us.
-    if (MODE != kModeBlock && direct) return launch_cfg<128, 128, 4, 2, MODE, true>(a, stream);
+    // Row/column modes that the persistent kernel does not take (fp32 or fp8 results, rows that take no 16-byte
+    // stores, K not a multiple of 128): 128 x 128 tiles.  The 256 x 256 instantiation of these modes does not fit the
+    // registers (40 spilled): fp32 results, M = 4096, N = 7168: K = 2304 438 -> 124 us, K = 16384 3129 -> 467 us;
+    // K = 4160 (loads through registers), M = N = 4096, bf16: fp8 382 -> 107 us, int8 755 -> 129 us.
+    if (MODE != kModeBlock)
+      return direct ? launch_cfg<128, 128, 4, 2, MODE, true>(a, stream) : launch_cfg<128, 128, 4, 2, MODE, false>(a, stream);
+    // block scales through registers: 256 x 256 tiles once they fill the compute units (M = N = 4096, K = 4160: 98
+    // against 120 us), 128 x 128 below (M = 1024: 88 -> 43 us; M = 256: 83 -> 34 us)
+    if (!direct && ceil_div(a.M, 256) * ceil_div(a.N, 256) < cu_count()) return launch_cfg<128, 128, 4, 2, MODE, false>(a, stream);
     return direct ? launch_cfg<256, 256, 4, 2, MODE, true>(a, stream)
                   : launch_cfg<256, 256, 4, 2, MODE, false>(a, stream);
   }

@@ -40,7 +40,8 @@ def _quantized_inputs(M, N, K, seed=0):
     return xq, wq, xs, ws
 
 
-REF_SHAPES = [(128, 256, 512), (64, 128, 128), (256, 256, 256), (83, 7748, 3884), (84, 7168, 3884)]
+REF_SHAPES = [(128, 256, 512), (64, 128, 128), (256, 256, 256), (83, 7748, 3884), (84, 7168, 3884),
+              (300, 520, 3884), (1100, 1000, 1000)]  # K not a multiple of 128 above 128 rows
 
 
 @pytest.mark.parametrize("M,N,K", REF_SHAPES)

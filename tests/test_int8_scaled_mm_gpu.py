@@ -42,7 +42,9 @@ def _exact(a, b, sa, sb):
                                    (1, 4096, 4096), (8, 2112, 7168), (16, 7168, 2304), (32, 1024, 8192), (5, 24592, 384),
                                    (12, 32768, 512), (20, 520, 1024),
                                    # 33..64 rows: the kernel with the activations of a K range in LDS
-                                   (33, 2112, 7168), (64, 4096, 4096), (48, 24576, 1536), (40, 264, 512)])
+                                   (33, 2112, 7168), (64, 4096, 4096), (48, 24576, 1536), (40, 264, 512),
+                                   # K that is not a multiple of 128 above 128 rows
+                                   (300, 1040, 4160), (1030, 528, 1040)])
 @pytest.mark.parametrize("kinds", [("scalar", "scalar"), ("vector", "vector"), ("vector", "scalar")])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16])
 def test_int8_cutlass_scaled_mm(M, N, K, kinds, out_dtype):

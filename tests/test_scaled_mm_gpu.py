@@ -24,6 +24,8 @@ MNK = [
     (512, 16384, 128), (512, 24576, 128), (8, 20496, 1536),
     # few 256 x 256 tiles with a long K: compute units share tiles and add their sums through the workspace
     (384, 5632, 8320), (300, 3088, 8448),
+    # K that is not a multiple of 128 (operands go through registers), above and below 128 rows
+    (300, 1040, 4160), (1030, 2064, 1040), (40, 528, 400),
 ]
 
 
