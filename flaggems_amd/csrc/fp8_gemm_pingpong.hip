@@ -623,28 +623,40 @@ __device__ __forceinline__ void finish_cut_tile(const PpArgs& a, const v4f (&acc
   if (lane == 0) prev = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   prev = (unsigned int)__builtin_amdgcn_readfirstlane((int)prev);
   if (prev != (unsigned int)(cuts - 1)) return;
-  v4f r[kTN][JN];
-  for (int q = 0; q < cuts; ++q) {
-    const float* const src = uniform_ptr(a.partials + ((size_t)((tile << a.cut_shift) + q) * 8 + wave) * kFloats);
-    v4f tmp[kTN][JN];
+  // Half of the piece at a time (its own sums are in the workspace like everybody's, so the accumulators are free),
+  // sixteen registers of partial sums in flight: with two fragments per wavefront more does not fit the registers.
+  constexpr int kPart = 4 / JN;  // MFMA tiles per load batch
 #pragma unroll
-    for (int t = 0; t < kTN; ++t)
+  for (int half = 0; half < 2; ++half) {
+    v4f r[kTN / 2][JN];
+    for (int q = 0; q < cuts; ++q) {
+      const float* const src = uniform_ptr(a.partials + ((size_t)((tile << a.cut_shift) + q) * 8 + wave) * kFloats);
 #pragma unroll
-      for (int j = 0; j < JN; ++j) load_x4_agent(tmp[t][j], src + (t * JN + j) * 256, lane_off);
+      for (int part = 0; part < kTN / 2 / kPart; ++part) {
+        v4f tmp[kPart][JN];
 #pragma unroll
-    for (int t = 0; t < kTN; ++t)
+        for (int t = 0; t < kPart; ++t)
 #pragma unroll
-      for (int j = 0; j < JN; ++j)  // the values are operands of the wait, so no use can move above it
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[t][j]) : : "memory");
+          for (int j = 0; j < JN; ++j)
+            load_x4_agent(tmp[t][j], src + ((half * (kTN / 2) + part * kPart + t) * JN + j) * 256, lane_off);
 #pragma unroll
-    for (int t = 0; t < kTN; ++t)
+        for (int t = 0; t < kPart; ++t)
 #pragma unroll
-      for (int j = 0; j < JN; ++j) {
-        if (q == 0) r[t][j] = tmp[t][j]; else r[t][j] += tmp[t][j];  // (no "0 + x" in the sum)
+          for (int j = 0; j < JN; ++j)  // the values are operands of the wait, so no use can move above it
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[t][j]) : : "memory");
+#pragma unroll
+        for (int t = 0; t < kPart; ++t)
+#pragma unroll
+          for (int j = 0; j < JN; ++j) {
+            const int tt = part * kPart + t;
+            if (q == 0) r[tt][j] = tmp[t][j]; else r[tt][j] += tmp[t][j];  // (no "0 + x" in the sum)
+          }
       }
+    }
+    store_tile<kModeBlock, false, SCATTER, JN, F16, kTN / 2>(a.g, r, m_base, n_base, l16, lg, m_end,
+                                                             SCATTER && a.c_rows > 0 ? a.row_index : nullptr, a.c_rows,
+                                                             a.row_weight, half * 2);
   }
-  store_tile<kModeBlock, false, SCATTER, JN, F16>(a.g, r, m_base, n_base, l16, lg, m_end, SCATTER && a.c_rows > 0 ? a.row_index : nullptr,
-                                                  a.c_rows, a.row_weight);
   if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the counted waits of the main loop start from zero
 }
@@ -1184,23 +1196,25 @@ constexpr size_t kCutSlotBytes = (size_t)8 * kTN * 256 * 4;  // a work item's pa
 constexpr int kMaxCutItems = 1024;                           // work items of a cut problem (64 MB of partial sums)
 // Largest number of cuts per tile of the last round, as a shift (the kernel picks among 0..this from the real tile
 // count): whole K-blocks, at least 8 per cut, and slots for a round short of one tile.
-int max_cut_shift(int grid, int KB) {
+int max_cut_shift(int grid, int KB, int jn) {
   int sh = 0;
-  while (sh < 2 && KB % (2 << sh) == 0 && (KB >> (sh + 1)) >= 8 && ((int64_t)(grid - 1) << (sh + 1)) <= kMaxCutItems) ++sh;
+  while (sh < 2 && KB % (2 << sh) == 0 && (KB >> (sh + 1)) >= 8 && ((int64_t)(grid - 1) << (sh + 1)) * jn <= kMaxCutItems) ++sh;
   return sh;
 }
 
 // The instantiation that serves a launch.
 struct KernelChoice {
-  bool grouped, short_tiles;
+  bool grouped;
+  int short_jn;  // grouped problems on short tiles: 16-row fragments per wavefront (1 or 2), else 0
   int mode;
   bool sk, aligned, pow2;
 };
 template <bool F16>
 void (*pick_kernel(const KernelChoice& c))(PpArgs) {
   if (c.grouped)
-    return c.short_tiles ? fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, 1, F16>
-                         : fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, kTM, F16>;
+    return c.short_jn == 1   ? fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, 1, F16>
+           : c.short_jn == 2 ? fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, 2, F16>
+                             : fp8_gemm_pingpong_kernel<false, kModeBlock, false, true, false, kTM, F16>;
   if (c.mode == kModeRowColI8) {
     if (c.sk)
       return c.aligned ? fp8_gemm_pingpong_kernel<true, kModeRowColI8, true, false, false, kTM, F16>
@@ -1255,15 +1269,26 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   PpArgs a = {};
   a.g = g;
   a.g.tiles_m = (int)ceil_div(g.M, kBM);
-  // Grouped problems whose segments average at most a short tile's rows take 64-row tiles (the JN = 1
-  // instantiation); the host sees only the total, and a segment longer than a tile then reads its weights once per
-  // 64 rows.  Measured on 8 segments, [28672, 4096] | [4096, 14336] weights each, 256-row -> 64-row tiles:
-  // 16 rows a segment on average 292 -> 202 | 200 -> 114 us, 32: 292 -> 214 | 206 -> 171, 64: 296 -> 291 | 221 -> 177,
-  // 128: 300 -> 415 | 204 -> 216.
-  const bool short_tiles = grouped != nullptr && g.M <= (int64_t)kShortTileRows * grouped->n_groups;
+  // Grouped problems with few rows per segment take tiles of 64 or 128 rows (the JN = 1 and 2 instantiations).  The
+  // host sees only the average; a segment longer than a tile reads its weights once per tile, and where the tiles
+  // are few (at most half the compute units when every segment has one) a longer segment also costs a round of its
+  // own, so those take the next tile height sooner.  Measured on 8 segments, [28672, 4096] | [4096, 14336] weights
+  // each (896 | 128 tiles), us for 256- / 64- / 128-row tiles by rows a segment on average:
+  //    16: 333 222 249 | 203 112 125     32: 295 223 240 | 207 170 128     64: 303 295 243 | 222 178 192
+  //    96: 303 336 288 | 219 181 189    128: 293 415 318 | 202 217 182     256: 404 705 463 | 213 351 269
+  int short_jn = 0;
+  if (grouped != nullptr) {
+    const int64_t E = grouped->n_groups;
+    const bool few_tiles = E * ceil_div(g.N, kBN) * 2 <= cu_count();
+    if (g.M <= 16 * E) short_jn = 1;
+    else if (g.M <= 32 * E) short_jn = few_tiles ? 2 : 1;
+    else if (g.M <= 96 * E) short_jn = 2;
+    else if (g.M <= 128 * E) short_jn = few_tiles ? 2 : 0;
+  }
+  const bool short_tiles = short_jn != 0;
   if (grouped != nullptr) {
     // every segment ends with at most one tile that is not full; the kernel counts the real tiles
-    const int tile_rows = short_tiles ? kShortTileRows : kBM;
+    const int tile_rows = short_tiles ? kShortTileRows * short_jn : kBM;
     const int64_t bound = g.M / tile_rows + grouped->n_groups;
     a.g.tiles_m = (int)(bound < g.M ? bound : g.M);
     a.groups = grouped->ends; a.n_groups = (int)grouped->n_groups;
@@ -1291,7 +1316,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   a.cut_steps = g.KB;
   if (short_tiles) {
     // (the grid is the compute units, also where the bound of the tile count is lower: cuts may fill them)
-    const int sh = max_cut_shift(cus, g.KB);
+    const int sh = max_cut_shift(cus, g.KB, short_jn);
     const size_t bytes = (size_t)kMaxCutItems * kCutSlotBytes;
     if (sh > 0 && workspace != nullptr && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= FG_WORKSPACE_COUNTER_BYTES + bytes &&
         (size_t)cus * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES) {
@@ -1336,7 +1361,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   const bool aligned = g.M % kBM == 0 && g.N % kBN == 0;
   const bool pow2 = mode == kModeBlock && grouped == nullptr && g.scales_pow2 != 0;
   const bool f16 = g.c_dtype == FG_F16;
-  const KernelChoice which = {grouped != nullptr, short_tiles, mode, a.sk != 0, aligned, pow2};
+  const KernelChoice which = {grouped != nullptr, short_jn, mode, a.sk != 0, aligned, pow2};
   void (*const kern)(PpArgs) = f16 ? pick_kernel<true>(which) : pick_kernel<false>(which);
   if (const int rc = allow_full_lds(kern)) return rc;
   if (tp.use && !a.sk && workspace != nullptr && workspace_bytes >= need && (size_t)tp.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&

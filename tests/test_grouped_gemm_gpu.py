@@ -57,6 +57,9 @@ CASES = [
     (96, 264, 2048, [0, 1, 1, 40, 40, 41, 90, 96]),    # N ends inside a tile; empty and one-row segments
     (300, 256, 3072, [0, 200, 200, 230, 299, 300, 300, 300]),  # a segment of several short tiles
     (16, 1024, 7168, None),                            # more segments than rows have tokens
+    # 33 .. 128 rows per segment on average: 128-row tiles, also cut along K
+    (512, 512, 4096, None),
+    (1000, 2144, 1024, [90, 130, 400, 401, 401, 640, 880, 1000]),
 ]
 
 
@@ -138,7 +141,8 @@ def test_unsupported_requests_fail_loudly():
                                                 ends.to(DEV), [128, 128])
 
 
-@pytest.mark.parametrize("T,N,K,top_k", [(64, 1024, 1024, 2), (700, 2144, 512, 2), (1500, 768, 2048, 1), (333, 640, 256, 4)])
+@pytest.mark.parametrize("T,N,K,top_k", [(64, 1024, 1024, 2), (700, 2144, 512, 2), (1500, 768, 2048, 1), (333, 640, 256, 4),
+                                         (256, 1024, 1024, 2), (200, 512, 4096, 2)])
 def test_rows_gathered_through_an_index(T, N, K, top_k):
     """row_index: the kernel reads row sorted_token_ids[m] // top_k of the token matrix for sorted row m, as the
     reference's MoE kernel does (src/flag_gems/fused/fused_moe.py:1111), instead of a copy of the activations in
@@ -193,7 +197,7 @@ def _aligned_layout(expert_of, E, block_m):
 
 @pytest.mark.parametrize("weighted", [False, True])
 @pytest.mark.parametrize("T,N,K,top_k,block_m", [(64, 1024, 1024, 2, 16), (700, 2144, 512, 2, 64), (333, 640, 256, 4, 64),
-                                                 (1500, 768, 2048, 1, 128)])
+                                                 (1500, 768, 2048, 1, 128), (256, 1024, 1024, 2, 32), (200, 512, 4096, 2, 16)])
 def test_results_scattered_and_weighted_like_the_moe_kernel(T, N, K, top_k, block_m, weighted):
     """The whole GEMM of the reference's MoE kernel (src/flag_gems/fused/fused_moe.py:1084-1125, 1484-1509): rows read
     through sorted_token_ids // top_k, results written to row sorted_token_ids[m] of a [T * top_k, N] matrix, padding
