@@ -308,7 +308,7 @@ int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_batch_stride
  * slower general path behind this entry point).
  * `workspace` (optional, 16-byte aligned, fg_grouped_block_fp8_gemm_workspace_bytes(M, N, K) bytes, first
  * FG_WORKSPACE_COUNTER_BYTES zero-filled once) lets row-major As be read from a transposed copy and, when the
- * groups average at most 64 rows (M <= 64 * n_groups), lets tiles be cut along K so that few tiles fill the GPU
+ * groups average at most 128 rows (M <= 128 * n_groups), lets tiles be cut along K so that few tiles fill the GPU
  * (64 MB of partial sums; the sums are added in a fixed order, but not in the order of the call without workspace).
  * row_index (optional DEVICE table of M int32): the kernel gathers its rows itself -- row m of the sorted order
  * (the order of group_ends and of C) is row row_index[m] / index_div of A and As, which then have a_rows rows
