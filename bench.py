@@ -254,6 +254,30 @@ def main():
                 row["read_floor_over_us"] = round(read_floor[(n, k)] / us, 4)
             detail.append(row)
 
+    # what the matrix pipes take of the kernel's own multiply phase when nothing else happens (fg_mfma_issue_probe:
+    # operands in registers, no LDS, no memory), on the bytes of a quantized weight of the sweep: the part holds a
+    # lower clock under matrix load than the one the published peak assumes
+    mfma_probe = fg_lib.load().fg_mfma_issue_probe
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    probe_ops = weights[DSV3_NK[0]][0][0]
+
+    def mfma_ceiling(with_fmas):
+        iters = 1500  # ~2.5 ms: long enough for the clock to settle
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        best = float("inf")
+        for rep in range(4):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            assert mfma_probe(probe_ops.data_ptr(), iters, with_fmas, None, stream) == 0
+            end.record()
+            end.synchronize()
+            if rep > 0:
+                best = min(best, start.elapsed_time(end) * 1e-3)
+        return iters * 32 * 65536.0 * 8 * cus / best / 1e12
+
+    ceiling_block = mfma_ceiling(1)
+    ceiling_plain = mfma_ceiling(0)
+
     big = [d for d in detail if d["M"] == 4096]
     big_flops = sum(gemm_flops(d["M"], d["N"], d["K"]) for d in big)
     big_time = sum(d["us"] for d in big) * 1e-6
@@ -267,7 +291,13 @@ def main():
                 "flops_per_launch": big_flops / len(big), "algorithmic_bytes_per_launch":
                     sum(gemm_bytes(d["M"], d["N"], d["K"]) for d in big) / len(big),
                 "avg_launch_us": round(big_time * 1e6 / len(big), 2),
-                "kernel": "fp8_gemm_pingpong_kernel (with the scale transposition that precedes it), the six M=4096 calls of the sweep"}
+                "kernel": "fp8_gemm_pingpong_kernel (with the scale transposition that precedes it), the six M=4096 calls of the sweep",
+                "mfma_issue_ceiling": {
+                    "block_scaled_mix": round(ceiling_block, 1), "mfma_only": round(ceiling_plain, 1), "unit": "TFLOP/s",
+                    "frac_of_block_scaled_mix": round(achieved / ceiling_block, 4),
+                    "what": "fg_mfma_issue_probe measured in this run: the kernel's multiply phase alone (8 wavefronts per "
+                            "compute unit, MFMA 16x16x128 e4m3 on a quantized weight's bytes held in registers, with / "
+                            "without the four scale FMAs per MFMA; no LDS, no memory, no barriers)"}}
     small = [d for d in detail if d["M"] <= 16]
     small_bytes = sum(gemm_bytes(d["M"], d["N"], d["K"]) for d in small)
     small_time = sum(d["us"] for d in small) * 1e-6

@@ -39,6 +39,7 @@ SIGNATURES = {
     "fg_last_error_string": (c_char_p, []),
     "fg_stream_capture_id": (c_uint64, [c_void_p]),
     "fg_stream_read_probe": (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
+    "fg_mfma_issue_probe": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "fg_group_quant_fp8": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64,

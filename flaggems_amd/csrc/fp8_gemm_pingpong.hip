@@ -1456,3 +1456,72 @@ int launch_pingpong(const GemmArgs& g, int mode, void* workspace, size_t workspa
 }
 
 }  // namespace fg
+
+// ---------------------------------------------------------------------------------------------
+// Measurement aid: the rate at which the matrix pipes take the multiply phase's instruction stream when nothing
+// else happens -- eight wavefronts per compute unit, operands in registers, 32 accumulator tiles per wavefront as in
+// the GEMM, no LDS, no memory, no barriers.  with_scale_fmas != 0: every MFMA starts from zero and four FMAs add
+// its result times a scale to the accumulators two steps later (the block-scaled form); 0: the MFMAs accumulate
+// (the row/column form).  The part holds a lower clock under matrix load than the one its peak is quoted at, and
+// how much lower depends on the operand bits: `operands` (at least 64 KB of device memory) supplies them, so a
+// benchmark can pass the bytes of its own quantized matrices.  The launch performs
+// iterations * 32 * 65536 * 8 * (compute units) flops.
+// ---------------------------------------------------------------------------------------------
+namespace fg {
+namespace {
+template <bool SCALE>
+__global__ __launch_bounds__(kThreads) void mfma_issue_kernel(const uint8_t* __restrict__ operands, int iterations, float* sink) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  v8i w[3], x[kTM];
+  // 7 fragments of 64 lanes x 32 bytes per wavefront, 8 wavefronts: 112 KB would be more than promised; the
+  // wavefronts of a block share four fragment sets
+  const uint8_t* const base = operands + (size_t)(wave & 3) * 7 * 2048;
+#pragma unroll
+  for (int i = 0; i < 3; ++i) w[i] = *reinterpret_cast<const v8i*>(base + (size_t)i * 2048 + lane * 32);
+#pragma unroll
+  for (int j = 0; j < kTM; ++j) x[j] = *reinterpret_cast<const v8i*>(base + (size_t)(3 + j) * 2048 + lane * 32);
+  float sc[kTM];
+#pragma unroll
+  for (int j = 0; j < kTM; ++j) sc[j] = 1.0f + 0.001f * (float)((lane + j) & 15);
+  v4f acc[kTN][kTM];
+#pragma unroll
+  for (int t = 0; t < kTN; ++t)
+#pragma unroll
+    for (int j = 0; j < kTM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+  for (int it = 0; it < iterations; ++it) {
+    if (SCALE) {
+      v4f p[3];
+#pragma unroll
+      for (int st = 0; st < kTN * kTM; ++st) {
+        p[st % 3] = mfma_partial(w[(st / kTM) % 3], x[st % kTM]);
+        if (st >= 2) scale_into<0>(acc[(st - 2) / kTM][(st - 2) % kTM], p[(st - 2) % 3], sc[(st - 2) % kTM]);
+      }
+      constexpr int L = kTN * kTM;
+      scale_into<0>(acc[(L - 2) / kTM][(L - 2) % kTM], p[(L - 2) % 3], sc[(L - 2) % kTM]);
+      scale_into<4>(acc[(L - 1) / kTM][(L - 1) % kTM], p[(L - 1) % 3], sc[(L - 1) % kTM]);
+    } else {
+#pragma unroll
+      for (int st = 0; st < kTN * kTM; ++st) mfma_accumulate(acc[st / kTM][st % kTM], w[(st / kTM) % 3], x[st % kTM]);
+    }
+  }
+  // the work must not be optimised away; the store happens for no real input
+  float sum = 0.f;
+#pragma unroll
+  for (int t = 0; t < kTN; ++t)
+#pragma unroll
+    for (int j = 0; j < kTM; ++j) sum += acc[t][j][0] + acc[t][j][1] + acc[t][j][2] + acc[t][j][3];
+  if (sum == 1.2345678e-30f && sink) sink[0] = sum;
+}
+}  // namespace
+}  // namespace fg
+
+extern "C" int fg_mfma_issue_probe(const void* operands, int iterations, int with_scale_fmas, void* sink, void* stream) {
+  using namespace fg;
+  if (!operands || (uintptr_t)operands % 32 != 0) FG_FAIL(FG_ERR_INVALID_ARG, "fg_mfma_issue_probe: operands must be a 32-byte aligned device pointer");
+  if (iterations < 1) FG_FAIL(FG_ERR_INVALID_ARG, "fg_mfma_issue_probe: %d iterations", iterations);
+  const dim3 grid((uint32_t)cu_count()), block(kThreads);
+  if (with_scale_fmas) FG_LAUNCH(mfma_issue_kernel<true>, grid, block, 0, (hipStream_t)stream, reinterpret_cast<const uint8_t*>(operands), iterations, reinterpret_cast<float*>(sink));
+  else FG_LAUNCH(mfma_issue_kernel<false>, grid, block, 0, (hipStream_t)stream, reinterpret_cast<const uint8_t*>(operands), iterations, reinterpret_cast<float*>(sink));
+  FG_CHECK_LAUNCH("mfma_issue_kernel");
+  return FG_OK;
+}

@@ -175,3 +175,23 @@ def test_decode_kernels_replayed_from_a_graph(M, N, K):
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
         assert not torch.equal(other, eager)
+
+
+def test_measurement_probes_run_and_check_their_arguments():
+    """fg_stream_read_probe and fg_mfma_issue_probe are what bench.py puts its figures next to: both must run on any
+    input they accept and refuse what they cannot take."""
+    lib = _lib.load()
+    stream = _lib.current_stream_ptr(torch.device(DEV))
+    buf = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device=DEV)
+    sink = torch.zeros(4, dtype=torch.int32, device=DEV)
+    assert lib.fg_stream_read_probe(buf.data_ptr(), buf.numel(), sink.data_ptr(), stream) == 0
+    assert lib.fg_stream_read_probe(buf.data_ptr(), 0, None, stream) == 0
+    assert lib.fg_stream_read_probe(buf.data_ptr() + 8, 1024, None, stream) == _lib.FG_ERR_INVALID_ARG
+    for with_fmas in (0, 1):
+        assert lib.fg_mfma_issue_probe(buf.data_ptr(), 3, with_fmas, None, stream) == 0
+        assert lib.fg_mfma_issue_probe(buf.data_ptr(), 1, with_fmas, sink.data_ptr(), stream) == 0
+    assert lib.fg_mfma_issue_probe(None, 3, 1, None, stream) == _lib.FG_ERR_INVALID_ARG
+    assert lib.fg_mfma_issue_probe(buf.data_ptr() + 8, 3, 1, None, stream) == _lib.FG_ERR_INVALID_ARG
+    assert lib.fg_mfma_issue_probe(buf.data_ptr(), 0, 1, None, stream) == _lib.FG_ERR_INVALID_ARG
+    torch.cuda.synchronize()
+    assert int(sink.abs().sum()) == 0  # the sinks are written for no real input
