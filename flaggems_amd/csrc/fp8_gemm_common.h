@@ -6,8 +6,11 @@
 namespace fg {
 
 // kModeRowColI8: int8 operands, int32 sums (kept as bit patterns in the fp32 accumulator registers), scales and
-// bias as kModeRowCol.  Only the tile kernel has it.
-enum { kModeBlock = 0, kModeRowCol = 1, kModeRowColI8 = 2 };
+// bias as kModeRowCol.
+// kModeRowColBF16 / kModeRowColF16 (persistent kernel only): bf16 / fp16 operands, whose rows the kernels take as
+// bytes (a 128-byte K-block is 64 elements); row and column scales, and the bias is added in fp32 before the one
+// rounding, as aten::_scaled_mm's generic kernel does (src/flag_gems/ops/scaled_mm.py:37-133).
+enum { kModeBlock = 0, kModeRowCol = 1, kModeRowColI8 = 2, kModeRowColBF16 = 3, kModeRowColF16 = 4 };
 
 struct GemmArgs {
   const uint8_t* X;  // activations [M, K]

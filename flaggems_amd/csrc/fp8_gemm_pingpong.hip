@@ -323,11 +323,16 @@ __device__ __forceinline__ void mfma_accumulate(v4f& c, const v8i& w, const v8i&
 // the K-block, 1: its second 16), int32 sums kept as bit patterns in the accumulator registers; the two instructions
 // take as long as the one fp8 instruction.  The multiply phase issues the two halves of one accumulator kTM
 // instructions apart, so that the matrix pipe never waits for the sum it has just started.
-__device__ __forceinline__ void mfma_accumulate_i8_half(v4f& c, const v8i& w, const v8i& x, int half) {
+// bf16 and fp16 operands (kModeRowColBF16 / F16) take the same route: a lane's 16 bytes are eight elements, the
+// fragment two 16x16x32 products into fp32 sums, and the pair again takes as long as the one fp8 instruction.
+template <int MODE>
+__device__ __forceinline__ void mfma_accumulate_half(v4f& c, const v8i& w, const v8i& x, int half) {
   typedef int v4i_ __attribute__((ext_vector_type(4)));
   const v4i_ wh = half ? v4i_{w[4], w[5], w[6], w[7]} : v4i_{w[0], w[1], w[2], w[3]};
   const v4i_ xh = half ? v4i_{x[4], x[5], x[6], x[7]} : v4i_{x[0], x[1], x[2], x[3]};
-  asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(c) : "v"(wh), "v"(xh));
+  if constexpr (MODE == kModeRowColBF16) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(wh), "v"(xh));
+  else if constexpr (MODE == kModeRowColF16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(wh), "v"(xh));
+  else asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(c) : "v"(wh), "v"(xh));
 }
 
 // Scales that are powers of two (POW2): the block-scaled form of the instruction multiplies the products by
@@ -470,8 +475,13 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[N
           const float r0 = acc[t][j][e0], r1 = acc[t][j][e0 + 1];
           const float s0 = MODE == kModeRowColI8 ? (float)__float_as_int(r0) : r0;
           const float s1 = MODE == kModeRowColI8 ? (float)__float_as_int(r1) : r1;
-          const float v0 = (s0 * sa) * sb[4 * (h >> 1) + e0];
-          const float v1 = (s1 * sa) * sb[4 * (h >> 1) + e0 + 1];
+          float v0 = (s0 * sa) * sb[4 * (h >> 1) + e0];
+          float v1 = (s1 * sa) * sb[4 * (h >> 1) + e0 + 1];
+          if (MODE >= kModeRowColBF16) {  // one rounding, the bias before it
+            if (a.bias) { v0 = v0 + bias[4 * (h >> 1) + e0]; v1 = v1 + bias[4 * (h >> 1) + e0 + 1]; }
+            w[h] = pack_out<F16>(v0, v1);
+            continue;
+          }
           w[h] = pack_out<F16>(v0, v1);
           if (a.bias)
             w[h] = pack_out<F16>(unpack_lo<F16>(w[h]) + bias[4 * (h >> 1) + e0],
@@ -983,17 +993,17 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
 
     // ================= multiply(T)
     __builtin_amdgcn_s_setprio(kMultiplyPrio);
-    if (MODE == kModeRowColI8) {
-      // int8: per row of tiles first the JN products of the lower K half, then those of the upper
+    if (MODE >= kModeRowColI8) {
+      // int8, bf16, fp16: per row of tiles first the JN products of the lower K half, then those of the upper
 #pragma unroll
       for (int t = 0; t < kTN; ++t) {
 #pragma unroll
         for (int j = 0; j < JN; ++j) {
-          mfma_accumulate_i8_half(acc[t][j], wr[t % 3], xf[j], 0);
+          mfma_accumulate_half<MODE>(acc[t][j], wr[t % 3], xf[j], 0);
           if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
         }
 #pragma unroll
-        for (int j = 0; j < JN; ++j) mfma_accumulate_i8_half(acc[t][j], wr[t % 3], xf[j], 1);
+        for (int j = 0; j < JN; ++j) mfma_accumulate_half<MODE>(acc[t][j], wr[t % 3], xf[j], 1);
       }
     } else if (MODE != kModeBlock) {
       // row/column mode: the matrix pipe accumulates; scales and bias wait for the epilogue
@@ -1222,6 +1232,13 @@ void (*pick_kernel(const KernelChoice& c))(PpArgs) {
     return c.aligned ? fp8_gemm_pingpong_kernel<false, kModeRowColI8, true, false, false, kTM, F16>
                      : fp8_gemm_pingpong_kernel<false, kModeRowColI8, false, false, false, kTM, F16>;
   }
+  // (16-bit operands: their entry point has no workspace, so tiles are never shared)
+  if (c.mode == kModeRowColBF16)
+    return c.aligned ? fp8_gemm_pingpong_kernel<false, kModeRowColBF16, true, false, false, kTM, F16>
+                     : fp8_gemm_pingpong_kernel<false, kModeRowColBF16, false, false, false, kTM, F16>;
+  if (c.mode == kModeRowColF16)
+    return c.aligned ? fp8_gemm_pingpong_kernel<false, kModeRowColF16, true, false, false, kTM, F16>
+                     : fp8_gemm_pingpong_kernel<false, kModeRowColF16, false, false, false, kTM, F16>;
   if (c.mode != kModeBlock) {
     if (c.sk)
       return c.aligned ? fp8_gemm_pingpong_kernel<true, kModeRowCol, true, false, false, kTM, F16>
@@ -1343,7 +1360,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     FG_CHECK_LAUNCH("transpose_scales_kernel");
     a.g.xs = xs_t; a.g.xs_rs = 1; a.g.xs_cs = scale_rows;
   }
-  if (sk.use && workspace != nullptr && workspace_bytes >= need && (size_t)sk.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
+  if (sk.use && mode < kModeRowColBF16 && workspace != nullptr && workspace_bytes >= need && (size_t)sk.grid * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES &&
       (uintptr_t)workspace % 16 == 0) {
     a.sk = 1; a.sk_q = sk.q; a.sk_r = sk.r; a.sk_split = sk.split;
     a.counters = reinterpret_cast<unsigned int*>(workspace);

@@ -46,7 +46,9 @@ CASES = [
     (torch.bfloat16, None, "rowwise_1d", True),
     (torch.bfloat16, torch.float16, "scalar", True),
 ]
-SHAPES = [(1, 1, 8), (16, 32, 64), (33, 65, 129), (128, 128, 32), (130, 250, 100), (256, 384, 512), (1000, 520, 2048)]
+SHAPES = [(1, 1, 8), (16, 32, 64), (33, 65, 129), (128, 128, 32), (130, 250, 100), (256, 384, 512), (1000, 520, 2048),
+          # enough 256 x 256 tiles for most compute units: 16-bit operands with 16-bit results take the persistent kernel
+          (2560, 4096, 256), (2500, 4200, 192)]
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: f"{str(c[0])[6:]}-{str(c[1])[6:] if c[1] else 'default'}-{c[2]}-bias{int(c[3])}")
