@@ -471,6 +471,14 @@ template <int MODE, bool ALIGNED, bool SCATTER = false, int JN = kTM, bool F16 =
 __device__ __forceinline__ void store_tile(const GemmArgs& a, const v4f (&acc)[NT][JN], int m_base, int n_base,
                                            int l16, int lg, int m_end, const int* out_index = nullptr, int c_rows = 0,
                                            const float* row_weight = nullptr, int q0 = 0) {
+  if constexpr (!ALIGNED && !SCATTER && NT % 4 == 0 && MODE == kModeBlock) {
+    // a wavefront's share that lies inside the matrix (uniform) takes the stores of whole tiles (block scales only:
+    // the row/column modes' instantiations with edges have no registers left for a second store path and spill)
+    if (m_base + 16 * JN <= m_end && piece_column(n_base, q0 + NT / 2, 0) <= a.N) {
+      store_tile<MODE, true, false, JN, F16, NT>(a, acc, m_base, n_base, l16, lg, m_end, nullptr, 0, nullptr, q0);
+      return;
+    }
+  }
   constexpr bool kPairs = ALIGNED && !SCATTER && NT % 4 == 0;  // whole tiles: pieces leave two at a time
   const bool odd = (l16 & 1) != 0;
   if (MODE != kModeBlock) {
