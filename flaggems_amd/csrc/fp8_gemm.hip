@@ -213,13 +213,17 @@ template <int BM, int BN, int WM, int WN, int MODE, bool DIRECT, bool SPLIT = fa
 __global__ __launch_bounds__(WM* WN * 64) void fp8_gemm_kernel(GemmArgs a) {
   using Cfg = TileCfg<BM, BN, WM, WN, NST>;
   static_assert(NST == 2 || (DIRECT && NST >= 3 && NST <= 5), "deep pipeline: direct loads, 3..5 stages");
-  if (!SPLIT && a.batch > 1) {  // uniform: this workgroup's entry of the batch
+  if (a.batch > 1) {  // uniform: this workgroup's entry of the batch
     const int64_t z = blockIdx.y;
     a.X += z * a.x_batch_bytes;
     a.W += z * a.w_batch_bytes;
     a.C = reinterpret_cast<uint8_t*>(a.C) + z * a.c_batch_bytes;
     a.xs += z * a.xs_batch_stride;
     a.ws += z * a.ws_batch_stride;
+    if (SPLIT && a.split_partials != nullptr) {
+      a.split_partials += z * a.split_partials_per_entry;
+      a.split_counters += z * (int64_t)(a.tiles_m * a.tiles_n * (Cfg::kThreads / 64));
+    }
   }
   constexpr int NT = Cfg::kThreads;
   constexpr int TM = Cfg::TM, TN = Cfg::TN;
@@ -655,12 +659,18 @@ struct PipePlan {
   size_t workspace_bytes;
 };
 constexpr int kPipeStages = 4;
-PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs) {
+// entries: equal problems launched together (blockIdx.y = entry): their tiles fill the compute units together, and
+// workspace_bytes is what all of them need.
+PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs, int64_t entries = 1) {
   PipePlan p = {false, 1, 0, 0};
-  if (M <= 64 || K <= 0 || K % 128 != 0) return p;
+  if (entries < 1) entries = 1;
+  if (M <= 32 || K <= 0 || K % 128 != 0) return p;
+  // 33..64 rows: the staged-activation kernel, except for batches with much weight (measured, [b, h, r] x [h, d, r] with
+  // d = 1024, b = 48: h = 16, r = 7168 (117 MB): 41 -> 34 us here; h = 8, r = 4096 (34 MB): 16 -> 20 us; h = 4, r = 2048: 10 -> 14 us)
+  if (M <= 64 && !(entries > 1 && entries * N * K > ((int64_t)64 << 20))) return p;
   if (xs_rs < 0 || xs_rs >= (1 << 21)) return p;  // 256 rows of scales addressed with 32-bit byte offsets
   const int64_t KB = K / 128;
-  const int64_t tiles = ceil_div(M, kSplitTile) * ceil_div(N, kSplitTile);
+  const int64_t tiles = ceil_div(M, kSplitTile) * ceil_div(N, kSplitTile) * entries;
   const int cus = cu_count();
   if (tiles > cus || KB < 4) return p;
   if (tiles * kSplitWaves * 4 > FG_WORKSPACE_COUNTER_BYTES) return p;
@@ -687,7 +697,8 @@ int launch_pipe(GemmArgs a, const PipePlan& plan, void* workspace, hipStream_t s
   a.splits = plan.splits;
   a.kb_per_split = plan.kb_per_split;
   a.split_counters = reinterpret_cast<unsigned int*>(workspace);
-  a.split_partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES) : nullptr;
+  a.split_partials = workspace && plan.splits > 1 ? reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + FG_WORKSPACE_COUNTER_BYTES) : nullptr;
+  a.split_partials_per_entry = (int64_t)a.tiles_m * a.tiles_n * a.splits * kSplitTile * kSplitTile;
   auto kern = fp8_gemm_kernel<kSplitTile, kSplitTile, kSplitWM, 2, MODE, true, true, kPipeStages>;
   static PerDeviceFlags lds_limit_raised = {};
   {
@@ -695,7 +706,7 @@ int launch_pipe(GemmArgs a, const PipePlan& plan, void* workspace, hipStream_t s
     if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", Cfg::kLdsBytes, hipGetErrorString(e));
   }
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n * a.splits;
-  FG_LAUNCH(kern, dim3((uint32_t)blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, a);
+  FG_LAUNCH(kern, dim3((uint32_t)blocks, (uint32_t)(a.batch > 1 ? a.batch : 1)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, a);
   FG_CHECK_LAUNCH("fp8_gemm_kernel (four stages)");
   return FG_OK;
 }
@@ -937,6 +948,10 @@ extern "C" size_t fg_batched_block_fp8_gemm_workspace_bytes(int64_t batch, int64
       if (all > need) need = all;
     }
   }
+  if (batch > 1) {
+    const fg::PipePlan pipe = fg::plan_pipe(M, N, K, 0, batch);
+    if (pipe.use && pipe.workspace_bytes > need) need = pipe.workspace_bytes;
+  }
   return need;
 }
 
@@ -985,6 +1000,12 @@ extern "C" int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_b
                            workspace_bytes >= FG_WORKSPACE_COUNTER_BYTES + (size_t)batch * per_entry &&
                            (size_t)batch * plan.n_chunks * sizeof(unsigned int) <= FG_WORKSPACE_COUNTER_BYTES);
         if (plan.use && fits) return launch_small_m(a, kModeBlock, plan, workspace, workspace_bytes, (hipStream_t)stream);
+      }
+      {
+        // few tiles in the whole batch: the four-stage tile kernel, K split over blocks until the compute units are full
+        const PipePlan pp = plan_pipe(M, N, K, as_row_stride, batch);
+        const bool fits = pp.splits == 1 || (workspace != nullptr && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= pp.workspace_bytes);
+        if (pp.use && fits) return launch_pipe<kModeBlock>(a, pp, workspace, (hipStream_t)stream);
       }
       if (M > 32 && M <= 128) {  // the staged-activation kernel, entry in blockIdx.z, under the same conditions
         const MidMPlan mid = plan_mid_m(M, N, K, batch);

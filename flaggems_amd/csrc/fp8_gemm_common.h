@@ -36,6 +36,9 @@ struct GemmArgs {
   // these many bytes (X, W, C) or floats (xs, ws) after the previous entry's; batch <= 1: one problem
   int batch;
   int64_t x_batch_bytes, w_batch_bytes, c_batch_bytes, xs_batch_stride, ws_batch_stride;
+  // a batch with K split over blocks: every entry has tiles x splits partial tiles of its own, these many floats in
+  // all, and tiles x wavefronts counters
+  int64_t split_partials_per_entry;
 };
 
 // s_waitcnt vmcnt(0) with expcnt/lgkmcnt left at their maxima (gfx9 encoding)

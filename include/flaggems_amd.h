@@ -286,11 +286,12 @@ int fg_block_fp8_gemm_noalloc(const void* A, int64_t lda, const void* B, int64_t
  * the scales, elements of c_dtype for C); row strides are free, so a [b, h, r] activation with h as the batch
  * takes lda = h * r and a_batch_stride = r.  Matrices too small to fill the GPU on their own go out in one launch
  * (the batch entry in the grid), larger ones one after the other on `stream`; the results are those of `batch`
- * calls of fg_block_fp8_gemm (the same bits, except that up to 128 rows K may be split over fewer blocks than for
- * a lone matrix, which changes the order of the fp32 partial sums), and the workspace rules are that entry point's
- * (one workspace serves the whole batch; fg_batched_block_fp8_gemm_workspace_bytes(batch, M, N, K) is what the
- * kernels can use: at most 32 rows per matrix, every entry keeps its own partial sums, and with less than that
- * the call takes a slower kernel instead of failing).
+ * calls of fg_block_fp8_gemm (the same bits, except that where K is split over blocks -- up to 128 rows, and beyond
+ * while the whole batch has no more 128 x 128 tiles than the GPU has compute units -- the batch is split into fewer
+ * ranges than a lone matrix, which changes the order of the fp32 partial sums), and the workspace rules are that
+ * entry point's (one workspace serves the whole batch; fg_batched_block_fp8_gemm_workspace_bytes(batch, M, N, K) is
+ * what the kernels can use: every entry keeps its own partial sums, and with less than that the call takes a slower
+ * kernel instead of failing).
  *
  * Stands in for w8a8_block_fp8_bmm (src/flag_gems/runtime/backend/_nvidia/hopper/ops/w8a8_block_fp8_bmm.py:629-779)
  * and, through it, fp8_einsum("bhr,hdr->bhd") (.../hopper/ops/fp8_einsum.py:22-68).

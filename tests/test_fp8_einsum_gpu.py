@@ -44,11 +44,12 @@ def test_einsum_large_batch_and_per_head_bits():
 
 
 @pytest.mark.parametrize("M", [1, 5, 17, 32, 33, 48, 64, 100, 128])
-@pytest.mark.parametrize("B,N,K", [(3, 384, 640), (12, 1024, 2048), (40, 128, 512), (2, 7168, 2304)])
+@pytest.mark.parametrize("B,N,K", [(3, 384, 640), (12, 1024, 2048), (40, 128, 512), (2, 7168, 2304), (10, 1024, 7168)])
 def test_batches_of_few_rows_go_out_in_one_launch(M, B, N, K):
-    """Up to 128 rows per matrix the weight-streaming kernels take the whole batch in one launch (the entry in the
-    grid, every entry with its own partial sums and counters); strided operands and outputs, and a second call on the
-    same workspace."""
+    """Up to 128 rows per matrix the weight-streaming kernels and the four-stage tile kernel take the whole batch in one
+    launch (the entry in the grid, every entry with its own partial sums and counters); strided operands and outputs,
+    and a second call on the same workspace.  The last shape has more than 64 MB of weights, which moves 33..64 rows to
+    the tile kernel as well."""
     xq, xs, yq, ys = O.make_fp8_einsum_inputs(M, B, K, N, seed=M + B)
     want = O.fp8_block_einsum_ref(xq, xs, yq, ys, [128, 128]).permute(1, 0, 2)       # [B, M, N]
     x, x_s = xq.permute(1, 0, 2).to(DEV), xs.permute(1, 0, 2).to(DEV)                # strided views, as fp8_einsum passes them
@@ -58,6 +59,23 @@ def test_batches_of_few_rows_go_out_in_one_launch(M, B, N, K):
         top = want.abs().max().item()
         torch.testing.assert_close(z[:, :, :N].cpu().float(), want, rtol=1e-2, atol=1e-2 * max(1.0, top / 8))
         assert torch.all(z[:, :, N:] == 3.0)
+
+
+@pytest.mark.parametrize("B,M,N,K", [(8, 256, 1024, 4096), (4, 384, 512, 2048), (5, 200, 640, 1024), (16, 130, 1024, 7168)])
+def test_batches_above_128_rows_with_few_tiles_in_all(B, M, N, K):
+    """While the whole batch has no more 128 x 128 tiles than the GPU has compute units it goes out as one launch of the
+    four-stage tile kernel with K split over blocks (64 ... 208 tiles here): against the oracle, rows that end inside a
+    tile, and the same bits on a second call."""
+    xq, xs, yq, ys = O.make_fp8_einsum_inputs(M, B, K, N, seed=B + M)
+    want = O.fp8_block_einsum_ref(xq, xs, yq, ys, [128, 128]).permute(1, 0, 2)       # [B, M, N]
+    x, x_s = xq.permute(1, 0, 2).to(DEV), xs.permute(1, 0, 2).to(DEV)
+    got = flag_gems.w8a8_block_fp8_bmm(x, yq.to(DEV), x_s, ys.to(DEV), [128, 128])
+    top = want.abs().max().item()
+    torch.testing.assert_close(got.cpu().float(), want, rtol=1e-2, atol=1e-2 * max(1.0, top / 8))
+    got32 = flag_gems.w8a8_block_fp8_bmm(x, yq.to(DEV), x_s, ys.to(DEV), [128, 128], output_dtype=torch.float32)
+    torch.testing.assert_close(got32.cpu(), want, rtol=1e-4, atol=1e-4 * max(1.0, top))
+    again = flag_gems.w8a8_block_fp8_bmm(x, yq.to(DEV), x_s, ys.to(DEV), [128, 128])
+    assert torch.equal(again.view(torch.int16), got.view(torch.int16))
 
 
 def test_bmm_into_callers_buffer_and_other_dtypes():
