@@ -665,9 +665,6 @@ PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs, int64_t entri
   PipePlan p = {false, 1, 0, 0};
   if (entries < 1) entries = 1;
   if (M <= 32 || K <= 0 || K % 128 != 0) return p;
-  // 33..64 rows: the staged-activation kernel, except for batches with much weight (measured, [b, h, r] x [h, d, r] with
-  // d = 1024, b = 48: h = 16, r = 7168 (117 MB): 41 -> 34 us here; h = 8, r = 4096 (34 MB): 16 -> 20 us; h = 4, r = 2048: 10 -> 14 us)
-  if (M <= 64 && !(entries > 1 && entries * N * K > ((int64_t)64 << 20))) return p;
   if (xs_rs < 0 || xs_rs >= (1 << 21)) return p;  // 256 rows of scales addressed with 32-bit byte offsets
   const int64_t KB = K / 128;
   const int64_t tiles = ceil_div(M, kSplitTile) * ceil_div(N, kSplitTile) * entries;
@@ -684,6 +681,13 @@ PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs, int64_t entri
   // with up to 128 K-blocks per block allowed here: M = 1024, N = 4096, K = 14336: 74 -> 82 us; with up to 64: M = 512,
   // same weights: 53 -> 45 us; N = 7168, K = 16384 at M = 256: 59 -> 50 us).
   if (p.kb_per_split > 64) return p;
+  // 33..64 rows: half of every tile is padding, and so is half of every partial tile a split writes; the
+  // staged-activation kernel is the alternative.  This kernel wins while K is split in two at most over ranges of
+  // eight K-blocks or more (measured at M = 64: N = 28672, K = 4096, 224 tiles unsplit: 46 -> 32 us; N = 24576, K = 1536:
+  // 16.2 -> 14.6 us; a batch of 16 x [1024, 7168], 128 tiles in two ranges, 48 rows: 41 -> 34 us; but N = 32768, K = 512,
+  // four K-blocks: 8.5 -> 9.8 us; N = 4096, K = 14336 in eight ranges: 23 -> 25 us; N = 4608, K = 7168 in seven: 17 -> 20 us;
+  // a batch of 8 x [1024, 4096] in four: 16 -> 20 us)
+  if (M <= 64 && !(p.splits <= 2 && p.kb_per_split >= 8)) return p;
   p.workspace_bytes = p.splits > 1 ? FG_WORKSPACE_COUNTER_BYTES + (size_t)tiles * p.splits * kSplitTile * kSplitTile * sizeof(float) : 0;
   p.use = true;
   return p;
@@ -734,6 +738,11 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
     // measured -- M = 128: N = 2112, K = 7168: 24.0 against 19.9 us; 7168 x 2304: 16.4 against 14.6; 4096 x 4096: 18.4
     // against 16.8 -- and only serves batches now)
     const bool mid_takes = mid.use && mid.tmx == 4;
+    if (a.M <= 64) {  // the four-stage tile kernel where its planner prefers it to the staged-activation kernel
+      const PipePlan pp = plan_pipe(a.M, a.N, a.K, MODE == kModeBlock ? a.xs_rs : 0);
+      const bool ws_ok = pp.splits == 1 || (workspace != nullptr && workspace_bytes >= pp.workspace_bytes && (uintptr_t)workspace % 16 == 0);
+      if (pp.use && ws_ok) return launch_pipe<MODE>(a, pp, workspace, stream);
+    }
     if (mid_takes && (mid.splits == 1 || (workspace != nullptr && workspace_bytes >= mid.workspace_bytes &&
                                           (uintptr_t)workspace % 16 == 0)))
       return launch_mid_m(a, MODE, mid, workspace, workspace_bytes, stream);
