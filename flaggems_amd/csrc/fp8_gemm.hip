@@ -204,7 +204,8 @@ struct TileCfg {
 // ---------------------------------------------------------------------------------------------
 // Main kernel
 // ---------------------------------------------------------------------------------------------
-// SPLIT: the grid is tiles x a.splits and a block computes a range of K-blocks of its tile.  Every wavefront
+// SPLIT: the grid is tiles x a.splits (times the batch in blockIdx.y, every entry with partial sums and counters of
+// its own) and a block computes a range of K-blocks of its tile.  Every wavefront
 // publishes its fp32 sums in the workspace and counts itself in (one counter per tile and wavefront position);
 // the one that arrives last adds the sums of all splits in split order -- the same order whoever comes last --
 // and runs the epilogue.  For problems with few tiles, which would leave most of the GPU idle while every

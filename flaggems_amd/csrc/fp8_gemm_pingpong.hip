@@ -36,7 +36,9 @@
 // lg = i >> 2 then holds eight consecutive columns per pair of tiles, and the four lanes that share an output
 // row (16 lanes apart) cover 64 contiguous bytes per store.  The memory side combines the lanes of one store
 // instruction, not the instructions: with 32 consecutive columns per lane (four stores of 16 bytes at a
-// 64-byte stride) results left at 3.1 TB/s, this way at 6.5 TB/s, and all compute units store at once.
+// 64-byte stride) results left at 3.1 TB/s, this way at 6.5 TB/s, and all compute units store at once.  Wavefront
+// shares that lie inside the matrix go one step further and pair the rows (store_piece_pair): the lanes of an even
+// row and of the odd row after it swap a piece each, and a store instruction writes whole 128-byte lines.
 //
 // Registers.  Two wavefronts per SIMD leave 256 registers each: 128 fp32 accumulators, the four activation
 // fragments of the K-block (32) and a ring of three weight fragments (24) that the multiply phase refills two
