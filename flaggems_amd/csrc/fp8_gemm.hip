@@ -665,7 +665,7 @@ constexpr int kPipeStages = 4;
 PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs, int64_t entries = 1) {
   PipePlan p = {false, 1, 0, 0};
   if (entries < 1) entries = 1;
-  if (M <= 32 || K <= 0 || K % 128 != 0) return p;
+  if (M <= 16 || (M <= 32 && entries > 1) || K <= 0 || K % 128 != 0) return p;
   if (xs_rs < 0 || xs_rs >= (1 << 21)) return p;  // 256 rows of scales addressed with 32-bit byte offsets
   const int64_t KB = K / 128;
   const int64_t tiles = ceil_div(M, kSplitTile) * ceil_div(N, kSplitTile) * entries;
@@ -688,7 +688,12 @@ PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs, int64_t entri
   // 16.2 -> 14.6 us; a batch of 16 x [1024, 7168], 128 tiles in two ranges, 48 rows: 41 -> 34 us; but N = 32768, K = 512,
   // four K-blocks: 8.5 -> 9.8 us; N = 4096, K = 14336 in eight ranges: 23 -> 25 us; N = 4608, K = 7168 in seven: 17 -> 20 us;
   // a batch of 8 x [1024, 4096] in four: 16 -> 20 us)
-  if (M <= 64 && !(p.splits <= 2 && p.kb_per_split >= 8)) return p;
+  if (M > 32 && M <= 64 && !((p.splits == 1 && p.kb_per_split >= 8) || (p.splits == 2 && p.kb_per_split >= 16))) return p;
+  // (two ranges of eight: N = 16384, K = 2048: 14 -> 17 us; of sixteen: N = 14336, K = 4096: 29 -> 22 us; N = 12288, K = 4096: 28 -> 20 us)
+  // 17..32 rows of a lone matrix: the decode kernels, except unsplit against very wide weights (M = 32: N = 24576,
+  // K = 1536: 18.3 -> 15.1 us; N = 28672, K = 4096: 34.9 -> 30.9 us; N = 32768, K = 1024: 15.8 -> 12.7 us), and up to 24
+  // rows only while K is short (M = 24, N = 28672, K = 4096: 34.0 -> 36.3 us, so not there; N = 20480, K = 3072: 24.8 -> 23.3 us)
+  if (M <= 32 && !(p.splits == 1 && p.kb_per_split >= 8 && (M > 24 || KB <= 24))) return p;
   p.workspace_bytes = p.splits > 1 ? FG_WORKSPACE_COUNTER_BYTES + (size_t)tiles * p.splits * kSplitTile * kSplitTile * sizeof(float) : 0;
   p.use = true;
   return p;
@@ -739,7 +744,7 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
     // measured -- M = 128: N = 2112, K = 7168: 24.0 against 19.9 us; 7168 x 2304: 16.4 against 14.6; 4096 x 4096: 18.4
     // against 16.8 -- and only serves batches now)
     const bool mid_takes = mid.use && mid.tmx == 4;
-    if (a.M <= 64) {  // the four-stage tile kernel where its planner prefers it to the staged-activation kernel
+    if (a.M <= 64) {  // the four-stage tile kernel where its planner prefers it to the staged-activation and decode kernels
       const PipePlan pp = plan_pipe(a.M, a.N, a.K, MODE == kModeBlock ? a.xs_rs : 0);
       const bool ws_ok = pp.splits == 1 || (workspace != nullptr && workspace_bytes >= pp.workspace_bytes && (uintptr_t)workspace % 16 == 0);
       if (pp.use && ws_ok) return launch_pipe<MODE>(a, pp, workspace, stream);

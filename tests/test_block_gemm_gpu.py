@@ -68,6 +68,20 @@ def test_quantized_linear_shapes_bf16(M, N, K):
     torch.testing.assert_close(got32.cpu(), want, rtol=1e-4, atol=2e-4)
 
 
+@pytest.mark.parametrize("M", [17, 24, 25, 32, 40, 64])
+@pytest.mark.parametrize("N,K", [(24576, 1536), (28672, 4096), (14336, 4096)])
+def test_few_rows_against_wide_weights(M, N, K):
+    """17 ... 64 rows against weights wide enough to give every compute unit a 128 x 128 tile (or half the units one, with
+    K in two ranges) leave the decode and staged-activation kernels for the four-stage tile kernel: all of them against
+    the oracle, whichever kernel the planner picks for the row count."""
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=M)
+    want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
+    got = flag_gems.w8a8_block_fp8_matmul(xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    torch.testing.assert_close(got.cpu().float(), want, rtol=1e-2, atol=1e-2)
+    got32 = flag_gems.w8a8_block_fp8_matmul(xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128], output_dtype=torch.float32)
+    torch.testing.assert_close(got32.cpu(), want, rtol=1e-4, atol=2e-4)
+
+
 def test_persistent_kernel_several_rounds_ragged_edges_and_strides():
     """M > 128 with 16-byte aligned rows takes the persistent 256x256 kernel: more tiles than compute units
     (a block walks several tiles), M and N that end inside a tile (N not a multiple of 32 either),
