@@ -9,15 +9,22 @@ loudly if the library has not been built (``python -m flaggems_amd.build``).
 from .act_quant import (  # noqa: F401
     SUPPORTED_FP8_DTYPE,
     act_quant_triton,
+    get_group_quant_rule,
     per_block_cast_to_fp8,
     per_token_cast_to_fp8,
     per_token_group_quant_fp8,
+    set_group_quant_rule,
     silu_and_mul_packed,
     silu_and_mul_per_token_group_quant_fp8,
 )
 from .cutlass_scaled_mm import SM_VERSION_NUM, cutlass_scaled_mm, get_sm_version_num  # noqa: F401
 from .fp8_einsum import fp8_einsum, w8a8_block_fp8_bmm  # noqa: F401
-from .grouped_block_fp8_matmul import group_ends_from_expert_ids, grouped_w8a8_block_fp8_matmul  # noqa: F401
+from .fused_moe import fused_experts_impl, moe_sort_slots, moe_sum  # noqa: F401
+from .grouped_block_fp8_matmul import (  # noqa: F401
+    group_ends_from_expert_ids,
+    grouped_w8a8_block_fp8_matmul,
+    local_rows_from_moe_align,
+)
 from .norm_quant import fused_add_rms_norm, rms_norm, rms_norm_per_token_group_quant_fp8  # noqa: F401
 from .registration import (  # noqa: F401
     all_registered_keys,
@@ -47,8 +54,13 @@ __all__ = [
     "fp8_matmul",
     "fp8_matmul_noop",
     "fused_add_rms_norm",
+    "fused_experts_impl",
+    "get_group_quant_rule",
     "grouped_w8a8_block_fp8_matmul",
     "group_ends_from_expert_ids",
+    "local_rows_from_moe_align",
+    "moe_sort_slots",
+    "moe_sum",
     "only_enable",
     "patch_empty_vllm",
     "per_block_cast_to_fp8",
@@ -58,6 +70,7 @@ __all__ = [
     "rms_norm_per_token_group_quant_fp8",
     "scaled_mm",
     "scaled_mm_out",
+    "set_group_quant_rule",
     "silu_and_mul_packed",
     "silu_and_mul_per_token_group_quant_fp8",
     "use_gems",

@@ -62,6 +62,7 @@ SIGNATURES = {
          c_int64, c_float, c_float, c_float, c_float, c_int, c_int, c_int, c_void_p],
     ),
     "fg_silu_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p]),
+    "fg_moe_sum": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p]),
     "fg_act_quant_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "fg_block_fp8_gemm": (
         c_int,
@@ -160,35 +161,94 @@ def require_gpu(t: torch.Tensor, what: str) -> None:
         )
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def current_stream_ptr(device: torch.device) -> int:
+    """The hipStream_t of torch's current stream on ``device`` (the raw getter skips building a Stream object, which
+    costs more host time than everything else the wrappers do around a launch)."""
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
 
 
-# Workspace of the GEMM kernels (arrival counters, split-K partial sums, transposed scales): one zero-filled buffer
-# per (device, stream), grown on demand.  Launches recorded into a HIP graph keep the raw address they were given, so
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(device: torch.device):
+    """``torch.cuda.device(device)``, or nothing at all when that device is already the current one (the usual case:
+    entering and leaving the context manager costs more host time than a decode-sized launch)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)
+
+
+_ws_bytes_cache = {}
+
+
+def cached_workspace_bytes(fn_name: str, *shape) -> int:
+    """``lib.<fn_name>(*shape)``, remembered per shape (the answer depends on the shape and the device's compute unit
+    count only; processes that mix GPU models would have to clear the table)."""
+    key = (fn_name, shape)
+    n = _ws_bytes_cache.get(key)
+    if n is None:
+        n = int(getattr(load(), fn_name)(*shape))
+        if len(_ws_bytes_cache) > 4096:
+            _ws_bytes_cache.clear()
+        _ws_bytes_cache[key] = n
+    return n
+
+
+# Workspace of the GEMM kernels (arrival counters, split-K partial sums, transposed scales): one buffer per
+# (device, stream) whose first FG_WORKSPACE_COUNTER_BYTES are zero, grown on demand.  Only the counter area needs the
+# zeros (every launch leaves it zero again); partial sums and transposed scales are written before they are read.
+# Launches recorded into a HIP graph keep the raw address they were given, so
 #   * a buffer that is replaced is retired, not released: a graph captured earlier may still write to it;
 #   * a buffer allocated while a capture is in progress comes from that graph's private memory pool and is handed out
-#     to launches of the same capture only (its zero fill is a kernel recorded in the graph; the counters are zero
-#     again after every launch, so refilling them on every replay changes nothing).
-# Growth at least doubles the size, so retired buffers add up to less than the live one.
+#     to launches of the same capture only.  The fill of its counter area is a 16 KB kernel recorded in the graph,
+#     which every replay repeats; `reserve_workspace()` on the capture stream before the capture avoids even that.
+# Growth at least doubles the size, so retired buffers add up to less than the live one; the list keeps the most
+# recent kMaxRetired of them (a graph that still uses an older one than that would have to be older than that many
+# growth steps of one stream).
 _workspaces = {}   # (device index, stream handle) -> (buffer, id of the capture it was allocated in, or 0)
 _retired = []
+kMaxRetired = 64
 
 
-def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    stream = torch.cuda.current_stream(device).cuda_stream
+def _capture_id(stream: int) -> int:
+    """0 unless the current stream is being captured into a graph (then the capture's id)."""
+    if not torch.cuda.is_current_stream_capturing():
+        return 0
+    return int(load().fg_stream_capture_id(stream))
+
+
+def workspace(device: torch.device, nbytes: int, stream: int = None) -> torch.Tensor:
+    if stream is None:
+        stream = current_stream_ptr(device)
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
-    capture = int(load().fg_stream_capture_id(stream))
+    capture = _capture_id(stream)
     need = max(int(nbytes), FG_WORKSPACE_COUNTER_BYTES)
     buf, made_in = _workspaces.get(key, (None, 0))
+    if buf is not None and made_in == capture and buf.numel() >= need:
+        return buf
     if buf is not None and made_in not in (0, capture):
         buf = None  # belongs to another graph's pool: that graph keeps the memory, this table must not hand it out
     if buf is None or buf.numel() < need:
         if buf is not None:
             if made_in == 0:
                 _retired.append(buf)
+                del _retired[:-kMaxRetired]
             need = max(need, 2 * buf.numel())
-        buf = torch.zeros(need, dtype=torch.uint8, device=device)
+        buf = torch.empty(need, dtype=torch.uint8, device=device)
+        buf[:FG_WORKSPACE_COUNTER_BYTES].zero_()
         # buffers of captures that have ended stay with their graphs; this table only drops its references
         for other in [k for k, (_, cap) in _workspaces.items() if cap not in (0, capture)]:
             del _workspaces[other]

@@ -18,6 +18,7 @@ true-quotient scale amax / 448 that the reference's device kernel and MoE fallba
 from __future__ import annotations
 
 import functools
+import os
 import logging
 from typing import Optional, Tuple
 
@@ -47,6 +48,40 @@ def _scale_rule_code(rule: Optional[str]) -> int:
     raise ValueError(f"scale_rule must be 'mul' or 'div', got {rule!r}")
 
 
+# Which of the reference's two formulations ``per_token_group_quant_fp8`` and the vLLM operator
+# ``_C::per_token_group_fp8_quant`` follow when the caller does not say (they differ in the last bit of about half of
+# all scales):
+#   "test_reference": scale = amax * fp32(1/448) with the floor ``eps`` rounded to the input's dtype -- the torch
+#                     helper the reference's unit test compares its kernel with
+#                     (tests/test_per_token_group_quant_fp8.py:23-48);
+#   "kernel":         scale = max(amax, eps) / 448 with ``eps`` as an fp32 value -- what the reference's device kernel
+#                     computes (src/flag_gems/ops/per_token_group_quant_fp8.py:55-70).
+# Process-wide; the environment variable FLAGGEMS_AMD_GROUP_QUANT_RULE sets the initial value.
+_GROUP_QUANT_RULES = ("test_reference", "kernel")
+_group_quant_rule = os.environ.get("FLAGGEMS_AMD_GROUP_QUANT_RULE", "test_reference")
+if _group_quant_rule not in _GROUP_QUANT_RULES:
+    raise ValueError(f"FLAGGEMS_AMD_GROUP_QUANT_RULE must be one of {_GROUP_QUANT_RULES}, got {_group_quant_rule!r}")
+
+
+def set_group_quant_rule(rule: str) -> str:
+    """Select the default formulation (see above); returns the previous one."""
+    global _group_quant_rule
+    if rule not in _GROUP_QUANT_RULES:
+        raise ValueError(f"rule must be one of {_GROUP_QUANT_RULES}, got {rule!r}")
+    previous, _group_quant_rule = _group_quant_rule, rule
+    return previous
+
+
+def get_group_quant_rule() -> str:
+    return _group_quant_rule
+
+
+def _default_rule_and_floor(eps: float, dtype: torch.dtype):
+    if _group_quant_rule == "kernel":
+        return _lib.FG_SCALE_DIV, _round_to_dtype(float(eps), torch.float32)
+    return _lib.FG_SCALE_MUL_INV, _round_to_dtype(float(eps), dtype)
+
+
 def _launch_group_quant(
     x2d: torch.Tensor,
     q2d: torch.Tensor,
@@ -63,7 +98,7 @@ def _launch_group_quant(
     _lib.require_gpu(x2d, "group quantizer")
     lib = _lib.load()
     rows, cols = x2d.shape
-    with torch.cuda.device(x2d.device):
+    with _lib.device_guard(x2d.device):
         status = lib.fg_group_quant_fp8(
             x2d.data_ptr(), _lib.DTYPE_CODE[x2d.dtype], rows, cols, x2d.stride(0) if rows > 1 else max(cols, x2d.stride(0)),
             q2d.data_ptr(), _lib.DTYPE_CODE[q2d.dtype], q2d.stride(0) if rows > 1 else max(cols, q2d.stride(0)),
@@ -165,10 +200,14 @@ def per_token_group_quant_fp8(
         s2d = x_s.view(-1, x_s.shape[-1])
     else:
         raise NotImplementedError("column_major_scales needs a 2-D input")
+    if scale_rule is None:
+        rule_code, floor = _default_rule_and_floor(eps, x.dtype)
+    else:
+        rule_code, floor = _scale_rule_code(scale_rule), _round_to_dtype(float(eps), x.dtype)
     _launch_group_quant(
         x2d, q2d, s2d, group_size,
-        floor=_round_to_dtype(float(eps), x.dtype), fp8_min=finfo.min, fp8_max=finfo.max,
-        scale_rule=_scale_rule_code(scale_rule), quotient_rule=_lib.FG_QUOT_DIV,
+        floor=floor, fp8_min=finfo.min, fp8_max=finfo.max,
+        scale_rule=rule_code, quotient_rule=_lib.FG_QUOT_DIV,
         pow2_rule=_lib.FG_POW2_LOG2 if scale_ue8m0 else _lib.FG_POW2_NONE,
     )
     return x_q, x_s
@@ -199,10 +238,11 @@ def per_token_group_fp8_quant_into(
         raise NotImplementedError("output_q must have unit stride in its last dimension")
     q2d = output_q if output_q.dim() == 2 else output_q.view(-1, input.shape[-1])
     s2d = output_s if output_s.dim() == 2 else output_s.view(-1, output_s.shape[-1])
+    rule_code, floor = _default_rule_and_floor(eps, input.dtype)
     _launch_group_quant(
         x2d, q2d, s2d, group_size,
-        floor=_round_to_dtype(float(eps), input.dtype), fp8_min=float(fp8_min), fp8_max=float(fp8_max),
-        scale_rule=_lib.FG_SCALE_MUL_INV, quotient_rule=_lib.FG_QUOT_DIV,
+        floor=floor, fp8_min=float(fp8_min), fp8_max=float(fp8_max),
+        scale_rule=rule_code, quotient_rule=_lib.FG_QUOT_DIV,
         pow2_rule=_lib.FG_POW2_LOG2 if scale_ue8m0 else _lib.FG_POW2_NONE,
     )
 
@@ -231,7 +271,7 @@ def per_block_cast_to_fp8(
         x = x.contiguous()
     _lib.require_gpu(x, "block quantizer")
     lib = _lib.load()
-    with torch.cuda.device(x.device):
+    with _lib.device_guard(x.device):
         status = lib.fg_block_quant_fp8(
             x.data_ptr(), _lib.DTYPE_CODE[x.dtype], m, n, x.stride(0) if m > 1 else max(n, x.stride(0)),
             q.data_ptr(), _lib.DTYPE_CODE[q.dtype], n,
@@ -292,7 +332,7 @@ def silu_and_mul_packed(x: torch.Tensor) -> torch.Tensor:
     x2d = _as_rows(x)
     _lib.require_gpu(x2d, "silu_and_mul")
     rows = x2d.shape[0]
-    with torch.cuda.device(x.device):
+    with _lib.device_guard(x.device):
         status = _lib.load().fg_silu_mul(
             x2d.data_ptr(), _lib.DTYPE_CODE[x.dtype], rows, d, x2d.stride(0) if rows > 1 else max(2 * d, x2d.stride(0)), d,
             out.data_ptr(), d, _lib.current_stream_ptr(x.device))
@@ -341,13 +381,17 @@ def silu_and_mul_per_token_group_quant_fp8(
     rows = x2d.shape[0]
     q2d = x_q.view(-1, d)
     s2d = x_s if x_s.dim() == 2 else x_s.view(-1, x_s.shape[-1])
-    with torch.cuda.device(x.device):
+    if scale_rule is None:  # the process-wide default, as in per_token_group_quant_fp8: the fused call stays its twin
+        rule_code, floor = _default_rule_and_floor(eps, x.dtype)
+    else:
+        rule_code, floor = _scale_rule_code(scale_rule), _round_to_dtype(float(eps), x.dtype)
+    with _lib.device_guard(x.device):
         status = _lib.load().fg_silu_mul_group_quant_fp8(
             x2d.data_ptr(), _lib.DTYPE_CODE[x.dtype], rows, d, x2d.stride(0) if rows > 1 else max(2 * d, x2d.stride(0)), d,
             q2d.data_ptr(), _lib.DTYPE_CODE[fp8_dtype], d,
             s2d.data_ptr(), s2d.stride(0), s2d.stride(1),
-            group_size, _round_to_dtype(float(eps), x.dtype), finfo.min, finfo.max, 1.0 / finfo.max,
-            _scale_rule_code(scale_rule), _lib.FG_QUOT_DIV, _lib.FG_POW2_LOG2 if scale_ue8m0 else _lib.FG_POW2_NONE,
+            group_size, floor, finfo.min, finfo.max, 1.0 / finfo.max,
+            rule_code, _lib.FG_QUOT_DIV, _lib.FG_POW2_LOG2 if scale_ue8m0 else _lib.FG_POW2_NONE,
             _lib.current_stream_ptr(x.device))
     _lib.check(status, "fg_silu_mul_group_quant_fp8")
     return x_q, x_s

@@ -47,10 +47,16 @@ inline void launch(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds_byt
 
 #define FG_LAUNCH(kern, grid, block, lds_bytes, stream, ...) ::fg::launch(kern, grid, block, lds_bytes, stream, __VA_ARGS__)
 
+// A failed launch also sets HIP's per-thread "last error", which would otherwise stay set after this library has
+// reported the failure through its own status and be raised by the caller's next launch check at an unrelated
+// operation: hipGetLastError() consumes it.  Nothing is read or cleared after a launch that succeeded.
 #define FG_CHECK_LAUNCH(what)                                                       \
   do {                                                                              \
     hipError_t e_ = ::fg::launch_status();                                          \
-    if (e_ != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e_)); \
+    if (e_ != hipSuccess) {                                                         \
+      (void)hipGetLastError();                                                      \
+      FG_FAIL(FG_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e_));                \
+    }                                                                               \
   } while (0)
 
 // Kernels that use more than 64 KB of dynamic LDS need the limit raised once per device (the attribute belongs to

@@ -885,11 +885,6 @@ constexpr size_t kScratchBytes = FG_NOALLOC_SCRATCH_BYTES;
 // code the name is only a handle for hipGetSymbolAddress.
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
-__global__ __launch_bounds__(256) void clear_counters_kernel(uint32_t* p, int n) {
-  const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
-  if (i < n) p[i] = 0u;
-}
-
 // device address of `scratch` on each device, looked up on the first call made with that device current
 struct ScratchTable {
   std::mutex lock;
@@ -900,10 +895,11 @@ ScratchTable& scratch_table() {
   return t;
 }
 
-// Address of the current device's copy (looked up once per device).  On the first use the counter area is cleared
-// by a kernel on the caller's stream, ahead of the launch that follows: a fill kernel, not a memset, so that the
-// call may be recorded into a graph.
-int scratch_of_current_device(hipStream_t stream, void** out) {
+// Address of the current device's copy (looked up once per device).  Nothing is enqueued here: a file-scope device
+// array without an initialiser is zero when the code object is loaded, which is the state the counter area has to
+// start from, and every launch leaves the counters zero again.  (A fill kernel on the first caller's stream would be
+// ordered against that stream only, and recorded into the caller's graph if the first call were made under capture.)
+int scratch_of_current_device(void** out) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) FG_FAIL(FG_ERR_LAUNCH, "fg_block_fp8_gemm_noalloc: hipGetDevice: %s", hipGetErrorString(e));
@@ -915,9 +911,6 @@ int scratch_of_current_device(hipStream_t stream, void** out) {
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess || p == nullptr)
       FG_FAIL(FG_ERR_LAUNCH, "fg_block_fp8_gemm_noalloc: hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
-    constexpr int kWords = FG_WORKSPACE_COUNTER_BYTES / 4;
-    FG_LAUNCH(clear_counters_kernel, dim3(kWords / 256), dim3(256), 0, stream, reinterpret_cast<uint32_t*>(p), kWords);
-    FG_CHECK_LAUNCH("clear_counters_kernel");
     t.ptr[dev] = p;
   }
   *out = t.ptr[dev];
@@ -941,7 +934,7 @@ extern "C" int fg_block_fp8_gemm_noalloc(const void* A, int64_t lda, const void*
             "%zu; call fg_block_fp8_gemm with a workspace of the caller's",
             (long long)M, (long long)N, (long long)K, need, kScratchBytes);
   void* ws = nullptr;
-  const int rc = scratch_of_current_device((hipStream_t)stream, &ws);
+  const int rc = scratch_of_current_device(&ws);
   if (rc != FG_OK) return rc;
   return fg_block_fp8_gemm(A, lda, B, ldb, As, as_row_stride, as_col_stride, Bs, bs_row_stride, bs_col_stride, C, ldc, c_dtype,
                            M, N, K, block_n, block_k, ws, kScratchBytes, stream);

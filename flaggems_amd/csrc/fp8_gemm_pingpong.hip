@@ -1003,6 +1003,8 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     // Past the last stage the loads are repeated from the last address into a slot nobody reads any more:
     // cheaper than a branch per load, and the wait counts below stay the same on every step.
     v8i xf[JN], wr[3];
+    v4f p_tail[2];  // results of the step's last two MFMAs, scaled into the sums after the barrier that ends the slot
+    (void)p_tail;
     issue_stage_part(0);
     xf[0] = read_frag(tx, 0, frag_off);
     issue_stage_part(1);
@@ -1089,9 +1091,10 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
         if (j == 0 && t + 2 < kTN) wr[(t + 2) % 3] = read_frag(tw, t + 2, frag_off);
         if (st >= 2) scale_into<0>(acc[(st - 2) / JN][(st - 2) % JN], p[(st - 2) % 3], sc[(st - 2) % JN]);
       }
-      constexpr int L = kTN * JN;
-      scale_into<0>(acc[(L - 2) / JN][(L - 2) % JN], p[(L - 2) % 3], sc[(L - 2) % JN]);
-      scale_into<4>(acc[(L - 1) / JN][(L - 1) % JN], p[(L - 1) % 3], sc[(L - 1) % JN]);
+      // The FMAs of the last two MFMAs wait until after the barrier below: they need the matrix pipe's last
+      // results (44 cycles after the last MFMA's issue), and while this wavefront waited for them before the barrier,
+      // the partner, whose MFMAs were ready, waited too.
+      p_tail[0] = p[(kTN * JN - 2) % 3]; p_tail[1] = p[(kTN * JN - 1) % 3];
     }
     __builtin_amdgcn_s_setprio(kFetchPrio);
     if (grp == 0) {  // A's share of stage T+1 has landed
@@ -1099,6 +1102,13 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     }
     flushed_prev = flushed_now;
     __builtin_amdgcn_s_barrier();
+    if (MODE == kModeBlock && !POW2) {
+      // (wait states between the last MFMA and the FMA that reads it: the four FMAs issued behind that MFMA, the
+      // priority change, the barrier, two here, four FMAs, two more)
+      constexpr int L = kTN * JN;
+      scale_into<2>(acc[(L - 2) / JN][(L - 2) % JN], p_tail[0], sc[(L - 2) % JN]);
+      scale_into<2>(acc[(L - 1) / JN][(L - 1) % JN], p_tail[1], sc[(L - 1) % JN]);
+    }
 
     // ================= next step; a finished tile is stored in this wavefront's next fetch slot
     rw_slot = (rw_slot + 1 == kWSt) ? 0 : rw_slot + 1;

@@ -35,8 +35,8 @@ def _launch_scaled_gemm(c, a, b, a_scale, b_scale, bias) -> None:
     m, k = a.shape
     n = b.shape[1]
     dev = a.device
-    with torch.cuda.device(dev):
-        ws_bytes = lib.fg_scaled_fp8_gemm_workspace_bytes(m, n, k)
+    with _lib.device_guard(dev):
+        ws_bytes = _lib.cached_workspace_bytes("fg_scaled_fp8_gemm_workspace_bytes", m, n, k)
         ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
         status = lib.fg_scaled_fp8_gemm(
             a.data_ptr(), a.stride(0) if m > 1 else max(k, a.stride(0)),
@@ -59,8 +59,8 @@ def _launch_scaled_int8_gemm(c, a, b, a_scale, b_scale, bias) -> None:
     m, k = a.shape
     n = b.shape[1]
     dev = a.device
-    with torch.cuda.device(dev):
-        ws_bytes = lib.fg_scaled_int8_gemm_workspace_bytes(m, n, k)
+    with _lib.device_guard(dev):
+        ws_bytes = _lib.cached_workspace_bytes("fg_scaled_int8_gemm_workspace_bytes", m, n, k)
         ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
         status = lib.fg_scaled_int8_gemm(
             a.data_ptr(), a.stride(0) if m > 1 else max(k, a.stride(0)),
@@ -84,7 +84,7 @@ def _launch_scaled_generic_gemm(c, a, b, a_scale, b_scale, bias) -> None:
     m, k = a.shape
     n = b.shape[1]
     dev = a.device
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         status = lib.fg_scaled_gemm(
             a.data_ptr(), a.stride(0) if m > 1 else max(k, a.stride(0)),
             b.data_ptr(), b.stride(1) if n > 1 else max(k, b.stride(1)), _lib.DTYPE_CODE[a.dtype],

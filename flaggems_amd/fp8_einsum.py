@@ -62,8 +62,8 @@ def w8a8_block_fp8_bmm(
     _lib.require_gpu(x, "batched block fp8 gemm")
     lib = _lib.load()
     dev = x.device
-    with torch.cuda.device(dev):
-        ws_bytes = lib.fg_batched_block_fp8_gemm_workspace_bytes(B, M, N, K)
+    with _lib.device_guard(dev):
+        ws_bytes = _lib.cached_workspace_bytes("fg_batched_block_fp8_gemm_workspace_bytes", B, M, N, K)
         ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
         status = lib.fg_batched_block_fp8_gemm(
             x.data_ptr(), x.stride(1) if M > 1 else max(K, x.stride(1)), x.stride(0),

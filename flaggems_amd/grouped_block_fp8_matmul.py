@@ -27,16 +27,46 @@ def _cdiv(a: int, b: int) -> int:
 
 def group_ends_from_expert_ids(expert_ids: torch.Tensor, block_m: int, num_experts: int) -> torch.Tensor:
     """The ``offs`` table of ``grouped_w8a8_block_fp8_matmul`` from the per-block expert table that the reference's
-    ``moe_align_block_size`` returns (one entry per ``block_m`` sorted rows, -1 for blocks past the padded end;
-    src/flag_gems/fused/moe_align_block_size.py:404-517, consumed at src/flag_gems/fused/fused_moe.py:1105).  Blocks
-    of one expert are consecutive and experts ascend, so expert e ends after ``block_m`` times the number of blocks
-    with an id in [0, e].  Stays on the device of ``expert_ids`` and does not synchronise."""
+    ``moe_align_block_size`` returns WITHOUT an ``expert_map`` (one entry per ``block_m`` sorted rows, ascending
+    expert ids, -1 only for the blocks past the padded end; src/flag_gems/fused/moe_align_block_size.py:404-517,
+    consumed at src/flag_gems/fused/fused_moe.py:1105).  Expert e then ends after ``block_m`` times the number of
+    blocks with an id in [0, e].  Stays on the device of ``expert_ids`` and does not synchronise.
+
+    A table that went through ``expert_map`` (moe_align_block_size.py:817-818) can hold -1 in front of or between
+    the local experts' blocks and local ids out of order; cumulative ends cannot express that.  Use
+    ``local_rows_from_moe_align`` for such tables."""
     assert expert_ids.ndim == 1 and block_m >= 1 and num_experts >= 1
     ids = expert_ids.to(torch.int64)
     used = (ids >= 0) & (ids < num_experts)
     counts = torch.zeros(num_experts, dtype=torch.int64, device=expert_ids.device)
     counts.scatter_add_(0, ids.clamp(0, num_experts - 1), used.to(torch.int64))
     return (torch.cumsum(counts, 0) * block_m).to(torch.int32)
+
+
+def local_rows_from_moe_align(sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor, block_m: int, num_experts: int):
+    """``(row_index, offs)`` for ``grouped_w8a8_block_fp8_matmul`` from the tables of the reference's
+    ``moe_align_block_size`` after ``expert_map`` has been applied (src/flag_gems/fused/moe_align_block_size.py:
+    771-819): ``expert_ids`` holds a LOCAL expert or -1 per block of ``block_m`` sorted rows, in any order.
+
+    The blocks are reordered, ascending by local expert with the -1 blocks last (a stable sort of at most a few
+    thousand block numbers on the device), and the rows of the -1 blocks are replaced by the padding value
+    ``sorted_token_ids.numel()``: the GEMM never multiplies them and stores nothing for them.  The reference writes
+    zeros for those rows (``write_zeros_to_output``, src/flag_gems/fused/fused_moe.py:804-820, 1114); pass
+    ``zero_unwritten_rows=True`` to the GEMM for the same result.  No synchronisation."""
+    assert sorted_token_ids.ndim == 1 and expert_ids.ndim == 1 and block_m >= 1 and num_experts >= 1
+    nb = expert_ids.numel()
+    assert sorted_token_ids.numel() == nb * block_m, "one expert id per block of block_m sorted rows"
+    ids = expert_ids.to(torch.int64)
+    local = (ids >= 0) & (ids < num_experts)
+    key = torch.where(local, ids, torch.full_like(ids, num_experts))
+    order = torch.argsort(key, stable=True)
+    rows = sorted_token_ids.view(nb, block_m).to(torch.int32)
+    pad = torch.full_like(rows, sorted_token_ids.numel())
+    rows = torch.where(local[:, None], rows, pad)[order].reshape(-1).contiguous()
+    counts = torch.zeros(num_experts + 1, dtype=torch.int64, device=expert_ids.device)
+    counts.scatter_add_(0, key, torch.ones_like(key))
+    offs = (torch.cumsum(counts[:num_experts], 0) * block_m).to(torch.int32)
+    return rows, offs
 
 
 def grouped_w8a8_block_fp8_matmul(
@@ -51,6 +81,7 @@ def grouped_w8a8_block_fp8_matmul(
     index_divisor: int = 1,
     scatter_rows: Optional[int] = None,
     row_weights: Optional[torch.Tensor] = None,
+    zero_unwritten_rows: bool = False,
 ) -> torch.Tensor:
     """C[offs[e-1]:offs[e]] = block_fp8_matmul(A[offs[e-1]:offs[e]], B[e]) for every group e.
 
@@ -69,6 +100,10 @@ def grouped_w8a8_block_fp8_matmul(
     ``torch.empty`` gave them.  ``row_weights`` (fp32 [R]) multiplies the fp32 sums of sorted row m by
     ``row_weights[row_index[m]]`` before the cast.  Both follow the epilogue of the reference's MoE kernel
     (src/flag_gems/fused/fused_moe.py:1484-1509: ``offs_token``, ``token_mask``, ``MUL_ROUTED_WEIGHT``).
+
+    ``zero_unwritten_rows``: the result starts as zeros instead of ``torch.empty``, so rows that no group covers (the
+    slots of experts that live on another device) read as zeros, which is what the reference's kernel stores for
+    them (src/flag_gems/fused/fused_moe.py:1114).
     """
     logger.debug("GEMS GROUPED_W8A8_BLOCK_FP8_MATMUL")
     assert len(block_size) == 2
@@ -105,14 +140,14 @@ def grouped_w8a8_block_fp8_matmul(
     if B.stride(2) != 1:
         B = B.contiguous()
 
-    C = A.new_empty((c_rows if c_rows else M, N), dtype=output_dtype)
+    C = (A.new_zeros if zero_unwritten_rows else A.new_empty)((c_rows if c_rows else M, N), dtype=output_dtype)
     if M == 0 or N == 0:
         return C
     _lib.require_gpu(A, "grouped block fp8 gemm")
     lib = _lib.load()
     dev = A.device
-    with torch.cuda.device(dev):
-        ws_bytes = lib.fg_grouped_block_fp8_gemm_workspace_bytes(max(M, T), N, K)
+    with _lib.device_guard(dev):
+        ws_bytes = _lib.cached_workspace_bytes("fg_grouped_block_fp8_gemm_workspace_bytes", max(M, T), N, K)
         ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
         status = lib.fg_grouped_block_fp8_gemm(
             A.data_ptr(), A.stride(0) if T > 1 else max(K, A.stride(0)),

@@ -14,7 +14,14 @@ from typing import Optional, Sequence, Tuple
 import torch
 
 from . import _lib
-from .act_quant import SUPPORTED_FP8_DTYPE, _FP8_DTYPES, _IN_DTYPES, _round_to_dtype, _scale_rule_code
+from .act_quant import (
+    SUPPORTED_FP8_DTYPE,
+    _FP8_DTYPES,
+    _IN_DTYPES,
+    _default_rule_and_floor,
+    _round_to_dtype,
+    _scale_rule_code,
+)
 
 logger = logging.getLogger(__name__)
 
@@ -34,12 +41,16 @@ def _launch(x2d, residual2d, weight, eps, y2d, q2d, s2d, group_size, quant_eps, 
 
     if q2d is not None:
         finfo = torch.finfo(fp8_dtype)
+        if scale_rule is None:  # the process-wide default of per_token_group_quant_fp8, whose twin the fused call is
+            rule_code, floor = _default_rule_and_floor(quant_eps, x2d.dtype)
+        else:
+            rule_code, floor = _scale_rule_code(scale_rule), _round_to_dtype(float(quant_eps), x2d.dtype)
         qargs = (q2d.data_ptr(), _lib.DTYPE_CODE[fp8_dtype], stride(q2d), s2d.data_ptr(), s2d.stride(0), s2d.stride(1),
-                 group_size, _round_to_dtype(float(quant_eps), x2d.dtype), finfo.min, finfo.max, 1.0 / finfo.max,
-                 _scale_rule_code(scale_rule), _lib.FG_QUOT_DIV, _lib.FG_POW2_LOG2 if scale_ue8m0 else _lib.FG_POW2_NONE)
+                 group_size, floor, finfo.min, finfo.max, 1.0 / finfo.max,
+                 rule_code, _lib.FG_QUOT_DIV, _lib.FG_POW2_LOG2 if scale_ue8m0 else _lib.FG_POW2_NONE)
     else:
         qargs = (None, 0, 0, None, 0, 0, 0, 0.0, 0.0, 0.0, 0.0, 0, 0, 0)
-    with torch.cuda.device(x2d.device):
+    with _lib.device_guard(x2d.device):
         status = _lib.load().fg_rms_norm_group_quant_fp8(
             x2d.data_ptr(), _lib.DTYPE_CODE[x2d.dtype], rows, cols, stride(x2d),
             residual2d.data_ptr() if residual2d is not None else None, stride(residual2d) if residual2d is not None else 0,

@@ -12,6 +12,7 @@ operator, so no vendor detection, condition lambdas or tuning tables are involve
 from __future__ import annotations
 
 import logging
+import os
 import warnings
 from typing import Iterable, List, Optional, Tuple
 
@@ -80,14 +81,41 @@ def _as_list(names) -> List[str]:
     return list(names)
 
 
+class _LogOncePerLocation(logging.Filter):
+    """Passes the first record of every call site (file, line) and drops the repeats: with ``once=True`` the record
+    file lists each operator call site once instead of once per call
+    (the reference's LogOncePerLocationFilter, src/flag_gems/logging_utils.py:34-45)."""
+
+    def __init__(self):
+        super().__init__()
+        self.seen = set()
+
+    def filter(self, record):
+        key = (record.pathname, record.lineno)
+        if key in self.seen:
+            return False
+        self.seen.add(key)
+        return True
+
+
 def _setup_logging(record: bool, once: bool, path: Optional[str]) -> None:
+    """The reference's setup_flaggems_logging (src/flag_gems/logging_utils.py:60-84): with ``record`` a file handler
+    on the ``flag_gems`` logger (a new call replaces the previous one's), the same line format, DEBUG level, no
+    propagation; ``once`` filters repeats per call site.  Default file: ~/.flaggems/oplist.log."""
     if not record:
         return
-    handler = logging.FileHandler(path or "./gems.log", mode="w")
-    handler.setFormatter(logging.Formatter("[%(levelname)s] %(name)s: %(message)s"))
+    _teardown_logging()
+    filename = os.path.expanduser(path) if path else os.path.join(os.path.expanduser("~"), ".flaggems", "oplist.log")
+    parent = os.path.dirname(os.path.abspath(filename))
+    os.makedirs(parent, exist_ok=True)
+    handler = logging.FileHandler(filename, mode="w")
+    handler.setFormatter(logging.Formatter("[%(levelname)s] %(name)s.%(funcName)s: %(message)s"))
     handler.set_name("flag_gems_record")
+    if once:
+        handler.addFilter(_LogOncePerLocation())
     logger.addHandler(handler)
     logger.setLevel(logging.DEBUG)
+    logger.propagate = False
 
 
 def _teardown_logging() -> None:

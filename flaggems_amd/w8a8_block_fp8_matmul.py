@@ -28,14 +28,16 @@ def _cdiv(a: int, b: int) -> int:
 
 
 def _launch_block_gemm(a2d, b, as2d, bs, c2d, block_n: int, block_k: int, scales_pow2: bool = False) -> None:
-    _lib.require_gpu(a2d, "block fp8 gemm")
+    dev = a2d.device
+    if dev.type != "cuda":
+        _lib.require_gpu(a2d, "block fp8 gemm")
     lib = _lib.load()
     m, k = a2d.shape
     n = b.shape[0]
-    dev = a2d.device
-    with torch.cuda.device(dev):
-        ws_bytes = lib.fg_block_fp8_gemm_workspace_bytes(m, n, k)
-        ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
+    with _lib.device_guard(dev):
+        stream = _lib.current_stream_ptr(dev)
+        ws_bytes = _lib.cached_workspace_bytes("fg_block_fp8_gemm_workspace_bytes", m, n, k)
+        ws = _lib.workspace(dev, ws_bytes, stream) if ws_bytes else None
         entry = lib.fg_block_fp8_gemm_pow2_scales if scales_pow2 else lib.fg_block_fp8_gemm
         status = entry(
             a2d.data_ptr(), a2d.stride(0) if m > 1 else max(k, a2d.stride(0)),
@@ -45,9 +47,10 @@ def _launch_block_gemm(a2d, b, as2d, bs, c2d, block_n: int, block_k: int, scales
             c2d.data_ptr(), c2d.stride(0) if m > 1 else max(n, c2d.stride(0)), _lib.DTYPE_CODE[c2d.dtype],
             m, n, k, block_n, block_k,
             ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
-            _lib.current_stream_ptr(dev),
+            stream,
         )
-    _lib.check(status, "fg_block_fp8_gemm")
+    if status:
+        _lib.check(status, "fg_block_fp8_gemm")
 
 
 def w8a8_block_fp8_matmul(

@@ -164,6 +164,18 @@ int fg_silu_mul(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t 
                 void* out, int64_t out_row_stride, void* stream);
 
 /*
+ * Sum over the top-k slots of every token, the last step of an expert layer:
+ *     out[t, h] = cast( sum_{k < top_k} in[t, k, h] )   (fp32 running sum in slot order, one rounding)
+ * in: [tokens, top_k, hidden] of dtype FG_BF16 / FG_F16 / FG_F32 with element strides in_token_stride and
+ * in_slot_stride (unit stride along hidden); out: [tokens, hidden] of the same dtype, rows out_token_stride apart.
+ * hidden a multiple of 8; in, out and every row 16-byte aligned, else FG_ERR_UNSUPPORTED.
+ * Stands in for moe_sum (src/flag_gems/fused/moe_sum.py:34-90), which the reference's expert layer calls on the
+ * scattered, weighted results of its second GEMM (src/flag_gems/fused/fused_moe.py:2177-2182).
+ */
+int fg_moe_sum(const void* in, int dtype, int64_t tokens, int64_t top_k, int64_t hidden, int64_t in_token_stride,
+               int64_t in_slot_stride, void* out, int64_t out_token_stride, void* stream);
+
+/*
  * RMSNorm (optionally preceded by the residual add) fused into the quantizer: every row of x [rows, cols] is
  * normalised, multiplied by weight [cols] (x's type), rounded to x's type as a separate norm kernel would have
  * stored it, and quantized exactly as fg_group_quant_fp8 quantizes that stored tensor (same codes and scales, bit
@@ -270,8 +282,9 @@ int fg_block_fp8_gemm_pow2_scales(const void* A, int64_t lda, const void* B, int
  * fg_block_fp8_gemm_workspace_bytes(M, N, K) exceeds FG_NOALLOC_SCRATCH_BYTES is refused with FG_ERR_WORKSPACE (use
  * fg_block_fp8_gemm with a workspace of the caller's).  All calls on one GPU share that GPU's array: calls that may
  * overlap on one GPU (two streams, two threads) race on the counters and partial sums and must be serialised by the
- * caller.  The first call on a device looks the array's address up and clears its counter area with a kernel on
- * `stream`; every launch leaves the counters zero for the next.
+ * caller.  The first call on a device looks the array's address up; nothing but the GEMM's own kernels is ever
+ * enqueued, so a call may be recorded into a graph like any other launch.  The counter area starts as zeros (a device
+ * array without an initialiser is zero when the library's code is loaded) and every launch leaves it zero.
  */
 #define FG_NOALLOC_SCRATCH_BYTES (32u << 20)
 int fg_block_fp8_gemm_noalloc(const void* A, int64_t lda, const void* B, int64_t ldb,

@@ -145,6 +145,25 @@ def per_token_group_quant_fp8_div_ref(
     return x_quant, x_scales
 
 
+def per_token_group_quant_fp8_kernel_ref(
+    x: torch.Tensor, group_size: int, eps: float = 1e-10, dtype: torch.dtype = FP8_DTYPE, scale_ue8m0: bool = False
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The arithmetic of the reference's DEVICE kernel ``_per_token_group_quant_fp8``
+    (src/flag_gems/ops/per_token_group_quant_fp8.py:55-70), which its torch test helper does not follow to the bit:
+    the group is widened to fp32 first, the floor ``eps`` is an fp32 value (not rounded to the input's dtype), the
+    scale is the true quotient ``max(amax, eps) / fp8_max``, optionally ``exp2(ceil(log2(max(|scale|, 1e-10))))``, and the codes
+    are ``clamp(y / scale, fp8_min, fp8_max)`` with a true division."""
+    assert x.shape[-1] % group_size == 0
+    finfo = torch.finfo(dtype)
+    y = x.reshape(x.numel() // group_size, group_size).to(torch.float32)
+    amax = torch.maximum(y.abs().max(dim=-1, keepdim=True)[0], torch.tensor(eps, dtype=torch.float32))
+    y_s = amax / finfo.max
+    if scale_ue8m0:
+        y_s = torch.exp2(torch.ceil(torch.log2(torch.maximum(y_s.abs(), torch.tensor(1e-10, dtype=torch.float32)))))
+    y_q = (y / y_s).clamp(min=finfo.min, max=finfo.max).to(dtype)
+    return y_q.reshape(x.shape), y_s.reshape(x.shape[:-1] + (x.shape[-1] // group_size,))
+
+
 def silu_and_mul_ref(x: torch.Tensor) -> torch.Tensor:
     """``silu(x[..., :d]) * x[..., d:]`` the way the reference's activation kernel computes it
     (src/flag_gems/fused/silu_and_mul.py:13-18, src/flag_gems/fused/fused_moe.py:795-800): the gate in
@@ -381,6 +400,58 @@ def grouped_block_fp8_matmul_ref(
             )
         begin = max(begin, end)
     return c
+
+
+def block_fp8_moe_ref(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    w1_scale: torch.Tensor,
+    w2_scale: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    block_shape: List[int],
+    expert_map: Optional[torch.Tensor] = None,
+    tokens: Optional[torch.Tensor] = None,
+    kernel_activation: bool = True,
+) -> torch.Tensor:
+    """Restates ``torch_w8a8_block_fp8_moe`` (reference tests/test_fused_experts_impl.py:604-662): every routed slot
+    (token t, choice j) goes through quantize (``amax / 448``) -> ``torch_w8a8_block_matmul`` with W1 of its expert
+    -> SiLU-and-mul -> quantize -> ``torch_w8a8_block_matmul`` with W2, each GEMM rounded to the activations' dtype,
+    and the slot results are weighted and summed per token in that dtype.
+
+    ``expert_map`` (global expert -> local expert or -1): slots of experts that are not local contribute zeros, as
+    the reference's kernel writes them (src/flag_gems/fused/fused_moe.py:1114, 2128-2129).  ``tokens``: evaluate
+    only these token rows (the full-size configurations are checked on a sample).  ``kernel_activation``: the
+    activation rounds once (``silu_and_mul_ref``, what the reference's kernel does) instead of twice in the
+    activations' dtype (the torch expression at :629-633); both are within the test's tolerance of each other.
+    The weighted sum follows the reference's expression: slot result times weight rounded to the dtype, summed over
+    the choices by torch in that dtype."""
+    if tokens is not None:
+        hidden_states, topk_weights, topk_ids = hidden_states[tokens], topk_weights[tokens], topk_ids[tokens]
+    batch, hidden = hidden_states.shape
+    topk = topk_ids.size(1)
+    _, block_k = block_shape
+    expanded = hidden_states.view(batch, -1, hidden).repeat(1, topk, 1).reshape(-1, hidden)
+    out = torch.zeros(batch * topk, w2.shape[1], dtype=hidden_states.dtype)
+    flat_ids = topk_ids.reshape(-1).to(torch.int64)
+    if expert_map is not None:
+        flat_ids = expert_map.to(torch.int64)[flat_ids]
+    hq, hs = per_token_group_quant_fp8_div_ref(expanded.contiguous(), block_k)
+
+    def activation(x):
+        if kernel_activation:
+            return silu_and_mul_ref(x)
+        d = x.shape[-1] // 2
+        return torch.nn.functional.silu(x[..., :d]) * x[..., d:]
+
+    for e in range(w1.shape[0]):
+        mask = flat_ids == e
+        if mask.sum():
+            inter = block_fp8_matmul_tiled_ref(hq[mask], w1[e], hs[mask], w1_scale[e], block_shape, hidden_states.dtype)
+            aq, a_s = per_token_group_quant_fp8_div_ref(activation(inter).contiguous(), block_k)
+            out[mask] = block_fp8_matmul_tiled_ref(aq, w2[e], a_s, w2_scale[e], block_shape, hidden_states.dtype)
+    return (out.view(batch, -1, w2.shape[1]) * topk_weights.reshape(batch, -1, 1).to(out.dtype)).sum(dim=1)
 
 
 def fp8_block_einsum_ref(

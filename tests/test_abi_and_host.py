@@ -196,3 +196,26 @@ def test_group_ends_from_the_per_block_expert_table():
     ends = flag_gems.group_ends_from_expert_ids(ids, 64, 5)
     assert ends.dtype == torch.int32 and ends.tolist() == [128, 128, 192, 384, 384]
     assert flag_gems.group_ends_from_expert_ids(torch.tensor([-1], dtype=torch.int32), 16, 2).tolist() == [0, 0]
+
+
+def test_record_once_lists_every_call_site_once(tmp_path):
+    """enable(record=True, once=True): the record file names each operator call site once, however often it runs
+    (the reference's LogOncePerLocationFilter, src/flag_gems/logging_utils.py:34-45); once=False lists every call."""
+    import logging
+
+    from flaggems_amd import registration
+
+    child = logging.getLogger("flag_gems.some_operator")
+    for once, want in ((True, 2), (False, 4)):
+        path = tmp_path / f"ops_{once}.log"
+        registration._setup_logging(True, once, str(path))
+        try:
+            for _ in range(3):
+                child.debug("GEMS SOME_OPERATOR")   # one call site, three calls
+            child.debug("GEMS SOME_OPERATOR")       # another call site
+        finally:
+            registration._teardown_logging()
+        lines = path.read_text().splitlines()
+        assert len(lines) == want, lines
+        assert lines[0] == "[DEBUG] flag_gems.some_operator.test_record_once_lists_every_call_site_once: GEMS SOME_OPERATOR"
+    assert not [h for h in logging.getLogger("flag_gems").handlers if h.get_name() == "flag_gems_record"]

@@ -7,7 +7,9 @@ would take minutes, so the oracle is evaluated on a sample: a handful of activat
 tile boundaries; for expert layers the first and last row of every segment) times whole 128-column scale blocks of
 the weight (first, second, one in the middle, the last, which may be ragged).  Every output element is a dot product
 of one activation row and one weight row, so any indexing mistake that moves rows, columns, K-blocks or scales
-shows in such a sample; on top, a second call must give the same bits.
+shows in such a sample; on top, a second call must give the same bits, and the whole result is compared on the
+device with torch's own fp32 GEMM of the dequantised operands (an independent implementation that sees every tile,
+K cut and tail launch the planner issues for the shape).
 
 Tolerance: |got - want| <= 1e-2 + 1e-2 |want| for the bf16 result against the float64 dequantised matmul
 (reference tests/test_w8a8_block_fp8_matmul.py:76-100 restated; the reference's own bar is looser)."""
@@ -60,6 +62,34 @@ def _oracle_on_sample(xq, wq, xs, ws, rows, blocks):
     return r, cols, want
 
 
+def _dequantized_weight(wq, ws):
+    """fp32 W[n, k] * Ws[n // 128, k // 128] on the device."""
+    N, K = wq.shape
+    s = ws.repeat_interleave(128, dim=0)[:N].repeat_interleave(128, dim=1)[:, :K]
+    return wq.float() * s
+
+
+def _assert_whole_matrix(got, xq, xs, w_deq, what=""):
+    """Every element of `got` against torch's own fp32 GEMM of the dequantised operands, computed on the device in
+    row chunks.  This is a cross-check, not the oracle: torch.matmul shares no code with libflaggems_amd.so, and
+    unlike the sampled oracle comparison it sees every tile, every K cut and every tail launch of the call."""
+    M, K = xq.shape
+    bad, worst, where = 0, 0.0, None
+    for r0 in range(0, M, 1024):
+        r1 = min(M, r0 + 1024)
+        x_deq = xq[r0:r1].float() * xs[r0:r1].repeat_interleave(128, dim=1)[:, :K]
+        ref = x_deq @ w_deq.t()
+        excess = (got[r0:r1].float() - ref).abs() - (1e-2 + 1e-2 * ref.abs())
+        n_bad = int((excess > 0).sum())
+        if n_bad:
+            bad += n_bad
+            top = float(excess.max())
+            if top > worst:
+                idx = int(excess.argmax())
+                worst, where = top, (r0 + idx // ref.shape[1], idx % ref.shape[1])
+    assert bad == 0, f"{what}: {bad} of {got.numel()} elements outside rtol/atol 1e-2 of the fp32 product, worst excess {worst:.3g} at {where}"
+
+
 def _check_block_gemm(M, N, K):
     xq, xs = _activation(M, K)
     wq, ws = _weight(N, K)
@@ -74,6 +104,7 @@ def _check_block_gemm(M, N, K):
     again = flag_gems.w8a8_block_fp8_matmul(xq, wq, xs, ws, [128, 128])
     assert torch.equal(again.view(torch.int16), got.view(torch.int16)), "two runs of one problem differ"
     assert torch.isfinite(got.float()).all()
+    _assert_whole_matrix(got, xq, xs, _dequantized_weight(wq, ws), f"M={M} N={N} K={K}")
 
 
 LLAMA3_8B = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]
@@ -125,6 +156,16 @@ def test_cutlass_scaled_mm_8192_square(M, use_bias):
     c2 = torch.empty_like(c)
     flag_gems.cutlass_scaled_mm(c2, a, b, sa, sb, bias)
     assert torch.equal(c2.view(torch.int16), c.view(torch.int16))
+    # every element against torch's fp32 GEMM of the scaled operands, on the device in row chunks (a cross-check
+    # that sees every tile of the launch; the allowance is the one of the sampled oracle comparison above)
+    b_deq = b.float() * sb
+    for r0 in range(0, M, 1024):
+        r1 = min(M, r0 + 1024)
+        prod_d = (a[r0:r1].float() * sa[r0:r1]) @ b_deq
+        exact_d = prod_d + bias.float() if use_bias else prod_d
+        allow_d = 1e-2 * (prod_d.abs() + (bias.float().abs() if use_bias else 0.0)) + 1e-2
+        err_d = (c[r0:r1].float() - exact_d).abs()
+        assert bool((err_d <= allow_d).all()), f"rows {r0}..{r1}: max excess {(err_d - allow_d).max().item()}"
 
 
 @functools.lru_cache(maxsize=2)
@@ -164,5 +205,11 @@ def test_mixtral_expert_layers(T, N, K):
             checked += len(rows)
         begin = end
     assert checked >= 8
+    begin = 0
+    for e in range(8):  # every row of every expert's segment against torch's fp32 GEMM on the device
+        end = int(ends[e])
+        if end > begin:
+            _assert_whole_matrix(got[begin:end], xq[begin:end], xs[begin:end], _dequantized_weight(wq[e], ws[e]), f"expert {e}")
+        begin = end
     again = flag_gems.grouped_w8a8_block_fp8_matmul(xq, wq, xs, ws, ends.to(DEV), [128, 128])
     assert torch.equal(again.view(torch.int16), got.view(torch.int16))

@@ -235,3 +235,60 @@ def test_einsum_ref_per_head_and_f64():
     np.testing.assert_allclose(got[:2, 1, :9].double().numpy(), want, rtol=1e-5, atol=1e-6)
     # scales of this input maker are powers of two and every group's largest code is +-448 or the group is tiny
     assert torch.all(torch.frexp(xs)[0] == 0.5) and torch.all(torch.frexp(ys)[0] == 0.5)
+
+
+def _moe_inputs(tokens, experts, hidden, inter, topk, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(tokens, hidden, generator=g).bfloat16()
+    w1 = (torch.randn(experts, 2 * inter, hidden, generator=g) / hidden**0.5).to(FP8)
+    w2 = (torch.randn(experts, hidden, inter, generator=g) / inter**0.5).to(FP8)
+    s1 = torch.rand(experts, 2 * inter // 128, hidden // 128, generator=g) + 0.5
+    s2 = torch.rand(experts, hidden // 128, inter // 128, generator=g) + 0.5
+    gate = torch.randn(tokens, experts, generator=g)
+    tw, ti = torch.topk(torch.softmax(gate, dim=-1), topk, dim=-1)
+    tw = (tw / tw.sum(dim=-1, keepdim=True)).bfloat16()
+    return x, w1, w2, s1, s2, tw, ti
+
+
+def _dense_mlp_f64(x, w1, w2, s1, s2):
+    """One expert's quantize -> GEMM -> SiLU-and-mul -> quantize -> GEMM through the *dequantised float64* GEMM
+    oracle (an algorithm other than the tiled one the MoE restatement calls), rounded to bf16 where the layer
+    rounds."""
+    q, s = O.per_token_group_quant_fp8_div_ref(x.contiguous(), 128)
+    h = O.block_fp8_matmul_dequant_ref(q, w1, s, s1, [128, 128], torch.bfloat16, torch.float64)
+    q2, s2a = O.per_token_group_quant_fp8_div_ref(O.silu_and_mul_ref(h).contiguous(), 128)
+    return O.block_fp8_matmul_dequant_ref(q2, w2, s2a, s2, [128, 128], torch.bfloat16, torch.float64)
+
+
+def test_moe_ref_with_identical_experts_is_the_dense_layer():
+    """Every expert holds the same weights and the routing weights of a token sum to one: whatever the routing, the
+    layer is the dense MLP (a wrong slot -> token map, a dropped weight or a missed slot breaks this).  The GEMM
+    results differ from the float64 route by a bf16 rounding here and there, which the second quantization can
+    amplify to a few percent of a row's largest element."""
+    x, w1, w2, s1, s2, tw, ti = _moe_inputs(12, 4, 256, 128, 2, seed=3)
+    w1[:] = w1[0]; w2[:] = w2[0]; s1[:] = s1[0]; s2[:] = s2[0]
+    got = O.block_fp8_moe_ref(x, w1, w2, s1, s2, tw, ti, [128, 128]).float()
+    want = _dense_mlp_f64(x, w1[0], w2[0], s1[0], s2[0]).float()
+    torch.testing.assert_close(got, want, rtol=3e-2, atol=3e-2 * float(want.abs().max()))
+
+
+def test_moe_ref_top1_picks_the_routed_expert_and_the_map_zeroes_foreign_slots():
+    x, w1, w2, s1, s2, _, _ = _moe_inputs(10, 3, 256, 128, 1, seed=5)
+    ids = torch.tensor([0, 2, 1, 1, 0, 2, 2, 0, 1, 0]).view(-1, 1)
+    ones = torch.ones(10, 1).bfloat16()
+    got = O.block_fp8_moe_ref(x, w1, w2, s1, s2, ones, ids, [128, 128]).float()
+    for e in range(3):
+        rows = (ids[:, 0] == e).nonzero()[:, 0]
+        want = _dense_mlp_f64(x[rows], w1[e], w2[e], s1[e], s2[e]).float()
+        torch.testing.assert_close(got[rows], want, rtol=3e-2, atol=3e-2 * float(want.abs().max()))
+    # half weights halve the result exactly (a power of two)
+    half = O.block_fp8_moe_ref(x, w1, w2, s1, s2, 0.5 * ones, ids, [128, 128]).float()
+    assert torch.equal(half, 0.5 * got)
+    # global experts 0 and 2 live elsewhere; global 1 is local expert 0
+    emap = torch.tensor([-1, 0, -1])
+    local = O.block_fp8_moe_ref(x, w1[1:2], w2[1:2], s1[1:2], s2[1:2], ones, ids, [128, 128], expert_map=emap).float()
+    mine = ids[:, 0] == 1
+    assert torch.equal(local[mine], got[mine]) and float(local[~mine].abs().max()) == 0.0
+    # a sample of tokens gives the rows of the full evaluation
+    pick = torch.tensor([7, 2, 3])
+    assert torch.equal(O.block_fp8_moe_ref(x, w1, w2, s1, s2, ones, ids, [128, 128], tokens=pick).float(), got[pick])

@@ -105,6 +105,21 @@ def test_group_quant_div_ref_vs_brute_force():
     assert np.array_equal(s.numpy().view(np.uint32), scales.view(np.uint32))
 
 
+@pytest.mark.parametrize("kind", ["randn", "wide"])
+def test_group_quant_kernel_ref_vs_brute_force(kind):
+    """The device kernel's formula: fp32 floor, amax / 448, true division.  A row of zeros shows the floor: with
+    bf16 inputs the torch helper floors at bf16(1e-10), the kernel at fp32(1e-10)."""
+    x = _rand_bf16(4, 512, 8, kind)
+    x[1, :128] = 0
+    y, s = O.per_token_group_quant_fp8_kernel_ref(x, 128)
+    codes, scales = _brute_quant(x.float().numpy(), 128, 1e-10, "div", "div")
+    assert np.array_equal(y.view(torch.uint8).numpy(), codes)
+    assert np.array_equal(s.numpy().view(np.uint32), scales.view(np.uint32))
+    assert s[1, 0].item() == np.float32(1e-10) / np.float32(448.0)
+    _, s_helper = O.per_token_group_quant_fp8_div_ref(x, 128)
+    assert s_helper[1, 0].item() != s[1, 0].item()
+
+
 def test_mul_and_div_scale_rules_really_differ():
     # the two scale formulas disagree in the last bit for about half of all amax
     # values, so a test that passes with the wrong rule would show here

@@ -193,6 +193,42 @@ def test_vllm_op_writes_callers_buffers():
         assert_codes_equal(q, want_q)
 
 
+def test_process_wide_rule_selects_the_kernels_formula():
+    """set_group_quant_rule("kernel"): the default of per_token_group_quant_fp8, of the fused producers and of the
+    vLLM operator becomes the reference's device-kernel arithmetic (fp32 floor, amax / 448, true division:
+    src/flag_gems/ops/per_token_group_quant_fp8.py:55-70); "test_reference" is the torch helper's.  Both against
+    their formulas, bit for bit; a group of zeros shows the floor, which is where the fp32 and the bf16 eps differ."""
+    flag_gems.patch_empty_vllm()
+    x = _x((61, 1024), 11)
+    x[3, 128:256] = 0
+    x[:, 512:640] *= 1e-9
+    xd = x.to(DEV)
+    assert flag_gems.get_group_quant_rule() == "test_reference"
+    try:
+        for rule, ref in (("kernel", O.per_token_group_quant_fp8_kernel_ref), ("test_reference", O.per_token_group_quant_fp8_ref)):
+            flag_gems.set_group_quant_rule(rule)
+            for ue8m0 in (False, True):
+                want_q, want_s = ref(x, 128, scale_ue8m0=ue8m0)
+                q, s = flag_gems.per_token_group_quant_fp8(xd, 128, scale_ue8m0=ue8m0)
+                assert_scales_equal(s, want_s, f"{rule} ue8m0={ue8m0}")
+                assert_codes_equal(q, want_q, f"{rule} ue8m0={ue8m0}")
+                q2 = torch.empty_like(q)
+                s2 = torch.empty_like(s)
+                torch.ops._C.per_token_group_fp8_quant(xd, q2, s2, 128, 1e-10, -448.0, 448.0, ue8m0)
+                assert_scales_equal(s2, want_s, f"vLLM op, {rule}")
+                assert_codes_equal(q2, want_q, f"vLLM op, {rule}")
+        flag_gems.set_group_quant_rule("kernel")
+        # an explicit scale_rule keeps its own meaning whatever the default is
+        want_q, want_s = O.per_token_group_quant_fp8_div_ref(x, 128)
+        q, s = flag_gems.per_token_group_quant_fp8(xd, 128, scale_rule="div")
+        assert_scales_equal(s, want_s)
+        assert_codes_equal(q, want_q)
+    finally:
+        flag_gems.set_group_quant_rule("test_reference")
+    with pytest.raises(ValueError):
+        flag_gems.set_group_quant_rule("fast")
+
+
 def test_empty_inputs():
     y, s = flag_gems.act_quant_triton(torch.empty(0, 256, dtype=torch.bfloat16, device=DEV))
     assert y.shape == (0, 256) and s.shape == (0, 2)
