@@ -26,6 +26,12 @@ Prints ONE JSON line with the driver's fields plus
   mixtral_moe_grouped_gemm
                 Mixtral-8x7B expert layers: 8 experts, top-2 over T tokens with Zipf(1.1) expert loads, rows sorted by
                 expert; the grouped block-fp8 GEMM with W1 [8,28672,4096] and W2 [8,4096,14336]; not part of `value`
+  mixtral_moe_layer
+                the whole expert layer on those weights (fused_experts_impl: quantize, GEMM 1 with gathered rows,
+                SiLU-and-mul + quantize, GEMM 2 with scattered weighted rows, sum over the slots), end to end
+  eager_host_overhead
+                host time per eager call (no graph) of fp8_matmul, of its allocation-only twin fp8_matmul_noop and of the
+                bare C-ABI call, at M = 1 on the smallest and the largest weight, next to the kernel's time
 """
 from __future__ import annotations
 
@@ -496,11 +502,13 @@ def main():
     # Mixtral-8x7B expert layers: grouped block-fp8 GEMM over rows sorted by expert
     moe = []
     experts = 8
+    moe_w = {}
     for (n, k) in [(28672, 4096), (4096, 14336)]:
         parts = [make_weight(n, k, gen, dev) for _ in range(experts)]
         wq = torch.stack([q for (q, _) in parts])
         ws = torch.stack([s_ for (_, s_) in parts])
         del parts
+        moe_w[(n, k)] = (wq, ws)
         for tokens in (64, 1024, 4096):
             rows = 2 * tokens
             ends = moe_row_ends(tokens, experts, 2, 0).to(dev)
@@ -512,6 +520,68 @@ def main():
                         "tflops": round(tf, 1), "gbps": round(nbytes / us / 1e3, 1),
                         "frac_mfma": round(tf / PEAK_FP8_TFLOPS, 4), "frac_hbm": round(nbytes / us / 1e3 / PEAK_HBM_GBPS, 4)})
         del wq, ws
+
+    # the whole expert layer: quantize -> grouped GEMM 1 (gather) -> SiLU-and-mul + quantize -> grouped GEMM 2 (scatter,
+    # routing weight) -> sum over the two slots of a token (fused_experts_impl), bf16 [T, 4096] in and out, the same
+    # Zipf(1.1) expert loads; flops = 2 * 2T * (28672 * 4096 + 4096 * 14336)
+    moe_layer = []
+    (w1q, w1s), (w2q, w2s) = moe_w[(28672, 4096)], moe_w[(4096, 14336)]
+    for tokens in (64, 1024, 4096):
+        ends = moe_row_ends(tokens, experts, 2, 0)
+        counts = torch.diff(ends, prepend=torch.zeros(1, dtype=torch.int32))
+        ids = torch.repeat_interleave(torch.arange(experts), counts.long())
+        ids = ids[torch.randperm(ids.numel(), generator=torch.Generator().manual_seed(tokens))].view(tokens, 2).to(dev)
+        tw = torch.rand(tokens, 2, device=dev, generator=gen) + 0.1
+        tw = (tw / tw.sum(dim=1, keepdim=True)).bfloat16()
+        hs = torch.randn(tokens, 4096, device=dev, generator=gen).bfloat16()
+        us = time_eager(lambda: flag_gems.fused_experts_impl(hs, w1q, w2q, tw, ids, use_fp8_w8a8=True, w1_scale=w1s,
+                                                             w2_scale=w2s, block_shape=[128, 128]), 10)
+        fl = 2.0 * 2 * tokens * (28672 * 4096 + 4096 * 14336)
+        gemm_rows = [r for r in moe if r["tokens"] == tokens]
+        moe_layer.append({"tokens": tokens, "us": round(us, 2), "tflops": round(fl / us / 1e6, 1),
+                          "frac_mfma": round(fl / us / 1e6 / PEAK_FP8_TFLOPS, 4),
+                          "weight_gbps": round(experts * (28672 * 4096 + 4096 * 14336) / us / 1e3, 1),
+                          "the_two_gemms_alone_us": round(sum(r["us"] for r in gemm_rows), 2)})
+    del moe_w, w1q, w1s, w2q, w2s
+
+    # ---- host time of an eager call (no graph): what a decode step pays per launch on the host, next to the kernel's
+    # own time.  fp8_matmul = checks + allocation + launch; fp8_matmul_noop = checks + allocation (the reference's
+    # probe of its binding overhead, cpp/lib/fp8_matmul.cpp:104-125); the bare C-ABI call through ctypes with all
+    # arguments prepared = the launch alone.  Host time = wall time of enqueueing, the queue never full (a
+    # synchronisation every 200 calls, outside the clock).
+    eager = []
+    lib = fg_lib.load()
+    for (n, k) in [(2112, 7168), (7168, 16384)]:
+        xq, xs = acts[(1, k)]
+        wq, ws = weights[(n, k)][0]
+
+        def host_us(fn, calls=2000, burst=200):
+            for _ in range(50):
+                fn()
+            torch.cuda.synchronize()
+            spent = 0.0
+            for _ in range(calls // burst):
+                t0 = time.perf_counter()
+                for _ in range(burst):
+                    fn()
+                spent += time.perf_counter() - t0
+                torch.cuda.synchronize()
+            return spent / calls * 1e6
+
+        c = torch.empty(1, n, dtype=torch.bfloat16, device=dev)
+        need = lib.fg_block_fp8_gemm_workspace_bytes(1, n, k)
+        wsp = torch.zeros(max(need, 16384), dtype=torch.uint8, device=dev)
+        raw = (xq.data_ptr(), k, wq.data_ptr(), k, xs.data_ptr(), xs.stride(0), xs.stride(1), ws.data_ptr(), ws.stride(0),
+               ws.stride(1), c.data_ptr(), n, 0, 1, n, k, 128, 128, wsp.data_ptr(), wsp.numel(),
+               fg_lib.current_stream_ptr(dev))
+        kernel_us = [d["us"] for d in detail if (d["M"], d["N"], d["K"]) == (1, n, k)][0]
+        eager.append({"M": 1, "N": n, "K": k,
+                      "fp8_matmul_host_us": round(host_us(lambda: flag_gems.fp8_matmul(xq, xs, wq, ws)), 2),
+                      "w8a8_block_fp8_matmul_host_us": round(host_us(lambda: flag_gems.w8a8_block_fp8_matmul(xq, wq, xs, ws, [128, 128])), 2),
+                      "fp8_matmul_noop_host_us": round(host_us(lambda: flag_gems.fp8_matmul_noop(xq, xs, wq, ws)), 2),
+                      "bare_c_abi_call_host_us": round(host_us(lambda: lib.fg_block_fp8_gemm(*raw)), 2),
+                      "kernel_us_in_a_graph": kernel_us})
+        del c, wsp
 
     # ---- CPU baseline: the oracle on the host cores, bounded samples
     cpu = None
@@ -608,6 +678,8 @@ def main():
         "fp8_einsum_bhr_hdr": einsum,
         "llama3_8b_linears": llama,
         "mixtral_moe_grouped_gemm": moe,
+        "mixtral_moe_layer": moe_layer,
+        "eager_host_overhead": eager,
         "cpu_baseline": cpu,
         "cpu_baseline_other_configs": cpu_configs,
         "detail": detail,

@@ -181,12 +181,16 @@ class _NoGuard:
 
 
 _NO_GUARD = _NoGuard()
+_single_gpu = None  # this process sees exactly one GPU (asked once): there is no other device to guard against
 
 
 def device_guard(device: torch.device):
     """``torch.cuda.device(device)``, or nothing at all when that device is already the current one (the usual case:
     entering and leaving the context manager costs more host time than a decode-sized launch)."""
-    if device.index is None or device.index == torch.cuda.current_device():
+    global _single_gpu
+    if _single_gpu is None:
+        _single_gpu = torch.cuda.device_count() == 1
+    if _single_gpu or device.index is None or device.index == torch.cuda.current_device():
         return _NO_GUARD
     return torch.cuda.device(device)
 

@@ -102,8 +102,30 @@ def w8a8_block_fp8_matmul(
         B = B.contiguous()
     a2d = A.view(M, K)
     as2d = As if As.dim() == 2 else As.reshape(M, As.shape[-1])
+    if (block_n, block_k) != (128, 128):
+        as2d, Bs, block_n, block_k = _scales_at_128(as2d, Bs, N, K, block_n, block_k)
     _launch_block_gemm(a2d, B, as2d, Bs, C.view(M, N), block_n, block_k, pow2)
     return C
+
+
+def _scales_at_128(as2d: torch.Tensor, bs: torch.Tensor, n: int, k: int, block_n: int, block_k: int):
+    """Scale blocks that are whole multiples of 128 restated at the kernels' 128 x 128 granularity: every 128-wide
+    piece of a larger block gets a copy of the block's scale, so each product is multiplied by the same fp32 value at
+    the same place of the sum and the result is what a kernel with the larger blocks would give (the reference's
+    kernel takes any ``block_size``: src/flag_gems/ops/w8a8_block_fp8_matmul.py:51-122).  Blocks that are not multiples
+    of 128 would need another matrix instruction shape per scale block and are refused."""
+    if block_n <= 0 or block_k <= 0 or block_n % 128 != 0 or block_k % 128 != 0:
+        raise NotImplementedError(
+            f"w8a8_block_fp8_matmul: block_size [{block_n}, {block_k}]: scale blocks must be multiples of 128 in both "
+            "directions (the kernels apply one scale product per 128 x 128 block of the weight and 128-wide K-block)")
+    rn, rk = block_n // 128, block_k // 128
+    kb, nb = _cdiv(k, 128), _cdiv(n, 128)
+    if rk > 1:
+        as2d = as2d.repeat_interleave(rk, dim=1)[:, :kb]
+        bs = bs.repeat_interleave(rk, dim=1)[:, :kb]
+    if rn > 1:
+        bs = bs.repeat_interleave(rn, dim=0)[:nb]
+    return as2d.contiguous(), bs.contiguous(), 128, 128
 
 
 def fp8_matmul(

@@ -395,7 +395,30 @@ def test_host_side_assertions():
         flag_gems.w8a8_block_fp8_matmul(A, B, As[:, :1], Bs, [128, 128])
     with pytest.raises(AssertionError):
         flag_gems.w8a8_block_fp8_matmul(A.t(), B, As, Bs, [128, 128])
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(NotImplementedError):  # scale blocks that are not multiples of 128 are refused, by name
         flag_gems.w8a8_block_fp8_matmul(A, B, As.repeat(1, 2), Bs.repeat(2, 2), [64, 64])
     out = flag_gems.w8a8_block_fp8_matmul(A[:0], B, As[:0], Bs, [128, 128])
     assert out.shape == (0, 256)
+
+
+@pytest.mark.parametrize("block_size", [[256, 128], [128, 256], [256, 256], [384, 512]])
+@pytest.mark.parametrize("M,N,K", [(7, 640, 1024), (100, 1000, 1536), (300, 2304, 4096), (4096, 2112, 7168)])
+def test_scale_blocks_that_are_multiples_of_128(M, N, K, block_size):
+    """block_size other than [128, 128] (the reference's kernel takes any: src/flag_gems/ops/w8a8_block_fp8_matmul.py:
+    173-232): blocks of whole multiples of 128, ragged at the edges of N and K, against the oracle evaluated with the
+    same block_size."""
+    block_n, block_k = block_size
+    g = torch.Generator().manual_seed(M + N + K + block_n)
+    A = torch.randn(M, K, generator=g).to(FP8)
+    B = torch.randn(N, K, generator=g).to(FP8)
+    As = 0.01 * torch.rand(M, -(-K // block_k), generator=g) + 0.005
+    Bs = 0.01 * torch.rand(-(-N // block_n), -(-K // block_k), generator=g) + 0.005
+    got = flag_gems.w8a8_block_fp8_matmul(A.to(DEV), B.to(DEV), As.to(DEV), Bs.to(DEV), block_size).cpu().float()
+    rows = torch.arange(M) if M <= 300 else torch.tensor([0, 1, 255, 256, 257, M // 2, M - 1])
+    want = O.block_fp8_matmul_dequant_ref(A[rows], B, As[rows], Bs, block_size, torch.float32, torch.float64)
+    torch.testing.assert_close(got[rows], want, rtol=1e-2, atol=1e-2)
+    # and the bits of the call with the scales written out per 128 x 128 block
+    As128 = As.repeat_interleave(block_k // 128, dim=1)[:, : -(-K // 128)].contiguous()
+    Bs128 = Bs.repeat_interleave(block_n // 128, dim=0)[: -(-N // 128)].repeat_interleave(block_k // 128, dim=1)[:, : -(-K // 128)].contiguous()
+    same = flag_gems.w8a8_block_fp8_matmul(A.to(DEV), B.to(DEV), As128.to(DEV), Bs128.to(DEV), [128, 128]).cpu().float()
+    assert torch.equal(same, got)
