@@ -143,6 +143,39 @@ def load() -> ctypes.CDLL:
     return _lib
 
 
+_fast = None
+_addresses = {}
+
+
+def fast():
+    """The CPython marshalling module for the decode-critical calls (csrc/fastcall.c, built next to the library by
+    flaggems_amd/build.py).  A ctypes call converts its 20-odd arguments in 2-3 us, as long as a decode kernel runs;
+    this module takes the function's address and the arguments as plain Python ints and floats."""
+    global _fast
+    if _fast is None:
+        import importlib.util
+
+        from .build import fastcall_path
+
+        path = fastcall_path()
+        if not os.path.exists(path):
+            raise ImportError(f"{path} is missing: build it with `python -m flaggems_amd.build`")
+        spec = importlib.util.spec_from_file_location("_fg_fastcall", path)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        _fast = mod
+    return _fast
+
+
+def address(name: str) -> int:
+    """Address of an exported C function, for the calls that go through `fast()`."""
+    a = _addresses.get(name)
+    if a is None:
+        a = ctypes.cast(getattr(load(), name), c_void_p).value
+        _addresses[name] = a
+    return a
+
+
 def check(status: int, what: str) -> None:
     if status == FG_OK:
         return

@@ -96,10 +96,10 @@ def _launch_group_quant(
 ) -> None:
     """x2d [R, C] unit column stride; q2d same shape; s2d [R, C/g] any strides."""
     _lib.require_gpu(x2d, "group quantizer")
-    lib = _lib.load()
     rows, cols = x2d.shape
     with _lib.device_guard(x2d.device):
-        status = lib.fg_group_quant_fp8(
+        status = _lib.fast().group_quant_fp8(
+            _lib.address("fg_group_quant_fp8"),
             x2d.data_ptr(), _lib.DTYPE_CODE[x2d.dtype], rows, cols, x2d.stride(0) if rows > 1 else max(cols, x2d.stride(0)),
             q2d.data_ptr(), _lib.DTYPE_CODE[q2d.dtype], q2d.stride(0) if rows > 1 else max(cols, q2d.stride(0)),
             s2d.data_ptr(), s2d.stride(0), s2d.stride(1),

@@ -56,6 +56,32 @@ def _run(cmd):
     return out
 
 
+FASTCALL_SRC = os.path.join(CSRC, "fastcall.c")
+
+
+def fastcall_path() -> str:
+    import sysconfig
+
+    return os.path.join(HERE, "_fg_fastcall" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+
+
+def build_fastcall(verbose: bool = True) -> str:
+    """Compile the CPython argument-marshalling module (csrc/fastcall.c) with the host C compiler.  It links nothing
+    of libflaggems_amd.so: the Python host hands it function addresses."""
+    import sysconfig
+
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        raise RuntimeError("no host C compiler (gcc / cc) for csrc/fastcall.c")
+    out = fastcall_path()
+    tmp = out + ".tmp"
+    _run([cc, "-O2", "-shared", "-fPIC", "-Wall", "-I" + sysconfig.get_paths()["include"], FASTCALL_SRC, "-o", tmp])
+    os.replace(tmp, out)
+    if verbose:
+        print("[flaggems_amd.build] built", out, flush=True)
+    return out
+
+
 def build(verbose: bool = True, jobs: int = 4) -> str:
     """Compile every HIP source for gfx950 and link the shared library.  Always recompiles."""
     hipcc = _hipcc()
@@ -78,6 +104,7 @@ def build(verbose: bool = True, jobs: int = 4) -> str:
     os.replace(tmp, LIB_PATH)
     if verbose:
         print("[flaggems_amd.build] linked", LIB_PATH, flush=True)
+    build_fastcall(verbose)
     return LIB_PATH
 
 

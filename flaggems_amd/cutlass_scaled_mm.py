@@ -31,14 +31,14 @@ SM_VERSION_NUM = get_sm_version_num()
 
 def _launch_scaled_gemm(c, a, b, a_scale, b_scale, bias) -> None:
     _lib.require_gpu(a, "scaled fp8 gemm")
-    lib = _lib.load()
     m, k = a.shape
     n = b.shape[1]
     dev = a.device
     with _lib.device_guard(dev):
         ws_bytes = _lib.cached_workspace_bytes("fg_scaled_fp8_gemm_workspace_bytes", m, n, k)
         ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
-        status = lib.fg_scaled_fp8_gemm(
+        status = _lib.fast().scaled_gemm(
+            _lib.address("fg_scaled_fp8_gemm"),
             a.data_ptr(), a.stride(0) if m > 1 else max(k, a.stride(0)),
             b.data_ptr(), b.stride(1) if n > 1 else max(k, b.stride(1)),
             a_scale.data_ptr(), 1 if a_scale.numel() > 1 or m == 1 else 0,
@@ -55,14 +55,14 @@ def _launch_scaled_gemm(c, a, b, a_scale, b_scale, bias) -> None:
 
 def _launch_scaled_int8_gemm(c, a, b, a_scale, b_scale, bias) -> None:
     _lib.require_gpu(a, "scaled int8 gemm")
-    lib = _lib.load()
     m, k = a.shape
     n = b.shape[1]
     dev = a.device
     with _lib.device_guard(dev):
         ws_bytes = _lib.cached_workspace_bytes("fg_scaled_int8_gemm_workspace_bytes", m, n, k)
         ws = _lib.workspace(dev, ws_bytes) if ws_bytes else None
-        status = lib.fg_scaled_int8_gemm(
+        status = _lib.fast().scaled_gemm(
+            _lib.address("fg_scaled_int8_gemm"),
             a.data_ptr(), a.stride(0) if m > 1 else max(k, a.stride(0)),
             b.data_ptr(), b.stride(1) if n > 1 else max(k, b.stride(1)),
             a_scale.data_ptr(), 1 if a_scale.numel() > 1 or m == 1 else 0,

@@ -27,30 +27,42 @@ def _cdiv(a: int, b: int) -> int:
     return (a + b - 1) // b
 
 
+def _launch_raw(dev, a_ptr, lda, b_ptr, ldb, as_ptr, as_rs, as_cs, bs_ptr, bs_rs, bs_cs, c_ptr, ldc, c_code, m, n, k,
+                block_n: int, block_k: int, scales_pow2: bool) -> None:
+    """The C-ABI call with everything already reduced to addresses and integers (decode-sized calls are host-bound:
+    every tensor method that is not needed per call is kept out of this path)."""
+    with _lib.device_guard(dev):
+        stream = _lib.current_stream_ptr(dev)
+        ws_bytes = _lib.cached_workspace_bytes("fg_block_fp8_gemm_workspace_bytes", m, n, k)
+        if ws_bytes:
+            ws = _lib.workspace(dev, ws_bytes, stream)
+            ws_ptr, ws_len = ws.data_ptr(), ws.numel()
+        else:
+            ws_ptr, ws_len = None, 0
+        status = _lib.fast().block_fp8_gemm(
+            _lib.address("fg_block_fp8_gemm_pow2_scales" if scales_pow2 else "fg_block_fp8_gemm"),
+            a_ptr, lda, b_ptr, ldb, as_ptr, as_rs, as_cs, bs_ptr, bs_rs, bs_cs, c_ptr, ldc, c_code,
+            m, n, k, block_n, block_k, ws_ptr, ws_len, stream,
+        )
+    if status:
+        _lib.check(status, "fg_block_fp8_gemm")
+
+
 def _launch_block_gemm(a2d, b, as2d, bs, c2d, block_n: int, block_k: int, scales_pow2: bool = False) -> None:
     dev = a2d.device
     if dev.type != "cuda":
         _lib.require_gpu(a2d, "block fp8 gemm")
-    lib = _lib.load()
     m, k = a2d.shape
     n = b.shape[0]
-    with _lib.device_guard(dev):
-        stream = _lib.current_stream_ptr(dev)
-        ws_bytes = _lib.cached_workspace_bytes("fg_block_fp8_gemm_workspace_bytes", m, n, k)
-        ws = _lib.workspace(dev, ws_bytes, stream) if ws_bytes else None
-        entry = lib.fg_block_fp8_gemm_pow2_scales if scales_pow2 else lib.fg_block_fp8_gemm
-        status = entry(
-            a2d.data_ptr(), a2d.stride(0) if m > 1 else max(k, a2d.stride(0)),
-            b.data_ptr(), b.stride(0) if n > 1 else max(k, b.stride(0)),
-            as2d.data_ptr(), as2d.stride(0), as2d.stride(1),
-            bs.data_ptr(), bs.stride(0), bs.stride(1),
-            c2d.data_ptr(), c2d.stride(0) if m > 1 else max(n, c2d.stride(0)), _lib.DTYPE_CODE[c2d.dtype],
-            m, n, k, block_n, block_k,
-            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
-            stream,
-        )
-    if status:
-        _lib.check(status, "fg_block_fp8_gemm")
+    _launch_raw(
+        dev,
+        a2d.data_ptr(), a2d.stride(0) if m > 1 else max(k, a2d.stride(0)),
+        b.data_ptr(), b.stride(0) if n > 1 else max(k, b.stride(0)),
+        as2d.data_ptr(), as2d.stride(0), as2d.stride(1),
+        bs.data_ptr(), bs.stride(0), bs.stride(1),
+        c2d.data_ptr(), c2d.stride(0) if m > 1 else max(n, c2d.stride(0)), _lib.DTYPE_CODE[c2d.dtype],
+        m, n, k, block_n, block_k, scales_pow2,
+    )
 
 
 def w8a8_block_fp8_matmul(
@@ -100,11 +112,11 @@ def w8a8_block_fp8_matmul(
         return C
     if B.stride(1) != 1:
         B = B.contiguous()
-    a2d = A.view(M, K)
+    a2d = A if A.dim() == 2 else A.view(M, K)
     as2d = As if As.dim() == 2 else As.reshape(M, As.shape[-1])
     if (block_n, block_k) != (128, 128):
         as2d, Bs, block_n, block_k = _scales_at_128(as2d, Bs, N, K, block_n, block_k)
-    _launch_block_gemm(a2d, B, as2d, Bs, C.view(M, N), block_n, block_k, pow2)
+    _launch_block_gemm(a2d, B, as2d, Bs, C if C.dim() == 2 else C.view(M, N), block_n, block_k, pow2)
     return C
 
 
@@ -153,12 +165,20 @@ def fp8_matmul(
     if pow2:
         a_s = a_s.to(torch.float32)
         b_s = b_s.to(torch.float32)
-    out_shape = (*a.size()[:-1], N)
-    C = torch.empty((M, N), device=a.device, dtype=torch.bfloat16)
+    C = torch.empty((*a.size()[:-1], N), device=a.device, dtype=torch.bfloat16)
     if M == 0 or N == 0:
-        return C.view(out_shape)
-    _launch_block_gemm(a.view(M, K), b, a_s.view(M, -1), b_s, C, GROUP_SIZE, GROUP_SIZE, pow2)
-    return C.view(out_shape)
+        return C
+    dev = a.device
+    if dev.type != "cuda":
+        _lib.require_gpu(a, "block fp8 gemm")
+    # every operand is contiguous (asserted above), so the leading dimensions follow from the shapes: no views, no
+    # stride queries (the reference's direct wrapper exists for the same reason: cpp/lib/fp8_matmul_direct.cpp:62-63)
+    kb = a_s.numel() // M
+    assert kb * M == a_s.numel(), "a_s must hold one row of scales per row of a"
+    bs_cols = b_s.size(-1)
+    _launch_raw(dev, a.data_ptr(), K, b.data_ptr(), K, a_s.data_ptr(), kb, 1, b_s.data_ptr(), bs_cols, 1,
+                C.data_ptr(), N, _lib.FG_BF16, M, N, K, GROUP_SIZE, GROUP_SIZE, pow2)
+    return C
 
 
 def fp8_matmul_noop(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Tensor) -> torch.Tensor:
@@ -172,6 +192,5 @@ def fp8_matmul_noop(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: to
     M = a.numel() // K if K else 0
     N = b.size(0)
     assert b.size(1) == K, "a and b must have the same K dimension"
-    a_s.view(M, -1)  # the scales must fold to one row per activation row, as the launch would require
-    C = torch.empty((M, N), device=a.device, dtype=torch.bfloat16)
-    return C.view(*a.size()[:-1], N)
+    assert M == 0 or (a_s.numel() // M) * M == a_s.numel(), "a_s must hold one row of scales per row of a"
+    return torch.empty((*a.size()[:-1], N), device=a.device, dtype=torch.bfloat16)

@@ -219,3 +219,28 @@ def test_record_once_lists_every_call_site_once(tmp_path):
         assert len(lines) == want, lines
         assert lines[0] == "[DEBUG] flag_gems.some_operator.test_record_once_lists_every_call_site_once: GEMS SOME_OPERATOR"
     assert not [h for h in logging.getLogger("flag_gems").handlers if h.get_name() == "flag_gems_record"]
+
+
+def test_fastcall_module_marshals_the_decode_critical_calls():
+    """csrc/fastcall.c: the CPython module through which the hosts of the block GEMM, the group quantizer and the
+    scaled GEMM call the C ABI (a ctypes call spends 2-3 us on converting their 20-odd arguments).  On a host without
+    a GPU only calls that launch nothing can run: empty problems return FG_OK, a wrong argument count raises."""
+    import pytest
+
+    from flaggems_amd import _lib
+
+    f = _lib.fast()
+    assert f.block_fp8_gemm(_lib.address("fg_block_fp8_gemm"), None, 0, None, 0, None, 0, 0, None, 0, 0, None, 0, _lib.FG_BF16,
+                            0, 8, 128, 128, 128, None, 0, None) == _lib.FG_OK
+    # a negative size comes back as the library's status, with its message behind fg_last_error_string
+    assert f.block_fp8_gemm(_lib.address("fg_block_fp8_gemm"), None, 0, None, 0, None, 0, 0, None, 0, 0, None, 0, _lib.FG_BF16,
+                            -1, 8, 128, 128, 128, None, 0, None) == _lib.FG_ERR_INVALID_ARG
+    assert b"negative" in _lib.load().fg_last_error_string()
+    assert f.group_quant_fp8(_lib.address("fg_group_quant_fp8"), None, _lib.FG_BF16, 0, 0, 0, None, _lib.FG_FP8_E4M3FN, 0, None, 0, 1,
+                             128, 1e-10, -448.0, 448.0, 1.0 / 448.0, 0, 1, 0, None) == _lib.FG_OK
+    assert f.scaled_gemm(_lib.address("fg_scaled_fp8_gemm"), None, 0, None, 0, None, 0, None, 0, None, 0, None, 0, _lib.FG_BF16,
+                         0, 8, 128, None, 0, None) == _lib.FG_OK
+    with pytest.raises(TypeError):
+        f.block_fp8_gemm(_lib.address("fg_block_fp8_gemm"), 1, 2, 3)
+    with pytest.raises(TypeError):
+        f.scaled_gemm(_lib.address("fg_scaled_fp8_gemm"), "not a pointer", 0, None, 0, None, 0, None, 0, None, 0, None, 0, 0, 0, 8, 128, None, 0, None)
