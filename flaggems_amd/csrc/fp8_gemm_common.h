@@ -214,6 +214,7 @@ struct SmallMPlan {
   int q;          // staged: 4-row weight groups the kernel loads per chunk (<= 4 * rg)
   bool xlds;      // staged: the block keeps the activations of its K range in LDS
   bool own;       // staged: every wavefront has a chunk of its own and walks all of K
+  bool ring;      // staged, xlds: two slots of activations per wavefront, refilled pair by pair
   int waves;      // wavefronts per block: 4 or 8
   int kpw;        // K-blocks (K-block pairs when staged) per wavefront
   int splits;     // blocks along K that share one 64-row output chunk

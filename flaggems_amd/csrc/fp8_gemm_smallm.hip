@@ -292,14 +292,18 @@ __device__ __forceinline__ void dma_to_lds_4(uint32_t byte_off, const void* base
 // and the weight scales into LDS with a handful of global -> LDS copies (no barrier: a pair is multiplied by the
 // wavefront that copied for it, and the wait for its first weights is also the wait for its copies, which were
 // issued earlier and complete in order); the ring holds one pair, whose refill goes out as soon as it is in the slab,
-// and the chunk has no more 4-row groups than its rows need.  OWN (wide weights): every wavefront has a chunk of
+// and the chunk has no more 4-row groups than its rows need.  RING: the activations of a wavefront's pairs do not
+// fit LDS all at once (M = 16 with K of 7168 and more), so it keeps two slots and copies for pair i + 1 after pair i
+// is in the slab and before the refill goes out: the wait for the refilled weights is again the wait for the copies.
+// OWN (wide weights): every wavefront has a chunk of
 // its own and walks all of K, so the block shares the activations (one barrier) and nothing is added across
 // wavefronts.  Without XLDS (activations too large for LDS, or too few pairs per wavefront to pay for the copies)
 // the activation fragments travel in the register ring next to the weights.
-template <int TMX, int Q, int DEPTH, int WAVES, int MODE, bool XLDS, bool OWN = false>
+template <int TMX, int Q, int DEPTH, int WAVES, int MODE, bool XLDS, bool OWN = false, bool RING = false>
 __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArgs a) {
   static_assert(!XLDS || TMX == 1, "activations are kept in LDS for M <= 16 only");
   static_assert(!OWN || XLDS, "wavefronts with chunks of their own share the activations through LDS");
+  static_assert(!RING || (XLDS && !OWN && DEPTH == 1), "the two-slot form belongs to the per-wavefront copies with one pair in the ring");
   constexpr int RG = (Q + 3) / 4;
   constexpr int kRows = 16 * RG;
   constexpr int kSlab = kRows * 256;  // one K-block pair of the chunk
@@ -345,6 +349,8 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
 
   // ---- activations and their scales -> LDS (issued before the first weight load: they arrive first)
   constexpr bool PW = XLDS && !OWN;  // every wavefront copies what its own pairs of K-blocks need: no barrier
+  // RING: a wavefront keeps two slots only and copies pair i + 1 while it multiplies pair i (activations of the whole
+  // K range too large for LDS)
   const uint32_t lds_x = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + WAVES * kSlab;
   // shared form (OWN): rows x_lds_stride apart, 16-byte pieces permuted; [M][kbc] activation scales; [2][kbc] weight
   // scales per wavefront
@@ -356,11 +362,39 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
   // weight scales
   // (the block's pairs are dealt round-robin, so wavefront w's slots begin after those of the wavefronts before it)
   const int blk_pairs = pair_end - pair_lo;
-  const uint32_t slot0 = (uint32_t)(wave * (blk_pairs / WAVES) + min(wave, blk_pairs % WAVES));
+  const uint32_t slot0 = RING ? (uint32_t)(wave * 2) : (uint32_t)(wave * (blk_pairs / WAVES) + min(wave, blk_pairs % WAVES));
   const uint32_t pw_x = lds_x + slot0 * (uint32_t)g.M * 256u;
   const uint32_t pw_xs = lds_x + (uint32_t)(a.pw_pairs * g.M) * 256u + slot0 * (uint32_t)(2 * g.M) * 4u;
   const uint32_t pw_ws = lds_x + (uint32_t)(a.pw_pairs * g.M) * (256u + 8u) + slot0 * 16u;
-  if (PW) {
+  // RING: the i-th pair of this wavefront -> slot i & 1 (same layout as below, one pair at a time)
+  auto copy_pair = [&](int i) __attribute__((always_inline)) {
+    const int p = pair_lo + wave + i * WAVES;
+    const uint32_t s = (uint32_t)(i & 1);
+    const bool two = p * 2 + 1 < g.KB;
+    for (int j = 0; j * 4 < g.M; ++j) {
+      const int m = j * 4 + lg;
+      if (m < g.M) {
+        int piece = l16 ^ (m & 15);
+        if (!two && piece >= 8) piece -= 8;
+        dma_to_lds_16((uint32_t)m * (uint32_t)g.ldx + (uint32_t)p * 256u + (uint32_t)piece * 16u, x_base,
+                      pw_x + s * (uint32_t)g.M * 256u + (uint32_t)j * 1024u);
+      }
+    }
+    if (MODE == kModeBlock) {
+      if (lane < 2 * g.M) {  // lane = b * M + row
+        const int b = lane >= g.M ? 1 : 0, m = lane - b * g.M;
+        const int kb = p * 2 + ((b && two) ? 1 : 0);
+        dma_to_lds_4(((uint32_t)m * (uint32_t)g.xs_rs + (uint32_t)kb * xs_cs) * 4u, xs_base, pw_xs + s * (uint32_t)(2 * g.M) * 4u);
+      }
+      if (lane < 4) {  // lane = scale block * 2 + b
+        const int kb = p * 2 + (((lane & 1) && two) ? 1 : 0);
+        dma_to_lds_4((uint32_t)((int64_t)kb * g.ws_cs + ((lane & 2) ? ws_second : 0)) * 4u, ws_base, pw_ws + s * 16u);
+      }
+    }
+  };
+  if (RING) {
+    if (pair_lo + wave < pair_end) copy_pair(0);
+  } else if (PW) {
     const int first = pair_lo + wave;
     const int my_pairs = first < pair_end ? (pair_end - first + WAVES - 1) / WAVES : 0;
     const int recip = a.m_recip;
@@ -514,14 +548,15 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
   auto multiply = [&](const PairRegs<TMX, Q>& u, int pair) __attribute__((always_inline)) {
     const int kb = pair * 2;
     const bool two = kb + 1 < g.KB;
+    const int rs = RING ? (slot & 1) : slot;  // where this pair's activations and scales lie
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       if (b == 1 && !two) break;
       float ws1 = 1.f, ws2 = 1.f;
       if (MODE == kModeBlock) {
         if (PW) {
-          ws1 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(pw_ws + (uint32_t)(slot * 4 + b) * 4u);
-          ws2 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(pw_ws + (uint32_t)(slot * 4 + 2 + b) * 4u);
+          ws1 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(pw_ws + (uint32_t)(rs * 4 + b) * 4u);
+          ws2 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(pw_ws + (uint32_t)(rs * 4 + 2 + b) * 4u);
         } else if (XLDS) {
           ws1 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(lds_ws + (uint32_t)(kb + b - kb_lo) * 4u);
           ws2 = *reinterpret_cast<const __attribute__((address_space(3))) float*>(lds_ws + (uint32_t)(kbc + kb + b - kb_lo) * 4u);
@@ -536,12 +571,12 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
       for (int t = 0; t < TMX; ++t) {
         if (PW) {
           // the pair's 16 pieces are permuted as a whole: logical piece b*8 + lg (+4) sits at that number ^ perm
-          const uint32_t at = pw_x + ((uint32_t)(slot * g.M) + mrow) * 256u;
+          const uint32_t at = pw_x + ((uint32_t)(rs * g.M) + mrow) * 256u;
           const u32x4 lo = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + (((uint32_t)(b * 8 + lg) ^ perm) << 4));
           const u32x4 hi = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + (((uint32_t)(b * 8 + lg + 4) ^ perm) << 4));
           xf[t] = join(lo, hi);
           xsc[t] = (MODE == kModeBlock)
-                       ? *reinterpret_cast<const __attribute__((address_space(3))) float*>(pw_xs + ((uint32_t)((slot * 2 + b) * g.M) + mrow) * 4u)
+                       ? *reinterpret_cast<const __attribute__((address_space(3))) float*>(pw_xs + ((uint32_t)((rs * 2 + b) * g.M) + mrow) * 4u)
                        : 1.f;
         } else if (XLDS) {
           const uint32_t at = lds_xrow[t] + (uint32_t)(kb + b - kb_lo) * 128u;
@@ -608,6 +643,12 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
         // With the activations in LDS the ring holds weights only and its registers are free once they are in
         // the slab: the refill goes out before the multiplication, so the slab double-buffers the ring.  With
         // activation fragments in the ring the refill has to follow the multiplication.
+        if (RING) {
+          // the slot of pair i + 1 was last read by the multiplication of pair i - 1; its copies go out ahead of the
+          // refill, so the wait for the refilled weights is the wait for them as well
+          asm volatile("" ::: "memory");
+          if (refill < pair_end) copy_pair(slot + 1);
+        }
         if (XLDS && refill < pair_end) load_w(ring[d], refill);
         multiply(ring[d], pair);
         if (!XLDS && refill < pair_end) {
@@ -669,7 +710,7 @@ inline int64_t decode_lds_bytes_per_wave(int q, int waves, int64_t M, int64_t pa
   return (int64_t)waves * 16 * ((q + 3) / 4) * 256 + pairs * (M * 256 + 2 * M * 4 + 16);
 }
 
-template <int TMX, int Q, int DEPTH, int WAVES, bool XLDS, bool OWN = false>
+template <int TMX, int Q, int DEPTH, int WAVES, bool XLDS, bool OWN = false, bool RING = false>
 int launch_transpose(const SmallArgs& sa, int mode, hipStream_t stream) {
   // WAVES slabs of 4 KB per 16 rows; the reduction buffer (WAVES * 16*TMX * rows floats) reuses the same memory
   constexpr int kSlabs = WAVES * 16 * ((Q + 3) / 4) * 256;
@@ -678,9 +719,9 @@ int launch_transpose(const SmallArgs& sa, int mode, hipStream_t stream) {
   if (lds_bytes > kDecodeLdsLimit) FG_FAIL(FG_ERR_LAUNCH, "fp8 gemm (small M): %d bytes of LDS planned", lds_bytes);
   const dim3 grid((uint32_t)(OWN ? ceil_div(sa.n_chunks, WAVES) : sa.n_chunks), (uint32_t)sa.splits, (uint32_t)(sa.g.batch > 1 ? sa.g.batch : 1));
   const dim3 block(WAVES * 64);
-  auto kb = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeBlock, XLDS, OWN>;
-  auto kr = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeRowCol, XLDS, OWN>;
-  auto ki = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeRowColI8, XLDS, OWN>;
+  auto kb = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeBlock, XLDS, OWN, RING>;
+  auto kr = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeRowCol, XLDS, OWN, RING>;
+  auto ki = fp8_gemm_transpose_kernel<TMX, Q, DEPTH, WAVES, kModeRowColI8, XLDS, OWN, RING>;
   static PerDeviceFlags lds_limit_raised = {};  // per instantiation
   {
     const hipError_t e = raise_dynamic_lds_limit(lds_limit_raised, XLDS ? kDecodeLdsLimit : kSlabs, reinterpret_cast<const void*>(kb), reinterpret_cast<const void*>(kr),
@@ -746,6 +787,14 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
     auto round_q = [&](int need) { int q = 16; for (int i = 7; i >= 0; --i) if (kQ[i] >= need) q = kQ[i]; return q; };
     int q = round_q(p.q);
     p.xlds = p.tmx == 1 && kpw >= (M > 8 ? 2 : 3) && decode_lds_bytes_per_wave(q, p.waves, M, std::min<int64_t>(pairs, kpw * p.waves)) <= kDecodeLdsLimit;
+    // Too large for LDS as a whole: two slots per wavefront, pair i + 1 copied while pair i is multiplied.  Only for
+    // chunks with at least as many rows as there are activation rows (N = 7168, K = 16384, M = 16: 25.9 -> 22.9 us;
+    // N = 4608, K = 7168: 11.0 -> 10.0; N = K = 8192: 17.9 -> 16.8; narrower chunks move more activation than weight
+    // bytes and do better with fewer, taller chunks below: N = 1024, K = 8192, M = 16: 7.9 us there, 9.8 us here).
+    // Where everything fits, the copies up front win: the same loop on N = 2112, K = 7168 takes 7.4 instead of 5.7 us.
+    p.ring = !p.xlds && p.tmx == 1 && kpw >= (M > 8 ? 2 : 3) && ceil_div(N, chunks) >= M &&
+             decode_lds_bytes_per_wave(q, p.waves, M, 2 * p.waves) <= kDecodeLdsLimit;
+    if (p.ring) p.xlds = true;
     if (!p.xlds && p.tmx == 1 && M > 4 && N <= 64 * B) {
       // every block fetches all M activation rows of its K range per pair of K-blocks: chunks of fewer rows than
       // that move more activation than weight bytes (N = 2048, K = 1024, M = 16: 256 chunks of 8 rows 3.8 us,
@@ -776,7 +825,7 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   p.own = p.tmx == 1 && KB >= 2 && KB <= 32 && ceil_div(N, 16) * entries >= 5 * (int64_t)cu_count() &&
           decode_lds_bytes(4, 4, M, KB) <= kDecodeLdsLimit / 2;
   if (p.own) {
-    p.staged = true; p.xlds = true; p.q = 4; p.rg = 1; p.waves = 4; splits = 1; kpw = (KB + 1) / 2;
+    p.staged = true; p.xlds = true; p.ring = false; p.q = 4; p.rg = 1; p.waves = 4; splits = 1; kpw = (KB + 1) / 2;
     p.n_chunks = (int)ceil_div(N, 16);
   }
   p.kpw = (int)kpw;
@@ -799,7 +848,7 @@ int launch_small_m(const GemmArgs& g, int mode, const SmallMPlan& plan, void* wo
   sa.rows_rem = (int)(g.N % plan.n_chunks);
   sa.x_lds_stride = plan.xlds ? x_lds_stride_for(std::min<int64_t>(g.KB, (int64_t)plan.kpw * plan.waves * 2)) : 0;
   sa.m_recip = (int)(65535 / g.M + 1);
-  sa.pw_pairs = (int)std::min<int64_t>((g.KB + 1) / 2, (int64_t)plan.kpw * plan.waves);
+  sa.pw_pairs = plan.ring ? 2 * plan.waves : (int)std::min<int64_t>((g.KB + 1) / 2, (int64_t)plan.kpw * plan.waves);
   sa.partials = nullptr;
   sa.counters = nullptr;
   sa.partials_per_entry = 0;
@@ -827,6 +876,18 @@ int launch_small_m(const GemmArgs& g, int mode, const SmallMPlan& plan, void* wo
               (long long)g.ldx, (long long)g.ldw);
     if (g.batch > 65535) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm (small M): at most 65535 batch entries per launch, got %d", g.batch);
     if (plan.own) return launch_transpose<1, 4, 1, 4, true, true>(sa, mode, stream);
+    if (plan.xlds && plan.ring) {
+      switch (plan.q) {
+        case 1: return launch_transpose<1, 1, 1, 8, true, false, true>(sa, mode, stream);
+        case 2: return launch_transpose<1, 2, 1, 8, true, false, true>(sa, mode, stream);
+        case 3: return launch_transpose<1, 3, 1, 8, true, false, true>(sa, mode, stream);
+        case 4: return launch_transpose<1, 4, 1, 8, true, false, true>(sa, mode, stream);
+        case 6: return launch_transpose<1, 6, 1, 8, true, false, true>(sa, mode, stream);
+        case 8: return launch_transpose<1, 8, 1, 8, true, false, true>(sa, mode, stream);
+        case 12: return launch_transpose<1, 12, 1, 8, true, false, true>(sa, mode, stream);
+        default: return launch_transpose<1, 16, 1, 8, true, false, true>(sa, mode, stream);
+      }
+    }
     if (plan.xlds) {
       switch (plan.q) {
         case 1: return launch_transpose<1, 1, 1, 8, true>(sa, mode, stream);

@@ -179,15 +179,18 @@ def test_33_to_128_rows(M, N, K, dtype):
 @pytest.mark.parametrize("M,N,K", [(1, 2112, 7168), (16, 2112, 7168), (5, 1000, 7168), (3, 200, 8192), (7, 300, 16512),
                                    (16, 4608, 7168), (12, 7168, 16384), (2, 7168, 16384), (1, 24576, 1536),
                                    (32, 2112, 7168), (20, 4608, 4096), (1, 9, 1024), (4, 130, 2048), (9, 4099, 7296),
-                                   (16, 32768, 512), (5, 24580, 384), (2, 20480, 256), (16, 28672, 4096)])
+                                   (16, 32768, 512), (5, 24580, 384), (2, 20480, 256), (16, 28672, 4096),
+                                   (16, 4612, 7296), (13, 7168, 16512), (16, 8192, 8192), (10, 5000, 12416), (8, 7168, 16384)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_up_to_32_rows_uneven_chunks(M, N, K, dtype):
     """M <= 32 takes the kernel that deals the weight rows out evenly over the compute units: chunks that differ by a
     row and begin anywhere (so that a chunk's rows lie in two 128-row scale blocks), chunks of fewer than 16 rows, N
     that is no multiple of 4, K split over blocks, an odd number of K-blocks, activations kept in LDS (long K, M <=
-    16) or fetched per K-block (short K, M = 12 with K = 16384, M > 16), wide weights (a wavefront per 16 rows, the
-    last four shapes: K of 2, 3 and 4 K-blocks, N that ends inside a 16-row group, activations too large to share),
-    column-major activation scales; against the oracle and bit-identical on reruns."""
+    16) or fetched per K-block (short K, M > 16), wide weights (a wavefront per 16 rows, the four shapes from
+    (16, 32768, 512) on: K of 2, 3 and 4 K-blocks, N that ends inside a 16-row group, activations too large to share),
+    activations too large for LDS as a whole and copied pair by pair into two slots per wavefront (M = 12 with
+    K = 16384 and the last five shapes: an odd number of K-blocks, chunks that begin anywhere), column-major activation
+    scales; against the oracle and bit-identical on reruns."""
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=17)
     want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
     args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
@@ -202,10 +205,11 @@ def test_up_to_32_rows_uneven_chunks(M, N, K, dtype):
     assert torch.equal(cm.view(torch.int8), got.view(torch.int8))
 
 
-def test_rows_of_a_small_batch_do_not_depend_on_its_size():
+@pytest.mark.parametrize("N,K", [(2112, 7168), (4608, 7168)])
+def test_rows_of_a_small_batch_do_not_depend_on_its_size(N, K):
     """Row m of the product is the same bits whether the call has 1, 8 or 16 activation rows: the kernels for M <= 16
-    differ only in where the activations are kept."""
-    N, K = 2112, 7168
+    differ only in where the activations are kept (all of them in LDS, or two slots per wavefront refilled pair by
+    pair: N = 4608 with 16 rows)."""
     xq, wq, xs, ws = _quantized_inputs(16, N, K, seed=23)
     xq, wq, xs, ws = xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV)
     full = flag_gems.w8a8_block_fp8_matmul(xq, wq, xs, ws, [128, 128], output_dtype=torch.float32)

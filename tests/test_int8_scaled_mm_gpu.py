@@ -117,7 +117,7 @@ def test_int8_sums_are_exact_in_bf16_above_128_rows():
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 512, 8192), (4, 2112, 7168), (16, 4096, 4096), (9, 24576, 1536), (32, 768, 2048),
-                                   (33, 512, 8192), (64, 2112, 7168)])
+                                   (33, 512, 8192), (64, 2112, 7168), (16, 4608, 7168)])
 def test_int8_sums_are_exact_up_to_64_rows(M, N, K):
     """The kernels for few rows split K over wavefronts and blocks: the int32 partial sums are added as integers, so
     the fp32 result is the one rounding of the exact sum, also where the sum needs more than 24 bits."""

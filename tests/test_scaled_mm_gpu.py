@@ -22,6 +22,8 @@ MNK = [
     (32, 8192, 4096), (32, 16384, 4096), (33, 1024, 1024), (33, 8192, 128), (64, 2048, 512), (64, 16384, 1024),
     (100, 8192, 512), (100, 1024, 4096), (48, 640, 4096), (128, 32768, 4096), (256, 4096, 4096), (512, 256, 1024), (512, 8192, 4096),
     (512, 16384, 128), (512, 24576, 128), (8, 20496, 1536),
+    # 16 rows against long K: the activations pass through two LDS slots per wavefront, pair by pair
+    (16, 4608, 7296), (13, 7168, 16384),
     # few 256 x 256 tiles with a long K: compute units share tiles and add their sums through the workspace
     (384, 5632, 8320), (300, 3088, 8448),
     # K that is not a multiple of 128 (operands go through registers), above and below 128 rows
