@@ -33,6 +33,9 @@ from .grouped_block_fp8_matmul import grouped_w8a8_block_fp8_matmul
 
 logger = logging.getLogger("flag_gems." + __name__.split(".")[-1])
 
+_SORT_MAX_SLOTS = 65536   # limits of fg_moe_sort_slots
+_SORT_MAX_EXPERTS = 960
+
 
 def moe_sort_slots(
     topk_ids: torch.Tensor, num_experts: int, expert_map: Optional[torch.Tensor] = None
@@ -44,11 +47,34 @@ def moe_sort_slots(
     ties in slot order, and the cumulative int32 ends of the ``num_experts`` local experts' segments.  With
     ``expert_map`` (global expert -> local expert or -1, the reference's convention:
     src/flag_gems/fused/moe_align_block_size.py:817-818) slots of experts that are not local sort last, behind
-    ``offs[-1]``.  Everything stays on the device of ``topk_ids``; nothing synchronises.
+    ``offs[-1]``, as do slots whose id names no expert at all.  Everything stays on the device of ``topk_ids``; nothing
+    synchronises.  Up to 65536 slots and 960 experts the table comes from one kernel (``fg_moe_sort_slots``, a stable
+    counting sort in a single block); larger tables from torch's stable sort, with the same result.
     """
-    flat = topk_ids.reshape(-1).to(torch.int64)
+    flat = topk_ids.reshape(-1)
+    n_slots = flat.numel()
+    if (flat.is_cuda and n_slots <= _SORT_MAX_SLOTS and 1 <= num_experts <= _SORT_MAX_EXPERTS
+            and flat.dtype in (torch.int32, torch.int64)
+            and (expert_map is None or (expert_map.dtype in (torch.int32, torch.int64) and expert_map.device == flat.device))):
+        # one kernel: a stable counting sort in a single block
+        flat = flat.contiguous()
+        emap = None if expert_map is None else expert_map.reshape(-1).contiguous()
+        sorted_slots = torch.empty(n_slots, dtype=torch.int32, device=flat.device)
+        offs = torch.empty(num_experts, dtype=torch.int32, device=flat.device)
+        with _lib.device_guard(flat.device):
+            status = _lib.load().fg_moe_sort_slots(
+                flat.data_ptr(), flat.element_size(), n_slots, num_experts,
+                None if emap is None else emap.data_ptr(), 0 if emap is None else emap.element_size(),
+                0 if emap is None else emap.numel(), sorted_slots.data_ptr(), offs.data_ptr(),
+                _lib.current_stream_ptr(flat.device))
+        _lib.check(status, "fg_moe_sort_slots")
+        return sorted_slots, offs
+    # tables beyond the kernel's limits: the same table from torch's stable sort
+    flat = flat.to(torch.int64)
     if expert_map is not None:
-        flat = expert_map.to(torch.int64)[flat]
+        inside = (flat >= 0) & (flat < expert_map.numel())
+        flat = torch.where(inside, expert_map.reshape(-1).to(torch.int64)[flat.clamp(0, max(expert_map.numel() - 1, 0))],
+                           torch.full_like(flat, -1))
     key = torch.where((flat >= 0) & (flat < num_experts), flat, torch.full_like(flat, num_experts))
     sorted_slots = torch.argsort(key, stable=True).to(torch.int32)
     counts = torch.zeros(num_experts + 1, dtype=torch.int64, device=flat.device)

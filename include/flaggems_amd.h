@@ -176,6 +176,22 @@ int fg_moe_sum(const void* in, int dtype, int64_t tokens, int64_t top_k, int64_t
                int64_t in_slot_stride, void* out, int64_t out_token_stride, void* stream);
 
 /*
+ * Routing table of an expert layer for fg_grouped_block_fp8_gemm: the routed slots sorted by expert.
+ *     key(s) = local expert of slot s, or num_experts if it has none
+ *     sorted_slots = the slot numbers 0 .. n_slots-1 in ascending order of key, ties in slot order (int32 [n_slots])
+ *     offs[e]      = number of slots with key <= e (int32 [num_experts]: the cumulative ends of the experts' segments)
+ * topk_ids: [n_slots] integers of id_bytes (4 or 8) bytes, slot t * top_k + j = the j-th expert of token t.
+ * expert_map (may be NULL): [map_len] integers of map_bytes (4 or 8) bytes, global expert -> local expert or -1; an id
+ * outside [0, map_len), a map entry outside [0, num_experts) and, without a map, an id outside [0, num_experts) all
+ * mean "no local expert": such slots sort behind offs[num_experts - 1].  One block, no workspace, nothing synchronises;
+ * at most 960 experts and 65536 slots (FG_ERR_UNSUPPORTED beyond).
+ * Stands in for the sorting stages of moe_align_block_size (src/flag_gems/fused/moe_align_block_size.py:405-519, the
+ * expert_map convention of :817-818) without the padding to a block multiple, which the grouped GEMM here does not need.
+ */
+int fg_moe_sort_slots(const void* topk_ids, int id_bytes, int64_t n_slots, int64_t num_experts, const void* expert_map,
+                      int map_bytes, int64_t map_len, int32_t* sorted_slots, int32_t* offs, void* stream);
+
+/*
  * RMSNorm (optionally preceded by the residual add) fused into the quantizer: every row of x [rows, cols] is
  * normalised, multiplied by weight [cols] (x's type), rounded to x's type as a separate norm kernel would have
  * stored it, and quantized exactly as fg_group_quant_fp8 quantizes that stored tensor (same codes and scales, bit

@@ -173,6 +173,44 @@ def test_moe_align_tables_with_interior_foreign_blocks():
                 assert float(got[st[b * block_m:(b + 1) * block_m]].abs().max()) == 0.0
 
 
+def _sorted_table(ids, experts, emap):
+    """The table by definition, on the host: key = local expert or `experts`; a stable sort by key; cumulative counts."""
+    flat = ids.reshape(-1).cpu().long()
+    if emap is not None:
+        m = emap.cpu().long()
+        inside = (flat >= 0) & (flat < m.numel())
+        flat = torch.where(inside, m[flat.clamp(0, max(m.numel() - 1, 0))], torch.full_like(flat, -1))
+    key = torch.where((flat >= 0) & (flat < experts), flat, torch.full_like(flat, experts))
+    order = torch.sort(key, stable=True).indices.to(torch.int32)
+    offs = torch.cumsum(torch.bincount(key, minlength=experts + 1)[:experts], 0).to(torch.int32)
+    return order, offs
+
+
+@pytest.mark.parametrize("slots", [0, 1, 63, 64, 65, 1000, 1024, 1025, 8192, 32768, 65536, 70000])
+@pytest.mark.parametrize("experts", [1, 8, 256, 960, 1000])
+def test_moe_sort_slots_is_a_stable_sort_by_expert(slots, experts):
+    """The routing table against its definition: every size around the kernel's 1024-slot rounds and its limits
+    (65536 slots, 960 experts; beyond them the table comes from torch's sort and must be the same), int32 and int64
+    ids, ids that name no expert (-1, too large), an expert_map of either width with foreign experts."""
+    g = torch.Generator().manual_seed(slots * 7 + experts)
+    for id_dtype, map_dtype in ((torch.int64, None), (torch.int32, torch.int32), (torch.int64, torch.int64), (torch.int32, None)):
+        global_experts = experts if map_dtype is None else experts + 5
+        ids = torch.randint(-1, global_experts + 2, (slots,), generator=g).to(id_dtype)
+        if slots > 100:  # a long run of one expert, and one expert that never occurs
+            ids[10:90] = 0
+            ids[ids == min(1, global_experts - 1)] = 0
+        emap = None
+        if map_dtype is not None:
+            perm = torch.randperm(global_experts, generator=g)
+            emap = torch.full((global_experts,), -1, dtype=map_dtype)
+            emap[perm[:experts]] = torch.arange(experts, dtype=map_dtype)
+        got_rows, got_offs = flag_gems.moe_sort_slots(ids.to(DEV), experts, None if emap is None else emap.to(DEV))
+        want_rows, want_offs = _sorted_table(ids, experts, emap)
+        assert got_rows.dtype == torch.int32 and got_offs.dtype == torch.int32
+        assert torch.equal(got_offs.cpu(), want_offs), f"offs, {slots} slots, {experts} experts, {id_dtype}, map {map_dtype}"
+        assert torch.equal(got_rows.cpu(), want_rows), f"order, {slots} slots, {experts} experts, {id_dtype}, map {map_dtype}"
+
+
 def test_moe_sum_rounds_once():
     for dtype in (torch.bfloat16, torch.float16, torch.float32):
         x = (torch.randn(37, 6, 264, device=DEV) * 3).to(dtype)
