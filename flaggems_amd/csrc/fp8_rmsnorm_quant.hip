@@ -88,7 +88,11 @@ __device__ __forceinline__ void narrow_chunk(const float (&v)[8], uint32_t (&w)[
 // QUANT: 0 = the norm alone, 1 = with the quantizer and its rules taken from the arguments, 2 = with the quantizer
 // under the rules of per_token_group_quant_fp8's defaults (scale = amax * (1 / max), true division, no power-of-two
 // rounding, e4m3), which lets the compiler drop every rule switch from the loop.
-template <int XDT, int CHUNKS, int QUANT>
+// LPG: lanes per quantization group when known at compile time (16 = groups of 128 elements), 0 = from the arguments:
+// the group maximum is then four DPP instructions instead of a chain of six tests.
+// A wavefront whose 64 chunks of a round all lie past the row's end (rows of 7168 elements: the last round of
+// wavefronts 2 and 3) skips the round; its zeros would not have changed any sum.
+template <int XDT, int CHUNKS, int QUANT, int LPG = 0>
 __global__ __launch_bounds__(kNormThreads) void rms_norm_quant_kernel(NormQuantArgs a) {
   if (QUANT == 2) {
     a.q.scale_rule = FG_SCALE_MUL_INV;
@@ -102,6 +106,7 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_quant_kernel(NormQuantA
   __shared__ float wave_sums[2][kNormWaves];
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t wave_first = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid & ~63u));  // chunk of lane 0 in round 0
   const bool add_residual = a.residual != nullptr;
   constexpr bool quantize = QUANT != 0;
   const Raw* wp = reinterpret_cast<const Raw*>(a.weight);
@@ -118,6 +123,11 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_quant_kernel(NormQuantA
     for (int i = 0; i < CHUNKS; ++i) {
       const uint32_t c = tid + (uint32_t)i * kNormThreads;
       const bool live = c < a.chunks_per_row;
+      if (wave_first + (uint32_t)i * kNormThreads >= a.chunks_per_row) {  // uniform: nothing of this round in this wavefront
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] = 0.0f;
+        continue;
+      }
       uint32_t rw[kWords];
       if (live) {
         uint32_t w[kWords];
@@ -161,6 +171,7 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_quant_kernel(NormQuantA
     for (int i = 0; i < CHUNKS; ++i) {
       const uint32_t c = tid + (uint32_t)i * kNormThreads;
       const bool live = c < a.chunks_per_row;
+      if (wave_first + (uint32_t)i * kNormThreads >= a.chunks_per_row) continue;
       uint32_t ww[kWords];
       float wv[8];
       if (live) load_chunk<XDT, kWords>(wp + (size_t)c * 8, ww);
@@ -187,14 +198,16 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_quant_kernel(NormQuantA
       if (live && a.y) store_chunk<XDT, kWords>(reinterpret_cast<Raw*>(a.y) + (int64_t)row * a.y_row_stride + (size_t)c * 8, yw);
       if (quantize) {  // uniform over the workgroup
         float yv[8];
-        const uint32_t m = group_max_lanes(widen_chunk<XDT, kWords>(yw, yv), a.lanes_per_group);
+        const uint32_t own = widen_chunk<XDT, kWords>(yw, yv);
+        const uint32_t m = LPG != 0 ? group_max_u32<LPG>(own) : group_max_lanes(own, a.lanes_per_group);
         uint32_t w0, w1;
         const float s = quantize_chunk<XDT>(yv, m, a.q, w0, w1);
         if (live) {
           const u32x2 out = {w0, w1};
           *reinterpret_cast<u32x2*>(a.q.q + (int64_t)row * a.q.q_row_stride + (size_t)c * 8) = out;
-          if (c % a.lanes_per_group == 0)
-            a.q.s[(int64_t)row * a.q.s_row_stride + (int64_t)(c / a.lanes_per_group) * a.q.s_col_stride] = s;
+          const uint32_t lpg = LPG != 0 ? (uint32_t)LPG : a.lanes_per_group;
+          if (c % lpg == 0)
+            a.q.s[(int64_t)row * a.q.s_row_stride + (int64_t)(c / lpg) * a.q.s_col_stride] = s;
         }
       }
     }
@@ -213,6 +226,7 @@ int launch_norm(const NormQuantArgs& a, int cus, hipStream_t stream) {
   do {                                                                                                               \
     if (quant == 0) FG_LAUNCH((rms_norm_quant_kernel<XDT, C, 0>), g, b, 0, stream, a);                      \
     else if (quant == 1) FG_LAUNCH((rms_norm_quant_kernel<XDT, C, 1>), g, b, 0, stream, a);                 \
+    else if (a.lanes_per_group == 16) FG_LAUNCH((rms_norm_quant_kernel<XDT, C, 2, 16>), g, b, 0, stream, a); \
     else FG_LAUNCH((rms_norm_quant_kernel<XDT, C, 2>), g, b, 0, stream, a);                                 \
   } while (0)
   if (per_thread <= 1) FG_NORM_LAUNCH(1);
