@@ -118,6 +118,7 @@ struct PpArgs {
   uint64_t group4_magic;  // ceil(2^40 / (4 * tiles_n)) when that divides every tile number exactly, else 0 (see tile_of_sid)
 };
 
+constexpr int kMaxCutItems = 1024;  // 64 KB slots of partial sums for cut tiles (64 MB): a work item of a 64 JN-row tile takes JN of them
 constexpr int kPartialFloatsPerWave = 64 * 128;                      // one wavefront's 64 x 128 results
 constexpr int kPartialFloatsPerSlot = 8 * kPartialFloatsPerWave;     // a whole 256 x 256 tile
 constexpr size_t kPartialSlotBytes = (size_t)kPartialFloatsPerSlot * 4;  // 256 KB
@@ -691,39 +692,41 @@ __device__ __forceinline__ void finish_cut_tile(const PpArgs& a, const v4f (&acc
   if (lane == 0) prev = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   prev = (unsigned int)__builtin_amdgcn_readfirstlane((int)prev);
   if (prev != (unsigned int)(cuts - 1)) return;
-  // Half of the piece at a time (its own sums are in the workspace like everybody's, so the accumulators are free),
-  // sixteen registers of partial sums in flight: with two fragments per wavefront more does not fit the registers.
-  constexpr int kPart = 4 / JN;  // MFMA tiles per load batch
+  // A part of the piece at a time (its own sums are in the workspace like everybody's, so the accumulators are free):
+  // halves for short tiles, quarters for 256-row tiles; sixteen registers of partial sums in flight.
+  constexpr int kParts = JN == kTM ? 4 : 2;   // parts of the piece
+  constexpr int kNT = kTN / kParts;           // MFMA tiles per part
+  constexpr int kBatch = 4 / JN;              // MFMA tiles per load batch
 #pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    v4f r[kTN / 2][JN];
+  for (int part = 0; part < kParts; ++part) {
+    v4f r[kNT][JN];
     for (int q = 0; q < cuts; ++q) {
       const float* const src = uniform_ptr(a.partials + ((size_t)((tile << a.cut_shift) + q) * 8 + wave) * kFloats);
 #pragma unroll
-      for (int part = 0; part < kTN / 2 / kPart; ++part) {
-        v4f tmp[kPart][JN];
+      for (int b = 0; b < kNT / kBatch; ++b) {
+        v4f tmp[kBatch][JN];
 #pragma unroll
-        for (int t = 0; t < kPart; ++t)
+        for (int t = 0; t < kBatch; ++t)
 #pragma unroll
           for (int j = 0; j < JN; ++j)
-            load_x4_agent(tmp[t][j], src + ((half * (kTN / 2) + part * kPart + t) * JN + j) * 256, lane_off);
+            load_x4_agent(tmp[t][j], src + ((part * kNT + b * kBatch + t) * JN + j) * 256, lane_off);
 #pragma unroll
-        for (int t = 0; t < kPart; ++t)
+        for (int t = 0; t < kBatch; ++t)
 #pragma unroll
           for (int j = 0; j < JN; ++j)  // the values are operands of the wait, so no use can move above it
             asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[t][j]) : : "memory");
 #pragma unroll
-        for (int t = 0; t < kPart; ++t)
+        for (int t = 0; t < kBatch; ++t)
 #pragma unroll
           for (int j = 0; j < JN; ++j) {
-            const int tt = part * kPart + t;
+            const int tt = b * kBatch + t;
             if (q == 0) r[tt][j] = tmp[t][j]; else r[tt][j] += tmp[t][j];  // (no "0 + x" in the sum)
           }
       }
     }
-    store_tile<kModeBlock, false, SCATTER, JN, F16, kTN / 2>(a.g, r, m_base, n_base, l16, lg, m_end,
-                                                             SCATTER && a.c_rows > 0 ? a.row_index : nullptr, a.c_rows,
-                                                             a.row_weight, half * 2);
+    store_tile<kModeBlock, false, SCATTER, JN, F16, kNT>(a.g, r, m_base, n_base, l16, lg, m_end,
+                                                         SCATTER && a.c_rows > 0 ? a.row_index : nullptr, a.c_rows,
+                                                         a.row_weight, part * (kNT / 2));
   }
   if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the counted waits of the main loop start from zero
@@ -744,7 +747,12 @@ template <bool SK, int MODE, bool ALIGNED, bool GROUPED = false, bool POW2 = fal
 __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   static_assert(JN == kTM || (GROUPED && JN >= 1 && JN < kTM), "short tiles: grouped problems only");
   constexpr int kTileRows = 64 * JN;
-  constexpr bool kCuts = GROUPED && JN < kTM;  // tiles may be cut along K (cut_shift = 0: they are not)
+  constexpr bool kCuts = GROUPED;  // tiles may be cut along K (cut_shift = 0: they are not)
+  // Short tiles finish a cut tile in the fetch slot that follows it, like a whole tile.  With 128 accumulators that
+  // code does not fit the registers of the hot loop (242 spilled), and the walk of a block is [whole tiles][its cut
+  // work items] anyway: the loop runs once for the whole tiles and once per work item, which is finished between
+  // the runs, as the shared tiles of a stream-K launch are.
+  constexpr bool kCutsInLoop = kCuts && JN < kTM;
   // Short tiles stream weights for next to no arithmetic, and what sets their pace is how many weight bytes a compute
   // unit has in flight: the activation stages shrink to the tile's rows and the LDS they leave holds a fourth weight
   // stage, so that group B loads three steps ahead instead of two.
@@ -782,6 +790,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
       const int full = n_tiles / grid * grid, rest = n_tiles - full;
       int best = 0, best_cost = g.KB;
       for (int sh = 1; sh <= a.cut_shift; ++sh) {
+        if ((rest << sh) * JN > kMaxCutItems) break;  // slots for the partial sums
         const int cost = ((rest << sh) + grid - 1) / grid * ((g.KB >> sh) + 8);
         if (cost < best_cost) { best_cost = cost; best = sh; }
       }
@@ -949,7 +958,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     pending = false;
   };
   auto flush_whole_tile = [&]() __attribute__((always_inline)) {
-    if constexpr (kCuts) {
+    if constexpr (kCutsInLoop) {
       if (pend_idx >= a.cut_full) {
         wait_vmem<0>();
         finish_cut_tile<GROUPED, JN, F16>(a, acc, pend_idx - a.cut_full, pend_m, pend_n, pend_m_end, wave, lane, l16, lg);
@@ -1143,6 +1152,16 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     } else if (pending) {
       flush_whole_tile();
     }
+  } else if (kCuts && !kCutsInLoop) {
+    const int n_whole = a.cut_shift != 0 ? a.cut_full / (int)gridDim.x * g.KB : total;
+    run_steps(0, n_whole);
+    if (pending) flush_whole_tile();
+    for (int t0 = n_whole; t0 < total; t0 += a.cut_steps) {  // this block's work items of cut tiles
+      run_steps(t0, t0 + a.cut_steps);
+      wait_vmem<0>();
+      finish_cut_tile<GROUPED, JN, F16>(a, acc, pend_idx - a.cut_full, pend_m, pend_n, pend_m_end, wave, lane, l16, lg);
+      clear_acc();
+    }
   } else {
     run_steps(0, total);
     if (pending) flush_whole_tile();
@@ -1271,12 +1290,13 @@ size_t transposed_scales_bytes(int64_t M, int64_t KB) { return (size_t)((M * KB 
 // Short tiles of grouped problems (the JN = 1 instantiation) and their cuts along K.
 constexpr int kShortTileRows = 64;
 constexpr size_t kCutSlotBytes = (size_t)8 * kTN * 256 * 4;  // a work item's partial sums: 8 wavefronts x 16 x 128 floats
-constexpr int kMaxCutItems = 1024;                           // work items of a cut problem (64 MB of partial sums)
 // Largest number of cuts per tile of the last round, as a shift (the kernel picks among 0..this from the real tile
 // count): whole K-blocks, at least 8 per cut, and slots for a round short of one tile.
+// (256-row tiles, jn = 4: a round short of one tile would need four times the slots; the kernel, which knows how many
+// tiles the last round really holds, takes a shift only while their work items fit)
 int max_cut_shift(int grid, int KB, int jn) {
   int sh = 0;
-  while (sh < 2 && KB % (2 << sh) == 0 && (KB >> (sh + 1)) >= 8 && ((int64_t)(grid - 1) << (sh + 1)) * jn <= kMaxCutItems) ++sh;
+  while (sh < 2 && KB % (2 << sh) == 0 && (KB >> (sh + 1)) >= 8 && (jn == kTM || ((int64_t)(grid - 1) << (sh + 1)) * jn <= kMaxCutItems)) ++sh;
   return sh;
 }
 
@@ -1399,9 +1419,9 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   if (sk.use || grouped != nullptr || mode != kModeBlock) tp.use = false;
   size_t sk_bytes = sk.use ? (size_t)sk.grid * 2 * kPartialSlotBytes : (tp.use ? (size_t)tp.grid * 2 * kPartialSlotBytes : 0);
   a.cut_steps = g.KB;
-  if (short_tiles) {
+  if (grouped != nullptr) {
     // (the grid is the compute units, also where the bound of the tile count is lower: cuts may fill them)
-    const int sh = max_cut_shift(cus, g.KB, short_jn);
+    const int sh = max_cut_shift(cus, g.KB, short_tiles ? short_jn : kTM);
     const size_t bytes = (size_t)kMaxCutItems * kCutSlotBytes;
     if (sh > 0 && workspace != nullptr && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= FG_WORKSPACE_COUNTER_BYTES + bytes &&
         (size_t)cus * 8 * 4 <= FG_WORKSPACE_COUNTER_BYTES) {

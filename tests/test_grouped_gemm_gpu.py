@@ -89,6 +89,38 @@ def test_grouped_gemm_equals_plain_gemm_where_the_tiles_coincide():
     assert torch.equal(got, plain)
 
 
+@pytest.mark.parametrize("M,N,K,ends", [(16700, 1024, 4096, [5000, 5001, 16700]), (9000, 2048, 2048, [100, 4100, 4100, 9000])])
+def test_last_round_of_256_row_tiles_is_cut_along_k(M, N, K, ends):
+    """More 256-row tiles than compute units, a few of them left for a last round (268 = 256 + 12 and 296 = 256 + 40):
+    those are cut into work items along K whose sums meet in the workspace.  Every row against the plain GEMM of its
+    segment (another kernel instantiation; whole tiles give the same bits there, cut tiles sums in another order),
+    sampled rows against the oracle, and the same bits on a second call."""
+    g = torch.Generator().manual_seed(M)
+    xq = torch.randn(M, K, generator=g).to(FP8)
+    xs = torch.rand(M, K // 128, generator=g) * 0.02 + 0.005
+    E = len(ends)
+    wq = (0.5 * torch.randn(E, N, K, generator=g)).to(FP8)
+    ws = torch.rand(E, N // 128, K // 128, generator=g) * 0.02 + 0.005
+    ends_t = torch.tensor(ends, dtype=torch.int32)
+    got = _run(xq, wq, xs, ws, ends_t)
+    assert torch.equal(got, _run(xq, wq, xs, ws, ends_t))
+    begin, same = 0, 0
+    for e, end in enumerate(ends):
+        if end > begin:
+            plain = flag_gems.w8a8_block_fp8_matmul(xq[begin:end].to(DEV), wq[e].to(DEV), xs[begin:end].to(DEV), ws[e].to(DEV), [128, 128])
+            torch.testing.assert_close(got[begin:end].float(), plain.float(), rtol=1e-2, atol=1e-2)
+            same += int((got[begin:end] == plain).sum())
+        begin = end
+    assert same > 0.9 * M * N  # most tiles are whole and coincide bit for bit
+    rows = torch.randperm(M, generator=g)[:96].sort().values
+    seg = torch.bucketize(rows, ends_t.long(), right=True)
+    for e in range(E):
+        pick = rows[seg == e]
+        if pick.numel():
+            want = O.block_fp8_matmul_dequant_ref(xq[pick], wq[e], xs[pick], ws[e], [128, 128], torch.float32, torch.float64)
+            torch.testing.assert_close(got[pick.to(DEV)].cpu().float(), want, rtol=1e-2, atol=1e-2)
+
+
 def test_group_table_is_forced_into_range():
     """Ends that go backwards or past the rows are forced into [previous end, M]: no row is read or written
     outside the operands, and the result is that of the forced table."""
