@@ -747,6 +747,7 @@ template <bool SK, int MODE, bool ALIGNED, bool GROUPED = false, bool POW2 = fal
 __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   static_assert(JN == kTM || (GROUPED && JN >= 1 && JN < kTM), "short tiles: grouped problems only");
   constexpr int kTileRows = 64 * JN;
+  constexpr bool kDeferTail = JN == kTM;  // the FMAs of a step's last two MFMAs run after the barrier that ends the slot
   constexpr bool kCuts = GROUPED;  // tiles may be cut along K (cut_shift = 0: they are not)
   // Short tiles finish a cut tile in the fetch slot that follows it, like a whole tile.  With 128 accumulators that
   // code does not fit the registers of the hot loop (242 spilled), and the walk of a block is [whole tiles][its cut
@@ -1102,8 +1103,15 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
       }
       // The FMAs of the last two MFMAs wait until after the barrier below: they need the matrix pipe's last
       // results (44 cycles after the last MFMA's issue), and while this wavefront waited for them before the barrier,
-      // the partner, whose MFMAs were ready, waited too.
-      p_tail[0] = p[(kTN * JN - 2) % 3]; p_tail[1] = p[(kTN * JN - 1) % 3];
+      // the partner, whose MFMAs were ready, waited too.  (Short tiles keep them here: their steps are set by the
+      // weight stream, and with the FMAs behind the barrier a step of 64-row tiles took a quarter longer.)
+      if (kDeferTail) {
+        p_tail[0] = p[(kTN * JN - 2) % 3]; p_tail[1] = p[(kTN * JN - 1) % 3];
+      } else {
+        constexpr int L = kTN * JN;
+        scale_into<0>(acc[(L - 2) / JN][(L - 2) % JN], p[(L - 2) % 3], sc[(L - 2) % JN]);
+        scale_into<4>(acc[(L - 1) / JN][(L - 1) % JN], p[(L - 1) % 3], sc[(L - 1) % JN]);
+      }
     }
     __builtin_amdgcn_s_setprio(kFetchPrio);
     if (grp == 0) {  // A's share of stage T+1 has landed
@@ -1111,7 +1119,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
     }
     flushed_prev = flushed_now;
     __builtin_amdgcn_s_barrier();
-    if (MODE == kModeBlock && !POW2) {
+    if (MODE == kModeBlock && !POW2 && kDeferTail) {
       // (wait states between the last MFMA and the FMA that reads it: the four FMAs issued behind that MFMA, the
       // priority change, the barrier, two here, four FMAs, two more)
       constexpr int L = kTN * JN;
