@@ -831,9 +831,8 @@ int block_fp8_gemm(const char* who, int scales_pow2, const void* A, int64_t lda,
                                  void* C, int64_t ldc, int c_dtype,
                                  int64_t M, int64_t N, int64_t K, int64_t block_n, int64_t block_k,
                                  void* workspace, size_t workspace_bytes, void* stream) {
-  if (block_n != 128 || block_k != 128)
-    FG_FAIL(FG_ERR_UNSUPPORTED, "%s: only 128x128 scale blocks are implemented (got %lld x %lld)", who,
-            (long long)block_n, (long long)block_k);
+  if (block_n < 1 || block_k < 1)
+    FG_FAIL(FG_ERR_INVALID_ARG, "%s: scale block %lld x %lld", who, (long long)block_n, (long long)block_k);
   if (c_dtype != FG_BF16 && c_dtype != FG_F16 && c_dtype != FG_F32)
     FG_FAIL(FG_ERR_INVALID_ARG, "%s: c_dtype %d", who, c_dtype);
   int rc = check_common(A, B, C, lda, ldb, ldc, M, N, K, who);
@@ -848,6 +847,9 @@ int block_fp8_gemm(const char* who, int scales_pow2, const void* A, int64_t lda,
   a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)ceil_div(K, 128);
   a.c_dtype = c_dtype;
   a.scales_pow2 = scales_pow2;
+  // the matrix-instruction kernels apply one scale product per 128 x 128 block; every other block size takes the
+  // plain kernel (the host side restates multiples of 128 at 128 x 128 first, so they do not come here)
+  if (block_n != 128 || block_k != 128) return launch_anyblock(a, block_n, block_k, (hipStream_t)stream);
   return launch_gemm<kModeBlock>(a, workspace, workspace_bytes, (hipStream_t)stream);
 }
 }  // namespace

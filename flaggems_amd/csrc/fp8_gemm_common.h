@@ -221,6 +221,9 @@ struct SmallMPlan {
   int n_chunks;   // ceil(N / (16 * rg))
   size_t workspace_bytes;
 };
+// fp8_gemm_anyblock.hip: block-scaled product for scale blocks of any size (a plain fp32 tile kernel).
+int launch_anyblock(const GemmArgs& g, int64_t block_n, int64_t block_k, hipStream_t stream);
+
 SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries = 1);
 int launch_small_m(const GemmArgs& a, int mode, const SmallMPlan& plan, void* workspace, size_t workspace_bytes,
                    hipStream_t stream);

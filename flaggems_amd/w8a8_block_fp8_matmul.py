@@ -114,8 +114,9 @@ def w8a8_block_fp8_matmul(
         B = B.contiguous()
     a2d = A if A.dim() == 2 else A.view(M, K)
     as2d = As if As.dim() == 2 else As.reshape(M, As.shape[-1])
-    if (block_n, block_k) != (128, 128):
+    if (block_n, block_k) != (128, 128) and block_n % 128 == 0 and block_k % 128 == 0:
         as2d, Bs, block_n, block_k = _scales_at_128(as2d, Bs, N, K, block_n, block_k)
+    # (any other block size goes to the library as it is: a plain kernel serves it, see csrc/fp8_gemm_anyblock.hip)
     _launch_block_gemm(a2d, B, as2d, Bs, C if C.dim() == 2 else C.view(M, N), block_n, block_k, pow2)
     return C
 
@@ -124,12 +125,8 @@ def _scales_at_128(as2d: torch.Tensor, bs: torch.Tensor, n: int, k: int, block_n
     """Scale blocks that are whole multiples of 128 restated at the kernels' 128 x 128 granularity: every 128-wide
     piece of a larger block gets a copy of the block's scale, so each product is multiplied by the same fp32 value at
     the same place of the sum and the result is what a kernel with the larger blocks would give (the reference's
-    kernel takes any ``block_size``: src/flag_gems/ops/w8a8_block_fp8_matmul.py:51-122).  Blocks that are not multiples
-    of 128 would need another matrix instruction shape per scale block and are refused."""
-    if block_n <= 0 or block_k <= 0 or block_n % 128 != 0 or block_k % 128 != 0:
-        raise NotImplementedError(
-            f"w8a8_block_fp8_matmul: block_size [{block_n}, {block_k}]: scale blocks must be multiples of 128 in both "
-            "directions (the kernels apply one scale product per 128 x 128 block of the weight and 128-wide K-block)")
+    kernel takes any ``block_size``: src/flag_gems/ops/w8a8_block_fp8_matmul.py:51-122)."""
+    assert block_n > 0 and block_k > 0 and block_n % 128 == 0 and block_k % 128 == 0
     rn, rk = block_n // 128, block_k // 128
     kb, nb = _cdiv(k, 128), _cdiv(n, 128)
     if rk > 1:

@@ -399,8 +399,6 @@ def test_host_side_assertions():
         flag_gems.w8a8_block_fp8_matmul(A, B, As[:, :1], Bs, [128, 128])
     with pytest.raises(AssertionError):
         flag_gems.w8a8_block_fp8_matmul(A.t(), B, As, Bs, [128, 128])
-    with pytest.raises(NotImplementedError):  # scale blocks that are not multiples of 128 are refused, by name
-        flag_gems.w8a8_block_fp8_matmul(A, B, As.repeat(1, 2), Bs.repeat(2, 2), [64, 64])
     out = flag_gems.w8a8_block_fp8_matmul(A[:0], B, As[:0], Bs, [128, 128])
     assert out.shape == (0, 256)
 
@@ -426,3 +424,29 @@ def test_scale_blocks_that_are_multiples_of_128(M, N, K, block_size):
     Bs128 = Bs.repeat_interleave(block_n // 128, dim=0)[: -(-N // 128)].repeat_interleave(block_k // 128, dim=1)[:, : -(-K // 128)].contiguous()
     same = flag_gems.w8a8_block_fp8_matmul(A.to(DEV), B.to(DEV), As128.to(DEV), Bs128.to(DEV), [128, 128]).cpu().float()
     assert torch.equal(same, got)
+
+
+@pytest.mark.parametrize("block_size", [[64, 64], [64, 128], [128, 64], [32, 96], [100, 60], [128, 200], [1, 7], [4096, 32]])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (7, 640, 1000), (100, 1000, 1536), (300, 2112, 4096), (2100, 330, 777)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_scale_blocks_of_any_size(M, N, K, block_size, dtype):
+    """block_size that is no multiple of 128 (64-wide groups, blocks that divide nothing, a block wider than N, a
+    K-group of 7): the plain kernel, against the oracle evaluated with the same block_size; M, N and K that end inside
+    its 64 x 64 tiles and 32-element rounds."""
+    block_n, block_k = block_size
+    if dtype == torch.float32 and (M, N, K) not in ((7, 640, 1000), (2100, 330, 777)):
+        pytest.skip("fp32 output on two shapes")
+    g = torch.Generator().manual_seed(M + N + K + block_n + block_k)
+    A = torch.randn(M, K, generator=g).to(FP8)
+    B = torch.randn(N, K, generator=g).to(FP8)
+    As = 0.01 * torch.rand(M, -(-K // block_k), generator=g) + 0.005
+    Bs = 0.01 * torch.rand(-(-N // block_n), -(-K // block_k), generator=g) + 0.005
+    got = flag_gems.w8a8_block_fp8_matmul(A.to(DEV), B.to(DEV), As.to(DEV), Bs.to(DEV), block_size, output_dtype=dtype)
+    assert got.dtype == dtype and got.shape == (M, N)
+    want = O.block_fp8_matmul_dequant_ref(A, B, As, Bs, block_size, torch.float32, torch.float64)
+    tol = dict(rtol=1e-4, atol=2e-4) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(got.cpu().float(), want, **tol)
+    # strided scales (column-major activation scales) give the same bits
+    as_cm = As.to(DEV).t().contiguous().t()
+    again = flag_gems.w8a8_block_fp8_matmul(A.to(DEV), B.to(DEV), as_cm, Bs.to(DEV), block_size, output_dtype=dtype)
+    assert torch.equal(again.view(torch.int8), got.view(torch.int8))
