@@ -42,8 +42,10 @@ def test_c_abi_argument_validation_needs_no_gpu():
                                 128, 1e-4, -448.0, 448.0, 1.0 / 448.0, 0, 0, 0, None)
     assert rc == _lib.FG_ERR_INVALID_ARG
     assert b"divisible" in lib.fg_last_error_string()
-    rc = lib.fg_block_fp8_gemm(1, 128, 1, 128, 1, 1, 1, 1, 1, 1, 1, 128, _lib.FG_BF16, 4, 4, 128, 64, 64, None, 0, None)
-    assert rc == _lib.FG_ERR_UNSUPPORTED
+    # a scale block of no size is refused before any launch (every positive size is served)
+    rc = lib.fg_block_fp8_gemm(1, 128, 1, 128, 1, 1, 1, 1, 1, 1, 1, 128, _lib.FG_BF16, 4, 4, 128, 0, 64, None, 0, None)
+    assert rc == _lib.FG_ERR_INVALID_ARG
+    assert b"scale block" in lib.fg_last_error_string()
     rc = lib.fg_block_fp8_gemm(None, 128, None, 128, None, 1, 1, None, 1, 1, None, 128, _lib.FG_BF16, 4, 4, 128, 128, 128, None, 0, None)
     assert rc == _lib.FG_ERR_INVALID_ARG
     # empty problems are accepted without touching the device
