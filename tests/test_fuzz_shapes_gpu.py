@@ -103,3 +103,69 @@ def test_row_column_scaled_shapes_walk():
         tol = 1.6e-2 * want.abs() + 2.5e-3 * want.abs().max().item() + 1e-3
         n_bad = int((err > tol).sum())
         assert n_bad == 0, f"{tag}: {n_bad} elements outside the bar, max error {err.max().item():.4g}"
+
+
+def test_grouped_shapes_walk():
+    """Grouped (expert) products with random segment tables: 1 .. 16 experts, empty and one-row segments, few rows per
+    segment (64- and 128-row tiles) up to thousands (256-row tiles, more tiles than compute units, the last round cut
+    along K), rows gathered through an index, results scattered and weighted, bf16 and fp16 -- every element against
+    torch's fp32 GEMM of the dequantised operands, segment by segment."""
+    rng = random.Random(4711)
+    torch.manual_seed(2)
+    for it in range(60):
+        E = rng.choice([1, 2, 3, 8, 16])
+        K = 128 * rng.choice([1, 4, 8, 16, 24, 32, 56, 64])
+        N = rng.choice([128 * rng.randint(1, 32), 8 * rng.randint(16, 500), 256 * rng.randint(1, 16)])
+        avg = rng.choice([3, 20, 60, 100, 200, 700, 2500])
+        counts = [max(0, int(rng.gauss(avg, avg / 2))) if rng.random() > 0.15 else rng.choice([0, 1]) for _ in range(E)]
+        if sum(counts) == 0:
+            counts[0] = 5
+        while sum(counts) * (N + K) > 3.0e8:  # keep a case under a few hundred MB
+            counts = [c // 2 for c in counts]
+        M = sum(counts)
+        ends = torch.tensor([sum(counts[: i + 1]) for i in range(E)], dtype=torch.int32, device=DEV)
+        mode = rng.choice(["sorted", "gather", "scatter", "scatter+weights"])
+        odt = rng.choice([torch.bfloat16, torch.float16])
+        top_k = rng.choice([1, 2, 4]) if mode != "sorted" else 1
+        tag = f"case {it}: grouped E={E} rows={counts} N={N} K={K} {mode} top_k={top_k} {odt}"
+        print(tag, flush=True)
+        w = torch.randn(E, N, K, device=DEV).to(FP8)
+        ws = torch.rand(E, (N + 127) // 128, K // 128, device=DEV) + 0.25
+        if mode == "sorted":
+            x = torch.randn(M, K, device=DEV).to(FP8)
+            xs = torch.rand(M, K // 128, device=DEV) + 0.25
+            got = flag_gems.grouped_w8a8_block_fp8_matmul(x, w, xs, ws, ends, [128, 128], odt)
+            x_rows, xs_rows, out_rows, wts = x, xs, None, None
+        else:
+            T = (M + top_k - 1) // top_k  # tokens; slot s reads token s // top_k
+            x = torch.randn(T, K, device=DEV).to(FP8)
+            xs = torch.rand(T, K // 128, device=DEV) + 0.25
+            slots = torch.randperm(T * top_k, device=DEV)[:M].to(torch.int32)  # sorted row m is slot slots[m]
+            src = (slots.long() // top_k)
+            x_rows, xs_rows = x[src], xs[src]
+            kw = dict(row_index=slots, index_divisor=top_k)
+            out_rows, wts = None, None
+            if mode != "gather":
+                kw["scatter_rows"] = T * top_k
+                out_rows = slots.long()
+                if mode == "scatter+weights":
+                    wts = torch.rand(T * top_k, device=DEV) + 0.5
+                    kw["row_weights"] = wts
+            got = flag_gems.grouped_w8a8_block_fp8_matmul(x, w, xs, ws, ends, [128, 128], odt, **kw)
+        begin = 0
+        for e in range(E):
+            end = int(ends[e])
+            if end > begin:
+                want = _block_reference(x_rows[begin:end], xs_rows[begin:end], w[e], ws[e])
+                if out_rows is None:
+                    mine = got[begin:end].float()
+                else:
+                    mine = got[out_rows[begin:end]].float()
+                    if wts is not None:
+                        want = want * wts[out_rows[begin:end]][:, None]
+                assert torch.isfinite(mine).all(), tag
+                err = (mine - want).abs()
+                tol = 1e-2 * want.abs() + 2.5e-3 * want.abs().max().item() + 1e-3
+                n_bad = int((err > tol).sum())
+                assert n_bad == 0, f"{tag}: expert {e}: {n_bad} elements outside the bar, max error {err.max().item():.4g}"
+            begin = end
