@@ -83,6 +83,47 @@ def moe_sort_slots(
     return sorted_slots, offs
 
 
+def moe_align_block_size(
+    topk_ids: torch.Tensor,
+    block_size: int,
+    num_experts: int,
+    expert_map: Optional[torch.Tensor] = None,
+    pad_sorted_ids: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The reference's routing table (src/flag_gems/fused/moe_align_block_size.py:771-819): ``(sorted_ids, expert_ids,
+    num_tokens_post_pad)`` with every expert's slots padded to a multiple of ``block_size`` by the value
+    ``topk_ids.numel()``, the expert of every block (``expert_map`` applied, -1 where it has none) and the padded length.
+    Same shapes as the reference allocates.  Inside an expert's run the slots are in ascending order (the reference's
+    atomics leave that order open).  The expert layer of this package does not need this table (``moe_sort_slots``);
+    it is here for callers that keep the reference's format, and ``local_rows_from_moe_align`` takes it from there."""
+    logger.debug("GEMS MOE ALIGN BLOCK SIZE")
+    numel = topk_ids.numel()
+    cap = numel + num_experts * (block_size - 1)
+    if pad_sorted_ids:
+        cap = -(-cap // block_size) * block_size
+    n_blocks = -(-cap // block_size)
+    dev = topk_ids.device
+    flat = topk_ids.reshape(-1)
+    if not (flat.is_cuda and numel <= _SORT_MAX_SLOTS and 1 <= num_experts <= _SORT_MAX_EXPERTS
+            and flat.dtype in (torch.int32, torch.int64)):
+        raise NotImplementedError(
+            f"moe_align_block_size: up to {_SORT_MAX_SLOTS} slots and {_SORT_MAX_EXPERTS} experts, int32 or int64 ids on the "
+            f"GPU (got {numel} slots, {num_experts} experts, {flat.dtype} on {dev})")
+    flat = flat.contiguous()
+    sorted_ids = torch.empty(cap, dtype=torch.int32, device=dev)
+    expert_ids = torch.empty(n_blocks, dtype=torch.int32, device=dev)
+    num_tokens_post_pad = torch.empty(1, dtype=torch.int32, device=dev)
+    with _lib.device_guard(dev):
+        status = _lib.load().fg_moe_align_block_size(
+            flat.data_ptr(), flat.element_size(), numel, num_experts, block_size, sorted_ids.data_ptr(), cap,
+            expert_ids.data_ptr(), n_blocks, num_tokens_post_pad.data_ptr(), _lib.current_stream_ptr(dev))
+    _lib.check(status, "fg_moe_align_block_size")
+    if expert_map is not None:
+        mapped = expert_map.reshape(-1).to(torch.int32)[expert_ids.clamp(min=0).long()]
+        expert_ids = torch.where(expert_ids >= 0, mapped, expert_ids)
+    return sorted_ids, expert_ids, num_tokens_post_pad
+
+
 def moe_sum(input: torch.Tensor, output: torch.Tensor) -> None:
     """``output[t] = sum_k input[t, k]`` with an fp32 running sum in slot order and one rounding
     (src/flag_gems/fused/moe_sum.py:70-90)."""

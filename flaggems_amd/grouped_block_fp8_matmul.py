@@ -55,13 +55,18 @@ def local_rows_from_moe_align(sorted_token_ids: torch.Tensor, expert_ids: torch.
     ``zero_unwritten_rows=True`` to the GEMM for the same result.  No synchronisation."""
     assert sorted_token_ids.ndim == 1 and expert_ids.ndim == 1 and block_m >= 1 and num_experts >= 1
     nb = expert_ids.numel()
-    assert sorted_token_ids.numel() == nb * block_m, "one expert id per block of block_m sorted rows"
+    n_sorted = sorted_token_ids.numel()
+    # (the reference allocates numel + num_experts * (block_m - 1) sorted entries and one expert id per started block:
+    # the last block may be short unless pad_sorted_ids was set; its missing entries count as padding)
+    assert (nb - 1) * block_m < n_sorted <= nb * block_m, "one expert id per (started) block of block_m sorted rows"
+    if n_sorted < nb * block_m:
+        sorted_token_ids = torch.cat([sorted_token_ids, sorted_token_ids.new_full((nb * block_m - n_sorted,), n_sorted)])
     ids = expert_ids.to(torch.int64)
     local = (ids >= 0) & (ids < num_experts)
     key = torch.where(local, ids, torch.full_like(ids, num_experts))
     order = torch.argsort(key, stable=True)
     rows = sorted_token_ids.view(nb, block_m).to(torch.int32)
-    pad = torch.full_like(rows, sorted_token_ids.numel())
+    pad = torch.full_like(rows, n_sorted)
     rows = torch.where(local[:, None], rows, pad)[order].reshape(-1).contiguous()
     counts = torch.zeros(num_experts + 1, dtype=torch.int64, device=expert_ids.device)
     counts.scatter_add_(0, key, torch.ones_like(key))

@@ -192,6 +192,23 @@ int fg_moe_sort_slots(const void* topk_ids, int id_bytes, int64_t n_slots, int64
                       int map_bytes, int64_t map_len, int32_t* sorted_slots, int32_t* offs, void* stream);
 
 /*
+ * The padded routing table of the reference's moe_align_block_size (src/flag_gems/fused/moe_align_block_size.py:771-819,
+ * kernels :405-519), same layout and meaning:
+ *     sorted_ids [sorted_cap]   expert e's slots, in slot order, start at entry (sum over e' < e of ceil(count[e'] /
+ *                               block_size)) * block_size; every entry that holds no slot is n_slots (the padding value)
+ *     expert_ids [expert_ids_cap]  the expert of every block of block_size entries, -1 for blocks past the padded length
+ *     num_tokens_post_pad [1]   the padded length, sum over e of ceil(count[e] / block_size) * block_size
+ * topk_ids: [n_slots] integers of id_bytes (4 or 8) bytes in [0, num_experts); ids outside that range take no entry.
+ * sorted_cap >= n_slots + num_experts * (block_size - 1) and expert_ids_cap >= ceil(that / block_size), the sizes the
+ * reference allocates (FG_ERR_INVALID_ARG otherwise).  The reference leaves the order inside an expert's run to its
+ * atomics; here it is the slot order.  expert_map is applied by the caller to expert_ids afterwards, as in the reference
+ * (:817-818).  One block, no workspace; at most 960 experts and 65536 slots (FG_ERR_UNSUPPORTED beyond).
+ */
+int fg_moe_align_block_size(const void* topk_ids, int id_bytes, int64_t n_slots, int64_t num_experts, int64_t block_size,
+                            int32_t* sorted_ids, int64_t sorted_cap, int32_t* expert_ids, int64_t expert_ids_cap,
+                            int32_t* num_tokens_post_pad, void* stream);
+
+/*
  * RMSNorm (optionally preceded by the residual add) fused into the quantizer: every row of x [rows, cols] is
  * normalised, multiplied by weight [cols] (x's type), rounded to x's type as a separate norm kernel would have
  * stored it, and quantized exactly as fg_group_quant_fp8 quantizes that stored tensor (same codes and scales, bit

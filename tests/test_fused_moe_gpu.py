@@ -211,6 +211,73 @@ def test_moe_sort_slots_is_a_stable_sort_by_expert(slots, experts):
         assert torch.equal(got_rows.cpu(), want_rows), f"order, {slots} slots, {experts} experts, {id_dtype}, map {map_dtype}"
 
 
+@pytest.mark.parametrize("slots,experts,block_m", [(0, 4, 16), (1, 1, 16), (130, 8, 16), (1000, 8, 64), (4096, 64, 16), (8192, 8, 128),
+                                                   (20000, 256, 64), (65536, 960, 16), (333, 512, 1)])
+@pytest.mark.parametrize("pad_sorted_ids", [False, True])
+def test_moe_align_block_size_layout(slots, experts, block_m, pad_sorted_ids):
+    """The padded table in the reference's format (src/flag_gems/fused/moe_align_block_size.py:771-819) against its
+    definition: shapes as the reference allocates them, every expert's slots in ascending order from a block boundary,
+    the padding value everywhere else, the expert of every block, the padded length."""
+    g = torch.Generator().manual_seed(slots + experts)
+    ids = torch.randint(0, experts, (slots,), generator=g)
+    if slots > 100:
+        ids[ids == experts // 2] = 0  # an expert without slots (when there is more than one)
+    for dtype in (torch.int64, torch.int32):
+        sorted_ids, expert_ids, post = flag_gems.moe_align_block_size(ids.to(dtype).to(DEV), block_m, experts, pad_sorted_ids=pad_sorted_ids)
+        cap = slots + experts * (block_m - 1)
+        if pad_sorted_ids:
+            cap = -(-cap // block_m) * block_m
+        assert sorted_ids.shape == (cap,) and sorted_ids.dtype == torch.int32
+        assert expert_ids.shape == (-(-cap // block_m),) and post.shape == (1,)
+        counts = torch.bincount(ids, minlength=experts)
+        padded = (counts + block_m - 1) // block_m * block_m
+        want_sorted = torch.full((cap,), slots, dtype=torch.int32)
+        want_blocks = torch.full((-(-cap // block_m),), -1, dtype=torch.int32)
+        start = 0
+        order = torch.sort(ids, stable=True).indices.to(torch.int32)
+        taken = 0
+        for e in range(experts):
+            c, p = int(counts[e]), int(padded[e])
+            want_sorted[start:start + c] = order[taken:taken + c]
+            want_blocks[start // block_m:(start + p) // block_m] = e
+            start += p
+            taken += c
+        assert int(post) == start
+        assert torch.equal(sorted_ids.cpu(), want_sorted)
+        assert torch.equal(expert_ids.cpu(), want_blocks)
+
+
+def test_moe_align_table_feeds_the_grouped_gemm_under_expert_map():
+    """The reference's flow end to end: moe_align_block_size with an expert_map (two local experts out of five, in
+    swapped order), local_rows_from_moe_align, the grouped GEMM with scattered rows: every slot of a local expert gets
+    its own expert's product, every other slot zeros."""
+    tokens, top_k, N, K, block_m = 200, 2, 384, 256, 16
+    g = torch.Generator().manual_seed(3)
+    ids = torch.randint(0, 5, (tokens, top_k), generator=g)
+    emap = torch.tensor([-1, 1, -1, 0, -1], dtype=torch.int32)  # global 3 -> local 0, global 1 -> local 1
+    sorted_ids, expert_ids, _ = flag_gems.moe_align_block_size(ids.to(DEV), block_m, 5, expert_map=emap.to(DEV))
+    rows, offs = flag_gems.local_rows_from_moe_align(sorted_ids, expert_ids, block_m, 2)
+    x = torch.randn(tokens, K, generator=g).bfloat16()
+    xq, xs = O.act_quant_ref(x, 128)
+    wq, ws = [], []
+    for _ in range(2):
+        q, s = O.per_block_cast_to_fp8_ref((0.02 * torch.randn(N, K, generator=g)).bfloat16())
+        wq.append(q); ws.append(s)
+    wq, ws = torch.stack(wq), torch.stack(ws)
+    got = flag_gems.grouped_w8a8_block_fp8_matmul(
+        xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), offs, [128, 128], row_index=rows, index_divisor=top_k,
+        scatter_rows=tokens * top_k, zero_unwritten_rows=True).cpu().float()
+    flat = ids.reshape(-1)
+    want = torch.zeros(tokens * top_k, N)
+    for local, glob in ((0, 3), (1, 1)):
+        slots_e = torch.nonzero(flat == glob).reshape(-1)
+        tok = slots_e // top_k
+        want[slots_e] = O.block_fp8_matmul_tiled_ref(xq[tok], wq[local], xs[tok], ws[local], [128, 128], torch.float32)
+    torch.testing.assert_close(got, want, rtol=1e-2, atol=1e-2)
+    foreign = ~((flat == 3) | (flat == 1))
+    assert float(got[foreign].abs().max()) == 0.0
+
+
 def test_moe_sum_rounds_once():
     for dtype in (torch.bfloat16, torch.float16, torch.float32):
         x = (torch.randn(37, 6, 264, device=DEV) * 3).to(dtype)
