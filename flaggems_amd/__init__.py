@@ -19,7 +19,13 @@ from .act_quant import (  # noqa: F401
 )
 from .cutlass_scaled_mm import SM_VERSION_NUM, cutlass_scaled_mm, get_sm_version_num  # noqa: F401
 from .fp8_einsum import fp8_einsum, w8a8_block_fp8_bmm  # noqa: F401
-from .fused_moe import fused_experts_impl, moe_align_block_size, moe_sort_slots, moe_sum  # noqa: F401
+from .fused_moe import (  # noqa: F401
+    fused_experts_impl,
+    moe_align_block_size,
+    moe_align_block_size_triton,
+    moe_sort_slots,
+    moe_sum,
+)
 from .grouped_block_fp8_matmul import (  # noqa: F401
     group_ends_from_expert_ids,
     grouped_w8a8_block_fp8_matmul,
@@ -61,6 +67,7 @@ __all__ = [
     "local_rows_from_moe_align",
     "moe_sort_slots",
     "moe_align_block_size",
+    "moe_align_block_size_triton",
     "moe_sum",
     "only_enable",
     "patch_empty_vllm",

@@ -83,6 +83,37 @@ def moe_sort_slots(
     return sorted_slots, offs
 
 
+def moe_align_block_size_triton(
+    topk_ids: torch.Tensor,
+    num_experts: int,
+    block_size: int,
+    sorted_token_ids: torch.Tensor,
+    expert_ids: torch.Tensor,
+    num_tokens_post_pad: torch.Tensor,
+) -> None:
+    """The reference's in-place form under its own name (src/flag_gems/fused/moe_align_block_size.py:520-770; what
+    vLLM's ``_moe_C::moe_align_block_size`` is patched with, src/flag_gems/patches/patch_vllm_all.py:306-321): fills
+    the caller's three int32 buffers.  One kernel here, whatever the name says."""
+    logger.debug("GEMS MOE ALIGN BLOCK SIZE")
+    numel = topk_ids.numel()
+    flat = topk_ids.reshape(-1)
+    if not (flat.is_cuda and numel <= _SORT_MAX_SLOTS and 1 <= num_experts <= _SORT_MAX_EXPERTS
+            and flat.dtype in (torch.int32, torch.int64)):
+        raise NotImplementedError(
+            f"moe_align_block_size: up to {_SORT_MAX_SLOTS} slots and {_SORT_MAX_EXPERTS} experts, int32 or int64 ids on the "
+            f"GPU (got {numel} slots, {num_experts} experts, {flat.dtype} on {flat.device})")
+    for t in (sorted_token_ids, expert_ids, num_tokens_post_pad):
+        assert t.dtype == torch.int32 and t.is_contiguous() and t.device == flat.device
+    assert num_tokens_post_pad.numel() >= 1
+    flat = flat.contiguous()
+    with _lib.device_guard(flat.device):
+        status = _lib.load().fg_moe_align_block_size(
+            flat.data_ptr(), flat.element_size(), numel, num_experts, block_size, sorted_token_ids.data_ptr(),
+            sorted_token_ids.numel(), expert_ids.data_ptr(), expert_ids.numel(), num_tokens_post_pad.data_ptr(),
+            _lib.current_stream_ptr(flat.device))
+    _lib.check(status, "fg_moe_align_block_size")
+
+
 def moe_align_block_size(
     topk_ids: torch.Tensor,
     block_size: int,
@@ -96,28 +127,16 @@ def moe_align_block_size(
     Same shapes as the reference allocates.  Inside an expert's run the slots are in ascending order (the reference's
     atomics leave that order open).  The expert layer of this package does not need this table (``moe_sort_slots``);
     it is here for callers that keep the reference's format, and ``local_rows_from_moe_align`` takes it from there."""
-    logger.debug("GEMS MOE ALIGN BLOCK SIZE")
     numel = topk_ids.numel()
     cap = numel + num_experts * (block_size - 1)
     if pad_sorted_ids:
         cap = -(-cap // block_size) * block_size
     n_blocks = -(-cap // block_size)
     dev = topk_ids.device
-    flat = topk_ids.reshape(-1)
-    if not (flat.is_cuda and numel <= _SORT_MAX_SLOTS and 1 <= num_experts <= _SORT_MAX_EXPERTS
-            and flat.dtype in (torch.int32, torch.int64)):
-        raise NotImplementedError(
-            f"moe_align_block_size: up to {_SORT_MAX_SLOTS} slots and {_SORT_MAX_EXPERTS} experts, int32 or int64 ids on the "
-            f"GPU (got {numel} slots, {num_experts} experts, {flat.dtype} on {dev})")
-    flat = flat.contiguous()
     sorted_ids = torch.empty(cap, dtype=torch.int32, device=dev)
     expert_ids = torch.empty(n_blocks, dtype=torch.int32, device=dev)
     num_tokens_post_pad = torch.empty(1, dtype=torch.int32, device=dev)
-    with _lib.device_guard(dev):
-        status = _lib.load().fg_moe_align_block_size(
-            flat.data_ptr(), flat.element_size(), numel, num_experts, block_size, sorted_ids.data_ptr(), cap,
-            expert_ids.data_ptr(), n_blocks, num_tokens_post_pad.data_ptr(), _lib.current_stream_ptr(dev))
-    _lib.check(status, "fg_moe_align_block_size")
+    moe_align_block_size_triton(topk_ids, num_experts, block_size, sorted_ids, expert_ids, num_tokens_post_pad)
     if expert_map is not None:
         mapped = expert_map.reshape(-1).to(torch.int32)[expert_ids.clamp(min=0).long()]
         expert_ids = torch.where(expert_ids >= 0, mapped, expert_ids)

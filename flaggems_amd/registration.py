@@ -20,6 +20,7 @@ import torch
 
 from .act_quant import per_token_group_fp8_quant_into
 from .cutlass_scaled_mm import cutlass_scaled_mm
+from .fused_moe import moe_align_block_size_triton, moe_sum
 from .scaled_mm import scaled_mm, scaled_mm_out
 
 logger = logging.getLogger("flag_gems")
@@ -203,6 +204,29 @@ _VLLM_IMPLS = {
     "per_token_group_fp8_quant": custom_per_token_group_fp8_quant,
 }
 
+# the two operators of vLLM's ``_moe_C`` namespace that the expert layer of this path uses
+# (src/flag_gems/patches/patch_util.py:74-85, patch_vllm_all.py:306-321, 356-359)
+_VLLM_MOE_OPS_SIGNATURES = {
+    "moe_align_block_size": "(Tensor topk_ids, int num_experts, "
+    "int block_size, Tensor(a!) sorted_token_ids, Tensor(b!) experts_ids, "
+    "Tensor(c!) num_tokens_post_pad) -> ()",
+    "moe_sum": "(Tensor input, Tensor(a!) output) -> ()",
+}
+
+
+def custom_moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids, num_tokens_post_pad):
+    moe_align_block_size_triton(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids, num_tokens_post_pad)
+
+
+def custom_moe_sum(input, output):
+    moe_sum(input, output)
+
+
+_VLLM_MOE_IMPLS = {
+    "moe_align_block_size": custom_moe_align_block_size,
+    "moe_sum": custom_moe_sum,
+}
+
 _vllm_libs: List[torch.library.Library] = []
 _vllm_patched = False
 
@@ -216,20 +240,22 @@ def _op_defined(namespace: str, name: str) -> bool:
 
 
 def patch_empty_vllm(verbose: bool = False) -> None:
-    """Define (when vLLM has not) and implement the two ``_C`` operators of this path.  Idempotent."""
+    """Define (when vLLM has not) and implement the ``_C`` and ``_moe_C`` operators of this path.  Idempotent."""
     global _vllm_patched
     if _vllm_patched:
         return
-    for name, schema in _VLLM_OPS_SIGNATURES.items():
-        if not _op_defined("_C", name):
-            def_lib = torch.library.Library("_C", "FRAGMENT")
-            def_lib.define(name + schema)
-            _vllm_libs.append(def_lib)
-        impl_lib = torch.library.Library("_C", "IMPL")
-        impl_lib.impl(name, _VLLM_IMPLS[name], DISPATCH_KEY)
-        _vllm_libs.append(impl_lib)
-        if verbose:
-            logger.info("patched _C::%s", name)
+    for namespace, signatures, impls in (("_C", _VLLM_OPS_SIGNATURES, _VLLM_IMPLS),
+                                        ("_moe_C", _VLLM_MOE_OPS_SIGNATURES, _VLLM_MOE_IMPLS)):
+        for name, schema in signatures.items():
+            if not _op_defined(namespace, name):
+                def_lib = torch.library.Library(namespace, "FRAGMENT")
+                def_lib.define(name + schema)
+                _vllm_libs.append(def_lib)
+            impl_lib = torch.library.Library(namespace, "IMPL")
+            impl_lib.impl(name, impls[name], DISPATCH_KEY)
+            _vllm_libs.append(impl_lib)
+            if verbose:
+                logger.info("patched %s::%s", namespace, name)
     _vllm_patched = True
 
 

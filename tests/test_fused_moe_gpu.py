@@ -278,6 +278,25 @@ def test_moe_align_table_feeds_the_grouped_gemm_under_expert_map():
     assert float(got[foreign].abs().max()) == 0.0
 
 
+def test_vllm_moe_ops_write_the_callers_buffers():
+    """``_moe_C::moe_align_block_size`` and ``_moe_C::moe_sum`` as vLLM calls them, with buffers it allocated
+    (src/flag_gems/patches/patch_vllm_all.py:306-321, 356-359; schemas of patch_util.py:74-85)."""
+    flag_gems.patch_empty_vllm()
+    ids = torch.randint(0, 8, (300, 2), generator=torch.Generator().manual_seed(5)).to(DEV)
+    block_m = 16
+    cap = ids.numel() + 8 * (block_m - 1)
+    sorted_ids = torch.empty(cap, dtype=torch.int32, device=DEV)
+    expert_ids = torch.empty(-(-cap // block_m), dtype=torch.int32, device=DEV)
+    post = torch.empty(1, dtype=torch.int32, device=DEV)
+    torch.ops._moe_C.moe_align_block_size(ids, 8, block_m, sorted_ids, expert_ids, post)
+    a, b, c = flag_gems.moe_align_block_size(ids, block_m, 8)
+    assert torch.equal(sorted_ids, a) and torch.equal(expert_ids, b) and torch.equal(post, c)
+    x = torch.randn(40, 2, 256, device=DEV).bfloat16()
+    out = torch.empty(40, 256, device=DEV, dtype=torch.bfloat16)
+    torch.ops._moe_C.moe_sum(x, out)
+    assert torch.equal(out, (x[:, 0].float() + x[:, 1].float()).bfloat16())
+
+
 def test_moe_sum_rounds_once():
     for dtype in (torch.bfloat16, torch.float16, torch.float32):
         x = (torch.randn(37, 6, 264, device=DEV) * 3).to(dtype)
