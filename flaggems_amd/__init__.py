@@ -21,6 +21,8 @@ from .cutlass_scaled_mm import SM_VERSION_NUM, cutlass_scaled_mm, get_sm_version
 from .fp8_einsum import fp8_einsum, w8a8_block_fp8_bmm  # noqa: F401
 from .fused_moe import (  # noqa: F401
     fused_experts_impl,
+    inplace_fused_experts,
+    outplace_fused_experts,
     moe_align_block_size,
     moe_align_block_size_triton,
     moe_sort_slots,
@@ -66,6 +68,8 @@ __all__ = [
     "group_ends_from_expert_ids",
     "local_rows_from_moe_align",
     "moe_sort_slots",
+    "inplace_fused_experts",
+    "outplace_fused_experts",
     "moe_align_block_size",
     "moe_align_block_size_triton",
     "moe_sum",

@@ -252,3 +252,18 @@ def fused_experts_impl(
     )
     moe_sum(cache3.view(T, top_k, H), out)
     return out
+
+
+def inplace_fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, topk_weights: torch.Tensor,
+                          topk_ids: torch.Tensor, activation: str = "silu", **options) -> None:
+    """``fused_experts_impl(..., inplace=True)``: the result replaces ``hidden_states``; returns nothing
+    (src/flag_gems/fused/fused_moe.py:2188-2238; the remaining keywords are ``fused_experts_impl``'s)."""
+    assert "inplace" not in options
+    fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, inplace=True, activation=activation, **options)
+
+
+def outplace_fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, topk_weights: torch.Tensor,
+                           topk_ids: torch.Tensor, activation: str = "silu", **options) -> torch.Tensor:
+    """``fused_experts_impl(..., inplace=False)``: a new tensor (src/flag_gems/fused/fused_moe.py:2241-2291)."""
+    assert "inplace" not in options
+    return fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, inplace=False, activation=activation, **options)

@@ -91,6 +91,13 @@ def test_reference_configurations(config, randn_scales):
     _assert_close(got, want, f"config {config}")
     again = _run(*args)
     assert torch.equal(again.view(torch.int16), got.view(torch.int16)), "two runs of one layer differ"
+    # the two wrappers of the reference (src/flag_gems/fused/fused_moe.py:2188-2291)
+    x, w1, w2, s1, s2, tw, ti = args
+    kw = dict(use_fp8_w8a8=True, w1_scale=s1, w2_scale=s2, block_shape=[128, 128])
+    assert torch.equal(flag_gems.outplace_fused_experts(x, w1, w2, tw, ti, **kw), got)
+    y = x.clone()
+    assert flag_gems.inplace_fused_experts(y, w1, w2, tw, ti, **kw) is None
+    assert torch.equal(y, got)
 
 
 @pytest.mark.parametrize("tokens", [1, 16, 64, 1024, 4096])
