@@ -90,8 +90,8 @@ __device__ __forceinline__ void narrow_chunk(const float (&v)[8], uint32_t (&w)[
 // rounding, e4m3), which lets the compiler drop every rule switch from the loop.
 // LPG: lanes per quantization group when known at compile time (16 = groups of 128 elements), 0 = from the arguments:
 // the group maximum is then four DPP instructions instead of a chain of six tests.
-// A wavefront whose 64 chunks of a round all lie past the row's end (rows of 7168 elements: the last round of
-// wavefronts 2 and 3) skips the round; its zeros would not have changed any sum.
+// A wavefront whose 64 chunks of a pass all lie past the row's end (rows of 7168 elements: the last pass of
+// wavefronts 2 and 3) skips the pass; its zeros would not have changed any sum.
 template <int XDT, int CHUNKS, int QUANT, int LPG = 0>
 __global__ __launch_bounds__(kNormThreads) void rms_norm_quant_kernel(NormQuantArgs a) {
   if (QUANT == 2) {
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_quant_kernel(NormQuantA
   __shared__ float wave_sums[2][kNormWaves];
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  const uint32_t wave_first = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid & ~63u));  // chunk of lane 0 in round 0
+  const uint32_t wave_first = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid & ~63u));  // chunk of lane 0 in the first pass over the row
   const bool add_residual = a.residual != nullptr;
   constexpr bool quantize = QUANT != 0;
   const Raw* wp = reinterpret_cast<const Raw*>(a.weight);
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_quant_kernel(NormQuantA
     for (int i = 0; i < CHUNKS; ++i) {
       const uint32_t c = tid + (uint32_t)i * kNormThreads;
       const bool live = c < a.chunks_per_row;
-      if (wave_first + (uint32_t)i * kNormThreads >= a.chunks_per_row) {  // uniform: nothing of this round in this wavefront
+      if (wave_first + (uint32_t)i * kNormThreads >= a.chunks_per_row) {  // uniform: this wavefront holds nothing of this pass
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[i][e] = 0.0f;
         continue;

@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_slots_kernel(const void
       if (block_m == 0 || pos < sorted_cap) sorted[pos] = s;
     }
     __syncthreads();
-    for (int i = tid; i < K; i += kSortThreads) {  // the key's base moves past this round's slots; sizes back to zero
+    for (int i = tid; i < K; i += kSortThreads) {  // the key's base moves past the slots just placed; sizes back to zero
       int t = 0;
 #pragma unroll
       for (int w = 0; w < kSortWaves; ++w) {
