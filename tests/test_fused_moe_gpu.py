@@ -304,6 +304,30 @@ def test_vllm_moe_ops_write_the_callers_buffers():
     assert torch.equal(out, (x[:, 0].float() + x[:, 1].float()).bfloat16())
 
 
+def test_expert_layer_under_graph_capture():
+    """The layer recorded into a HIP graph on a side stream after a warm-up call (the serving flow) and replayed on
+    new inputs written into the captured buffers: every replay equals the eager call on the same inputs.  Nothing
+    in the chain synchronises or allocates outside torch's graph pool."""
+    tokens, experts, hidden, inter, topk = 48, 8, 512, 1024, 2
+    x, w1, w2, s1, s2, tw, ti = _layer(tokens, experts, hidden, inter, topk, seed=77)
+    static_x, static_tw, static_ti = x.clone(), tw.clone(), ti.clone()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        _run(static_x, w1, w2, s1, s2, static_tw, static_ti)  # warm-up: workspaces, first-launch work
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            static_out = _run(static_x, w1, w2, s1, s2, static_tw, static_ti)
+    torch.cuda.synchronize()
+    for seed in (78, 79, 80):
+        nx, _, _, _, _, ntw, nti = _layer(tokens, experts, hidden, inter, topk, seed=seed)
+        static_x.copy_(nx); static_tw.copy_(ntw); static_ti.copy_(nti)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = _run(nx, w1, w2, s1, s2, ntw, nti)  # eager work between the replays
+        assert torch.equal(static_out.view(torch.int16), want.view(torch.int16)), f"replay with seed {seed}"
+
+
 def test_moe_sum_rounds_once():
     for dtype in (torch.bfloat16, torch.float16, torch.float32):
         x = (torch.randn(37, 6, 264, device=DEV) * 3).to(dtype)
