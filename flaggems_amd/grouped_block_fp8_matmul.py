@@ -87,6 +87,7 @@ def grouped_w8a8_block_fp8_matmul(
     scatter_rows: Optional[int] = None,
     row_weights: Optional[torch.Tensor] = None,
     zero_unwritten_rows: bool = False,
+    out: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """C[offs[e-1]:offs[e]] = block_fp8_matmul(A[offs[e-1]:offs[e]], B[e]) for every group e.
 
@@ -108,7 +109,7 @@ def grouped_w8a8_block_fp8_matmul(
 
     ``zero_unwritten_rows``: the result starts as zeros instead of ``torch.empty``, so rows that no group covers (the
     slots of experts that live on another device) read as zeros, which is what the reference's kernel stores for
-    them (src/flag_gems/fused/fused_moe.py:1114).
+    them (src/flag_gems/fused/fused_moe.py:1114).  ``out``: write into this ``[rows, N]`` tensor instead of a new one.
     """
     logger.debug("GEMS GROUPED_W8A8_BLOCK_FP8_MATMUL")
     assert len(block_size) == 2
@@ -145,7 +146,12 @@ def grouped_w8a8_block_fp8_matmul(
     if B.stride(2) != 1:
         B = B.contiguous()
 
-    C = (A.new_zeros if zero_unwritten_rows else A.new_empty)((c_rows if c_rows else M, N), dtype=output_dtype)
+    if out is not None:  # the caller's buffer: [rows, N] with unit stride along N
+        assert out.shape == (c_rows if c_rows else M, N) and out.dtype == output_dtype and out.device == A.device
+        assert out.stride(1) == 1
+        C = out.zero_() if zero_unwritten_rows else out
+    else:
+        C = (A.new_zeros if zero_unwritten_rows else A.new_empty)((c_rows if c_rows else M, N), dtype=output_dtype)
     if M == 0 or N == 0:
         return C
     _lib.require_gpu(A, "grouped block fp8 gemm")
