@@ -200,6 +200,24 @@ def test_group_ends_from_the_per_block_expert_table():
     assert flag_gems.group_ends_from_expert_ids(torch.tensor([-1], dtype=torch.int32), 16, 2).tolist() == [0, 0]
 
 
+def test_local_rows_from_the_aligners_tables_on_the_host():
+    """The reorder of an aligner table (pure torch, so it runs here): foreign (-1) blocks in front of and between
+    the local experts' blocks, local ids out of order, and the reference's unpadded table length
+    (numel + num_experts * (block_m - 1) entries, the last block short)."""
+    block_m = 4
+    expert_ids = torch.tensor([-1, 1, 0, -1, 1], dtype=torch.int32)
+    sorted_ids = torch.arange(100, 100 + 18, dtype=torch.int32)  # 18 entries: the fifth block has 2 of its 4
+    rows, offs = flag_gems.local_rows_from_moe_align(sorted_ids, expert_ids, block_m, 2)
+    pad = 18
+    assert offs.tolist() == [4, 12]                      # one block of expert 0, two of expert 1
+    assert rows.tolist() == ([108, 109, 110, 111]        # expert 0: block 2
+                             + [104, 105, 106, 107]      # expert 1: blocks 1 and 4, in table order
+                             + [116, 117, pad, pad]
+                             + [pad] * 8)                # the two foreign blocks, turned into padding
+    with pytest.raises(AssertionError):
+        flag_gems.local_rows_from_moe_align(sorted_ids[:16], expert_ids, block_m, 2)  # a whole block without entries
+
+
 def test_record_once_lists_every_call_site_once(tmp_path):
     """enable(record=True, once=True): the record file names each operator call site once, however often it runs
     (the reference's LogOncePerLocationFilter, src/flag_gems/logging_utils.py:34-45); once=False lists every call."""
