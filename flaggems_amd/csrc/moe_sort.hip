@@ -167,7 +167,7 @@ extern "C" int fg_moe_align_block_size(const void* topk_ids, int id_bytes, int64
   using namespace fg;
   const char* me = "fg_moe_align_block_size";
   if (block_size < 1 || block_size > 65536) FG_FAIL(FG_ERR_INVALID_ARG, "%s: block size %lld", me, (long long)block_size);
-  if (!sorted_ids || !expert_ids || !num_tokens_post_pad) FG_FAIL(FG_ERR_INVALID_ARG, "%s: null pointer", me);
+  if ((!sorted_ids && sorted_cap > 0) || (!expert_ids && expert_ids_cap > 0) || !num_tokens_post_pad) FG_FAIL(FG_ERR_INVALID_ARG, "%s: null pointer", me);
   if (num_experts >= 1 && num_experts <= kSortMaxExperts && n_slots >= 0) {
     // the largest padded length: every expert's run rounded up
     const int64_t need = n_slots + num_experts * (block_size - 1);

@@ -218,7 +218,7 @@ def test_moe_sort_slots_is_a_stable_sort_by_expert(slots, experts):
         assert torch.equal(got_rows.cpu(), want_rows), f"order, {slots} slots, {experts} experts, {id_dtype}, map {map_dtype}"
 
 
-@pytest.mark.parametrize("slots,experts,block_m", [(0, 4, 16), (1, 1, 16), (130, 8, 16), (1000, 8, 64), (4096, 64, 16), (8192, 8, 128),
+@pytest.mark.parametrize("slots,experts,block_m", [(0, 4, 16), (0, 3, 1), (1, 1, 16), (130, 8, 16), (1000, 8, 64), (4096, 64, 16), (8192, 8, 128),
                                                    (20000, 256, 64), (65536, 960, 16), (333, 512, 1)])
 @pytest.mark.parametrize("pad_sorted_ids", [False, True])
 def test_moe_align_block_size_layout(slots, experts, block_m, pad_sorted_ids):
