@@ -6,6 +6,7 @@
 #include <stdio.h>
 
 #include "../../include/flaggems_amd.h"
+#include "../../include/flaggems_amd_probes.h"
 
 namespace fg {
 

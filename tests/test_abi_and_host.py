@@ -16,7 +16,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "flaggems_amd.h")).read()
+    text = "".join(open(os.path.join(ROOT, "include", name)).read() for name in sorted(os.listdir(os.path.join(ROOT, "include")))
+                   if name.endswith(".h"))
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(fg_[a-z0-9_]+)\s*\(", text)))
 
