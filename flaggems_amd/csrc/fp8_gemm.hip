@@ -1091,7 +1091,7 @@ extern "C" int fg_grouped_block_fp8_gemm(const void* A, int64_t lda,
   a.xs_rs = as_row_stride; a.xs_cs = as_col_stride; a.ws_rs = bs_row_stride; a.ws_cs = bs_col_stride;
   a.M = (int)M; a.N = (int)N; a.K = (int)K; a.KB = (int)(K / 128);
   a.c_dtype = c_dtype;
-  GroupedGemm grouped = {group_ends, n_groups, b_group_stride, bs_group_stride, row_index, index_div, row_index ? a_rows : M,
+  GroupedGemm grouped = {group_ends, n_groups, b_group_stride, bs_group_stride, row_index, index_div, (row_index && index_div != 0) ? a_rows : M,
                          c_rows, row_weight};
   return launch_grouped(a, grouped, workspace, workspace_bytes, (hipStream_t)stream);
 }

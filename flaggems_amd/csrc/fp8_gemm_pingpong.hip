@@ -102,6 +102,9 @@ struct PpArgs {
   // sorted_token_ids // top_k, src/flag_gems/fused/fused_moe.py:1111); entries are forced into [0, x_rows).
   const int* row_index;
   int index_div, x_rows;
+  // the table the loaders gather through: row_index, or null when the rows are already in sorted order and row_index
+  // only addresses the scattered result (index_div == 0)
+  const int* gather_index;
   // Scattered results (c_rows > 0, with row_index): the result of sorted row m goes to row row_index[m] of C, which
   // has c_rows rows; entries outside [0, c_rows) are padding and store nothing.  With row_weight the fp32 sums are
   // multiplied by row_weight[row_index[m]] before the cast.  This is where and how the reference's MoE kernel
@@ -836,9 +839,9 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   lw.start(a, first_idx, first_kb, n_tiles, tiles_m);
   LoadShare share = {};
   auto set_load_tile = [&]() __attribute__((always_inline)) {
-    if (GROUPED && a.row_index != nullptr && wave < 4) {
+    if (GROUPED && a.gather_index != nullptr && wave < 4) {
       const int valid = lw.m_end - lw.m0;
-      share.set_gathered(g, a.row_index, a.index_div, a.x_rows, lw.m0, valid < kTileRows ? valid : kTileRows, lane, wave);
+      share.set_gathered(g, a.gather_index, a.index_div, a.x_rows, lw.m0, valid < kTileRows ? valid : kTileRows, lane, wave);
     } else {
       share.template set_tile<kTileRows>(g, lw.m0, lw.n0, wave, lane, lw.m_end, GROUPED ? (int64_t)lw.group * a.w_group_stride : 0);
     }
@@ -881,7 +884,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
   uint32_t xs_off[kTM] = {0u, 0u, 0u, 0u};
   const float* xs_ptr = g.xs;
   // offsets are relative to the tile's first row; rows past the edge read the last row's scale
-  const bool gathered = GROUPED && a.row_index != nullptr;  // uniform
+  const bool gathered = GROUPED && a.gather_index != nullptr;  // uniform
   auto set_scale_offsets = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < kTM; ++j) {
@@ -889,7 +892,7 @@ __global__ __launch_bounds__(kThreads) void fp8_gemm_pingpong_kernel(PpArgs a) {
       const int last = sw.m_end - 1 - sw.m0;
       r = r < last ? r : last;
       if (gathered) {  // the scales of the source row, relative to the first row of the scale matrix
-        int src = a.row_index[sw.m0 + r] / a.index_div;
+        int src = a.gather_index[sw.m0 + r] / a.index_div;
         r = src < 0 ? 0 : (src < a.x_rows ? src : a.x_rows - 1);
       }
       xs_off[j] = (uint32_t)r * (uint32_t)g.xs_rs * 4u;
@@ -1407,6 +1410,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
     a.groups = grouped->ends; a.n_groups = (int)grouped->n_groups;
     a.w_group_stride = grouped->w_group_stride; a.ws_group_stride = grouped->ws_group_stride;
     a.row_index = grouped->row_index; a.index_div = (int)grouped->index_div; a.x_rows = (int)grouped->x_rows;
+    a.gather_index = grouped->index_div > 0 ? grouped->row_index : nullptr;
     a.c_rows = (int)grouped->c_rows; a.row_weight = grouped->row_weight;
   }
   a.g.tiles_n = (int)ceil_div(g.N, kBN);
@@ -1442,7 +1446,7 @@ int launch_block(const GemmArgs& g, int mode, void* workspace, size_t workspace_
   }
   const size_t need = FG_WORKSPACE_COUNTER_BYTES + sk_bytes;
   // rows of the activation-scale matrix: the rows of X, which a gathered problem reads through its index
-  const int64_t scale_rows = (grouped != nullptr && grouped->row_index != nullptr) ? grouped->x_rows : (int64_t)g.M;
+  const int64_t scale_rows = (grouped != nullptr && grouped->row_index != nullptr && grouped->index_div > 0) ? grouped->x_rows : (int64_t)g.M;
   // workspace: [counters][partial tiles, if the shape is one that shares tiles][transposed activation scales]
   // (a grouped problem's tile count is an upper bound that a few hundred rows spread over many segments inflate:
   // there the gathers are few and the transposition, ~5 us whatever the size, does not pay)
@@ -1554,7 +1558,9 @@ int launch_grouped(const GemmArgs& g, const GroupedGemm& grouped, void* workspac
   if (!(g.xs_rs >= 0 && g.xs_cs >= 0 && g.ws_rs >= 0 && g.ws_cs >= 0 && (int64_t)g.M * g.xs_rs < (1ll << 29)))
     FG_FAIL(FG_ERR_UNSUPPORTED, "grouped fp8 gemm: scale strides must be non-negative and M * row stride below 2^29");
   if (grouped.n_groups <= 0 || grouped.n_groups > 65536) FG_FAIL(FG_ERR_INVALID_ARG, "grouped fp8 gemm: 1..65536 groups");
-  if (grouped.row_index != nullptr) {
+  if (grouped.row_index != nullptr && grouped.index_div == 0 && grouped.c_rows == 0)
+    FG_FAIL(FG_ERR_INVALID_ARG, "grouped fp8 gemm: index divisor 0 (rows not gathered) leaves row_index without a use unless the results are scattered");
+  if (grouped.row_index != nullptr && grouped.index_div != 0) {
     if (grouped.index_div < 1 || grouped.index_div > 0x7FFFFFFF) FG_FAIL(FG_ERR_INVALID_ARG, "grouped fp8 gemm: index divisor %lld", (long long)grouped.index_div);
     if (grouped.x_rows < 1 || grouped.x_rows > 0x7FFFFFFF || grouped.x_rows * g.ldx >= (1ll << 32) || grouped.x_rows * g.xs_rs >= (1ll << 29))
       FG_FAIL(FG_ERR_UNSUPPORTED, "grouped fp8 gemm: %lld gathered rows: the rows of A and of its scales must fit 32-bit byte offsets",

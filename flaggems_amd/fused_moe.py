@@ -7,11 +7,11 @@ expert in torch (tests/test_fused_experts_impl.py:604-662).  The steps are the r
 
   1. the activations are quantized per token and 128-group (``moe_kernel_quantize_input`` -> per_token_group_quant_fp8,
      fused_moe.py:674-683);
-  2. GEMM 1 reads token ``slot // top_k`` for every routed slot and writes the result at the slot's own row
-     (fused_moe.py:1111, 1484-1509);
-  3. SiLU-and-mul and the second quantization (fused_moe.py:2108-2122) -- one kernel here;
-  4. GEMM 2 reads and writes slot rows and multiplies the fp32 sums by the slot's routing weight
-     (``MUL_ROUTED_WEIGHT``, fused_moe.py:1495-1502);
+  2. GEMM 1 reads token ``slot // top_k`` for every routed slot (fused_moe.py:1111); the reference writes the result
+     at the slot's own row (fused_moe.py:1484-1509), here it stays where it is computed, in expert order;
+  3. SiLU-and-mul and the second quantization (fused_moe.py:2108-2122) -- one kernel here, row by row;
+  4. GEMM 2 reads its rows (in place here, through the table in the reference), multiplies the fp32 sums by the slot's
+     routing weight (``MUL_ROUTED_WEIGHT``, fused_moe.py:1495-1502) and writes every result at its slot's row;
   5. ``moe_sum`` adds the top-k slot rows of every token (fused_moe.py:2177-2182).
 
 What differs is the routing table.  The reference pads every expert's rows to a multiple of the kernel's BLOCK_M
@@ -237,19 +237,29 @@ def fused_experts_impl(
     weights = topk_weights.reshape(-1).to(torch.float32).contiguous()
 
     xq, xs = per_token_group_quant_fp8(hidden_states, block_shape[1], scale_rule=quant_scale_rule)
-    # GEMM 1: slot m of the sorted order reads token sorted_slots[m] // top_k and writes row sorted_slots[m]
-    cache1 = grouped_w8a8_block_fp8_matmul(
-        xq, w1, xs, w1_scale, offs, block_shape, dtype, row_index=sorted_slots, index_divisor=top_k,
-        scatter_rows=slots, row_weights=weights if apply_router_weight_on_input else None,
-    )
-    # rows of slots whose expert lives elsewhere were never written: they are quantized like the rest and never read
-    aq, a_s = silu_and_mul_per_token_group_quant_fp8(cache1, block_shape[1], scale_rule=quant_scale_rule)
-    # GEMM 2: reads and writes slot rows; a slot that no local expert serves contributes zeros
-    cache3 = grouped_w8a8_block_fp8_matmul(
-        aq, w2, a_s, w2_scale, offs, block_shape, dtype, row_index=sorted_slots, index_divisor=1,
-        scatter_rows=slots, row_weights=None if apply_router_weight_on_input else weights,
-        zero_unwritten_rows=expert_map is not None,
-    )
+    if apply_router_weight_on_input:
+        # the routing weight multiplies GEMM 1's fp32 sums, which the kernel does where it scatters: both GEMMs read
+        # and write slot rows, as the reference's kernel does
+        cache1 = grouped_w8a8_block_fp8_matmul(
+            xq, w1, xs, w1_scale, offs, block_shape, dtype, row_index=sorted_slots, index_divisor=top_k,
+            scatter_rows=slots, row_weights=weights)
+        aq, a_s = silu_and_mul_per_token_group_quant_fp8(cache1, block_shape[1], scale_rule=quant_scale_rule)
+        cache3 = grouped_w8a8_block_fp8_matmul(
+            aq, w2, a_s, w2_scale, offs, block_shape, dtype, row_index=sorted_slots, index_divisor=1,
+            scatter_rows=slots, zero_unwritten_rows=expert_map is not None)
+    else:
+        # The rows between the two GEMMs stay in expert order: GEMM 1 gathers token sorted_slots[m] // top_k for sorted
+        # row m and stores the row where it is (whole-line stores, no scatter), the activation and its quantizer work
+        # row by row whatever the order, and GEMM 2 reads its rows in place and scatters sorted row m to slot row
+        # sorted_slots[m], times the slot's routing weight.  Same values as with slot-ordered rows in between (the
+        # reference's layout, fused_moe.py:1111, 1484-1509); rows of slots that no local expert serves are never
+        # written by GEMM 1 (they lie behind the last segment), quantized like the rest and never read.
+        cache1 = grouped_w8a8_block_fp8_matmul(
+            xq, w1, xs, w1_scale, offs, block_shape, dtype, row_index=sorted_slots, index_divisor=top_k)
+        aq, a_s = silu_and_mul_per_token_group_quant_fp8(cache1, block_shape[1], scale_rule=quant_scale_rule)
+        cache3 = grouped_w8a8_block_fp8_matmul(
+            aq, w2, a_s, w2_scale, offs, block_shape, dtype, row_index=sorted_slots, index_divisor=0,
+            scatter_rows=slots, row_weights=weights, zero_unwritten_rows=expert_map is not None)
     moe_sum(cache3.view(T, top_k, H), out)
     return out
 

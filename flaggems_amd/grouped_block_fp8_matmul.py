@@ -100,6 +100,9 @@ def grouped_w8a8_block_fp8_matmul(
     reads its tokens (``sorted_token_ids // top_k``, src/flag_gems/fused/fused_moe.py:1111); the result still has
     M = ``row_index.numel()`` rows in sorted order.
 
+    ``index_divisor=0`` (with ``scatter_rows``): A and As are in sorted order themselves and ``row_index`` only says
+    where the results go -- the second GEMM of an expert layer whose intermediate rows stayed in expert order.
+
     With ``scatter_rows`` = R as well, the result has R rows and sorted row m is written to row ``row_index[m]``;
     entries outside ``[0, R)`` are padding (the reference pads ``sorted_token_ids`` with ``numel``,
     src/flag_gems/fused/moe_align_block_size.py:404-517) and store nothing, rows no entry names keep what
@@ -120,8 +123,11 @@ def grouped_w8a8_block_fp8_matmul(
     M = T
     if row_index is not None:
         assert row_index.ndim == 1 and row_index.dtype == torch.int32 and row_index.is_contiguous()
-        assert row_index.device == A.device and index_divisor >= 1
+        assert row_index.device == A.device and index_divisor >= 0
         M = row_index.numel()
+        if index_divisor == 0:  # rows already in sorted order: the index only addresses the scattered result
+            assert scatter_rows is not None and T == M, "index_divisor=0 needs scatter_rows and A in sorted order"
+
     c_rows = 0
     if scatter_rows is not None:
         assert row_index is not None, "scattered results are addressed through row_index"

@@ -356,6 +356,8 @@ int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_batch_stride
  * (entries are forced into [0, a_rows); a_rows * lda must fit 32 bits).  This is how the reference's MoE kernel
  * reads its tokens (rows = sorted_token_ids // top_k, src/flag_gems/fused/fused_moe.py:1111): the caller need not
  * materialise the activations in expert order.  NULL: A and As are already in sorted order (a_rows ignored).
+ * index_div == 0 (with c_rows > 0): A and As are in sorted order as well and row_index only addresses the scattered
+ * result -- the second GEMM of an expert layer whose intermediate rows stayed in expert order.
  * c_rows > 0 (needs row_index): the results are scattered as well -- C has c_rows rows, the result of sorted row m
  * goes to row row_index[m], and entries outside [0, c_rows) are padding that stores nothing (the reference's
  * sorted_token_ids pads every expert to a multiple of its block with the value numel,

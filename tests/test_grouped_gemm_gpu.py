@@ -269,6 +269,13 @@ def test_results_scattered_and_weighted_like_the_moe_kernel(T, N, K, top_k, bloc
         xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), ends.to(DEV), [128, 128], row_index=sorted_ids.to(DEV),
         index_divisor=top_k, scatter_rows=slots, row_weights=weights.to(DEV) if weighted else None)
     assert torch.equal(again, got)
+    # index_divisor = 0: the rows are handed over in sorted order already and the index only addresses the result
+    src_rows = (sorted_ids.clamp(0, slots - 1) // top_k).long()
+    presorted = flag_gems.grouped_w8a8_block_fp8_matmul(
+        xq.to(DEV)[src_rows.to(DEV)].contiguous(), wq.to(DEV), xs.to(DEV)[src_rows.to(DEV)].contiguous(), ws.to(DEV), ends.to(DEV),
+        [128, 128], row_index=sorted_ids.to(DEV), index_divisor=0, scatter_rows=slots,
+        row_weights=weights.to(DEV) if weighted else None)
+    assert torch.equal(presorted, got)
 
 
 def test_scatter_skips_padding_and_rows_out_of_range():
