@@ -391,6 +391,22 @@ def main():
     def time_eager(fn, reps):
         return time_graph(lambda r: fn(), launches=max(reps, 20))
 
+    # inverse RoPE fused into the group quantizer, the largest shape of the reference's benchmark
+    # (benchmark/core_shapes.yaml "fused_inv_rope_fp8_quant": 4096 tokens, 128 heads of 512 in 8 groups, bf16)
+    rope_tokens, rope_heads = 4096, 128
+    r_o = torch.randn(rope_tokens, rope_heads, 512, device=dev, generator=gen).bfloat16()
+    r_pos = torch.randint(0, 8192, (rope_tokens,), device=dev, generator=gen)
+    r_freq = torch.outer(torch.arange(8192, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(0, 32, dtype=torch.float32) / 32)))
+    r_cache = torch.cat((r_freq.cos(), r_freq.sin()), dim=-1).to(dev)
+    rope_bytes = rope_tokens * rope_heads * 512 * 3 + rope_tokens * rope_heads * 4 * 4
+    rope_us = time_eager(lambda: flag_gems.fused_inv_rope_fp8_quant(r_o, r_pos, r_cache, 8, rope_heads // 8), 10)
+    rope_packed_us = time_eager(lambda: flag_gems.fused_inv_rope_fp8_quant(r_o, r_pos, r_cache, 8, rope_heads // 8,
+                                                                             tma_aligned_scales=True), 10)
+    inv_rope = {"shape": [rope_tokens, rope_heads, 512], "groups": 8, "us": round(rope_us, 2),
+                "gbps": round(rope_bytes / rope_us / 1e3, 1), "frac_hbm": round(rope_bytes / rope_us / 1e3 / PEAK_HBM_GBPS, 4),
+                "packed_ue8m0_us": round(rope_packed_us, 2)}
+    del r_o, r_pos, r_cache
+
     # the M = 4096 GEMMs of the sweep once more with power-of-two scales (ue8m0 quantization: act_quant scale_fmt
     # "ue8m0", per_block_cast_to_fp8 use_ue8m0), through the entry point that hands the scales to the matrix
     # instruction; the same call without that promise beside it
@@ -450,13 +466,14 @@ def main():
     for dt, peak in ((torch.bfloat16, 2500.0), (torch.float16, 2500.0), (torch.float32, 157.3)):
         gb = torch.randn(4096, 4096, device=dev, generator=gen).to(dt).t()
         g_sb = torch.rand(1, 4096, device=dev, generator=gen) + 0.5
-        for m in (64, 4096):
+        for m in (1, 64, 4096):
             ga = torch.randn(m, 4096, device=dev, generator=gen).to(dt)
             g_sa = torch.rand(m, 1, device=dev, generator=gen) + 0.5
             us = time_eager(lambda: flag_gems.scaled_mm(ga, gb, g_sa, g_sb), 10)
             tf = gemm_flops(m, 4096, 4096) / us / 1e6
+            g_bytes = (m * 4096 + 4096 * 4096 + m * 4096) * ga.element_size()
             generic.append({"dtype": str(dt)[6:], "M": m, "N": 4096, "K": 4096, "us": round(us, 2), "tflops": round(tf, 1),
-                            "frac_mfma": round(tf / peak, 4)})
+                            "gbps": round(g_bytes / us / 1e3, 1), "frac_mfma": round(tf / peak, 4)})
         del ga, gb
 
     # fp8_einsum("bhr,hdr->bhd") at the first shape group of the reference's benchmark (h = 8, r = 4096, d = 1024)
@@ -671,6 +688,7 @@ def main():
         "weight_quantizer_128x128": weight_quant,
         "silu_mul_quantizer": fused,
         "rms_norm_quantizer": norm_quant,
+        "inv_rope_quantizer": inv_rope,
         "block_fp8_gemm_pow2_scales_m4096": pow2_summary,
         "cutlass_scaled_mm_n8192_k8192_bias": scaled,
         "cutlass_scaled_mm_int8_n8192_k8192_bias": scaled_i8,

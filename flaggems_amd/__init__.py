@@ -19,6 +19,7 @@ from .act_quant import (  # noqa: F401
 )
 from .cutlass_scaled_mm import SM_VERSION_NUM, cutlass_scaled_mm, get_sm_version_num  # noqa: F401
 from .fp8_einsum import fp8_einsum, w8a8_block_fp8_bmm  # noqa: F401
+from .fused_inv_rope_fp8_quant import fused_inv_rope_fp8_quant  # noqa: F401
 from .fused_moe import (  # noqa: F401
     fused_experts_impl,
     inplace_fused_experts,
@@ -63,6 +64,7 @@ __all__ = [
     "fp8_matmul_noop",
     "fused_add_rms_norm",
     "fused_experts_impl",
+    "fused_inv_rope_fp8_quant",
     "get_group_quant_rule",
     "grouped_w8a8_block_fp8_matmul",
     "group_ends_from_expert_ids",

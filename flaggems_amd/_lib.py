@@ -61,6 +61,11 @@ SIGNATURES = {
          c_void_p, c_int, c_int64, c_void_p, c_int64, c_int64,
          c_int64, c_float, c_float, c_float, c_float, c_int, c_int, c_int, c_void_p],
     ),
+    "fg_inv_rope_group_quant_fp8": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int64, c_int64,
+         c_int64, c_int64, c_int64, c_float, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p],
+    ),
     "fg_silu_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p]),
     "fg_moe_sum": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p]),
     "fg_moe_sort_slots": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_void_p, c_void_p]),

@@ -221,6 +221,42 @@ int fg_rms_norm_group_quant_fp8(const void* x, int x_dtype, int64_t rows, int64_
                                 void* stream);
 
 /*
+ * Inverse rotary embedding fused into the group quantizer: the producer of the quantized activations of
+ * DeepSeek-V4's grouped output projection (the "bhr,hdr->bhd" einsum that fg_batched_block_fp8_gemm serves).
+ *   o: [tokens, heads, head_dim] of FG_BF16 / FG_F16 / FG_F32, unit stride along head_dim, element strides
+ *      o_stride_token and o_stride_head; heads = groups * heads_per_group.
+ *   positions: [tokens], int32 or int64 (position_bytes 4 or 8); cos_sin_cache: fp32 [cache_rows, >= rope_dim]
+ *      with rows cache_stride apart, cos in the first rope_dim / 2 columns and sin in the next rope_dim / 2.
+ *      A position outside [0, cache_rows) reads the nearest row (the reference reads out of bounds there).
+ *   The last rope_dim values of every head are rotated back in fp32, pairs interleaved:
+ *      x[2i]' = x[2i] cos_i + x[2i+1] sin_i,   x[2i+1]' = x[2i+1] cos_i - x[2i] sin_i   (each operation rounded),
+ *   the first head_dim - rope_dim pass through, and every group_size values are quantized without an intermediate
+ *   rounding: amax = max(max|x|, eps), scale = amax * fp32(1/448), codes = e4m3fn(clamp(x / scale, -448, 448)).
+ *   q: e4m3fn, value (t, h, j) at q[(h / heads_per_group) * q_stride_group + t * q_stride_token
+ *      + (h % heads_per_group) * head_dim + j]  (the reference allocates [groups, tokens, heads_per_group * head_dim]
+ *      and returns its transpose, so that every group is a contiguous [tokens, K] operand).
+ *   scales, pack_ue8m0 == 0: fp32, group c of head h of token t at
+ *      scales[(h / heads_per_group) * scale_stride_group + t + ((h % heads_per_group) * chunks + c) * scale_stride_k],
+ *      chunks = head_dim / group_size: tokens have unit stride (column-major per group).
+ *   scales, pack_ue8m0 != 0: the scale is rounded up to a power of two, exp2(ceil(log2(max(scale, 1e-10)))), and one
+ *      int32 per head holds the exponent fields of its (at most four) groups, group c in byte c, at
+ *      scales[(h / heads_per_group) * scale_stride_group + t + (h % heads_per_group) * scale_stride_k].
+ *   Rows tokens <= t < padded_tokens of the scale columns are set to zero (the reference pads the token count to a
+ *   multiple of four); q has no such rows.
+ * group_size 64, 128, 256 or 512 with rope_dim <= group_size, both multiples of 8; heads of o 16-byte aligned,
+ * rows of q 8-byte aligned (FG_ERR_UNSUPPORTED otherwise).
+ * Stands in for fused_inv_rope_fp8_quant (src/flag_gems/fused/fused_inv_rope_fp8_quant.py:164-257, kernel :38-161).
+ */
+int fg_inv_rope_group_quant_fp8(const void* o, int o_dtype, int64_t tokens, int64_t heads, int64_t head_dim,
+                                int64_t o_stride_token, int64_t o_stride_head,
+                                const void* positions, int position_bytes,
+                                const float* cos_sin_cache, int64_t cache_rows, int64_t cache_stride,
+                                int64_t heads_per_group, int64_t rope_dim, int64_t group_size, float eps,
+                                void* q, int64_t q_stride_group, int64_t q_stride_token,
+                                void* scales, int64_t scale_stride_group, int64_t scale_stride_k,
+                                int64_t padded_tokens, int pack_ue8m0, void* stream);
+
+/*
  * act_quant with the reference's fixed rules (bf16 in, e4m3fn out, floor 1e-4,
  * scale = amax * fp32(1/448), reciprocal-multiply quotient, power-of-two scale when
  * round_scale != 0), contiguous [rows, cols] input and outputs.

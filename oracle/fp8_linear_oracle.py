@@ -32,6 +32,13 @@ the checks live in tests/test_oracle_*.py):
 * fp8_block_einsum_ref -- dequantise-then-einsum over [b, h, r] x [h, d, r]; pinned
   per head against block_fp8_matmul_tiled_ref (a different order of operations)
   and by a float64 loop on a tiny case.
+* inv_rope_ref, fused_inv_rope_fp8_quant_ref -- the rotation is pinned by known answers the mathematics fixes (a pair
+  (cos t, sin t) rotated back by t is (1, 0); forward rotation would give (cos 2t, sin 2t)), by a float64
+  evaluation with complex numbers (a different formula), by exact preservation of pair norms at the angles 0, pi/2
+  and pi, and by position 0 leaving the input untouched; the quantizer half is pinned by equality with
+  per_token_group_quant_fp8_kernel_ref's formulas on the same values (itself pinned by the brute-force quantizer),
+  and the layout and packed exponents by inputs whose group maxima are 448 * 2^k, so that scale k and byte 127 + k
+  are known in advance (tests/test_oracle_inv_rope.py).
 * silu_and_mul_ref -- pinned by a float64 evaluation (at most one rounding step of the
   output type apart), by torch.sigmoid (a different formula), and by the special
   cases silu(0) = 0, silu(g) = g for large g, silu(g) = -0 for very negative g and
@@ -162,6 +169,63 @@ def per_token_group_quant_fp8_kernel_ref(
         y_s = torch.exp2(torch.ceil(torch.log2(torch.maximum(y_s.abs(), torch.tensor(1e-10, dtype=torch.float32)))))
     y_q = (y / y_s).clamp(min=finfo.min, max=finfo.max).to(dtype)
     return y_q.reshape(x.shape), y_s.reshape(x.shape[:-1] + (x.shape[-1] // group_size,))
+
+
+def inv_rope_ref(o: torch.Tensor, positions: torch.Tensor, cos_sin_cache: torch.Tensor, nope_dim: int, rope_dim: int,
+                 round_rotated: bool = True) -> torch.Tensor:
+    """Restates ``_reference_inv_rope`` (reference tests/test_fused_inv_rope_fp8_quant.py:104-121): the last
+    ``rope_dim`` values of every head rotated back by the token's position, pairs interleaved (GPT-J style), in fp32:
+    ``x * cos + rotate(x) * (-sin)`` with ``rotate((a, b)) = (-b, a)``.  With ``round_rotated`` the rotated values are
+    rounded to ``o``'s dtype (the test helper); without, the result is fp32 and the rotated tail keeps its fp32
+    values (what the reference's device kernel quantizes, src/flag_gems/fused/fused_inv_rope_fp8_quant.py:96-113)."""
+    half = rope_dim // 2
+    cos_sin = cos_sin_cache.index_select(0, positions)
+    cos = cos_sin[:, :half].repeat_interleave(2, dim=-1).unsqueeze(1)
+    sin = -cos_sin[:, half:].repeat_interleave(2, dim=-1).unsqueeze(1)
+    o_pass = o[..., :nope_dim]
+    rot = o[..., nope_dim:].float()
+    x1, x2 = rot[..., ::2], rot[..., 1::2]
+    rotated_half = torch.stack((-x2, x1), dim=-1).flatten(-2)
+    rot = rot * cos + rotated_half * sin
+    if round_rotated:
+        return torch.cat((o_pass, rot.to(o.dtype)), dim=-1)
+    return torch.cat((o_pass.float(), rot), dim=-1)
+
+
+def fused_inv_rope_fp8_quant_ref(
+    o: torch.Tensor, positions: torch.Tensor, cos_sin_cache: torch.Tensor, n_groups: int, heads_per_group: int,
+    nope_dim: int = 448, rope_dim: int = 64, quant_group_size: int = 128, eps: float = 1e-10,
+    tma_aligned_scales: bool = False, round_rotated: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Restates ``native_fused_inv_rope_fp8_quant`` (reference tests/test_fused_inv_rope_fp8_quant.py:124-177):
+    inverse RoPE, then per group of ``quant_group_size`` values in fp32: amax floored at ``eps``,
+    scale = amax * fp32(1/448), optionally exp2(ceil(log2(max(scale, eps)))), codes = clamp(x / scale, +-448) cast
+    to e4m3fn.  Returns (codes [T, G, hpg * head_dim], scales [T, G, blocks] fp32 -- or, with ``tma_aligned_scales``,
+    int32 [T, G, hpg] holding the exponent fields of a head's scales, group c in byte c, as ``_pack_ue8m0_scales``,
+    :55-64, packs them).
+
+    ``round_rotated=True`` is the test helper to the letter (it rounds the rotated tail to ``o``'s dtype before
+    quantizing); the default ``False`` is the reference's device kernel, which quantizes the fp32 values
+    (src/flag_gems/fused/fused_inv_rope_fp8_quant.py:96-128) -- the two differ by that one rounding, which is why
+    the reference's own test compares them by cosine similarity."""
+    o_rot = inv_rope_ref(o, positions, cos_sin_cache, nope_dim, rope_dim, round_rotated)
+    num_tokens, _, head_dim = o_rot.shape
+    d = heads_per_group * head_dim
+    chunks_per_head = head_dim // quant_group_size
+    blocks = d // quant_group_size
+    o_blocks = o_rot.reshape(num_tokens, n_groups, d).float().reshape(num_tokens, n_groups, blocks, quant_group_size)
+    absmax = o_blocks.abs().amax(dim=-1).clamp(min=eps)
+    scales = absmax * (1.0 / FP8_MAX)
+    if tma_aligned_scales:
+        scales = torch.exp2(torch.ceil(torch.log2(scales.clamp(min=eps))))
+    codes = (o_blocks / scales.unsqueeze(-1)).clamp(-FP8_MAX, FP8_MAX).to(FP8_DTYPE).reshape(num_tokens, n_groups, d)
+    if not tma_aligned_scales:
+        return codes, scales
+    exps = (scales.reshape(num_tokens, n_groups, heads_per_group, chunks_per_head).contiguous().view(torch.int32) >> 23) & 0xFF
+    packed = torch.zeros(exps.shape[:-1], dtype=torch.int32)
+    for c in range(chunks_per_head):
+        packed |= exps[..., c] << (8 * c)
+    return codes, packed
 
 
 def silu_and_mul_ref(x: torch.Tensor) -> torch.Tensor:

@@ -48,7 +48,9 @@ CASES = [
 ]
 SHAPES = [(1, 1, 8), (16, 32, 64), (33, 65, 129), (128, 128, 32), (130, 250, 100), (256, 384, 512), (1000, 520, 2048),
           # enough 256 x 256 tiles for most compute units: 16-bit operands with 16-bit results take the persistent kernel
-          (2560, 4096, 256), (2500, 4200, 192)]
+          (2560, 4096, 256), (2500, 4200, 192),
+          # up to 128 rows: workgroups of 16 columns whose wavefronts share K, several runs of K steps per wavefront
+          (64, 272, 4096), (128, 48, 2088), (17, 16, 8200), (97, 100, 520)]
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: f"{str(c[0])[6:]}-{str(c[1])[6:] if c[1] else 'default'}-{c[2]}-bias{int(c[3])}")
