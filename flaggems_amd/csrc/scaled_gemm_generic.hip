@@ -414,7 +414,21 @@ extern "C" int fg_scaled_gemm(const void* A, int64_t lda, const void* B, int64_t
   g.C = C; g.c_dtype = c_dtype;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
   g.tiles_n = (int)tiles_n;
-  if (M <= 128 && ceil_div(N, 16) <= 0x7FFFFFFF) {
+  // Up to 128 rows: workgroups of 16 columns while that is the faster way.  Their time grows with N (every workgroup
+  // fetches the rows of A again), the 128 x 128 tiles' time only with the rounds of tiles over the compute units.
+  // Timed on both at K = 4096, us: bf16 M = 64: N = 8192 43 against 63, N = 16384 83 against 65; M = 128: N = 4096 44 against
+  // 64, N = 8192 84 against 64; fp32 M = 64: N = 16384 194 against 299, N = 28672 352 against 301; both scale with K.
+  // (With at most 32 rows of 16-bit operands the tiles load straight from global memory, 74-95 us: never faster.)
+  bool skinny = M <= 128 && ceil_div(N, 16) <= 0x7FFFFFFF;
+  if (skinny && (ab_dtype == FG_F32 || M > 32)) {
+    const int64_t slices = ceil_div(M, 64), fm = ceil_div(ceil_div(M, slices), 16);
+    const double k4 = (double)K / 4096.0, units = (double)ceil_div(N, 16) * (double)slices * (double)(fm + 1);
+    const double rounds = (double)ceil_div(tiles_m * tiles_n, (int64_t)cu_count());
+    const double t_skinny = 3.0 + (ab_dtype == FG_F32 ? 0.037 : 0.0155) * units * k4;
+    const double t_tiles = (ab_dtype == FG_F32 ? 5.0 + 290.0 * k4 : 10.0 + 52.0 * k4) * rounds;
+    skinny = t_skinny < t_tiles;
+  }
+  if (skinny) {
     if (ab_dtype == FG_BF16) launch_skinny<FG_BF16>(g, (hipStream_t)stream);
     else if (ab_dtype == FG_F16) launch_skinny<FG_F16>(g, (hipStream_t)stream);
     else launch_skinny<FG_F32>(g, (hipStream_t)stream);

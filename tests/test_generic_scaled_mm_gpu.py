@@ -50,7 +50,9 @@ SHAPES = [(1, 1, 8), (16, 32, 64), (33, 65, 129), (128, 128, 32), (130, 250, 100
           # enough 256 x 256 tiles for most compute units: 16-bit operands with 16-bit results take the persistent kernel
           (2560, 4096, 256), (2500, 4200, 192),
           # up to 128 rows: workgroups of 16 columns whose wavefronts share K, several runs of K steps per wavefront
-          (64, 272, 4096), (128, 48, 2088), (17, 16, 8200), (97, 100, 520)]
+          (64, 272, 4096), (128, 48, 2088), (17, 16, 8200), (97, 100, 520),
+          # 128 rows against a wide matrix: the 128 x 128 tiles again (16-bit operands; fp32 stays with the 16-column workgroups)
+          (128, 8192, 2048)]
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: f"{str(c[0])[6:]}-{str(c[1])[6:] if c[1] else 'default'}-{c[2]}-bias{int(c[3])}")
