@@ -178,7 +178,7 @@ __global__ __launch_bounds__(kRopeThreads) void inv_rope_quant_kernel(InvRopeArg
 template <int XDT, int LPG>
 int launch_inv_rope(const InvRopeArgs& a, int64_t padded_tokens, hipStream_t stream) {
   // 16 tokens and four heads per workgroup once that leaves workgroups enough to fill the GPU; else 4 tokens, one head
-  const bool wide = ceil_div(padded_tokens, (int64_t)16) * (a.heads / 4) >= 2048 && a.heads % 4 == 0;
+  const bool wide = ceil_div(padded_tokens, (int64_t)16) * (a.heads / 4) >= 1024 && a.heads % 4 == 0;
   const int64_t head_blocks = wide ? a.heads / 4 : a.heads;
   const int64_t blocks = ceil_div(padded_tokens, (int64_t)(wide ? 16 : 4)) * head_blocks;
   if (blocks > 0x7FFFFFFF) FG_FAIL(FG_ERR_UNSUPPORTED, "fg_inv_rope_group_quant_fp8: too many workgroups");
