@@ -407,6 +407,21 @@ def main():
                 "packed_ue8m0_us": round(rope_packed_us, 2)}
     del r_o, r_pos, r_cache
 
+    # routing in front of the expert layer: softmax + top-2 of 8 experts (Mixtral), group-limited top-8 of 256 experts in 8
+    # groups (DeepSeek-V3), 4096 tokens each; latency-bound launches, reported in microseconds only
+    rt_tokens = 4096
+    rt_g8 = torch.randn(rt_tokens, 8, device=dev, generator=gen)
+    rt_w = torch.empty(rt_tokens, 2, device=dev)
+    rt_i = torch.empty(rt_tokens, 2, device=dev, dtype=torch.int32)
+    rt_s = torch.empty(rt_tokens, 2, device=dev, dtype=torch.int32)
+    rt_softmax_us = time_eager(lambda: flag_gems.topk_softmax(rt_w, rt_i, rt_s, rt_g8, True), 20)
+    rt_g256 = torch.randn(rt_tokens, 256, device=dev, generator=gen).bfloat16()
+    rt_bias = torch.randn(256, device=dev, generator=gen).bfloat16()
+    rt_grouped_us = time_eager(lambda: flag_gems.grouped_topk(rt_g256, 8, 4, 8, True, 2.5, rt_bias, 1), 20)
+    routing = {"tokens": rt_tokens, "topk_softmax_8_experts_top2_us": round(rt_softmax_us, 2),
+               "grouped_topk_256_experts_8_groups_top8_us": round(rt_grouped_us, 2)}
+    del rt_g8, rt_g256
+
     # the M = 4096 GEMMs of the sweep once more with power-of-two scales (ue8m0 quantization: act_quant scale_fmt
     # "ue8m0", per_block_cast_to_fp8 use_ue8m0), through the entry point that hands the scales to the matrix
     # instruction; the same call without that promise beside it
@@ -689,6 +704,7 @@ def main():
         "silu_mul_quantizer": fused,
         "rms_norm_quantizer": norm_quant,
         "inv_rope_quantizer": inv_rope,
+        "moe_routing": routing,
         "block_fp8_gemm_pow2_scales_m4096": pow2_summary,
         "cutlass_scaled_mm_n8192_k8192_bias": scaled,
         "cutlass_scaled_mm_int8_n8192_k8192_bias": scaled_i8,

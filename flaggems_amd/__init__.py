@@ -34,6 +34,7 @@ from .grouped_block_fp8_matmul import (  # noqa: F401
     grouped_w8a8_block_fp8_matmul,
     local_rows_from_moe_align,
 )
+from .moe_routing import grouped_topk, topk_softmax  # noqa: F401
 from .norm_quant import fused_add_rms_norm, rms_norm, rms_norm_per_token_group_quant_fp8  # noqa: F401
 from .registration import (  # noqa: F401
     all_registered_keys,
@@ -66,6 +67,7 @@ __all__ = [
     "fused_experts_impl",
     "fused_inv_rope_fp8_quant",
     "get_group_quant_rule",
+    "grouped_topk",
     "grouped_w8a8_block_fp8_matmul",
     "group_ends_from_expert_ids",
     "local_rows_from_moe_align",
@@ -87,6 +89,7 @@ __all__ = [
     "set_group_quant_rule",
     "silu_and_mul_packed",
     "silu_and_mul_per_token_group_quant_fp8",
+    "topk_softmax",
     "use_gems",
     "w8a8_block_fp8_bmm",
     "w8a8_block_fp8_matmul",

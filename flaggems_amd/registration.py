@@ -21,6 +21,7 @@ import torch
 from .act_quant import per_token_group_fp8_quant_into
 from .cutlass_scaled_mm import cutlass_scaled_mm
 from .fused_moe import moe_align_block_size_triton, moe_sum
+from .moe_routing import grouped_topk, topk_softmax
 from .scaled_mm import scaled_mm, scaled_mm_out
 
 logger = logging.getLogger("flag_gems")
@@ -204,13 +205,17 @@ _VLLM_IMPLS = {
     "per_token_group_fp8_quant": custom_per_token_group_fp8_quant,
 }
 
-# the two operators of vLLM's ``_moe_C`` namespace that the expert layer of this path uses
-# (src/flag_gems/patches/patch_util.py:74-85, patch_vllm_all.py:306-321, 356-359)
+# the operators of vLLM's ``_moe_C`` namespace that the reference implements: routing, alignment, the sum over the slots
+# (src/flag_gems/patches/patch_util.py:74-85, patch_vllm_all.py:306-359, 628-633)
 _VLLM_MOE_OPS_SIGNATURES = {
     "moe_align_block_size": "(Tensor topk_ids, int num_experts, "
     "int block_size, Tensor(a!) sorted_token_ids, Tensor(b!) experts_ids, "
     "Tensor(c!) num_tokens_post_pad) -> ()",
     "moe_sum": "(Tensor input, Tensor(a!) output) -> ()",
+    "topk_softmax": "(Tensor(a!) topk_weights, Tensor(b!) topk_indices, Tensor(c!) token_expert_indices, "
+    "Tensor gating_output, bool renormalize=False) -> ()",
+    "grouped_topk": "(Tensor scores, int n_group, int topk_group, int topk, bool renormalize, "
+    "float routed_scaling_factor, Tensor bias, int scoring_func=0) -> (Tensor, Tensor)",
 }
 
 
@@ -222,9 +227,20 @@ def custom_moe_sum(input, output):
     moe_sum(input, output)
 
 
+def custom_topk_softmax(topk_weights, topk_indices, token_expert_indices, gating_output, renormalize=False):
+    topk_softmax(topk_weights, topk_indices, token_expert_indices, gating_output, renormalize)
+
+
+def custom_moe_grouped_topk(gating_output, n_group, topk_group, topk, renormalize, routed_scaling_factor, bias, scoring_func=0):
+    return grouped_topk(scores=gating_output, n_group=n_group, topk_group=topk_group, topk=topk, renormalize=renormalize,
+                        routed_scaling_factor=routed_scaling_factor, bias=bias, scoring_func=scoring_func)
+
+
 _VLLM_MOE_IMPLS = {
     "moe_align_block_size": custom_moe_align_block_size,
     "moe_sum": custom_moe_sum,
+    "topk_softmax": custom_topk_softmax,
+    "grouped_topk": custom_moe_grouped_topk,
 }
 
 _vllm_libs: List[torch.library.Library] = []

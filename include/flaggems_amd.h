@@ -157,6 +157,39 @@ int fg_moe_sum(const void* in, int dtype, int64_t tokens, int64_t top_k, int64_t
                int64_t in_slot_stride, void* out, int64_t out_token_stride, void* stream);
 
 /*
+ * Routing by softmax: probabilities p = exp(x - max) / (sum + 1e-8) over the experts of a token (fp32), then topk rounds
+ * of "largest remaining probability, the lower expert on ties".  gating: [tokens, experts] of FG_BF16 / FG_F16 / FG_F32,
+ * rows row_stride elements apart; topk_weights: fp32 [tokens, topk], in descending order, divided by
+ * (their sum + 1e-8) when renormalize != 0; topk_indices: [tokens, topk] of 4- or 8-byte integers (index_bytes);
+ * token_expert_indices: int32 [tokens, topk] = k * tokens + t, or NULL.  topk <= 32 and <= experts <= 1024.
+ * Stands in for topk_softmax (src/flag_gems/fused/topk_softmax.py:85-137, kernel :24-82), the vLLM operator
+ * _moe_C::topk_softmax (src/flag_gems/patches/patch_vllm_all.py:348-353).
+ */
+int fg_topk_softmax(const void* gating, int dtype, int64_t tokens, int64_t experts, int64_t row_stride,
+                    int64_t topk, int renormalize, float* topk_weights, void* topk_indices, int index_bytes,
+                    int* token_expert_indices, void* stream);
+
+/*
+ * Group-limited routing (DeepSeek): with s = scores (scoring_func 0) or sigmoid(scores) rounded to the scores' type
+ * (scoring_func 1) and sb = s + bias rounded to that type,
+ *   group score  = the sum of the two largest sb of the group's experts/n_group consecutive experts (the largest counted
+ *                  twice when it occurs twice), rounded to the scores' type; NaN and +inf count as -inf;
+ *   groups       = the topk_group largest group scores, ties to the lower group;
+ *   experts      = topk rounds of "largest remaining sb among the experts of those groups, the lower expert on ties";
+ *   weights      = s of the selected experts * routed_scaling_factor, over (their sum + 1e-20) when renormalize != 0.
+ * When no group score is above -inf the result is experts 0 .. topk-1 with weight 1 / topk each.
+ * scores: [tokens, experts] (score_stride elements between rows), bias: [experts], both FG_BF16 / FG_F16 / FG_F32;
+ * topk_values fp32 and topk_ids int32: [tokens, topk], out_stride elements between rows.
+ * n_group <= 32 divides experts <= 1024; topk <= 32.
+ * Stands in for grouped_topk (src/flag_gems/fused/grouped_topk.py:256-355, kernels :25-78 and :81-253), the vLLM
+ * operator _moe_C::grouped_topk (src/flag_gems/patches/patch_vllm_all.py:324-345).
+ */
+int fg_grouped_topk(const void* scores, int dtype, int64_t tokens, int64_t experts, int64_t score_stride,
+                    const void* bias, int64_t n_group, int64_t topk_group, int64_t topk, int renormalize,
+                    float routed_scaling_factor, int scoring_func, float* topk_values, int* topk_ids,
+                    int64_t out_stride, void* stream);
+
+/*
  * Routing table of an expert layer for fg_grouped_block_fp8_gemm: the routed slots sorted by expert.
  *     key(s) = local expert of slot s, or num_experts if it has none
  *     sorted_slots = the slot numbers 0 .. n_slots-1 in ascending order of key, ties in slot order (int32 [n_slots])

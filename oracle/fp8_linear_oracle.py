@@ -39,6 +39,12 @@ the checks live in tests/test_oracle_*.py):
   per_token_group_quant_fp8_kernel_ref's formulas on the same values (itself pinned by the brute-force quantizer),
   and the layout and packed exponents by inputs whose group maxima are 448 * 2^k, so that scale k and byte 127 + k
   are known in advance (tests/test_oracle_inv_rope.py).
+* topk_softmax_ref, grouped_topk_ref -- the reference tests both against vLLM's CUDA operators, which are absent here;
+  the restatements follow the reference's own Triton kernels and are pinned by library routines and closed forms:
+  torch.softmax + torch.topk on rows without ties, rows of equal logits (experts 0 .. k-1 at 1 / E each), weights that
+  sum to 1 after renormalisation, the published DeepSeek-V3 routing written with masks and torch.topk (a different
+  algorithm text) on rows without ties, a pure-Python loop over sorted lists on tiny inputs with ties, one group =
+  plain top-k of score + bias, and the fixed answer when every score is -inf (tests/test_oracle_routing.py).
 * silu_and_mul_ref -- pinned by a float64 evaluation (at most one rounding step of the
   output type apart), by torch.sigmoid (a different formula), and by the special
   cases silu(0) = 0, silu(g) = g for large g, silu(g) = -0 for very negative g and
@@ -558,6 +564,78 @@ def make_fp8_einsum_inputs(b: int, h: int, r: int, d: int, seed: int = 0):
     for i in range(h):
         yq[i], ys[i] = per_block_cast_to_fp8_ref(y[i], use_ue8m0=True)
     return xq.view(b, h, r), xs.view(b, h, -1), yq, ys
+
+
+def topk_softmax_ref(gating: torch.Tensor, topk: int, renormalize: bool = False):
+    """Restates the reference's routing kernel ``topk_gating_softmax_kernel``
+    (src/flag_gems/fused/topk_softmax.py:44-82; its own test compares with vLLM's CUDA operator, which is not in
+    this image): fp32 probabilities exp(x - max) / (sum + 1e-8), then ``topk`` rounds of (largest remaining value,
+    first index that holds it), the taken entry set to -inf; with ``renormalize`` the selected values are divided by
+    (their running sum + 1e-8).  Returns (weights fp32 [T, k], indices int64 [T, k], token_expert_indices int32
+    [T, k] = k * T + t)."""
+    x = gating.float()
+    tokens = x.shape[0]
+    e = torch.exp(x - x.max(dim=1, keepdim=True).values)
+    probs = e / (e.sum(dim=1, keepdim=True) + 1e-8)
+    weights = torch.empty(tokens, topk, dtype=torch.float32)
+    indices = torch.empty(tokens, topk, dtype=torch.int64)
+    selected_sum = torch.zeros(tokens, dtype=torch.float32)
+    for ki in range(topk):
+        cur, arg = torch.max(probs, dim=1)          # the first maximal value's index
+        weights[:, ki], indices[:, ki] = cur, arg
+        selected_sum = selected_sum + cur
+        probs = probs.scatter(1, arg.unsqueeze(1), float("-inf"))
+    if renormalize:
+        weights = weights / (selected_sum + 1e-8).unsqueeze(1)
+    source = (torch.arange(topk, dtype=torch.int32).unsqueeze(0) * tokens + torch.arange(tokens, dtype=torch.int32).unsqueeze(1))
+    return weights, indices, source
+
+
+def grouped_topk_ref(scores: torch.Tensor, n_group: int, topk_group: int, topk: int, renormalize: bool,
+                     routed_scaling_factor: float, bias: torch.Tensor, scoring_func: int = 0):
+    """Restates the reference's group-limited routing (src/flag_gems/fused/grouped_topk.py:256-355 with its kernels
+    ``topk_with_k2_triton`` :25-78 and ``group_idx_and_topk_triton`` :81-253; its own test compares with vLLM's CUDA
+    operator, which is not in this image).  All sums of 16-bit tensors are rounded to their type as the kernels'
+    loads and stores round them: s = scores or sigmoid(scores) in the scores' type, sb = s + bias, group score = the
+    two largest sb of the group added (rounded), not-finite group scores = -inf, the ``topk_group`` largest groups
+    (ties: lower group), ``topk`` rounds of (largest remaining sb among their experts, first index), weights = s of
+    the selected * factor, over (their sum + 1e-20) with ``renormalize``; experts 0 .. topk-1 at 1 / topk each when no
+    group score is above -inf.  Returns (fp32 [T, topk], int32 [T, topk])."""
+    tokens, experts = scores.shape
+    per = experts // n_group
+    bias = bias.to(scores.dtype).flatten()
+    s = torch.sigmoid(scores.float()).to(scores.dtype) if scoring_func == 1 else scores
+    sb = s + bias
+    grouped = sb.float().view(tokens, n_group, per)
+    max1 = grouped.max(dim=-1).values
+    if per >= 2:
+        max2 = grouped.topk(2, dim=-1).values[..., 1]
+    else:
+        max2 = torch.full_like(max1, float("-inf"))
+    gs = (max1 + max2).to(scores.dtype).float()
+    gs = torch.where(torch.isfinite(gs) | (gs == float("-inf")), gs, torch.full_like(gs, float("-inf")))
+    proceed = gs.max(dim=1).values != float("-inf")
+    order = torch.sort(gs, dim=1, descending=True, stable=True).indices[:, : min(topk_group, n_group)]
+    chosen = torch.zeros(tokens, n_group, dtype=torch.bool).scatter(1, order, True)
+    sel = torch.where(chosen.repeat_interleave(per, dim=1), sb.float(), torch.full((tokens, experts), float("-inf")))
+    values = torch.empty(tokens, topk, dtype=torch.float32)
+    ids = torch.empty(tokens, topk, dtype=torch.int64)
+    for ki in range(topk):
+        arg = torch.max(sel, dim=1).indices
+        ids[:, ki] = arg
+        values[:, ki] = s.float().gather(1, arg.unsqueeze(1)).squeeze(1)
+        sel = sel.scatter(1, arg.unsqueeze(1), float("-inf"))
+    if renormalize:
+        total = torch.zeros(tokens, dtype=torch.float32)
+        for ki in range(topk):
+            total = total + values[:, ki]
+        scale = torch.tensor(routed_scaling_factor, dtype=torch.float32) / (total + 1e-20)
+        values = values * scale.unsqueeze(1)
+    else:
+        values = values * torch.tensor(routed_scaling_factor, dtype=torch.float32)
+    values = torch.where(proceed.unsqueeze(1), values, torch.full_like(values, 1.0 / topk))
+    ids = torch.where(proceed.unsqueeze(1), ids, torch.arange(topk).expand(tokens, topk))
+    return values, ids.to(torch.int32)
 
 
 def make_moe_rows(tokens: int, experts: int = 8, top_k: int = 2, seed: int = 0) -> torch.Tensor:
