@@ -15,6 +15,7 @@ from .act_quant import (  # noqa: F401
     per_token_group_quant_fp8,
     set_group_quant_rule,
     silu_and_mul_packed,
+    silu_and_mul_packed_out,
     silu_and_mul_per_token_group_quant_fp8,
 )
 from .cutlass_scaled_mm import SM_VERSION_NUM, cutlass_scaled_mm, get_sm_version_num  # noqa: F401
@@ -35,7 +36,7 @@ from .grouped_block_fp8_matmul import (  # noqa: F401
     local_rows_from_moe_align,
 )
 from .moe_routing import grouped_topk, topk_softmax  # noqa: F401
-from .norm_quant import fused_add_rms_norm, rms_norm, rms_norm_per_token_group_quant_fp8  # noqa: F401
+from .norm_quant import fused_add_rms_norm, rms_norm, rms_norm_out, rms_norm_per_token_group_quant_fp8  # noqa: F401
 from .registration import (  # noqa: F401
     all_registered_keys,
     all_registered_ops,
@@ -83,11 +84,13 @@ __all__ = [
     "per_token_cast_to_fp8",
     "per_token_group_quant_fp8",
     "rms_norm",
+    "rms_norm_out",
     "rms_norm_per_token_group_quant_fp8",
     "scaled_mm",
     "scaled_mm_out",
     "set_group_quant_rule",
     "silu_and_mul_packed",
+    "silu_and_mul_packed_out",
     "silu_and_mul_per_token_group_quant_fp8",
     "topk_softmax",
     "use_gems",

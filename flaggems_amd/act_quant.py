@@ -327,6 +327,17 @@ def silu_and_mul_packed(x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError(f"silu_and_mul_packed: unsupported input dtype {x.dtype}")
     d = x.shape[-1] // 2
     out = torch.empty(x.shape[:-1] + (d,), dtype=x.dtype, device=x.device)
+    return silu_and_mul_packed_out(out, x)
+
+
+def silu_and_mul_packed_out(out: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """The same into ``out`` (x's shape with half the last dimension, contiguous): what vLLM's ``_C::silu_and_mul(out,
+    input)`` asks for (src/flag_gems/patches/patch_vllm_all.py:276-279)."""
+    assert x.shape[-1] % 2 == 0 and x.stride(-1) == 1
+    if x.dtype not in _IN_DTYPES:
+        raise NotImplementedError(f"silu_and_mul_packed: unsupported input dtype {x.dtype}")
+    d = x.shape[-1] // 2
+    assert out.shape == x.shape[:-1] + (d,) and out.dtype == x.dtype and out.device == x.device and out.is_contiguous()
     if out.numel() == 0:
         return out
     x2d = _as_rows(x)

@@ -25,7 +25,7 @@ from .act_quant import (
 
 logger = logging.getLogger(__name__)
 
-__all__ = ["rms_norm", "fused_add_rms_norm", "rms_norm_per_token_group_quant_fp8"]
+__all__ = ["rms_norm", "rms_norm_out", "fused_add_rms_norm", "rms_norm_per_token_group_quant_fp8"]
 
 
 def _launch(x2d, residual2d, weight, eps, y2d, q2d, s2d, group_size, quant_eps, fp8_dtype, scale_rule, scale_ue8m0):
@@ -76,6 +76,19 @@ def rms_norm(x: torch.Tensor, normalized_shape: Sequence[int], weight: torch.Ten
     if x.numel():
         _launch(x.view(rows, cols), None, weight.contiguous(), eps, y.view(rows, cols), None, None, 0, 0.0, None, None, False)
     return y
+
+
+def rms_norm_out(result: torch.Tensor, x: torch.Tensor, normalized_shape: Sequence[int], weight: torch.Tensor,
+                 eps: float = 1e-5) -> torch.Tensor:
+    """``rms_norm`` into ``result`` (x's shape and dtype, contiguous): what vLLM's ``_C::rms_norm(result, input, weight,
+    epsilon)`` asks for (src/flag_gems/patches/patch_vllm_all.py:610-613)."""
+    logger.debug("GEMS RMS_NORM OUT")
+    rows, cols = _rows_of(x, normalized_shape)
+    assert result.shape == x.shape and result.dtype == x.dtype and result.device == x.device and result.is_contiguous()
+    x = x.contiguous()
+    if x.numel():
+        _launch(x.view(rows, cols), None, weight.contiguous(), eps, result.view(rows, cols), None, None, 0, 0.0, None, None, False)
+    return result
 
 
 def fused_add_rms_norm(x: torch.Tensor, residual: torch.Tensor, normalized_shape: Sequence[int], weight: torch.Tensor,

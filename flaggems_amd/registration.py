@@ -18,10 +18,11 @@ from typing import Iterable, List, Optional, Tuple
 
 import torch
 
-from .act_quant import per_token_group_fp8_quant_into
+from .act_quant import per_token_group_fp8_quant_into, silu_and_mul_packed_out
 from .cutlass_scaled_mm import cutlass_scaled_mm
 from .fused_moe import moe_align_block_size_triton, moe_sum
 from .moe_routing import grouped_topk, topk_softmax
+from .norm_quant import rms_norm_out
 from .scaled_mm import scaled_mm, scaled_mm_out
 
 logger = logging.getLogger("flag_gems")
@@ -189,6 +190,8 @@ _VLLM_OPS_SIGNATURES = {
     "per_token_group_fp8_quant": "(Tensor input, Tensor(a!) output_q, "
     "Tensor(b!) output_s, int group_size, float eps, float fp8_min, "
     "float fp8_max, bool scale_ue8m0=False) -> ()",
+    "rms_norm": "(Tensor(a!) result, Tensor input, Tensor weight, float epsilon) -> ()",
+    "silu_and_mul": "(Tensor(a!) out, Tensor input) -> ()",
 }
 
 
@@ -200,9 +203,19 @@ def custom_per_token_group_fp8_quant(input, output_q, output_s, group_size, eps,
     per_token_group_fp8_quant_into(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0)
 
 
+def custom_rms_norm_out(result, input, weight, epsilon):
+    rms_norm_out(result, input, list(weight.size()), weight, epsilon)
+
+
+def custom_silu_and_mul(out, input):
+    silu_and_mul_packed_out(out, input)
+
+
 _VLLM_IMPLS = {
     "cutlass_scaled_mm": custom_cutlass_scaled_mm,
     "per_token_group_fp8_quant": custom_per_token_group_fp8_quant,
+    "rms_norm": custom_rms_norm_out,
+    "silu_and_mul": custom_silu_and_mul,
 }
 
 # the operators of vLLM's ``_moe_C`` namespace that the reference implements: routing, alignment, the sum over the slots

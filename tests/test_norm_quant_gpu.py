@@ -139,3 +139,25 @@ def test_unsupported_requests_fail_loudly():
         flag_gems.rms_norm(x, (256,), torch.ones(256, dtype=torch.float32, device=DEV))
     with pytest.raises(RuntimeError, match="group size"):
         flag_gems.rms_norm_per_token_group_quant_fp8(x, torch.ones(256, dtype=torch.bfloat16, device=DEV), 4)
+
+
+def test_vllm_rms_norm_and_silu_and_mul_write_the_callers_tensors():
+    """_C::rms_norm(result, input, weight, epsilon) and _C::silu_and_mul(out, input): the same bits as the operators
+    that allocate, in the tensor the caller passed."""
+    flag_gems.patch_empty_vllm()
+    g = torch.Generator().manual_seed(17)
+    for dtype in (torch.bfloat16, torch.float16):
+        x = torch.randn(3, 37, 1024, generator=g).to(dtype).to(DEV)
+        w = (1 + 0.1 * torch.randn(1024, generator=g)).to(dtype).to(DEV)
+        result = torch.full_like(x, 7.0)
+        assert torch.ops._C.rms_norm(result, x, w, 1e-6) is None
+        assert torch.equal(result, flag_gems.rms_norm(x, (1024,), w, 1e-6))
+        want = O.rms_norm_ref(x.cpu().reshape(-1, 1024), w.cpu(), 1e-6)
+        assert torch.equal(result.cpu().reshape(-1, 1024).view(torch.int16), want.view(torch.int16))
+        out = torch.full((3, 37, 512), 7.0, dtype=dtype, device=DEV)
+        assert torch.ops._C.silu_and_mul(out, x) is None
+        assert torch.equal(out, flag_gems.silu_and_mul_packed(x))
+    with pytest.raises(AssertionError):
+        flag_gems.silu_and_mul_packed_out(torch.empty(3, 37, 500, dtype=torch.float16, device=DEV), x)
+    with pytest.raises(AssertionError):
+        flag_gems.rms_norm_out(torch.empty(3, 37, 512, dtype=torch.float16, device=DEV), x, (1024,), w)
