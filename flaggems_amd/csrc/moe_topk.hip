@@ -12,7 +12,7 @@
 // Both are a few hundred bytes per token and bound by latency, not by any roofline: one wavefront per token, the
 // experts dealt to the lanes (expert e in lane e % 64, slot e / 64), every maximum a 64-bit key (order-preserving
 // image of the value above the complement of the index, so that the largest key is the largest value at the lowest
-// index) reduced over the wavefront with six exchanges.
+// index) reduced over the wavefront with six exchanges, four of them DPP moves inside a row of 16 lanes.
 
 #include "fg_common.h"
 
@@ -43,19 +43,39 @@ __device__ __forceinline__ uint32_t ordered(float v) {
 __device__ __forceinline__ float unordered(uint32_t o) { return bits_to_float((o & 0x80000000u) ? (o & 0x7FFFFFFFu) : ~o); }
 __device__ __forceinline__ uint64_t make_key(float v, uint32_t index) { return ((uint64_t)ordered(v) << 32) | (uint64_t)(~index); }
 
+// A value of another lane: the four exchanges inside a row of 16 lanes are DPP moves (quad swaps, then mirrors of 8 and
+// of 16 lanes: for a reduction any pairing across the halves serves), the two across rows go through the LDS crossbar.
+template <int STEP>
+__device__ __forceinline__ uint32_t from_partner(uint32_t v) {
+  if (STEP == 0) return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);   // quad_perm [1, 0, 3, 2]
+  if (STEP == 1) return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xF, 0xF, true);   // quad_perm [2, 3, 0, 1]
+  if (STEP == 2) return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x141, 0xF, 0xF, true);  // row_half_mirror
+  if (STEP == 3) return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x140, 0xF, 0xF, true);  // row_mirror
+  return (uint32_t)__shfl_xor((int)v, STEP == 4 ? 16 : 32, 64);
+}
+template <int STEP>
+__device__ __forceinline__ float from_partner_f32(float v) { return bits_to_float(from_partner<STEP>(float_to_bits(v))); }
+
+template <int STEP = 0>
 __device__ __forceinline__ uint64_t wave_max_key(uint64_t k) {
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)k, d, 64), hi = (uint32_t)__shfl_xor((int)(uint32_t)(k >> 32), d, 64);
-    const uint64_t o = ((uint64_t)hi << 32) | lo;
-    k = o > k ? o : k;
-  }
+  const uint64_t o = ((uint64_t)from_partner<STEP>((uint32_t)(k >> 32)) << 32) | from_partner<STEP>((uint32_t)k);
+  k = o > k ? o : k;
+  if constexpr (STEP < 5) return wave_max_key<STEP + 1>(k);
   return k;
 }
+template <int STEP = 0>
 __device__ __forceinline__ float wave_max_f32(float v) {
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) v = fmaxf(v, __shfl_xor(v, d, 64));
+  v = fmaxf(v, from_partner_f32<STEP>(v));
+  if constexpr (STEP < 5) return wave_max_f32<STEP + 1>(v);
   return v;
+}
+// (largest, second largest) over the wavefront of the lanes' (t1, t2) pairs
+template <int STEP = 0>
+__device__ __forceinline__ void wave_top2_f32(float& t1, float& t2) {
+  const float o1 = from_partner_f32<STEP>(t1), o2 = from_partner_f32<STEP>(t2);
+  t2 = fmaxf(fminf(t1, o1), fmaxf(t2, o2));
+  t1 = fmaxf(t1, o1);
+  if constexpr (STEP < 5) wave_top2_f32<STEP + 1>(t1, t2);
 }
 __device__ __forceinline__ float wave_sum_f32(float v) {
 #pragma unroll
@@ -158,12 +178,7 @@ __global__ __launch_bounds__(kTopkThreads) void grouped_topk_kernel(GroupedTopkA
       t2 = fmaxf(t2, fminf(t1, v));
       t1 = fmaxf(t1, v);
     }
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const float o1 = __shfl_xor(t1, d, 64), o2 = __shfl_xor(t2, d, 64);
-      t2 = fmaxf(fminf(t1, o1), fmaxf(t2, o2));
-      t1 = fmaxf(t1, o1);
-    }
+    wave_top2_f32(t1, t2);
     // (a group of one expert has no second score: -inf, as the reference's maximum over nothing)
     const float gs = round_like(t1 + t2, a.dt);
     if (lane == g) group_score = gs;
