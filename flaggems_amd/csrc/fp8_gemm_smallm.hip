@@ -301,7 +301,7 @@ __device__ __forceinline__ void dma_to_lds_4(uint32_t byte_off, const void* base
 // the activation fragments travel in the register ring next to the weights.
 template <int TMX, int Q, int DEPTH, int WAVES, int MODE, bool XLDS, bool OWN = false, bool RING = false>
 __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArgs a) {
-  static_assert(!XLDS || TMX == 1, "activations are kept in LDS for M <= 16 only");
+  static_assert(!XLDS || TMX == 1 || (OWN && TMX == 2), "activations in LDS: M <= 16, or M <= 32 where the block shares them");
   static_assert(!OWN || XLDS, "wavefronts with chunks of their own share the activations through LDS");
   static_assert(!RING || (XLDS && !OWN && DEPTH == 1), "the two-slot form belongs to the per-wavefront copies with one pair in the ring");
   constexpr int RG = (Q + 3) / 4;
@@ -499,9 +499,18 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
     lds_xrow[t] = lds_x + (uint32_t)m * x_stride;
     lds_xsrow[t] = lds_xs + (uint32_t)(m * kbc) * 4u;
   }
-  const uint32_t mrow = (uint32_t)(l16 < g.M ? l16 : g.M - 1);  // TMX == 1 when used
-  const uint32_t perm = PW ? (mrow & 15u) : ((mrow >> 1) & 7u);
-  const uint32_t x_lo_piece = ((uint32_t)lg ^ perm) << 4, x_hi_piece = ((uint32_t)(lg + 4) ^ perm) << 4;
+  const uint32_t mrow = (uint32_t)(l16 < g.M ? l16 : g.M - 1);  // per-wavefront copies: TMX == 1
+  const uint32_t perm = mrow & 15u;
+  // shared form: where this lane's two pieces of a K-block lie in row t * 16 + l16 (see the copies above)
+  uint32_t x_lo_piece[TMX], x_hi_piece[TMX];
+#pragma unroll
+  for (int t = 0; t < TMX; ++t) {
+    int m = t * 16 + l16;
+    m = m < g.M ? m : g.M - 1;
+    const uint32_t pm = ((uint32_t)m >> 1) & 7u;
+    x_lo_piece[t] = ((uint32_t)lg ^ pm) << 4;
+    x_hi_piece[t] = ((uint32_t)(lg + 4) ^ pm) << 4;
+  }
   int slot = 0;  // PW: index of the pair among this wavefront's
 
   v4f acc[RG][TMX];
@@ -580,8 +589,8 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
                        : 1.f;
         } else if (XLDS) {
           const uint32_t at = lds_xrow[t] + (uint32_t)(kb + b - kb_lo) * 128u;
-          const u32x4 lo = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + x_lo_piece);
-          const u32x4 hi = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + x_hi_piece);
+          const u32x4 lo = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + x_lo_piece[t]);
+          const u32x4 hi = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(at + x_hi_piece[t]);
           xf[t] = join(lo, hi);
           xsc[t] = (MODE == kModeBlock)
                        ? *reinterpret_cast<const __attribute__((address_space(3))) float*>(lds_xsrow[t] + (uint32_t)(kb + b - kb_lo) * 4u)
@@ -668,17 +677,21 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
     // lane holds m = l16, n = n0 + r*16 + 4*lg + [0,4); bf16 results of the block-scaled product take a short path
     // of their own (see finish_chunk)
     const bool plain = MODE == kModeBlock && g.c_dtype == FG_BF16;
-    uint16_t* const c_row = reinterpret_cast<uint16_t*>(g.C) + (int64_t)l16 * g.ldc + n0;
 #pragma unroll
-    for (int r = 0; r < RG; ++r)
+    for (int t = 0; t < TMX; ++t) {
+      const int m = t * 16 + l16;
+      uint16_t* const c_row = reinterpret_cast<uint16_t*>(g.C) + (int64_t)m * g.ldc + n0;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int nn = r * 16 + lg * 4 + i;
-        if (l16 < g.M && nn < rows_valid) {
-          if (plain) c_row[nn] = float_to_bf16_bits(acc[r][0][i]);
-          else store_output<MODE>(g, l16, n0 + nn, acc[r][0][i]);
+      for (int r = 0; r < RG; ++r)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int nn = r * 16 + lg * 4 + i;
+          if (m < g.M && nn < rows_valid) {
+            if (plain) c_row[nn] = float_to_bf16_bits(acc[r][t][i]);
+            else store_output<MODE>(g, m, n0 + nn, acc[r][t][i]);
+          }
         }
-      }
+    }
     return;
   }
   // a wavefront's sums (16*TMX x 16*RG floats) go into its own slab, which only it has used: no barrier before them
@@ -822,10 +835,19 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   // K = 512: 6.5 -> 6.1 us; N = 28672, K = 4096: 26.5 -> 25 us; N = 16384, K = 2048 (four groups per unit): no gain.
   // With more than 16 pairs of K-blocks the walk of a single wavefront gets long and the shared chunks are as fast
   // (N = 32768, K = 8192: 51 us shared, 53-56 us here), so this form stops at K = 4096.
-  p.own = p.tmx == 1 && KB >= 2 && KB <= 32 && ceil_div(N, 16) * entries >= 5 * (int64_t)cu_count() &&
-          decode_lds_bytes(4, 4, M, KB) <= kDecodeLdsLimit / 2;
+  // Up to 32 rows take the same form, with two 16-row images of the activations: against the 32-row chunks with the
+  // activations in the register ring and the four-stage tile kernel, us at M = 17 / 24 / 32, before -> after:
+  // N = 24576, K = 1536: 15.1 / 13.8 / 13.7 -> 10.5 / 11.3 / 12.3 (16 rows: 10.1); N = 49152, K = 1024: 20.4 / 21.3 / 22.6 ->
+  // 12.5 / 13.3 / 17.4; N = 32768, K = 512: 8.4 / 8.5 / 8.7 -> 7.0 / 7.6 / 8.4.
+  // Where two blocks of four wavefronts do not fit a compute unit but one of eight does, eight share the activations:
+  // N = 20480, K = 3072, M = 24 / 32: 23.2 / 21.3 -> 15.5 / 16.5; N = 28672, K = 4096, M = 16 / 17 / 24: 28.5 / 32.7 / 33.4 ->
+  // 27.4 / 26.6 / 27.3; N = 32768, K = 2048, M = 32: 20.8 -> 15.6.
+  const bool own_shape = p.tmx <= 2 && KB >= 2 && KB <= 32 && ceil_div(N, 16) * entries >= 5 * (int64_t)cu_count();
+  const int own_waves = !own_shape ? 0 : decode_lds_bytes(4, 4, M, KB) <= kDecodeLdsLimit / 2 ? 4
+                        : decode_lds_bytes(4, 8, M, KB) <= kDecodeLdsLimit ? 8 : 0;
+  p.own = own_waves != 0;
   if (p.own) {
-    p.staged = true; p.xlds = true; p.ring = false; p.q = 4; p.rg = 1; p.waves = 4; splits = 1; kpw = (KB + 1) / 2;
+    p.staged = true; p.xlds = true; p.ring = false; p.q = 4; p.rg = 1; p.waves = own_waves; splits = 1; kpw = (KB + 1) / 2;
     p.n_chunks = (int)ceil_div(N, 16);
   }
   p.kpw = (int)kpw;
@@ -875,7 +897,9 @@ int launch_small_m(const GemmArgs& g, int mode, const SmallMPlan& plan, void* wo
       FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm (small M): row strides of %lld / %lld bytes are beyond the kernel's 32-bit offsets",
               (long long)g.ldx, (long long)g.ldw);
     if (g.batch > 65535) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm (small M): at most 65535 batch entries per launch, got %d", g.batch);
-    if (plan.own) return launch_transpose<1, 4, 1, 4, true, true>(sa, mode, stream);
+    if (plan.own && plan.waves == 8)
+      return plan.tmx == 2 ? launch_transpose<2, 4, 1, 8, true, true>(sa, mode, stream) : launch_transpose<1, 4, 1, 8, true, true>(sa, mode, stream);
+    if (plan.own) return plan.tmx == 2 ? launch_transpose<2, 4, 1, 4, true, true>(sa, mode, stream) : launch_transpose<1, 4, 1, 4, true, true>(sa, mode, stream);
     if (plan.xlds && plan.ring) {
       switch (plan.q) {
         case 1: return launch_transpose<1, 1, 1, 8, true, false, true>(sa, mode, stream);

@@ -40,7 +40,7 @@ def _exact(a, b, sa, sb):
                                    (129, 264, 128), (700, 8, 384),
                                    # up to 32 rows: the weight-streaming kernels (K split over blocks for the first)
                                    (1, 4096, 4096), (8, 2112, 7168), (16, 7168, 2304), (32, 1024, 8192), (5, 24592, 384),
-                                   (12, 32768, 512), (20, 520, 1024),
+                                   (12, 32768, 512), (20, 520, 1024), (24, 32768, 512), (32, 24580, 1536),
                                    # 33..64 rows: the kernel with the activations of a K range in LDS
                                    (33, 2112, 7168), (64, 4096, 4096), (48, 24576, 1536), (40, 264, 512),
                                    # K that is not a multiple of 128 above 128 rows
