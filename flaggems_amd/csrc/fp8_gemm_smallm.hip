@@ -842,7 +842,15 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   // Where two blocks of four wavefronts do not fit a compute unit but one of eight does, eight share the activations:
   // N = 20480, K = 3072, M = 24 / 32: 23.2 / 21.3 -> 15.5 / 16.5; N = 28672, K = 4096, M = 16 / 17 / 24: 28.5 / 32.7 / 33.4 ->
   // 27.4 / 26.6 / 27.3; N = 32768, K = 2048, M = 32: 20.8 -> 15.6.
-  const bool own_shape = p.tmx <= 2 && KB >= 2 && KB <= 32 && ceil_div(N, 16) * entries >= 5 * (int64_t)cu_count();
+  // With 17 to 32 rows the alternatives are weaker and four groups per compute unit suffice while K is short (N = 16384,
+  // K = 1024, M = 17 / 24 / 32: 10.9 / 10.8 / 10.7 -> 7.3 / 7.5 / 8.2 us; N = 18432: 11.2 / 11.1 / 10.8 -> 8.2 / 8.7 / 9.3; K = 2048:
+  // 11.8 / 12.0 / 12.6 -> 11.2 / 11.6 / 12.0; three groups, N = 12288, K = 1536: 9.3 -> 9.4, and N = 14336, K = 4096: 17.8 -> 19.7).
+  // Up to 16 rows, K <= 2048: from the first row past 64 per compute unit on, where the shared chunks need a second round
+  // of blocks (N = 18432, K = 1024, M = 1 / 16: 8.0 / 9.1 -> 7.1 / 7.9 us; N = 17408, K = 1536: 9.2 / 10.3 -> 8.7 / 9.6; at exactly
+  // 64 rows, N = 16384, K = 2048: 8.7 -> 9.9, so not there).
+  const int64_t groups = ceil_div(N, 16) * entries, cus = cu_count();
+  const bool enough = KB > 16 ? groups >= 5 * cus : (p.tmx == 2 ? groups >= 4 * cus : groups > 4 * cus);
+  const bool own_shape = p.tmx <= 2 && KB >= 2 && KB <= 32 && enough;
   const int own_waves = !own_shape ? 0 : decode_lds_bytes(4, 4, M, KB) <= kDecodeLdsLimit / 2 ? 4
                         : decode_lds_bytes(4, 8, M, KB) <= kDecodeLdsLimit ? 8 : 0;
   p.own = own_waves != 0;

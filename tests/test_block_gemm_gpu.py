@@ -182,7 +182,8 @@ def test_33_to_128_rows(M, N, K, dtype):
                                    (16, 32768, 512), (5, 24580, 384), (2, 20480, 256), (16, 28672, 4096),
                                    (16, 4612, 7296), (13, 7168, 16512), (16, 8192, 8192), (10, 5000, 12416), (8, 7168, 16384),
                                    (17, 24576, 1536), (32, 32768, 512), (24, 20490, 640), (31, 49152, 1024), (32, 24584, 1536),
-                                   (19, 20480, 256), (32, 28672, 4096), (24, 20488, 3072), (32, 32768, 2048)])
+                                   (19, 20480, 256), (32, 28672, 4096), (24, 20488, 3072), (32, 32768, 2048),
+                                   (24, 16384, 1024), (17, 16400, 2048), (16, 18432, 1024), (3, 17416, 1536)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_up_to_32_rows_uneven_chunks(M, N, K, dtype):
     """M <= 32 takes the kernel that deals the weight rows out evenly over the compute units: chunks that differ by a
@@ -192,9 +193,9 @@ def test_up_to_32_rows_uneven_chunks(M, N, K, dtype):
     (16, 32768, 512) on: K of 2, 3 and 4 K-blocks, N that ends inside a 16-row group, activations that eight wavefronts share),
     activations too large for LDS as a whole and copied pair by pair into two slots per wavefront (M = 12 with
     K = 16384 and the five shapes from (16, 4612, 7296) on: an odd number of K-blocks, chunks that begin anywhere), wide
-    weights with 17 to 32 rows (the block shares two 16-row images of the activations; the last nine shapes, of which
-    (32, 28672, 4096) is too long in K for that and stays on the kernels for 32 rows and the last two take blocks of eight
-    wavefronts), column-major activation
+    weights with 17 to 32 rows (the block shares two 16-row images of the activations; the shapes from (17, 24576, 1536) on, of which
+    (32, 28672, 4096) is too long in K for that and stays on the kernels for 32 rows, two take blocks of eight
+    wavefronts, and the last four have just over four 16-row groups per compute unit), column-major activation
     scales; against the oracle and bit-identical on reruns."""
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=17)
     want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
