@@ -744,9 +744,9 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
     // measured -- M = 128: N = 2112, K = 7168: 24.0 against 19.9 us; 7168 x 2304: 16.4 against 14.6; 4096 x 4096: 18.4
     // against 16.8 -- and only serves batches now)
     const bool mid_takes = mid.use && mid.tmx == 4;
-    if (a.M > 16 && a.M <= 32) {
+    if (a.M > 16 && a.M <= 48) {
       // very wide weights against short K: a wavefront per 16 weight rows with the block's activations in LDS
-      // (N = 24576, K = 1536, M = 17 / 24 / 32: 15.1 / 13.8 / 13.7 us on the kernels below)
+      // (N = 24576, K = 1536, M = 17 / 24 / 32 / 40: 15.1 / 13.8 / 13.7 / 14.2 us on the kernels below)
       const SmallMPlan sp = plan_small_m(a.M, a.N, a.K);
       if (sp.use && sp.own) return launch_small_m(a, MODE, sp, workspace, workspace_bytes, stream);
     }

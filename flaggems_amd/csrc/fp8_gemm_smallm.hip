@@ -301,7 +301,7 @@ __device__ __forceinline__ void dma_to_lds_4(uint32_t byte_off, const void* base
 // the activation fragments travel in the register ring next to the weights.
 template <int TMX, int Q, int DEPTH, int WAVES, int MODE, bool XLDS, bool OWN = false, bool RING = false>
 __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArgs a) {
-  static_assert(!XLDS || TMX == 1 || (OWN && TMX == 2), "activations in LDS: M <= 16, or M <= 32 where the block shares them");
+  static_assert(!XLDS || TMX == 1 || OWN, "activations in LDS: M <= 16, or more rows where the block shares them");
   static_assert(!OWN || XLDS, "wavefronts with chunks of their own share the activations through LDS");
   static_assert(!RING || (XLDS && !OWN && DEPTH == 1), "the two-slot form belongs to the per-wavefront copies with one pair in the ring");
   constexpr int RG = (Q + 3) / 4;
@@ -849,8 +849,14 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   // of blocks (N = 18432, K = 1024, M = 1 / 16: 8.0 / 9.1 -> 7.1 / 7.9 us; N = 17408, K = 1536: 9.2 / 10.3 -> 8.7 / 9.6; at exactly
   // 64 rows, N = 16384, K = 2048: 8.7 -> 9.9, so not there).
   const int64_t groups = ceil_div(N, 16) * entries, cus = cu_count();
-  const bool enough = KB > 16 ? groups >= 5 * cus : (p.tmx == 2 ? groups >= 4 * cus : groups > 4 * cus);
-  const bool own_shape = p.tmx <= 2 && KB >= 2 && KB <= 32 && enough;
+  const bool enough = KB > 16 ? groups >= 5 * cus : (p.tmx >= 2 ? groups >= 4 * cus : groups > 4 * cus);
+  // 33 to 48 rows (four 16-row images): against the staged-activation and tile kernels it wins from twelve K-blocks on, and
+  // from eight against weights of up to five groups per compute unit at up to 40 rows; us at M = 33 / 40 / 48, before -> after:
+  // N = 49152, K = 2048: 38.8 / 38.6 / 39.0 -> 29.2 / 29.9 / 32.1; N = 24576, K = 1536: 15.0 / 14.2 / 14.2 -> 12.8 / 13.2 / 14.1;
+  // N = 16384, K = 1024: 10.9 / 10.9 -> 8.9 / 9.4.  Not with fewer K-blocks or more rows (N = 32768, K = 512: 8.1 -> 8.9;
+  // N = 49152, K = 1024, M = 48: 19.0 -> 20.5; 64 rows: 14.4 -> 15.9 and 10.8 -> 12.1 on the second and third shape above).
+  const bool rows_ok = p.tmx <= 2 || (p.tmx == 4 && ((KB >= 12 && M <= 48) || (KB >= 8 && groups <= 5 * cus && M <= 40)));
+  const bool own_shape = rows_ok && KB >= 2 && KB <= 32 && enough;
   const int own_waves = !own_shape ? 0 : decode_lds_bytes(4, 4, M, KB) <= kDecodeLdsLimit / 2 ? 4
                         : decode_lds_bytes(4, 8, M, KB) <= kDecodeLdsLimit ? 8 : 0;
   p.own = own_waves != 0;
@@ -905,6 +911,8 @@ int launch_small_m(const GemmArgs& g, int mode, const SmallMPlan& plan, void* wo
       FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm (small M): row strides of %lld / %lld bytes are beyond the kernel's 32-bit offsets",
               (long long)g.ldx, (long long)g.ldw);
     if (g.batch > 65535) FG_FAIL(FG_ERR_UNSUPPORTED, "fp8 gemm (small M): at most 65535 batch entries per launch, got %d", g.batch);
+    if (plan.own && plan.tmx == 4)
+      return plan.waves == 8 ? launch_transpose<4, 4, 1, 8, true, true>(sa, mode, stream) : launch_transpose<4, 4, 1, 4, true, true>(sa, mode, stream);
     if (plan.own && plan.waves == 8)
       return plan.tmx == 2 ? launch_transpose<2, 4, 1, 8, true, true>(sa, mode, stream) : launch_transpose<1, 4, 1, 8, true, true>(sa, mode, stream);
     if (plan.own) return plan.tmx == 2 ? launch_transpose<2, 4, 1, 4, true, true>(sa, mode, stream) : launch_transpose<1, 4, 1, 4, true, true>(sa, mode, stream);
