@@ -44,12 +44,12 @@ def test_einsum_large_batch_and_per_head_bits():
 
 
 @pytest.mark.parametrize("M", [1, 5, 17, 32, 33, 48, 64, 100, 128])
-@pytest.mark.parametrize("B,N,K", [(3, 384, 640), (12, 1024, 2048), (40, 128, 512), (2, 7168, 2304), (10, 1024, 7168)])
+@pytest.mark.parametrize("B,N,K", [(3, 384, 640), (12, 1024, 2048), (40, 128, 512), (2, 7168, 2304), (10, 1024, 7168), (20, 1024, 1024)])
 def test_batches_of_few_rows_go_out_in_one_launch(M, B, N, K):
     """Up to 128 rows per matrix the weight-streaming kernels and the four-stage tile kernel take the whole batch in one
     launch (the entry in the grid, every entry with its own partial sums and counters); strided operands and outputs,
     and a second call on the same workspace.  The last shape has more than 64 MB of weights, which moves 33..64 rows to
-    the tile kernel as well."""
+    the tile kernel as well; the one after it has enough 16-row groups in all for a wavefront per group (up to 32 rows)."""
     xq, xs, yq, ys = O.make_fp8_einsum_inputs(M, B, K, N, seed=M + B)
     want = O.fp8_block_einsum_ref(xq, xs, yq, ys, [128, 128]).permute(1, 0, 2)       # [B, M, N]
     x, x_s = xq.permute(1, 0, 2).to(DEV), xs.permute(1, 0, 2).to(DEV)                # strided views, as fp8_einsum passes them
