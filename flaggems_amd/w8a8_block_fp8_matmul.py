@@ -116,7 +116,7 @@ def w8a8_block_fp8_matmul(
     as2d = As if As.dim() == 2 else As.reshape(M, As.shape[-1])
     if (block_n, block_k) != (128, 128) and block_n % 128 == 0 and block_k % 128 == 0:
         as2d, Bs, block_n, block_k = _scales_at_128(as2d, Bs, N, K, block_n, block_k)
-    # (any other block size goes to the library as it is: a plain kernel serves it, see csrc/fp8_gemm_anyblock.hip)
+    # (any other block size goes to the library as it is: csrc/fp8_gemm_anyblock.hip serves it)
     _launch_block_gemm(a2d, B, as2d, Bs, C if C.dim() == 2 else C.view(M, N), block_n, block_k, pow2)
     return C
 

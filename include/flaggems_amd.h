@@ -307,9 +307,11 @@ int fg_act_quant_bf16(const void* x, void* y, float* s, int64_t rows, int64_t co
  * [ceil(N/block_n), ceil(K/block_k)] with both strides given.  C: [M, N] row stride ldc,
  * c_dtype in {FG_BF16, FG_F16, FG_F32}.  Products are accumulated in fp32 per K-block, scaled,
  * and accumulated in fp32 across K-blocks; the result is rounded once to c_dtype.
- * block_n == block_k == 128 takes the matrix-instruction kernels; every other positive block size takes a plain fp32
- * tile kernel (correct, about fifty times slower; callers with multiples of 128 do better to write the scales out per
- * 128 x 128 block and call with 128, which gives the same result).
+ * block_n == block_k == 128 takes the kernels built around the 16x16x128 matrix instruction.  Other block sizes with
+ * block_k a multiple of 32 and block_n of 16 (64 x 64, 128 x 64, 32 x 96 ...; K a multiple of 16, 16-byte aligned rows)
+ * take a tile kernel on the 16x16x32 instruction, about four times slower; everything else a plain fp32 tile kernel,
+ * about fifty times slower.  (Callers with multiples of 128 do better to write the scales out per 128 x 128 block and
+ * call with 128, which gives the same result.)
  * `workspace` holds split-K partial sums and, for long GEMMs, a transposed copy of As.
  * fg_block_fp8_gemm_workspace_bytes(M, N, K) says how much the kernels can use for the shape (0: none).
  * For M <= 32 that much is required when it is not 0 (FG_ERR_WORKSPACE otherwise); for larger M it is

@@ -434,14 +434,15 @@ def test_scale_blocks_that_are_multiples_of_128(M, N, K, block_size):
 
 
 @pytest.mark.parametrize("block_size", [[64, 64], [64, 128], [128, 64], [32, 96], [100, 60], [128, 200], [1, 7], [4096, 32]])
-@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (7, 640, 1000), (100, 1000, 1536), (300, 2112, 4096), (2100, 330, 777)])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (7, 640, 1000), (100, 1000, 1536), (300, 2112, 4096), (2100, 330, 777), (130, 200, 1008)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_scale_blocks_of_any_size(M, N, K, block_size, dtype):
     """block_size that is no multiple of 128 (64-wide groups, blocks that divide nothing, a block wider than N, a
-    K-group of 7): the plain kernel, against the oracle evaluated with the same block_size; M, N and K that end inside
-    its 64 x 64 tiles and 32-element rounds."""
+    K-group of 7): the tile kernel on the 16x16x32 matrix instruction where block_k is a multiple of 32, block_n of 16
+    and K of 16, the plain kernel otherwise, against the oracle evaluated with the same block_size; M, N and K that
+    end inside the tiles and K rounds of both."""
     block_n, block_k = block_size
-    if dtype == torch.float32 and (M, N, K) not in ((7, 640, 1000), (2100, 330, 777)):
+    if dtype == torch.float32 and (M, N, K) not in ((7, 640, 1000), (2100, 330, 777), (130, 200, 1008)):
         pytest.skip("fp32 output on two shapes")
     g = torch.Generator().manual_seed(M + N + K + block_n + block_k)
     A = torch.randn(M, K, generator=g).to(FP8)
