@@ -662,6 +662,15 @@ struct PipePlan {
 constexpr int kPipeStages = 4;
 // entries: equal problems launched together (blockIdx.y = entry): their tiles fill the compute units together, and
 // workspace_bytes is what all of them need.
+// Whether the staged-activation kernel's blocks run in two or more rounds with the last one under nine tenths full.
+bool mid_m_partial_round(const MidMPlan& mid, int cus) {
+  if (!mid.use) return false;
+  const int64_t blocks = ceil_div((int64_t)mid.n_chunks, (int64_t)mid.waves) * mid.splits;
+  const int64_t slots = (int64_t)cus * (mid.waves == 8 ? 1 : 2);  // four-wavefront blocks take half of LDS at most
+  const int64_t rounds = ceil_div(blocks, slots);
+  return rounds >= 2 && blocks * 10 < rounds * slots * 9;
+}
+
 PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs, int64_t entries = 1) {
   PipePlan p = {false, 1, 0, 0};
   if (entries < 1) entries = 1;
@@ -688,7 +697,14 @@ PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs, int64_t entri
   // 16.2 -> 14.6 us; a batch of 16 x [1024, 7168], 128 tiles in two ranges, 48 rows: 41 -> 34 us; but N = 32768, K = 512,
   // four K-blocks: 8.5 -> 9.8 us; N = 4096, K = 14336 in eight ranges: 23 -> 25 us; N = 4608, K = 7168 in seven: 17 -> 20 us;
   // a batch of 8 x [1024, 4096] in four: 16 -> 20 us)
-  if (M > 32 && M <= 64 && !((p.splits == 1 && p.kb_per_split >= 8) || (p.splits == 2 && p.kb_per_split >= 16))) return p;
+  // -- or while that kernel, one block of eight wavefronts per compute unit at these sizes, would run a second round
+  // of blocks that fills under nine tenths of the compute units (M = 48: N = 10240, K = 8192, 320 blocks: 38 -> 26 us;
+  // N = 7168, K = 8192, 280 blocks: 32.5 -> 23 us; N = 5120, K = 13824: 36 -> 25 us; N = 9216, K = 9216: 39 -> 27 us;
+  // N = 8192, K = 28672, 896 blocks: 75 -> 58 us; with full rounds it keeps the shape: N = 8192, K = 16384, 512 blocks: 39
+  // against 43 us here)
+  if (M > 32 && M <= 64 && !((p.splits == 1 && p.kb_per_split >= 8) || (p.splits == 2 && p.kb_per_split >= 16)) &&
+      !(entries == 1 && p.kb_per_split >= 16 && mid_m_partial_round(plan_mid_m(M, N, K), cus)))
+    return p;
   // (two ranges of eight: N = 16384, K = 2048: 14 -> 17 us; of sixteen: N = 14336, K = 4096: 29 -> 22 us; N = 12288, K = 4096: 28 -> 20 us)
   // 17..32 rows of a lone matrix: the decode kernels, except unsplit against very wide weights (M = 32: N = 24576,
   // K = 1536: 18.3 -> 15.1 us; N = 28672, K = 4096: 34.9 -> 30.9 us; N = 32768, K = 1024: 15.8 -> 12.7 us), and up to 24
