@@ -702,14 +702,17 @@ PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs, int64_t entri
   // N = 7168, K = 8192, 280 blocks: 32.5 -> 23 us; N = 5120, K = 13824: 36 -> 25 us; N = 9216, K = 9216: 39 -> 27 us;
   // N = 8192, K = 28672, 896 blocks: 75 -> 58 us; with full rounds it keeps the shape: N = 8192, K = 16384, 512 blocks: 39
   // against 43 us here)
-  if (M > 32 && M <= 64 && !((p.splits == 1 && p.kb_per_split >= 8) || (p.splits == 2 && p.kb_per_split >= 16)) &&
+  if (M > 32 && M <= 64 && !((p.splits == 1 && tiles * 2 > cus && p.kb_per_split >= 8) || (p.splits == 2 && p.kb_per_split >= 16)) &&
       !(entries == 1 && p.kb_per_split >= 16 && mid_m_partial_round(plan_mid_m(M, N, K), cus)))
     return p;
   // (two ranges of eight: N = 16384, K = 2048: 14 -> 17 us; of sixteen: N = 14336, K = 4096: 29 -> 22 us; N = 12288, K = 4096: 28 -> 20 us)
   // 17..32 rows of a lone matrix: the decode kernels, except unsplit against very wide weights (M = 32: N = 24576,
   // K = 1536: 18.3 -> 15.1 us; N = 28672, K = 4096: 34.9 -> 30.9 us; N = 32768, K = 1024: 15.8 -> 12.7 us), and up to 24
   // rows only while K is short (M = 24, N = 28672, K = 4096: 34.0 -> 36.3 us, so not there; N = 20480, K = 3072: 24.8 -> 23.3 us)
-  if (M <= 32 && !(p.splits == 1 && p.kb_per_split >= 8 && (M > 24 || KB <= 24))) return p;
+  // (one range because the tiles fill the compute units, not because K is too short to split: N = 8192, K = 1024, 64 tiles,
+  // 10.5 us here whatever M; M = 17 ... 32: 5.2-5.7 us on the decode kernels, 33 ... 64: 7.5-7.9 us on the staged-activation
+  // kernel; N = 16384, K = 1024, 128 tiles, M = 48 / 64: 10.9 / 11.0 -> 8.1 / 8.5 us)
+  if (M <= 32 && !(p.splits == 1 && tiles * 2 > cus && p.kb_per_split >= 8 && (M > 24 || KB <= 24))) return p;
   p.workspace_bytes = p.splits > 1 ? FG_WORKSPACE_COUNTER_BYTES + (size_t)tiles * p.splits * kSplitTile * kSplitTile * sizeof(float) : 0;
   p.use = true;
   return p;

@@ -767,8 +767,9 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   // long as the compute unit with most bytes to fetch.  Narrow weights get chunks of at least `rows_min` rows and K
   // split over blocks below; weights with more than 64 rows per compute unit get whole rounds of blocks.
   const int64_t B = std::max<int64_t>(1, cu_count() / entries);
-  auto deal_rows = [&](int64_t rows_min) {
-    chunks = N <= 64 * B ? std::min<int64_t>(B, ceil_div(N, rows_min)) : ceil_div(N, 64 * B) * B;
+  auto deal_rows = [&](int64_t rows_min, int64_t blocks = 0) {
+    if (blocks < 1) blocks = B;
+    chunks = N <= 64 * blocks ? std::min<int64_t>(blocks, ceil_div(N, rows_min)) : ceil_div(N, 64 * blocks) * blocks;
     const int64_t rows_max = ceil_div(N, chunks);
     p.q = (int)ceil_div(rows_max, 4);
     p.rg = p.q <= 4 ? 1 : (p.q <= 8 ? 2 : 4);
@@ -799,22 +800,44 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
     static const int kQ[] = {1, 2, 3, 4, 6, 8, 12, 16};
     auto round_q = [&](int need) { int q = 16; for (int i = 7; i >= 0; --i) if (kQ[i] >= need) q = kQ[i]; return q; };
     int q = round_q(p.q);
-    p.xlds = p.tmx == 1 && kpw >= (M > 8 ? 2 : 3) && decode_lds_bytes_per_wave(q, p.waves, M, std::min<int64_t>(pairs, kpw * p.waves)) <= kDecodeLdsLimit;
-    // Too large for LDS as a whole: two slots per wavefront, pair i + 1 copied while pair i is multiplied.  Only for
-    // chunks with at least as many rows as there are activation rows (N = 7168, K = 16384, M = 16: 25.9 -> 22.9 us;
-    // N = 4608, K = 7168: 11.0 -> 10.0; N = K = 8192: 17.9 -> 16.8; narrower chunks move more activation than weight
-    // bytes and do better with fewer, taller chunks below: N = 1024, K = 8192, M = 16: 7.9 us there, 9.8 us here).
-    // Where everything fits, the copies up front win: the same loop on N = 2112, K = 7168 takes 7.4 instead of 5.7 us.
-    p.ring = !p.xlds && p.tmx == 1 && kpw >= (M > 8 ? 2 : 3) && ceil_div(N, chunks) >= M &&
-             decode_lds_bytes_per_wave(q, p.waves, M, 2 * p.waves) <= kDecodeLdsLimit;
-    if (p.ring) p.xlds = true;
+    auto place_activations = [&]() {
+      p.xlds = p.tmx == 1 && kpw >= (M > 8 ? 2 : 3) && decode_lds_bytes_per_wave(q, p.waves, M, std::min<int64_t>(pairs, kpw * p.waves)) <= kDecodeLdsLimit;
+      // Too large for LDS as a whole: two slots per wavefront, pair i + 1 copied while pair i is multiplied.  Only for
+      // chunks with at least as many rows as there are activation rows (N = 7168, K = 16384, M = 16: 25.9 -> 22.9 us;
+      // N = 4608, K = 7168: 11.0 -> 10.0; N = K = 8192: 17.9 -> 16.8; narrower chunks move more activation than weight
+      // bytes and do better with fewer, taller chunks below: N = 1024, K = 8192, M = 16: 7.9 us there, 9.8 us here).
+      // Where everything fits, the copies up front win: the same loop on N = 2112, K = 7168 takes 7.4 instead of 5.7 us.
+      p.ring = !p.xlds && p.tmx == 1 && kpw >= (M > 8 ? 2 : 3) && ceil_div(N, chunks) >= M &&
+               decode_lds_bytes_per_wave(q, p.waves, M, 2 * p.waves) <= kDecodeLdsLimit;
+      if (p.ring) p.xlds = true;
+    };
+    place_activations();
     if (!p.xlds && p.tmx == 1 && M > 4 && N <= 64 * B) {
       // every block fetches all M activation rows of its K range per pair of K-blocks: chunks of fewer rows than
       // that move more activation than weight bytes (N = 2048, K = 1024, M = 16: 256 chunks of 8 rows 3.8 us,
-      // 128 of 16 rows 3.5 us; N = 1024, K = 8192: 9.1 against 7.9 us)
+      // 128 of 16 rows 3.5 us; N = 1024, K = 8192: 9.1 against 7.9 us); the K ranges of the taller chunks may fit LDS
+      // (N = 1024, K = 8192, M = 16, 64 chunks in two ranges: 7.9 -> 6.9 us; N = 1280: 8.2 -> 7.4 us)
       deal_rows((M + 3) / 4 * 4);
       split_k();
       q = round_q(p.q);
+      place_activations();
+    }
+    // Long K against narrow weights, 128 KB of activations or more: every block reads the activations of its K range,
+    // which at one range is as much as its weight rows or more.  Half the blocks with twice the rows (32 at most: taller
+    // chunks take the slower four-group form) on half of K each halve the activation bytes per block, and the half
+    // ranges may fit LDS.  us at M = 8 / 12 / 16, one range -> two: N = 2304, K = 16384: 15.6 / 14.7 / 17.6 -> 11.0 / 12.4 / 12.5;
+    // N = 3584, K = 18944: 17.7 / 20.9 / 19.8 -> 16.0 / 16.7 / 16.7; M = 12 / 16: N = 4096, K = 14336: 16.4 / 16.9 -> 14.9 / 15.0;
+    // N = 4096, K = 11008: 13.9 / 14.4 -> 12.7 / 12.9; M = 16: N = 3072, K = 8192: 10.3 -> 9.5.  Not below 128 KB (M = 8,
+    // K = 14336: 12.4 -> 13.9; M = 12, N = 3072, K = 8192: 7.7 -> 9.5), not where the activations fit LDS at one range
+    // (N = 2112, K = 7168, M = 16: 7.6 -> 8.0), not for taller chunks (N = 7168, K = 16384: 22.9 -> 27.5; N = 5120, K = 13824:
+    // 16.7 -> 20.5).
+    if (p.tmx == 1 && entries == 1 && M * KB >= 1024 && (!p.xlds || p.ring) && N <= 32 * (B / 2) && max_splits >= 2 && pairs >= 2 * 8) {
+      deal_rows((M + 3) / 4 * 4, B / 2);
+      p.n_chunks = (int)chunks;
+      splits = 2;
+      kpw = ceil_div(pairs, splits * p.waves);
+      q = round_q(p.q);
+      place_activations();
     }
     p.q = p.tmx == 1 ? q : 4 * p.rg;
   } else {

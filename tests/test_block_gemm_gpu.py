@@ -157,7 +157,7 @@ def test_129_to_512_tiles_of_128_rows(M, N, K, dtype):
 @pytest.mark.parametrize("M,N,K", [(33, 100, 384), (64, 2112, 7168), (50, 7168, 16384), (40, 24584, 1536), (64, 4104, 2304),
                                    (33, 49152, 2048), (48, 20490, 1536), (37, 16384, 1024), (33, 20480, 3072),
                                    (65, 520, 1024), (100, 2112, 4096), (128, 4096, 4096), (128, 7000, 2304),
-                                   (48, 8330, 6144), (64, 6650, 8192)])
+                                   (48, 8330, 6144), (64, 6650, 8192), (40, 8200, 1024), (64, 16384, 1152)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_33_to_128_rows(M, N, K, dtype):
     """33 <= M <= 64 (and 65 <= M <= 128 with small weights) takes the kernel that keeps the activations in LDS and
@@ -186,7 +186,9 @@ def test_33_to_128_rows(M, N, K, dtype):
                                    (16, 4612, 7296), (13, 7168, 16512), (16, 8192, 8192), (10, 5000, 12416), (8, 7168, 16384),
                                    (17, 24576, 1536), (32, 32768, 512), (24, 20490, 640), (31, 49152, 1024), (32, 24584, 1536),
                                    (19, 20480, 256), (32, 28672, 4096), (24, 20488, 3072), (32, 32768, 2048),
-                                   (24, 16384, 1024), (17, 16400, 2048), (16, 18432, 1024), (3, 17416, 1536)])
+                                   (24, 16384, 1024), (17, 16400, 2048), (16, 18432, 1024), (3, 17416, 1536),
+                                   (16, 2304, 16384), (9, 3590, 18944), (12, 4096, 11008), (16, 1280, 8192), (16, 1000, 8192),
+                                   (8, 2050, 16384), (24, 8192, 1024), (17, 2050, 1152)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_up_to_32_rows_uneven_chunks(M, N, K, dtype):
     """M <= 32 takes the kernel that deals the weight rows out evenly over the compute units: chunks that differ by a
@@ -198,8 +200,10 @@ def test_up_to_32_rows_uneven_chunks(M, N, K, dtype):
     K = 16384 and the five shapes from (16, 4612, 7296) on: an odd number of K-blocks, chunks that begin anywhere), wide
     weights with 17 to 32 rows (the block shares two 16-row images of the activations; the shapes from (17, 24576, 1536) on, of which
     (32, 28672, 4096) is too long in K for that and stays on the kernels for 32 rows, two take blocks of eight
-    wavefronts, and the last four have just over four 16-row groups per compute unit), column-major activation
-    scales; against the oracle and bit-identical on reruns."""
+    wavefronts, and the four up to (3, 17416, 1536) have just over four 16-row groups per compute unit), narrow weights
+    with 128 KB of activations or more (half the blocks on half of K each, the half ranges in LDS or in the two slots;
+    the six shapes from (16, 2304, 16384) on), 17 to 32 rows against short K and few tiles (the last two), column-major
+    activation scales; against the oracle and bit-identical on reruns."""
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=17)
     want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
     args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
