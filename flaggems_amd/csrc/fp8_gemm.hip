@@ -685,6 +685,15 @@ PipePlan plan_pipe(int64_t M, int64_t N, int64_t K, int64_t xs_rs, int64_t entri
   if (splits > KB / 5) splits = KB / 5;  // at least five K-blocks per block: a block starts with a full load latency
   if (splits > 8) splits = 8;            // the wavefront that finishes a tile reads the splits one after another
   if (splits < 1) splits = 1;
+  // 129 to 160 tiles unsplit leave over a third of the compute units idle for the whole launch; with long K three ranges
+  // (1.7 to 1.9 rounds of blocks) pay for their partial tiles: M = 128: N = 18432, K = 16384: 110 -> 91 us; K = 8192:
+  // 58 -> 53 us; N = 20480, K = 8192: 58 -> 55 us; M = 256: N = K = 9216: 66 -> 52 us; N = 10240, K = 8192: 53 -> 49 us.  Not with
+  // short K or more tiles (M = 128, N = 24576, K = 4096, 192 tiles: 35 -> 46 us; M = 256, N = 13312, K = 16384, 208 tiles:
+  // 89 -> 116 us), and two, five or seven ranges lose everywhere.  (Equal runs of K-blocks dealt out over the compute
+  // units whatever the tile borders -- every block then writes up to two partial tiles and the blocks of a tile run at
+  // different places in K -- were built and measured on 17 weight shapes x M = 128 / 256 / 512: faster on three of
+  // the 51 cases by 12-16 %, slower by up to 2x where several row tiles share a weight block, 5-45 % slower where K is short.)
+  if (splits == 1 && entries == 1 && M > 64 && tiles * 2 > cus && tiles * 16 <= (int64_t)cus * 10 && KB >= 64) splits = 3;
   p.kb_per_split = (int)ceil_div(KB, splits);
   p.splits = (int)ceil_div(KB, (int64_t)p.kb_per_split);
   // Long K loops stay with the persistent kernel, whose 256 x 256 tiles need half the LDS reads per MFMA (measured
