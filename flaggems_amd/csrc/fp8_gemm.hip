@@ -771,13 +771,16 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
     // (65..128 rows: the 128-row variant of that kernel loses to the four-stage tile kernel below on every shape
     // measured -- M = 128: N = 2112, K = 7168: 24.0 against 19.9 us; 7168 x 2304: 16.4 against 14.6; 4096 x 4096: 18.4
     // against 16.8 -- and only serves batches now)
-    const bool mid_takes = mid.use && mid.tmx == 4;
+    const bool mid_takes = mid.use && mid.tmx <= 4;
     if (a.M > 16 && a.M <= 48) {
       // very wide weights against short K: a wavefront per 16 weight rows with the block's activations in LDS
       // (N = 24576, K = 1536, M = 17 / 24 / 32 / 40: 15.1 / 13.8 / 13.7 / 14.2 us on the kernels below)
       const SmallMPlan sp = plan_small_m(a.M, a.N, a.K);
       if (sp.use && sp.own) return launch_small_m(a, MODE, sp, workspace, workspace_bytes, stream);
     }
+    // 21..32 rows against narrow weights with long K: the staged-activation kernel with 32 rows (its planner holds the rule)
+    if (a.M <= 32 && mid_takes && (mid.splits == 1 || (workspace != nullptr && workspace_bytes >= mid.workspace_bytes && (uintptr_t)workspace % 16 == 0)))
+      return launch_mid_m(a, MODE, mid, workspace, workspace_bytes, stream);
     if (a.M <= 64) {  // the four-stage tile kernel where its planner prefers it to the staged-activation and decode kernels
       const PipePlan pp = plan_pipe(a.M, a.N, a.K, MODE == kModeBlock ? a.xs_rs : 0);
       const bool ws_ok = pp.splits == 1 || (workspace != nullptr && workspace_bytes >= pp.workspace_bytes && (uintptr_t)workspace % 16 == 0);

@@ -41,6 +41,7 @@ def _exact(a, b, sa, sb):
                                    # up to 32 rows: the weight-streaming kernels (K split over blocks for the first)
                                    (1, 4096, 4096), (8, 2112, 7168), (16, 7168, 2304), (32, 1024, 8192), (5, 24592, 384),
                                    (12, 32768, 512), (20, 520, 1024), (24, 32768, 512), (32, 24580, 1536),
+                                   (32, 2112, 7168), (24, 4624, 7168), (16, 2304, 16384),
                                    # 33..64 rows: the kernel with the activations of a K range in LDS
                                    (33, 2112, 7168), (64, 4096, 4096), (48, 24576, 1536), (40, 264, 512),
                                    # K that is not a multiple of 128 above 128 rows
@@ -117,7 +118,8 @@ def test_int8_sums_are_exact_in_bf16_above_128_rows():
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 512, 8192), (4, 2112, 7168), (16, 4096, 4096), (9, 24576, 1536), (32, 768, 2048),
-                                   (33, 512, 8192), (64, 2112, 7168), (16, 4608, 7168)])
+                                   (33, 512, 8192), (64, 2112, 7168), (16, 4608, 7168), (32, 2112, 7168), (16, 2304, 16384),
+                                   (24, 2304, 16384)])
 def test_int8_sums_are_exact_up_to_64_rows(M, N, K):
     """The kernels for few rows split K over wavefronts and blocks: the int32 partial sums are added as integers, so
     the fp32 result is the one rounding of the exact sum, also where the sum needs more than 24 bits."""
@@ -153,7 +155,13 @@ def test_int8_sums_are_exact_up_to_64_rows(M, N, K):
     torch.cuda.synchronize()
     assert torch.equal(c2, c)
     if need:
-        assert call(None, 0) == -3  # FG_ERR_WORKSPACE
+        # 21..32 rows against narrow weights with long K: without a workspace the decode kernels take the shape in one K range
+        falls_back = (M, N, K) == (32, 2112, 7168)
+        c2.zero_()
+        assert call(None, 0) == (0 if falls_back else -3)  # FG_ERR_WORKSPACE
+        if falls_back:
+            torch.cuda.synchronize()
+            assert torch.equal(c2, c)
 
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
