@@ -756,7 +756,7 @@ bool mid_m_preferred(const MidMPlan& mid, int64_t M, int64_t N, int64_t K) {
   // 33..64 rows: always (measured against both alternatives on every DeepSeek-V3 and Llama-3 shape).  65..128 rows:
   // the splits' partial sums cost as much as the weights, which pays only while the weights are small: M = 128,
   // N = 6144, K = 4096: 31 -> 20 us; N = 7168, K = 2304: 19 -> 16 us; but N = 24576, K = 1536: 23 -> 28 us.
-  return mid.use && (mid.tmx == 4 || N * K <= (int64_t)28 << 20);
+  return mid.use && (mid.tmx <= 4 || N * K <= (int64_t)28 << 20);
 }
 
 template <int MODE>
@@ -1063,7 +1063,7 @@ extern "C" int fg_batched_block_fp8_gemm(const void* A, int64_t lda, int64_t a_b
                            (size_t)batch * mid.n_chunks * sizeof(unsigned int) <= FG_WORKSPACE_COUNTER_BYTES);
         // 65..128 rows: measured against the tile kernel on the same batch, b = 128: 8 x [1024, 4096]: 41 -> 26 us,
         // 16 x [1024, 7168]: 67 -> 81 us
-        const bool small_enough = mid.tmx == 4 || (int64_t)batch * N * K <= (int64_t)64 << 20;
+        const bool small_enough = mid.tmx <= 4 || (int64_t)batch * N * K <= (int64_t)64 << 20;
         if (mid_m_preferred(mid, M, N, K) && small_enough && fits) return launch_mid_m(a, kModeBlock, mid, workspace, workspace_bytes, (hipStream_t)stream);
       }
       // 256 x 256 tiles once the batch has one for every compute unit (measured, h = 8, r = 4096, d = 1024, 128-row against
