@@ -298,6 +298,8 @@ MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   // 33..48 rows stage 48: a quarter less LDS per K-block (21 fit), MFMA work and partial sums: 2-8 % faster than with 64 rows
   // on 13 of 14 shapes (M = 40: N = 7168, K = 16384: 40.2 -> 37.0 us; N = 2112, K = 7168: 13.0 -> 12.2; N = 4096, K = 14336: 22.4 -> 21.1;
   // N = 14336, K = 4096: 20.8 -> 21.1)
+  // (80 and 96 rows staged for 65..96 rows do not soften the step to the tile kernel at 65 rows: M = 80, N = 2112, K = 7168:
+  // 19.4 us there, 19.1 here; N = 7168, K = 16384: 40 against 58; N = K = 4096: 16.2 against 15.8; N = 24576, K = 1536: 14.8 against 17.7)
   const int tmx = M <= 32 ? 2 : M <= 48 ? 3 : M <= 64 ? 4 : 8;
   const int64_t kb_max = mid_kb_max(tmx);
   const int64_t min_splits = ceil_div(KB, kb_max);
