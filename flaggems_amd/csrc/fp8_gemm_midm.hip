@@ -324,6 +324,28 @@ MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   }
   while (rg < 4 && ceil_div(N, 16 * rg) > FG_WORKSPACE_COUNTER_BYTES / 4) rg <<= 1;
   if (tmx == 8 && rg > 2) return p;
+  if (tmx <= 4 && entries == 1 && ceil_div(N, 128) > cu_count()) {
+    // Weights too wide for the tile kernel's one round of 128 x 128 tiles run in several rounds of blocks here, and the
+    // wavefront count above says nothing about how full the last round is.  Take the split with the least
+    // rounds x (K-blocks per block + 2, + 4 with K split) instead (2: staging; 4: a block's partial sums, written and read
+    // back, are as many bytes as four K-blocks of its weights; N = 57344, K = 8192: eight ranges fill seven rounds exactly and
+    // take 150 us, four ranges in four rounds 134 us).  M = 64:
+    // N = 49152, K = 2048: two ranges, 768 blocks on 512 places, 40.5 us -> one range, 192 blocks, 29.9 us; N = 37888,
+    // K = 3584: two ranges, 296 blocks on 256 places, 58.4 -> three, 444 blocks, 49.5 us; M = 48: N = 40960, K = 5120: 84.4 -> 67.6 us;
+    // N = 152064, K = 3584: 163.5 -> 147.9 us.
+    const int64_t max_splits = KB / 8 > min_splits ? KB / 8 : min_splits;
+    const int64_t per_kb = mid_stage_bytes(tmx) + mid_rows(tmx) * 4;
+    int64_t best = splits, best_cost = 0;
+    for (int64_t s = min_splits; s <= max_splits; ++s) {
+      const int64_t kb_s = ceil_div(KB, s), s_eff = ceil_div(KB, kb_s);
+      const int64_t waves = kb_s * per_kb > 80 * 1024 ? 8 : 4;
+      const int64_t blocks = ceil_div(ceil_div(N, 16 * rg), waves) * s_eff;
+      const int64_t rounds = ceil_div(blocks, (int64_t)cu_count() * (waves == 8 ? 1 : 2));
+      const int64_t cost = rounds * (kb_s + 2 + (s_eff > 1 ? 4 : 0));
+      if (best_cost == 0 || cost < best_cost) { best = s_eff; best_cost = cost; }
+    }
+    splits = best;
+  }
   const int64_t kbps = ceil_div(KB, splits);
   splits = ceil_div(KB, kbps);
   p.tmx = tmx;
