@@ -802,13 +802,18 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
   }
   {
     const int64_t tiles128 = ceil_div(a.M, 128) * ceil_div(a.N, 128);
-    // 257..512 tiles of 128 x 128 with short K (up to 448 tiles for K up to 8192): at most the 512 workgroups that are
+    // 257..512 tiles of 128 x 128 with K up to 4096: at most the 512 workgroups that are
     // resident at a time, two on each compute unit (560 tiles: M = 1280, N = 7168, K = 2304 went from 36 to 51 us); the persistent kernel has a quarter of the tiles and spends its
     // time filling and draining.  Measured: M = 256, N = 24576, K = 1536: 27.7 -> 23.4 us; M = 768, N = 7168, K = 2304:
-    // 34.8 -> 28.9; N = 6144, K = 4096: 50.0 -> 43.4; M = 1024, N = 7168, K = 2304: 35.3 -> 29.6 (N = K = 8192: 86 -> 89).
+    // 34.8 -> 28.9; N = 6144, K = 4096: 50.0 -> 43.4; M = 1024, N = 7168, K = 2304: 35.3 -> 29.6.
     // The tile count decides, whatever M: M = 2048, N = 3072, K = 2048: 34.0 -> 24.8 us; M = 3072, N = K = 2048: 34.0 -> 24.2;
-    // M = 2048, N = K = 4096: 51.0 -> 45.2; M = 2048, N = 2112, K = 7168: 66.5 -> 63.5.
-    if (direct && a.M > 128 && tiles128 > 256 && ((tiles128 <= 512 && a.KB <= 32) || (tiles128 <= 448 && a.KB <= 64)))
+    // M = 2048, N = K = 4096: 51.0 -> 45.2.
+    // With longer K the persistent kernel, which shares tiles between compute units through the workspace, is ahead: the rule
+    // once reached to K = 8192 for up to 448 tiles, and without that M = 256, N = 20480, K = 8192 goes from 100 to 72 us; M = 512,
+    // N = 10240: 92 -> 65; M = 384, N = 14336: 91 -> 78; M = 768, N = 7168: 85 -> 65; M = 512, N = 9216, K = 6144: 73 -> 55; M = 256,
+    // N = 20480, K = 5120: 70 -> 56; M = 1024, N = 4608, K = 7168: 74 -> 58; M = 2048, N = 2112, K = 7168: 70 -> 62 (of 105 cases
+    // measured, five lose, by 3-8 %: M = 768, N = 20480, K = 5120: 73 -> 78).
+    if (direct && a.M > 128 && tiles128 > 256 && tiles128 <= 512 && a.KB <= 32)
       return launch_cfg<128, 128, 4, 2, MODE, true>(a, stream);  // eight wavefronts: 7-13 % faster than four on these shapes
   }
   const bool big = a.M > 128;
