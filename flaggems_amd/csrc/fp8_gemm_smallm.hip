@@ -822,7 +822,7 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
       q = round_q(p.q);
       place_activations();
     }
-    // Long K against narrow weights, 128 KB of activations or more: every block reads the activations of its K range,
+    // Long K against narrow weights, 125 KB of activations or more (9 rows of K = 14336: 16.7 -> 14.0 us): every block reads the activations of its K range,
     // which at one range is as much as its weight rows or more.  Half the blocks with twice the rows (32 at most: taller
     // chunks take the slower four-group form) on half of K each halve the activation bytes per block, and the half
     // ranges may fit LDS.  us at M = 8 / 12 / 16, one range -> two: N = 2304, K = 16384: 15.6 / 14.7 / 17.6 -> 11.0 / 12.4 / 12.5;
@@ -831,7 +831,7 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
     // K = 14336: 12.4 -> 13.9; M = 12, N = 3072, K = 8192: 7.7 -> 9.5), not where the activations fit LDS at one range
     // (N = 2112, K = 7168, M = 16: 7.6 -> 8.0), not for taller chunks (N = 7168, K = 16384: 22.9 -> 27.5; N = 5120, K = 13824:
     // 16.7 -> 20.5).
-    if (p.tmx == 1 && entries == 1 && M * KB >= 1024 && (!p.xlds || p.ring) && N <= 32 * (B / 2) && max_splits >= 2 && pairs >= 2 * 8) {
+    if (p.tmx == 1 && entries == 1 && M * KB >= 1000 && (!p.xlds || p.ring) && N <= 32 * (B / 2) && max_splits >= 2 && pairs >= 2 * 8) {
       deal_rows((M + 3) / 4 * 4, B / 2);
       p.n_chunks = (int)chunks;
       splits = 2;

@@ -193,7 +193,8 @@ def test_33_to_128_rows(M, N, K, dtype):
                                    (16, 2304, 16384), (9, 3590, 18944), (12, 4096, 11008), (16, 1280, 8192), (16, 1000, 8192),
                                    (8, 2050, 16384), (24, 8192, 1024), (17, 2050, 1152),
                                    (17, 2304, 16384), (32, 3590, 18944), (24, 4096, 14336),
-                                   (21, 2112, 7168), (32, 4608, 7168), (30, 4100, 4096), (25, 5000, 7296), (20, 2112, 7168)])
+                                   (21, 2112, 7168), (32, 4608, 7168), (30, 4100, 4096), (25, 5000, 7296), (20, 2112, 7168),
+                                   (9, 4096, 14336)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_up_to_32_rows_uneven_chunks(M, N, K, dtype):
     """M <= 32 takes the kernel that deals the weight rows out evenly over the compute units: chunks that differ by a
@@ -209,7 +210,7 @@ def test_up_to_32_rows_uneven_chunks(M, N, K, dtype):
     with 128 KB of activations or more (half the blocks on half of K each, the half ranges in LDS or in the two slots;
     the six shapes from (16, 2304, 16384) on, and the last three with 17 to 32 rows), 17 to 32 rows against short K and
     few tiles ((24, 8192, 1024) and the next), 21 to 32 rows against narrow weights with long K (the kernel of 33 to 64 rows
-    with 32 rows staged; (32, 3590, 18944), (24, 4096, 14336) and the last five, of which the last stays below its threshold), column-major
+    with 32 rows staged; (32, 3590, 18944), (24, 4096, 14336) and the five from (21, 2112, 7168) on, of which the last stays below its threshold), column-major
     activation scales; against the oracle and bit-identical on reruns."""
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=17)
     want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
