@@ -749,6 +749,13 @@ int launch_pipe(GemmArgs a, const PipePlan& plan, void* workspace, hipStream_t s
   return FG_OK;
 }
 
+// Whether 65..128 rows go to the staged-activation kernel as two halves (measurements at the call).
+bool two_halves_preferred(int64_t M, int64_t N, int64_t K) {
+  if (M <= 64 || M > 128) return false;
+  const int64_t bytes = N * K;
+  return bytes <= ((int64_t)8 << 20) || (N <= 3072 && bytes <= ((int64_t)34 << 20)) || (N <= 4096 && bytes <= ((int64_t)17 << 20));
+}
+
 // Whether the 33..64-row kernel is the one to take for the shape (it is compared with the K-split tile kernel and
 // the decode kernels, which take the same shapes).
 bool mid_m_preferred(const MidMPlan& mid, int64_t M, int64_t N, int64_t K) {
@@ -766,6 +773,34 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
   const bool direct = (a.K > 0) && (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) &&
                       (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
                       ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
+  // 65..128 rows against small weights: the staged-activation kernel over the two halves of the rows in one launch (the
+  // halves are the entries of a batch that shares the weights; 33..48 rows stage 48, 49..64 stage 64).  The weights are
+  // read twice, which small ones stand: us at M = 65 / 96 / 128, K-split tile kernel -> here: N = 2112, K = 7168:
+  // 19.3 / 19.6 / 19.9 -> 15.8 / 16.2 / 17.3; N = K = 4096: 15.9 / 16.2 / 16.7 -> 14.7 / 13.9 / 15.0; N = 1024, K = 8192: 17.9 / 18.4 / 19.0 ->
+  // 11.7 / 11.8 / 12.4; N = 8192, K = 1024: 10.7 / 11.0 / 11.2 -> 7.7 / 8.0 / 8.3; N = 2048, K = 16384: 23.3 / 25.1 / 26.2 -> 20.9 / 21.3 / 23.3.
+  // Wider or larger weights lose (N = 4608, K = 7168: 20 -> 33; N = 7168, K = 2304: 13.8 -> 14.4; N = 5120, K = 5120: 17.8 -> 20.2;
+  // N = 2304, K = 16384: 24.0 -> 26.5).
+  if (direct && a.batch <= 1 && two_halves_preferred(a.M, a.N, a.K)) {
+    const int64_t half = (a.M + 1) / 2;
+    const MidMPlan mh = plan_mid_m(half, a.N, a.K, 2);
+    const size_t per_entry = mh.splits > 1 ? mh.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES : 0;
+    const bool fits = mh.use && (mh.splits == 1 || (workspace != nullptr && (uintptr_t)workspace % 16 == 0 &&
+                                                    workspace_bytes >= FG_WORKSPACE_COUNTER_BYTES + 2 * per_entry &&
+                                                    2 * (size_t)mh.n_chunks * sizeof(unsigned int) <= FG_WORKSPACE_COUNTER_BYTES));
+    if (fits) {
+      GemmArgs h = a;
+      const int64_t c_elem = a.c_dtype == FG_F32 ? 4 : (a.c_dtype == FG_BF16 || a.c_dtype == FG_F16) ? 2 : 1;
+      h.M = (int)half;
+      h.batch = 2;
+      h.last_entry_rows = (int)(a.M - half);
+      h.x_batch_bytes = half * a.ldx;
+      h.w_batch_bytes = 0;
+      h.c_batch_bytes = half * a.ldc * c_elem;
+      h.xs_batch_stride = MODE == kModeBlock ? half * a.xs_rs : (a.xs_per_row ? half : 0);
+      h.ws_batch_stride = 0;
+      return launch_mid_m(h, MODE, mh, workspace, workspace_bytes, stream);
+    }
+  }
   if (direct) {
     const MidMPlan mid = plan_mid_m(a.M, a.N, a.K);
     // (65..128 rows: the 128-row variant of that kernel loses to the four-stage tile kernel below on every shape
@@ -858,6 +893,13 @@ extern "C" size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_
   if (plan.use && plan.workspace_bytes > need) need = plan.workspace_bytes;
   const fg::MidMPlan mid = fg::plan_mid_m(M, N, K);
   if (mid.use && mid.workspace_bytes > need) need = mid.workspace_bytes;
+  if (fg::two_halves_preferred(M, N, K)) {  // the same kernel over the two halves of the rows
+    const fg::MidMPlan mh = fg::plan_mid_m((M + 1) / 2, N, K, 2);
+    if (mh.use && mh.splits > 1) {
+      const size_t both = FG_WORKSPACE_COUNTER_BYTES + 2 * (mh.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES);
+      if (both > need) need = both;
+    }
+  }
   const size_t pp = fg::pingpong_workspace_bytes(M, N, K);
   return pp > need ? pp : need;
 }

@@ -39,6 +39,9 @@ struct GemmArgs {
   // a batch with K split over blocks: every entry has tiles x splits partial tiles of its own, these many floats in
   // all, and tiles x wavefronts counters
   int64_t split_partials_per_entry;
+  // staged-activation kernel over the two halves of a lone problem's rows (batch == 2, the weights shared): rows of the
+  // second half when it has fewer than M, else 0
+  int last_entry_rows;
 };
 
 // s_waitcnt vmcnt(0) with expcnt/lgkmcnt left at their maxima (gfx9 encoding)

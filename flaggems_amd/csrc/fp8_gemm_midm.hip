@@ -64,6 +64,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_midm_kernel(MidArgs a) {
     a.g.ws += z * a.g.ws_batch_stride;
     if (a.partials) a.partials += z * a.partials_per_entry;
     if (a.counters) a.counters += z * a.n_chunks;
+    if (a.g.last_entry_rows > 0 && z == a.g.batch - 1) a.g.M = a.g.last_entry_rows;
   }
   const GemmArgs& g = a.g;
   const int tid = threadIdx.x, lane = tid & 63;

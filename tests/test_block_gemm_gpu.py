@@ -158,7 +158,8 @@ def test_129_to_512_tiles_of_128_rows(M, N, K, dtype):
                                    (33, 49152, 2048), (48, 20490, 1536), (37, 16384, 1024), (33, 20480, 3072),
                                    (65, 520, 1024), (100, 2112, 4096), (128, 4096, 4096), (128, 7000, 2304),
                                    (48, 8330, 6144), (64, 6650, 8192), (40, 8200, 1024), (64, 16384, 1152), (70, 16650, 8192),
-                                   (64, 33040, 2048), (44, 36000, 2560)])
+                                   (64, 33040, 2048), (44, 36000, 2560),
+                                   (65, 2112, 7168), (97, 1030, 8192), (128, 8200, 1024), (81, 3000, 4224), (128, 2048, 16384)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_33_to_128_rows(M, N, K, dtype):
     """33 <= M <= 64 (and 65 <= M <= 128 with small weights) takes the kernel that keeps the activations in LDS and
@@ -167,7 +168,9 @@ def test_33_to_128_rows(M, N, K, dtype):
     on reruns.  The last line of shapes: that kernel's blocks would leave a second round of compute units mostly idle,
     so the four-stage tile kernel takes them with K in three and four ranges; the last shape has 131 tiles, which that kernel
     splits in three ranges rather than leave half of the compute units idle; the two after it are too wide for one round of tiles
-    and run in rounds of blocks whose K split is chosen by how full the rounds are."""
+    and run in rounds of blocks whose K split is chosen by how full the rounds are; the last five (and (65, 520, 1024),
+    (100, 2112, 4096), (128, 4096, 4096) above) have 65 to 128 rows against small weights, which the same kernel takes as two
+    halves of the rows in one launch (48 or 64 rows staged, a second half with fewer rows than the first)."""
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=13)
     want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
     args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])

@@ -42,6 +42,8 @@ def _exact(a, b, sa, sb):
                                    (1, 4096, 4096), (8, 2112, 7168), (16, 7168, 2304), (32, 1024, 8192), (5, 24592, 384),
                                    (12, 32768, 512), (20, 520, 1024), (24, 32768, 512), (32, 24580, 1536),
                                    (32, 2112, 7168), (24, 4624, 7168), (16, 2304, 16384),
+                                   # 65..128 rows against small weights: two halves of the rows in one launch
+                                   (65, 2112, 7168), (128, 1024, 8192), (99, 4096, 4096),
                                    # 33..64 rows: the kernel with the activations of a K range in LDS
                                    (33, 2112, 7168), (64, 4096, 4096), (48, 24576, 1536), (40, 264, 512),
                                    # K that is not a multiple of 128 above 128 rows
