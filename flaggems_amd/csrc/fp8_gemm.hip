@@ -749,11 +749,23 @@ int launch_pipe(GemmArgs a, const PipePlan& plan, void* workspace, hipStream_t s
   return FG_OK;
 }
 
-// Whether 65..128 rows go to the staged-activation kernel as two halves (measurements at the call).
-bool two_halves_preferred(int64_t M, int64_t N, int64_t K) {
-  if (M <= 64 || M > 128) return false;
+// Into how many equal parts of at most 64 rows the staged-activation kernel takes the rows of a lone problem above 64 rows
+// (measurements at the call); 0: not at all.
+int64_t row_parts(int64_t M, int64_t N, int64_t K) {
   const int64_t bytes = N * K;
-  return bytes <= ((int64_t)8 << 20) || (N <= 3072 && bytes <= ((int64_t)34 << 20)) || (N <= 4096 && bytes <= ((int64_t)17 << 20));
+  if (M > 64 && M <= 128 &&
+      (bytes <= ((int64_t)8 << 20) || (N <= 3072 && bytes <= ((int64_t)34 << 20)) || (N <= 4096 && bytes <= ((int64_t)17 << 20))))
+    return 2;
+  // more parts only for the smallest weights, which every part reads again: us at M = 129 / 192 / 256, N = 512, K = 7168:
+  // 16.7 / 17.5 / 18.2 -> 11.1 / 11.7 / 11.9; N = 1024, K = 4096: 14.8 / 15.2 / 15.8 -> 9.6 / 10.0 / 10.2; N = K = 2048: 12.6 / 12.7 / 13.0 ->
+  // 9.0 / 9.6 / 9.7; up to 192 rows, N = 1280, K = 8192: 18.6 / 18.8 -> 14.9 / 16.3; N = 1024, K = 8192: 18.1 / 18.6 -> 16.0 / 17.2 (N = 2112,
+  // K = 7168: 19.2 -> 20.9; N = K = 4096: 16.6 -> 23.2)
+  if (M > 128 && M <= 256 && bytes <= ((int64_t)4 << 20)) return ceil_div(M, (int64_t)64);
+  if (M > 128 && M <= 192 && bytes <= ((int64_t)10 << 20)) return 3;
+  // (257..512 rows: N = 1024, K = 2048: 12.6 -> 9.4; N = 256, K = 8192: 17.2 / 18.4 -> 12.0 / 12.3 at 257 / 512 rows; N = 512, K = 7168:
+  // 17.6 / 18.4 -> 15.2 / 17.0; N = 1024, K = 8192: 20.6 -> 21.2)
+  if (M > 256 && M <= 512 && bytes <= ((int64_t)2 << 20)) return ceil_div(M, (int64_t)64);
+  return 0;
 }
 
 // Whether the 33..64-row kernel is the one to take for the shape (it is compared with the K-split tile kernel and
@@ -780,23 +792,23 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
   // 11.7 / 11.8 / 12.4; N = 8192, K = 1024: 10.7 / 11.0 / 11.2 -> 7.7 / 8.0 / 8.3; N = 2048, K = 16384: 23.3 / 25.1 / 26.2 -> 20.9 / 21.3 / 23.3.
   // Wider or larger weights lose (N = 4608, K = 7168: 20 -> 33; N = 7168, K = 2304: 13.8 -> 14.4; N = 5120, K = 5120: 17.8 -> 20.2;
   // N = 2304, K = 16384: 24.0 -> 26.5).
-  if (direct && a.batch <= 1 && two_halves_preferred(a.M, a.N, a.K)) {
-    const int64_t half = (a.M + 1) / 2;
-    const MidMPlan mh = plan_mid_m(half, a.N, a.K, 2);
+  if (const int64_t parts = direct && a.batch <= 1 ? row_parts(a.M, a.N, a.K) : 0; parts > 1) {
+    const int64_t rows = ceil_div((int64_t)a.M, parts);
+    const MidMPlan mh = plan_mid_m(rows, a.N, a.K, parts);
     const size_t per_entry = mh.splits > 1 ? mh.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES : 0;
     const bool fits = mh.use && (mh.splits == 1 || (workspace != nullptr && (uintptr_t)workspace % 16 == 0 &&
-                                                    workspace_bytes >= FG_WORKSPACE_COUNTER_BYTES + 2 * per_entry &&
-                                                    2 * (size_t)mh.n_chunks * sizeof(unsigned int) <= FG_WORKSPACE_COUNTER_BYTES));
+                                                    workspace_bytes >= FG_WORKSPACE_COUNTER_BYTES + (size_t)parts * per_entry &&
+                                                    (size_t)parts * mh.n_chunks * sizeof(unsigned int) <= FG_WORKSPACE_COUNTER_BYTES));
     if (fits) {
       GemmArgs h = a;
       const int64_t c_elem = a.c_dtype == FG_F32 ? 4 : (a.c_dtype == FG_BF16 || a.c_dtype == FG_F16) ? 2 : 1;
-      h.M = (int)half;
-      h.batch = 2;
-      h.last_entry_rows = (int)(a.M - half);
-      h.x_batch_bytes = half * a.ldx;
+      h.M = (int)rows;
+      h.batch = (int)parts;
+      h.last_entry_rows = (int)(a.M - (parts - 1) * rows);
+      h.x_batch_bytes = rows * a.ldx;
       h.w_batch_bytes = 0;
-      h.c_batch_bytes = half * a.ldc * c_elem;
-      h.xs_batch_stride = MODE == kModeBlock ? half * a.xs_rs : (a.xs_per_row ? half : 0);
+      h.c_batch_bytes = rows * a.ldc * c_elem;
+      h.xs_batch_stride = MODE == kModeBlock ? rows * a.xs_rs : (a.xs_per_row ? rows : 0);
       h.ws_batch_stride = 0;
       return launch_mid_m(h, MODE, mh, workspace, workspace_bytes, stream);
     }
@@ -893,10 +905,10 @@ extern "C" size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_
   if (plan.use && plan.workspace_bytes > need) need = plan.workspace_bytes;
   const fg::MidMPlan mid = fg::plan_mid_m(M, N, K);
   if (mid.use && mid.workspace_bytes > need) need = mid.workspace_bytes;
-  if (fg::two_halves_preferred(M, N, K)) {  // the same kernel over the two halves of the rows
-    const fg::MidMPlan mh = fg::plan_mid_m((M + 1) / 2, N, K, 2);
+  if (const int64_t parts = fg::row_parts(M, N, K); parts > 1) {  // the same kernel over equal parts of the rows
+    const fg::MidMPlan mh = fg::plan_mid_m(fg::ceil_div(M, parts), N, K, parts);
     if (mh.use && mh.splits > 1) {
-      const size_t both = FG_WORKSPACE_COUNTER_BYTES + 2 * (mh.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES);
+      const size_t both = FG_WORKSPACE_COUNTER_BYTES + (size_t)parts * (mh.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES);
       if (both > need) need = both;
     }
   }

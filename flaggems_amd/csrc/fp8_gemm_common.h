@@ -39,8 +39,8 @@ struct GemmArgs {
   // a batch with K split over blocks: every entry has tiles x splits partial tiles of its own, these many floats in
   // all, and tiles x wavefronts counters
   int64_t split_partials_per_entry;
-  // staged-activation kernel over the two halves of a lone problem's rows (batch == 2, the weights shared): rows of the
-  // second half when it has fewer than M, else 0
+  // staged-activation kernel over equal parts of a lone problem's rows (the entries of a batch that shares the weights):
+  // rows of the last part when it has fewer than M, else 0
   int last_entry_rows;
 };
 

@@ -137,6 +137,27 @@ def test_tall_problems_against_narrow_weights(M, N, K):
         assert torch.equal(flag_gems.w8a8_block_fp8_matmul(*args).view(torch.int16), got.view(torch.int16))
 
 
+@pytest.mark.parametrize("M,N,K", [(129, 576, 7168), (200, 1030, 4096), (256, 2048, 2048), (190, 1280, 8192), (257, 1024, 2048),
+                                   (500, 260, 8192), (512, 1000, 1152)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_129_to_512_rows_against_tiny_weights(M, N, K, dtype):
+    """Weights of a few MB: the kernel of 33 to 64 rows takes the rows in three to eight equal parts in one launch (the
+    last part with fewer rows), each part reading the weights again.  Ragged M and N, column-major activation scales;
+    against the oracle and bit-identical on reruns."""
+    xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=29)
+    want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
+    args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
+    got = flag_gems.w8a8_block_fp8_matmul(*args, output_dtype=dtype)
+    assert got.dtype == dtype and got.shape == (M, N)
+    tol = dict(rtol=1e-4, atol=4e-4) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(got.cpu().float(), want, **tol)
+    for _ in range(2):
+        assert torch.equal(flag_gems.w8a8_block_fp8_matmul(*args, output_dtype=dtype).view(torch.int8), got.view(torch.int8))
+    xs_cm = xs.to(DEV).t().contiguous().t()
+    cm = flag_gems.w8a8_block_fp8_matmul(args[0], args[1], xs_cm, args[3], [128, 128], output_dtype=dtype)
+    assert torch.equal(cm.view(torch.int8), got.view(torch.int8))
+
+
 @pytest.mark.parametrize("M,N,K", [(700, 4000, 4096), (512, 6144, 4096), (1000, 3200, 8192), (300, 10000, 1024),
                                    (768, 7168, 2304), (256, 24576, 1536), (1000, 6100, 4096), (130, 40000, 512)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
