@@ -749,6 +749,22 @@ int launch_pipe(GemmArgs a, const PipePlan& plan, void* workspace, hipStream_t s
   return FG_OK;
 }
 
+// Parts of up to 16 rows in which the decode kernels take 17..64 rows of a lone problem (measurements at the call): the parts
+// start `stride` rows apart and the last one ends with the last row; where stride < rows neighbouring parts share rows,
+// which both compute alike.
+struct DecodeParts {
+  int64_t parts, stride, rows;  // parts == 0: not taken
+};
+DecodeParts decode_parts(int64_t M, int64_t N, int64_t K) {
+  DecodeParts d = {0, 0, 0};
+  if (!((M > 16 && M <= 32 && N <= 6144) || (M > 32 && M <= 64 && N * K <= ((int64_t)8 << 20)))) return d;
+  for (d.parts = ceil_div(M, (int64_t)16);; ++d.parts) {
+    d.stride = M / d.parts;
+    d.rows = M - (d.parts - 1) * d.stride;
+    if (d.rows <= 16) return d;
+  }
+}
+
 // Into how many equal parts of at most 64 rows the staged-activation kernel takes the rows of a lone problem above 64 rows
 // (measurements at the call); 0: not at all.
 int64_t row_parts(int64_t M, int64_t N, int64_t K) {
@@ -785,6 +801,37 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
   const bool direct = (a.K > 0) && (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) &&
                       (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
                       ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
+  // 17..32 rows against weights of up to 6144 rows, 33..64 rows against weights of up to 8 MB: parts of up to 16 rows on the
+  // decode kernels in one launch (the entries of a batch that shares the weights).  With 17 rows or more a decode block
+  // fetches 32 activation rows per 16-32 weight rows through registers; with up to 16 the activations of its K range lie in
+  // LDS.  us at M = 17 / 24 / 32, before (decode kernels for 32 rows, or 32 rows staged in the kernel of 33..64 rows) -> two parts:
+  // N = 2112, K = 7168: 10.2 / 10.8 / 10.8 -> 7.4 / 7.7 / 9.2; N = 3072, K = 8192: 11.8 / 12.4 / 12.7 -> 8.6 / 10.1 / 10.3; N = 1024, K = 8192:
+  // 8.4 / 9.6 / 10.2 -> 6.2 / 6.5 / 9.2; N = 4096, K = 14336: 18.8 / 19.6 / 20.0 -> 17.4 / 17.4 / 17.4; N = 576, K = 7168: 8.1 / 9.1 / 9.5 -> 5.7 / 6.0 / 6.3;
+  // N = K = 6144: 12.9 / 14.3 / 15.9 -> 11.7 / 12.1 / 13.4; N = K = 4096: 8.0 / 8.8 / 9.1 -> 8.0 / 7.9 / 8.0.  Wider weights lose (N = 7168,
+  // K = 2304: 7.1 -> 8.0; N = 10240, K = 8192: 23 -> 31; N = 28672, K = 4096: 27 -> 45).  33..64 rows in three or four parts,
+  // M = 33 / 48 / 64: N = 512, K = 7168: 10.2 / 10.2 / 10.8 -> 6.5 / 7.1 / 6.2; N = K = 2048: 8.6 / 8.7 / 9.2 -> 5.4 / 5.8 / 5.1; N = 1024, K = 8192:
+  // 11.4 / 11.5 / 11.9 -> 8.0 / 9.4 / 9.5; larger weights lose there (N = 2112, K = 7168: 12.2 -> 11.7 at 48 rows, 13.2 -> 13.4 at 64;
+  // N = K = 4096: 10.0 -> 14.0).
+  if (const DecodeParts dp = direct && a.batch <= 1 ? decode_parts(a.M, a.N, a.K) : DecodeParts{0, 0, 0}; dp.parts > 1) {
+    const int64_t parts = dp.parts, stride = dp.stride, rows = dp.rows;
+    const SmallMPlan sp = plan_small_m(rows, a.N, a.K, parts);
+    const size_t per_entry = sp.splits > 1 ? sp.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES : 0;
+    const bool fits = sp.use && (sp.splits == 1 || (workspace != nullptr && (uintptr_t)workspace % 16 == 0 &&
+                                                    workspace_bytes >= FG_WORKSPACE_COUNTER_BYTES + (size_t)parts * per_entry &&
+                                                    (size_t)parts * sp.n_chunks * sizeof(unsigned int) <= FG_WORKSPACE_COUNTER_BYTES));
+    if (fits) {
+      GemmArgs h = a;
+      const int64_t c_elem = a.c_dtype == FG_F32 ? 4 : (a.c_dtype == FG_BF16 || a.c_dtype == FG_F16) ? 2 : 1;
+      h.M = (int)rows;
+      h.batch = (int)parts;
+      h.x_batch_bytes = stride * a.ldx;
+      h.w_batch_bytes = 0;
+      h.c_batch_bytes = stride * a.ldc * c_elem;
+      h.xs_batch_stride = MODE == kModeBlock ? stride * a.xs_rs : (a.xs_per_row ? stride : 0);
+      h.ws_batch_stride = 0;
+      return launch_small_m(h, MODE, sp, workspace, workspace_bytes, stream);
+    }
+  }
   // 65..128 rows against small weights: the staged-activation kernel over the two halves of the rows in one launch (the
   // halves are the entries of a batch that shares the weights; 33..48 rows stage 48, 49..64 stage 64).  The weights are
   // read twice, which small ones stand: us at M = 65 / 96 / 128, K-split tile kernel -> here: N = 2112, K = 7168:
@@ -825,9 +872,6 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
       const SmallMPlan sp = plan_small_m(a.M, a.N, a.K);
       if (sp.use && sp.own) return launch_small_m(a, MODE, sp, workspace, workspace_bytes, stream);
     }
-    // 21..32 rows against narrow weights with long K: the staged-activation kernel with 32 rows (its planner holds the rule)
-    if (a.M <= 32 && mid_takes && (mid.splits == 1 || (workspace != nullptr && workspace_bytes >= mid.workspace_bytes && (uintptr_t)workspace % 16 == 0)))
-      return launch_mid_m(a, MODE, mid, workspace, workspace_bytes, stream);
     if (a.M <= 64) {  // the four-stage tile kernel where its planner prefers it to the staged-activation and decode kernels
       const PipePlan pp = plan_pipe(a.M, a.N, a.K, MODE == kModeBlock ? a.xs_rs : 0);
       const bool ws_ok = pp.splits == 1 || (workspace != nullptr && workspace_bytes >= pp.workspace_bytes && (uintptr_t)workspace % 16 == 0);
@@ -905,6 +949,13 @@ extern "C" size_t fg_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_
   if (plan.use && plan.workspace_bytes > need) need = plan.workspace_bytes;
   const fg::MidMPlan mid = fg::plan_mid_m(M, N, K);
   if (mid.use && mid.workspace_bytes > need) need = mid.workspace_bytes;
+  if (const fg::DecodeParts dp = fg::decode_parts(M, N, K); dp.parts > 1) {  // the decode kernels over parts of the rows
+    const fg::SmallMPlan sp = fg::plan_small_m(dp.rows, N, K, dp.parts);
+    if (sp.use && sp.splits > 1) {
+      const size_t all = FG_WORKSPACE_COUNTER_BYTES + (size_t)dp.parts * (sp.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES);
+      if (all > need) need = all;
+    }
+  }
   if (const int64_t parts = fg::row_parts(M, N, K); parts > 1) {  // the same kernel over equal parts of the rows
     const fg::MidMPlan mh = fg::plan_mid_m(fg::ceil_div(M, parts), N, K, parts);
     if (mh.use && mh.splits > 1) {

@@ -235,7 +235,7 @@ int launch_small_m(const GemmArgs& a, int mode, const SmallMPlan& plan, void* wo
 // 33 <= M <= 128 rows, fp8_gemm_midm.hip: activations staged in LDS once per block, weights streamed.
 struct MidMPlan {
   bool use;
-  int tmx;           // 16-row activation groups staged: 2 (M <= 32), 3 (M <= 48), 4 (M <= 64) or 8
+  int tmx;           // 16-row activation groups staged: 3 (M <= 48), 4 (M <= 64) or 8
   int rg;            // 16-row weight groups per wavefront: 1, 2 or 4
   int waves;         // wavefronts per block: 4 or 8
   int kb_per_split;  // K-blocks per block (<= 16)

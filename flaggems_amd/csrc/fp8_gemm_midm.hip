@@ -1,5 +1,4 @@
-// FP8 GEMM for 33 <= M <= 64 activation rows on gfx950 (up to 128 rows against small weights, and from 21 rows against
-// narrow weights with long K): the weight is
+// FP8 GEMM for 33 <= M <= 64 activation rows on gfx950 (and more rows against small weights, in parts of up to 64): the weight is
 // read once, straight from global memory into MFMA operand registers, and the activations come out of LDS.
 //
 // With up to 64 rows the activation slice of a K-block (64 x 128 bytes) is as large as the 64 weight rows a
@@ -11,7 +10,7 @@
 //
 //  * A wavefront owns 16 * RG weight rows (RG = 1, 2, 4) and the K-blocks [split * kb_per_split, ...): per K-block
 //    2 * RG 16-byte loads per lane (DEPTH K-blocks in flight, 64 VGPRs), 8 LDS reads, 4 * RG MFMAs.
-//  * K is split over gridDim.y blocks only as far as LDS (128 KB of activations: 32 K-blocks of 32 rows, 16 of 64 rows, 8 of
+//  * K is split over gridDim.y blocks only as far as LDS (128 KB of activations: 21 K-blocks of 48 rows, 16 of 64 rows, 8 of
 //    128 rows) or the number of wavefronts requires; each wavefront then publishes its sums and the one that arrives last adds the
 //    splits' sums in split order (a fixed order: results do not depend on timing) and resets the counter.
 //
@@ -23,8 +22,8 @@
 namespace fg {
 namespace {
 
-// TMX 16-row groups of activations are staged (32, 48, 64 or 128 rows; rows past M repeat the last one and are never
-// stored); a block keeps at most 128 KB of them in LDS: 32 K-blocks of 32 rows, 21 of 48, 16 of 64, 8 of 128.
+// TMX 16-row groups of activations are staged (48, 64 or 128 rows; rows past M repeat the last one and are never
+// stored); a block keeps at most 128 KB of them in LDS: 21 K-blocks of 48 rows, 16 of 64, 8 of 128.
 constexpr int mid_rows(int tmx) { return 16 * tmx; }
 constexpr int mid_stage_bytes(int tmx) { return mid_rows(tmx) * 128; }
 constexpr int mid_kb_max(int tmx) { return 64 / tmx; }
@@ -285,23 +284,17 @@ int launch_mid(const MidArgs& ma, int mode, hipStream_t stream) {
 MidMPlan plan_mid_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
   MidMPlan p = {};
   if (entries < 1) entries = 1;  // equal problems launched together: their wavefronts fill the GPU together
-  // (a 16-row variant of this kernel was slower than the decode kernels on every shape)
-  if (M <= 16 || M > 128 || N < 1 || K < 128 || K % 128 != 0) return p;
-  // 17..32 rows (32 staged): this kernel takes the same time whatever M while the decode kernels, which fetch 32
-  // activation rows per 16-32 weight rows, grow by 2-3 % a row; against narrow weights with long K it is ahead from 21
-  // rows on, with K = 4096 from 29.  us at M = 17 / 24 / 32, decode -> here: N = 2112, K = 7168: 10.2 / 11.9 / 14.0 -> 10.8 / 10.7 / 10.8;
-  // N = 4608, K = 7168: 13.4 / 14.9 / 16.8 -> 14.2 / 13.4 / 13.6; N = 4096, K = 14336: 19.0 / 20.6 / 22.3 -> 19.0 / 19.6 / 19.9; N = 2304,
-  // K = 16384: 16.6 / 18.7 / 20.4 -> 17.2 / 16.8 / 17.1; N = K = 4096: 7.8 / 8.8 / 9.7 -> 9.2 / 9.2 / 9.2.  Wider weights stay with
-  // the decode kernels (N = 7168, K = 16384: 28 / 31 / 34.5 -> 47 / 48 / 48; N = 7168, K = 2304: 7.0 / 7.3 / 7.7 -> 9.3; N = 6144,
-  // K = 4096: 9.6 / 10.6 / 11.6 -> 12.4; N = 1024, K = 8192: 8.5 / 9.6 / 10.6 -> 10.2; N = K = 8192: 19.2 / 20.6 / 22.2 -> 19.8 / 20.3 / 20.8, too close to call).
-  if (M <= 32 && !(entries == 1 && ((K >= 7168 && N >= 2048 && N <= 5120 && M >= 21) || (K >= 4096 && N <= 4608 && M >= 29)))) return p;
+  // (16- and 32-row variants of this kernel were measured against the decode kernels: the 16-row one slower on every shape;
+  // the 32-row one ahead from 21 rows against narrow weights with long K -- N = 2112, K = 7168, M = 24 / 32: 11.9 / 14.0 -> 10.7 / 10.8 us --
+  // until the decode kernels took 17..32 rows in two parts of up to 16: 7.7 / 9.2 us)
+  if (M <= 32 || M > 128 || N < 1 || K < 128 || K % 128 != 0) return p;
   const int64_t KB = K / 128;
   // 33..48 rows stage 48: a quarter less LDS per K-block (21 fit), MFMA work and partial sums: 2-8 % faster than with 64 rows
   // on 13 of 14 shapes (M = 40: N = 7168, K = 16384: 40.2 -> 37.0 us; N = 2112, K = 7168: 13.0 -> 12.2; N = 4096, K = 14336: 22.4 -> 21.1;
   // N = 14336, K = 4096: 20.8 -> 21.1)
   // (80 and 96 rows staged for 65..96 rows do not soften the step to the tile kernel at 65 rows: M = 80, N = 2112, K = 7168:
   // 19.4 us there, 19.1 here; N = 7168, K = 16384: 40 against 58; N = K = 4096: 16.2 against 15.8; N = 24576, K = 1536: 14.8 against 17.7)
-  const int tmx = M <= 32 ? 2 : M <= 48 ? 3 : M <= 64 ? 4 : 8;
+  const int tmx = M <= 48 ? 3 : M <= 64 ? 4 : 8;
   const int64_t kb_max = mid_kb_max(tmx);
   const int64_t min_splits = ceil_div(KB, kb_max);
   int rg;
@@ -387,11 +380,6 @@ int launch_mid_m(const GemmArgs& g, int mode, const MidMPlan& plan, void* worksp
   if (plan.tmx == 8) {
     if (plan.rg == 2) return plan.waves == 8 ? launch_mid<8, 2, 8, 4>(ma, mode, stream) : launch_mid<8, 2, 4, 4>(ma, mode, stream);
     return plan.waves == 8 ? launch_mid<8, 1, 8, 8>(ma, mode, stream) : launch_mid<8, 1, 4, 8>(ma, mode, stream);
-  }
-  if (plan.tmx == 2) {
-    if (plan.rg == 4) return plan.waves == 8 ? launch_mid<2, 4, 8, 2>(ma, mode, stream) : launch_mid<2, 4, 4, 2>(ma, mode, stream);
-    if (plan.rg == 2) return plan.waves == 8 ? launch_mid<2, 2, 8, 4>(ma, mode, stream) : launch_mid<2, 2, 4, 4>(ma, mode, stream);
-    return plan.waves == 8 ? launch_mid<2, 1, 8, 8>(ma, mode, stream) : launch_mid<2, 1, 4, 8>(ma, mode, stream);
   }
   if (plan.tmx == 3) {
     if (plan.rg == 4) return plan.waves == 8 ? launch_mid<3, 4, 8, 2>(ma, mode, stream) : launch_mid<3, 4, 4, 2>(ma, mode, stream);

@@ -839,16 +839,6 @@ SmallMPlan plan_small_m(int64_t M, int64_t N, int64_t K, int64_t entries) {
       q = round_q(p.q);
       place_activations();
     }
-    // The same with 17 to 32 rows (activations through the register ring, 32 rows of them per block whatever M), from
-    // about twice the bytes on: us at M = 17 / 24 / 32, N = 2304, K = 16384: 19.7 / 23.6 / 27.4 -> 16.8 / 18.7 / 20.4; N = 3584,
-    // K = 18944: 23.3 / 25.1 / 29.6 -> 21.8 / 22.8 / 24.6; N = 4096, K = 14336, M = 24 / 32: 22.0 / 25.5 -> 20.8 / 22.4 (17 rows: 18.9 -> 19.2;
-    // N = 4096, K = 11008, M = 17 / 24 / 32: 14.7 / 16.5 / 18.8 -> 15.9 / 17.0 / 17.9; N = K = 4096, M = 32: 9.8 -> 10.0; 256 KB: N = 3072, K = 8192, M = 32: 16.0 -> 13.9; N = 4096, K = 8192: 16.4 -> 15.0).
-    if (p.tmx == 2 && entries == 1 && M * KB >= 2048 && splits == 1 && N <= 32 * (B / 2) && max_splits >= 2 && pairs >= 2 * 8) {
-      deal_rows(16, B / 2);
-      p.n_chunks = (int)chunks;
-      splits = 2;
-      kpw = ceil_div(pairs, splits * p.waves);
-    }
     p.q = p.tmx == 1 ? q : 4 * p.rg;
   } else {
     // aim for ~8 wavefronts per CU on 256 CUs, each with at least one K-block

@@ -180,7 +180,8 @@ def test_129_to_512_tiles_of_128_rows(M, N, K, dtype):
                                    (65, 520, 1024), (100, 2112, 4096), (128, 4096, 4096), (128, 7000, 2304),
                                    (48, 8330, 6144), (64, 6650, 8192), (40, 8200, 1024), (64, 16384, 1152), (70, 16650, 8192),
                                    (64, 33040, 2048), (44, 36000, 2560),
-                                   (65, 2112, 7168), (97, 1030, 8192), (128, 8200, 1024), (81, 3000, 4224), (128, 2048, 16384)])
+                                   (65, 2112, 7168), (97, 1030, 8192), (128, 8200, 1024), (81, 3000, 4224), (128, 2048, 16384),
+                                   (33, 512, 7168), (47, 1030, 8192), (64, 2048, 2048), (50, 8200, 1024)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_33_to_128_rows(M, N, K, dtype):
     """33 <= M <= 64 (and 65 <= M <= 128 with small weights) takes the kernel that keeps the activations in LDS and
@@ -191,7 +192,8 @@ def test_33_to_128_rows(M, N, K, dtype):
     splits in three ranges rather than leave half of the compute units idle; the two after it are too wide for one round of tiles
     and run in rounds of blocks whose K split is chosen by how full the rounds are; the last five (and (65, 520, 1024),
     (100, 2112, 4096), (128, 4096, 4096) above) have 65 to 128 rows against small weights, which the same kernel takes as two
-    halves of the rows in one launch (48 or 64 rows staged, a second half with fewer rows than the first)."""
+    halves of the rows in one launch (48 or 64 rows staged, a second half with fewer rows than the first); the last four are
+    33 to 64 rows against weights of up to 8 MB, which the decode kernels take in three or four parts of up to 16 rows."""
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=13)
     want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
     args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
@@ -232,10 +234,11 @@ def test_up_to_32_rows_uneven_chunks(M, N, K, dtype):
     (32, 28672, 4096) is too long in K for that and stays on the kernels for 32 rows, two take blocks of eight
     wavefronts, and the four up to (3, 17416, 1536) have just over four 16-row groups per compute unit), narrow weights
     with 128 KB of activations or more (half the blocks on half of K each, the half ranges in LDS or in the two slots;
-    the six shapes from (16, 2304, 16384) on, and the last three with 17 to 32 rows), 17 to 32 rows against short K and
-    few tiles ((24, 8192, 1024) and the next), 21 to 32 rows against narrow weights with long K (the kernel of 33 to 64 rows
-    with 32 rows staged; (32, 3590, 18944), (24, 4096, 14336) and the five from (21, 2112, 7168) on, of which the last stays below its threshold), column-major
-    activation scales; against the oracle and bit-identical on reruns."""
+    the six shapes from (16, 2304, 16384) on and (9, 4096, 14336)), 17 to 32 rows against short K and few tiles
+    ((24, 8192, 1024) and the next), 17 to 32 rows against weights of up to 6144 rows (two parts of up to 16 rows in one
+    launch, sharing the middle row when the count is odd: (20, 4608, 4096), (17, 2050, 1152), the three from
+    (17, 2304, 16384) on and the five from (21, 2112, 7168) on), column-major activation scales; against the oracle and
+    bit-identical on reruns."""
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=17)
     want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
     args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])

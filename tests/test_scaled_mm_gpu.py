@@ -26,10 +26,12 @@ MNK = [
     (16, 4608, 7296), (13, 7168, 16384),
     # 17 to 32 rows against wide weights and short K: a wavefront per 16 weight rows, two 16-row images of the activations in LDS
     (24, 24576, 512), (32, 20496, 1536), (17, 32768, 256), (40, 24592, 1536), (33, 49152, 2048),
-    # 21 to 32 rows against narrow weights with long K: 32 activation rows of a K range in LDS; two K ranges on the decode kernels below that
+    # 17 to 32 rows against weights of up to 6144 rows: two parts of up to 16 rows on the decode kernels in one launch
     (32, 2112, 7168), (24, 4624, 7168), (30, 4096, 4096), (18, 2304, 16384),
     # 65 to 128 rows against small weights: the staged-activation kernel over the two halves of the rows
     (65, 2112, 7168), (100, 1040, 8192), (128, 4096, 4096), (77, 8192, 1024),
+    # 33 to 64 rows against weights of up to 8 MB: three or four parts of up to 16 rows on the decode kernels
+    (33, 512, 7168), (50, 1040, 8192), (64, 2048, 2048),
     # few 256 x 256 tiles with a long K: compute units share tiles and add their sums through the workspace
     (384, 5632, 8320), (300, 3088, 8448),
     # K that is not a multiple of 128 (operands go through registers), above and below 128 rows
