@@ -23,6 +23,9 @@ Prints ONE JSON line with the driver's fields plus
                 operands; Llama-3-8B
                 linears as GEMM alone and as act_quant + GEMM), graph replays of one shape at a time with ONE copy
                 of the weights (small-M figures there may be served by the 256 MB Infinity Cache), not part of `value`
+  rows_at_the_hand_over_points
+                the block GEMM at the row counts where one kernel hands over to the next (16 | 17, 32 | 33, 64 | 65,
+                128 | 129) on three weights, weights rotated through 512 MB; not part of `value`
   mixtral_moe_grouped_gemm
                 Mixtral-8x7B expert layers: 8 experts, top-2 over T tokens with Zipf(1.1) expert loads, rows sorted by
                 expert; the grouped block-fp8 GEMM with W1 [8,28672,4096] and W2 [8,4096,14336]; not part of `value`
@@ -531,6 +534,22 @@ def main():
                           "weight_copies": len(use)})
         del wq, ws, pool
 
+    # the row counts at which one kernel hands over to the next (16/17: decode kernels / two parts of up to 16 rows; 32/33: to
+    # the staged-activation kernel; 64/65: to two halves of it, or the K-split tile kernel; 128/129: tile kernel), weights rotated
+    handover = []
+    for (n, k) in [(2112, 7168), (4096, 4096), (7168, 16384)]:
+        wq, ws = make_weight(n, k, gen, dev)
+        copies = max(1, -(-CACHE_BYTES // (n * k)))
+        pool = [wq] + [wq.clone() for _ in range(copies - 1)]
+        row = {"N": n, "K": k, "us_by_rows": {}}
+        for m in (16, 17, 32, 33, 64, 65, 128, 129):
+            xq = torch.randn(m, k, device=dev, generator=gen).to(torch.float8_e4m3fn)
+            xs = torch.rand(m, k // 128, device=dev, generator=gen) + 0.5
+            us = time_graph(lambda r: flag_gems.w8a8_block_fp8_matmul(xq, pool[r % len(pool)], xs, ws, [128, 128]))
+            row["us_by_rows"][str(m)] = round(us, 2)
+        handover.append(row)
+        del wq, ws, pool
+
     # Mixtral-8x7B expert layers: grouped block-fp8 GEMM over rows sorted by expert
     moe = []
     experts = 8
@@ -711,6 +730,7 @@ def main():
         "scaled_mm_unquantized_operands": generic,
         "fp8_einsum_bhr_hdr": einsum,
         "llama3_8b_linears": llama,
+        "rows_at_the_hand_over_points": handover,
         "mixtral_moe_grouped_gemm": moe,
         "mixtral_moe_layer": moe_layer,
         "eager_host_overhead": eager,
