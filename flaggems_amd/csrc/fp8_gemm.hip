@@ -757,7 +757,7 @@ struct DecodeParts {
 };
 DecodeParts decode_parts(int64_t M, int64_t N, int64_t K) {
   DecodeParts d = {0, 0, 0};
-  if (!((M > 16 && M <= 32 && N <= 6144) || (M > 32 && M <= 64 && N * K <= ((int64_t)8 << 20)))) return d;
+  if (!((M > 16 && M <= 32 && N <= 6144) || (M > 32 && M <= 64 && N <= 8192 && N * K <= ((int64_t)8 << 20)))) return d;
   for (d.parts = ceil_div(M, (int64_t)16);; ++d.parts) {
     d.stride = M / d.parts;
     d.rows = M - (d.parts - 1) * d.stride;
@@ -770,17 +770,19 @@ DecodeParts decode_parts(int64_t M, int64_t N, int64_t K) {
 int64_t row_parts(int64_t M, int64_t N, int64_t K) {
   const int64_t bytes = N * K;
   if (M > 64 && M <= 128 &&
-      (bytes <= ((int64_t)8 << 20) || (N <= 3072 && bytes <= ((int64_t)34 << 20)) || (N <= 4096 && bytes <= ((int64_t)17 << 20))))
+      ((N <= 32768 && bytes <= ((int64_t)8 << 20)) || (N <= 3072 && bytes <= ((int64_t)34 << 20)) || (N <= 4096 && bytes <= ((int64_t)17 << 20))))
     return 2;
   // more parts only for the smallest weights, which every part reads again: us at M = 129 / 192 / 256, N = 512, K = 7168:
   // 16.7 / 17.5 / 18.2 -> 11.1 / 11.7 / 11.9; N = 1024, K = 4096: 14.8 / 15.2 / 15.8 -> 9.6 / 10.0 / 10.2; N = K = 2048: 12.6 / 12.7 / 13.0 ->
   // 9.0 / 9.6 / 9.7; up to 192 rows, N = 1280, K = 8192: 18.6 / 18.8 -> 14.9 / 16.3; N = 1024, K = 8192: 18.1 / 18.6 -> 16.0 / 17.2 (N = 2112,
   // K = 7168: 19.2 -> 20.9; N = K = 4096: 16.6 -> 23.2)
-  if (M > 128 && M <= 256 && bytes <= ((int64_t)4 << 20)) return ceil_div(M, (int64_t)64);
-  if (M > 128 && M <= 192 && bytes <= ((int64_t)10 << 20)) return 3;
+  // (very wide weights with one or two K-blocks lose: N = 65536, K = 128, M = 128: 11.9 -> 13.2; N = 32768, K = 128, M = 256: 9.8 -> 12.7;
+  // N = 16384, K = 512, M = 129: 9.0 -> 10.8; N = 16384, K = 128, M = 257: 8.4 -> 10.8)
+  if (M > 128 && M <= 256 && N <= 16384 && bytes <= ((int64_t)4 << 20)) return ceil_div(M, (int64_t)64);
+  if (M > 128 && M <= 192 && N <= 8192 && bytes <= ((int64_t)10 << 20)) return 3;
   // (257..512 rows: N = 1024, K = 2048: 12.6 -> 9.4; N = 256, K = 8192: 17.2 / 18.4 -> 12.0 / 12.3 at 257 / 512 rows; N = 512, K = 7168:
   // 17.6 / 18.4 -> 15.2 / 17.0; N = 1024, K = 8192: 20.6 -> 21.2)
-  if (M > 256 && M <= 512 && bytes <= ((int64_t)2 << 20)) return ceil_div(M, (int64_t)64);
+  if (M > 256 && M <= 512 && N <= 8192 && bytes <= ((int64_t)2 << 20)) return ceil_div(M, (int64_t)64);
   return 0;
 }
 
@@ -801,7 +803,7 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
   const bool direct = (a.K > 0) && (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) &&
                       (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
                       ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
-  // 17..32 rows against weights of up to 6144 rows, 33..64 rows against weights of up to 8 MB: parts of up to 16 rows on the
+  // 17..32 rows against weights of up to 6144 rows, 33..64 rows against weights of up to 8 MB and 8192 rows: parts of up to 16 rows on the
   // decode kernels in one launch (the entries of a batch that shares the weights).  With 17 rows or more a decode block
   // fetches 32 activation rows per 16-32 weight rows through registers; with up to 16 the activations of its K range lie in
   // LDS.  us at M = 17 / 24 / 32, before (decode kernels for 32 rows, or 32 rows staged in the kernel of 33..64 rows) -> two parts:
@@ -811,7 +813,8 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
   // K = 2304: 7.1 -> 8.0; N = 10240, K = 8192: 23 -> 31; N = 28672, K = 4096: 27 -> 45).  33..64 rows in three or four parts,
   // M = 33 / 48 / 64: N = 512, K = 7168: 10.2 / 10.2 / 10.8 -> 6.5 / 7.1 / 6.2; N = K = 2048: 8.6 / 8.7 / 9.2 -> 5.4 / 5.8 / 5.1; N = 1024, K = 8192:
   // 11.4 / 11.5 / 11.9 -> 8.0 / 9.4 / 9.5; larger weights lose there (N = 2112, K = 7168: 12.2 -> 11.7 at 48 rows, 13.2 -> 13.4 at 64;
-  // N = K = 4096: 10.0 -> 14.0).
+  // N = K = 4096: 10.0 -> 14.0), and so do wide ones with short K (N = 32768, K = 256: 5.8 -> 8.6 ... 11.6; N = 16384, K = 512: 5.6 -> 6.0 ... 8.3;
+  // N = 8192, K = 1024: 7.5 -> 6.5 ... 7.1 still ahead).
   if (const DecodeParts dp = direct && a.batch <= 1 ? decode_parts(a.M, a.N, a.K) : DecodeParts{0, 0, 0}; dp.parts > 1) {
     const int64_t parts = dp.parts, stride = dp.stride, rows = dp.rows;
     const SmallMPlan sp = plan_small_m(rows, a.N, a.K, parts);
