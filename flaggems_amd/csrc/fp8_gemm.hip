@@ -749,20 +749,23 @@ int launch_pipe(GemmArgs a, const PipePlan& plan, void* workspace, hipStream_t s
   return FG_OK;
 }
 
-// Parts of up to 16 rows in which the decode kernels take 17..64 rows of a lone problem (measurements at the call): the parts
-// start `stride` rows apart and the last one ends with the last row; where stride < rows neighbouring parts share rows,
+// Parts of up to 16 rows in which the decode kernels take 17..128 rows of a lone problem (measurements at the call): two, four
+// or eight parts (three, five and six were measured and are 20-60 % slower than the next power of two), which
+// start `stride` rows apart, the last one ending with the last row; where stride < rows neighbouring parts share rows,
 // which both compute alike.
 struct DecodeParts {
   int64_t parts, stride, rows;  // parts == 0: not taken
 };
 DecodeParts decode_parts(int64_t M, int64_t N, int64_t K) {
   DecodeParts d = {0, 0, 0};
-  if (!((M > 16 && M <= 32 && N <= 6144) || (M > 32 && M <= 64 && N <= 8192 && N * K <= ((int64_t)8 << 20)))) return d;
-  for (d.parts = ceil_div(M, (int64_t)16);; ++d.parts) {
-    d.stride = M / d.parts;
-    d.rows = M - (d.parts - 1) * d.stride;
-    if (d.rows <= 16) return d;
-  }
+  const int64_t bytes = N * K;
+  if (M > 16 && M <= 32 && N <= 6144) d.parts = 2;
+  else if (M > 32 && M <= 64 && N <= 8192 && (bytes <= ((int64_t)13 << 20) || (N <= 3072 && bytes <= ((int64_t)26 << 20)))) d.parts = 4;
+  else if (M > 64 && M <= 128 && N <= 4096 && bytes <= ((int64_t)23 << 19)) d.parts = 8;
+  else return d;
+  d.stride = M / d.parts;
+  d.rows = M - (d.parts - 1) * d.stride;  // <= 16: M <= 16 * parts
+  return d;
 }
 
 // Into how many equal parts of at most 64 rows the staged-activation kernel takes the rows of a lone problem above 64 rows
@@ -803,18 +806,23 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
   const bool direct = (a.K > 0) && (a.K % 128 == 0) && (a.ldx % 16 == 0) && (a.ldw % 16 == 0) &&
                       (a.ldx < (1 << 23)) && (a.ldw < (1 << 23)) &&
                       ((uintptr_t)a.X % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
-  // 17..32 rows against weights of up to 6144 rows, 33..64 rows against weights of up to 8 MB and 8192 rows: parts of up to 16 rows on the
-  // decode kernels in one launch (the entries of a batch that shares the weights).  With 17 rows or more a decode block
-  // fetches 32 activation rows per 16-32 weight rows through registers; with up to 16 the activations of its K range lie in
-  // LDS.  us at M = 17 / 24 / 32, before (decode kernels for 32 rows, or 32 rows staged in the kernel of 33..64 rows) -> two parts:
-  // N = 2112, K = 7168: 10.2 / 10.8 / 10.8 -> 7.4 / 7.7 / 9.2; N = 3072, K = 8192: 11.8 / 12.4 / 12.7 -> 8.6 / 10.1 / 10.3; N = 1024, K = 8192:
-  // 8.4 / 9.6 / 10.2 -> 6.2 / 6.5 / 9.2; N = 4096, K = 14336: 18.8 / 19.6 / 20.0 -> 17.4 / 17.4 / 17.4; N = 576, K = 7168: 8.1 / 9.1 / 9.5 -> 5.7 / 6.0 / 6.3;
-  // N = K = 6144: 12.9 / 14.3 / 15.9 -> 11.7 / 12.1 / 13.4; N = K = 4096: 8.0 / 8.8 / 9.1 -> 8.0 / 7.9 / 8.0.  Wider weights lose (N = 7168,
-  // K = 2304: 7.1 -> 8.0; N = 10240, K = 8192: 23 -> 31; N = 28672, K = 4096: 27 -> 45).  33..64 rows in three or four parts,
-  // M = 33 / 48 / 64: N = 512, K = 7168: 10.2 / 10.2 / 10.8 -> 6.5 / 7.1 / 6.2; N = K = 2048: 8.6 / 8.7 / 9.2 -> 5.4 / 5.8 / 5.1; N = 1024, K = 8192:
-  // 11.4 / 11.5 / 11.9 -> 8.0 / 9.4 / 9.5; larger weights lose there (N = 2112, K = 7168: 12.2 -> 11.7 at 48 rows, 13.2 -> 13.4 at 64;
-  // N = K = 4096: 10.0 -> 14.0), and so do wide ones with short K (N = 32768, K = 256: 5.8 -> 8.6 ... 11.6; N = 16384, K = 512: 5.6 -> 6.0 ... 8.3;
-  // N = 8192, K = 1024: 7.5 -> 6.5 ... 7.1 still ahead).
+  // 17..128 rows against narrow or small weights: parts of up to 16 rows on the decode kernels in one launch (the entries of a
+  // batch that shares the weights).  With 17 rows or more a decode block fetches 32 activation rows per 16-32 weight rows
+  // through registers; with up to 16 the activations of its K range lie in LDS.  Every part reads the weights again, so
+  // the more parts, the smaller the weights that stand it.
+  // 17..32 rows in two parts, weights of up to 6144 rows; us at M = 17 / 24 / 32, before (decode kernels for 32 rows, or 32 rows
+  // staged in the kernel of 33..64 rows) -> after: N = 2112, K = 7168: 10.2 / 10.8 / 10.8 -> 7.4 / 7.7 / 9.2; N = 3072, K = 8192: 11.8 / 12.4 / 12.7 ->
+  // 8.6 / 10.1 / 10.3; N = 1024, K = 8192: 8.4 / 9.6 / 10.2 -> 6.2 / 6.5 / 9.2; N = 4096, K = 14336: 18.8 / 19.6 / 20.0 -> 17.4 / 17.4 / 17.4; N = 576,
+  // K = 7168: 8.1 / 9.1 / 9.5 -> 5.7 / 6.0 / 6.3; N = K = 6144: 12.9 / 14.3 / 15.9 -> 11.7 / 12.1 / 13.4; N = 6144, K = 256: 4.3 -> 3.6.  Wider weights
+  // lose (N = 7168, K = 2304: 7.1 -> 8.0; N = 10240, K = 8192: 23 -> 31; N = 28672, K = 4096: 27 -> 45).
+  // 33..64 rows in four parts, up to 13 MB (26 MB with N <= 3072); M = 33 / 48 / 64, staged-activation kernel -> four parts:
+  // N = 2112, K = 7168: 12.2 / 12.2 / 13.1 -> 10.7 / 10.8 / 13.1; N = 1536, K = 7168: 11.4 / 11.4 / 12.0 -> 7.9 / 7.6 / 8.8; N = 1280, K = 8192:
+  // 11.7 / 11.7 / 12.2 -> 8.0 / 9.1 / 9.3; N = 1536, K = 12288: 16.5 / 16.8 / 17.9 -> 12.4 / 12.3 / 12.6; N = 8192, K = 1536: 11.4 / 11.4 / 15.0 ->
+  // 8.0 / 8.2 / 8.7; N = 512, K = 7168: 10.2 / 10.2 / 10.8 -> 5.8 / 5.8 / 6.1; not N = K = 4096: 10.0 -> 10.7, N = 6144, K = 4096: 13.1 -> 14.5,
+  // N = 32768, K = 256: 5.8 -> 8.6.
+  // 65..128 rows in eight parts, up to 11.5 MB and 4096 rows; M = 65 / 96 / 128, two halves on the staged-activation kernel ->
+  // eight parts: N = 512, K = 7168: 11.0 / 11.2 / 11.7 -> 5.8 / 6.2 / 6.3; N = K = 2048: 8.8 / 8.8 / 9.4 -> 6.6 / 6.7 / 6.8; N = 1024, K = 8192:
+  // 11.6 / 11.7 / 12.3 -> 8.8 / 9.9 / 10.0; N = 1536, K = 7168: 14.1 / 14.4 / 15.7 -> 10.9 / 11.1 / 13.7; not N = 2112, K = 7168: 15.7 -> 19.7.
   if (const DecodeParts dp = direct && a.batch <= 1 ? decode_parts(a.M, a.N, a.K) : DecodeParts{0, 0, 0}; dp.parts > 1) {
     const int64_t parts = dp.parts, stride = dp.stride, rows = dp.rows;
     const SmallMPlan sp = plan_small_m(rows, a.N, a.K, parts);

@@ -181,7 +181,8 @@ def test_129_to_512_tiles_of_128_rows(M, N, K, dtype):
                                    (48, 8330, 6144), (64, 6650, 8192), (40, 8200, 1024), (64, 16384, 1152), (70, 16650, 8192),
                                    (64, 33040, 2048), (44, 36000, 2560),
                                    (65, 2112, 7168), (97, 1030, 8192), (128, 8200, 1024), (81, 3000, 4224), (128, 2048, 16384),
-                                   (33, 512, 7168), (47, 1030, 8192), (64, 2048, 2048), (50, 8200, 1024)])
+                                   (33, 512, 7168), (47, 1030, 8192), (64, 2048, 2048), (50, 8200, 1024),
+                                   (40, 2112, 7168), (64, 1536, 12288), (35, 8192, 1536), (100, 1000, 8192), (128, 2048, 2048), (77, 1536, 7168)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_33_to_128_rows(M, N, K, dtype):
     """33 <= M <= 64 (and 65 <= M <= 128 with small weights) takes the kernel that keeps the activations in LDS and
@@ -192,8 +193,10 @@ def test_33_to_128_rows(M, N, K, dtype):
     splits in three ranges rather than leave half of the compute units idle; the two after it are too wide for one round of tiles
     and run in rounds of blocks whose K split is chosen by how full the rounds are; the last five (and (65, 520, 1024),
     (100, 2112, 4096), (128, 4096, 4096) above) have 65 to 128 rows against small weights, which the same kernel takes as two
-    halves of the rows in one launch (48 or 64 rows staged, a second half with fewer rows than the first); the last four are
-    33 to 64 rows against weights of up to 8 MB, which the decode kernels take in three or four parts of up to 16 rows."""
+    halves of the rows in one launch (48 or 64 rows staged, a second half with fewer rows than the first); the last two lines are
+    33 to 64 rows against weights of up to 13 MB (26 MB when narrow), which the decode kernels take in four parts of up to 16
+    rows that share rows where the count does not divide, and 65 to 128 rows against weights of up to 11.5 MB in eight parts
+    ((50, 8200, 1024) is just too wide for that and stays on the staged-activation kernel)."""
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=13)
     want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
     args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])

@@ -30,7 +30,7 @@ MNK = [
     (32, 2112, 7168), (24, 4624, 7168), (30, 4096, 4096), (18, 2304, 16384),
     # 65 to 128 rows against small weights: the staged-activation kernel over the two halves of the rows
     (65, 2112, 7168), (100, 1040, 8192), (128, 4096, 4096), (77, 8192, 1024),
-    # 33 to 64 rows against weights of up to 8 MB: three or four parts of up to 16 rows on the decode kernels
+    # 33 to 64 rows against small weights: four parts of up to 16 rows on the decode kernels ((100, 1040, 8192) above: eight)
     (33, 512, 7168), (50, 1040, 8192), (64, 2048, 2048),
     # few 256 x 256 tiles with a long K: compute units share tiles and add their sums through the workspace
     (384, 5632, 8320), (300, 3088, 8448),
