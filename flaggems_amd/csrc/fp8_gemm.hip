@@ -749,8 +749,8 @@ int launch_pipe(GemmArgs a, const PipePlan& plan, void* workspace, hipStream_t s
   return FG_OK;
 }
 
-// Parts of up to 16 rows in which the decode kernels take 17..128 rows of a lone problem (measurements at the call): two, four
-// or eight parts (three, five and six were measured and are 20-60 % slower than the next power of two), which
+// Parts of up to 16 rows in which the decode kernels take 17..512 rows of a lone problem (measurements at the call): two, four,
+// eight ... parts (three, five and six were measured and are 20-60 % slower than the next power of two), which
 // start `stride` rows apart, the last one ending with the last row; where stride < rows neighbouring parts share rows,
 // which both compute alike.
 struct DecodeParts {
@@ -762,6 +762,12 @@ DecodeParts decode_parts(int64_t M, int64_t N, int64_t K) {
   if (M > 16 && M <= 32 && N <= 6144) d.parts = 2;
   else if (M > 32 && M <= 64 && N <= 8192 && (bytes <= ((int64_t)13 << 20) || (N <= 3072 && bytes <= ((int64_t)26 << 20)))) d.parts = 4;
   else if (M > 64 && M <= 128 && N <= 4096 && bytes <= ((int64_t)23 << 19)) d.parts = 8;
+  // (sixteen and thirty-two parts against the very smallest weights; us at M = 129 / 192 / 256, four 64-row parts on the
+  // staged-activation kernel -> sixteen parts: N = 512, K = 7168: 11.1 / 11.7 / 11.8 -> 7.8 / 8.0 / 8.6; N = 256, K = 8192: 10.8 / 11.3 / 11.9 ->
+  // 5.9 / 6.2 / 8.2; N = K = 1024: 7.1 / 7.4 / 7.5 -> 5.0 / 5.0 / 5.1; not N = 1024, K = 4096: 9.5 -> 10.0; M = 257 / 512 in thirty-two:
+  // N = 256, K = 8192: 11.9 / 12.3 -> 8.2 / 9.8; N = K = 1024: 7.5 / 7.6 -> 5.9 / 6.6)
+  else if (M > 128 && M <= 256 && (bytes <= ((int64_t)2 << 20) || (N <= 768 && bytes <= ((int64_t)6 << 20)))) d.parts = 16;
+  else if (M > 256 && M <= 512 && N <= 4096 && bytes <= ((int64_t)2 << 20)) d.parts = 32;
   else return d;
   d.stride = M / d.parts;
   d.rows = M - (d.parts - 1) * d.stride;  // <= 16: M <= 16 * parts

@@ -138,12 +138,14 @@ def test_tall_problems_against_narrow_weights(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(129, 576, 7168), (200, 1030, 4096), (256, 2048, 2048), (190, 1280, 8192), (257, 1024, 2048),
-                                   (500, 260, 8192), (512, 1000, 1152)])
+                                   (500, 260, 8192), (512, 1000, 1152), (256, 1100, 4096), (300, 4100, 512)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_129_to_512_rows_against_tiny_weights(M, N, K, dtype):
     """Weights of a few MB: the kernel of 33 to 64 rows takes the rows in three to eight equal parts in one launch (the
-    last part with fewer rows), each part reading the weights again.  Ragged M and N, column-major activation scales;
-    against the oracle and bit-identical on reruns."""
+    last part with fewer rows), each part reading the weights again ((200, 1030, 4096), (256, 2048, 2048), (190, 1280, 8192),
+    (256, 1100, 4096), (300, 4100, 512)); against the very smallest the decode kernels take sixteen or thirty-two parts
+    of up to 16 rows (the others).  Ragged M and N, column-major activation scales; against the oracle and bit-identical
+    on reruns."""
     xq, wq, xs, ws = _quantized_inputs(M, N, K, seed=29)
     want = O.block_fp8_matmul_dequant_ref(xq, wq, xs, ws, [128, 128], torch.float32, torch.float64)
     args = (xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV), [128, 128])
