@@ -64,11 +64,11 @@ REPEATS = 6               # timed replays per shape; the first is dropped, the m
 # half of the copied bytes, factor 2.0; WRITE_SIZE read all of them, factor 1.0).  (N, K) -> (fetch, write) KiB.
 TRAFFIC_M4096_KIB = {
     (2112, 7168): (2.0 * 63360.5, 17792.0),
-    (24576, 1536): (2.0 * 111968.1, 196800.0),
-    (32768, 512): (2.0 * 48314.5, 262144.0),
-    (7168, 16384): (2.0 * 366716.2, 59392.0),
-    (4608, 7168): (2.0 * 123769.6, 70568.0),
-    (7168, 2304): (2.0 * 51600.8, 57632.0),
+    (24576, 1536): (2.0 * 112156.3, 196800.0),
+    (32768, 512): (2.0 * 48261.2, 262144.0),
+    (7168, 16384): (2.0 * 366004.8, 59392.0),
+    (4608, 7168): (2.0 * 123769.4, 70568.0),
+    (7168, 2304): (2.0 * 51600.6, 57632.0),
 }
 
 
