@@ -750,11 +750,11 @@ int launch_pipe(GemmArgs a, const PipePlan& plan, void* workspace, hipStream_t s
 }
 
 // Parts of up to 16 rows in which the decode kernels take 17..512 rows of a lone problem (measurements at the call): two, four,
-// eight ... parts (three, five and six were measured and are 20-60 % slower than the next power of two), which
-// start `stride` rows apart, the last one ending with the last row; where stride < rows neighbouring parts share rows,
-// which both compute alike.
+// eight ... parts of `rows` rows each (three, five and six were measured and are 20-60 % slower than the next power of
+// two); the last part starts `back` rows early so that it ends with the last row, and the rows it shares with the part
+// before are computed alike by both.
 struct DecodeParts {
-  int64_t parts, stride, rows;  // parts == 0: not taken
+  int64_t parts, rows, back;  // parts == 0: not taken
 };
 DecodeParts decode_parts(int64_t M, int64_t N, int64_t K) {
   DecodeParts d = {0, 0, 0};
@@ -769,8 +769,8 @@ DecodeParts decode_parts(int64_t M, int64_t N, int64_t K) {
   else if (M > 128 && M <= 256 && (bytes <= ((int64_t)2 << 20) || (N <= 768 && bytes <= ((int64_t)6 << 20)))) d.parts = 16;
   else if (M > 256 && M <= 512 && N <= 4096 && bytes <= ((int64_t)2 << 20)) d.parts = 32;
   else return d;
-  d.stride = M / d.parts;
-  d.rows = M - (d.parts - 1) * d.stride;  // <= 16: M <= 16 * parts
+  d.rows = ceil_div(M, d.parts);           // <= 16: M <= 16 * parts
+  d.back = d.parts * d.rows - M;           // < parts: rows that the last part shares with the one before
   return d;
 }
 
@@ -830,7 +830,7 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
   // eight parts: N = 512, K = 7168: 11.0 / 11.2 / 11.7 -> 5.8 / 6.2 / 6.3; N = K = 2048: 8.8 / 8.8 / 9.4 -> 6.6 / 6.7 / 6.8; N = 1024, K = 8192:
   // 11.6 / 11.7 / 12.3 -> 8.8 / 9.9 / 10.0; N = 1536, K = 7168: 14.1 / 14.4 / 15.7 -> 10.9 / 11.1 / 13.7; not N = 2112, K = 7168: 15.7 -> 19.7.
   if (const DecodeParts dp = direct && a.batch <= 1 ? decode_parts(a.M, a.N, a.K) : DecodeParts{0, 0, 0}; dp.parts > 1) {
-    const int64_t parts = dp.parts, stride = dp.stride, rows = dp.rows;
+    const int64_t parts = dp.parts, stride = dp.rows, rows = dp.rows;
     const SmallMPlan sp = plan_small_m(rows, a.N, a.K, parts);
     const size_t per_entry = sp.splits > 1 ? sp.workspace_bytes - FG_WORKSPACE_COUNTER_BYTES : 0;
     const bool fits = sp.use && (sp.splits == 1 || (workspace != nullptr && (uintptr_t)workspace % 16 == 0 &&
@@ -846,6 +846,9 @@ int launch_gemm(const GemmArgs& a, void* workspace, size_t workspace_bytes, hipS
       h.c_batch_bytes = stride * a.ldc * c_elem;
       h.xs_batch_stride = MODE == kModeBlock ? stride * a.xs_rs : (a.xs_per_row ? stride : 0);
       h.ws_batch_stride = 0;
+      h.last_x_back_bytes = dp.back * a.ldx;
+      h.last_c_back_bytes = dp.back * a.ldc * c_elem;
+      h.last_xs_back = MODE == kModeBlock ? dp.back * a.xs_rs : (a.xs_per_row ? dp.back : 0);
       return launch_small_m(h, MODE, sp, workspace, workspace_bytes, stream);
     }
   }

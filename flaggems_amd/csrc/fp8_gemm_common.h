@@ -42,6 +42,9 @@ struct GemmArgs {
   // staged-activation kernel over equal parts of a lone problem's rows (the entries of a batch that shares the weights):
   // rows of the last part when it has fewer than M, else 0
   int last_entry_rows;
+  // decode kernels over parts of a lone problem's rows: the last entry starts this much before where the batch strides
+  // would put it, so that it ends with the last row (bytes of X, bytes of C, floats of xs; 0 otherwise)
+  int64_t last_x_back_bytes, last_c_back_bytes, last_xs_back;
 };
 
 // s_waitcnt vmcnt(0) with expcnt/lgkmcnt left at their maxima (gfx9 encoding)

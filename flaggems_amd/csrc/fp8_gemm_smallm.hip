@@ -54,6 +54,11 @@ __device__ __forceinline__ void select_batch_entry(SmallArgs& a, int64_t z) {
     a.g.ws += z * a.g.ws_batch_stride;
     if (a.partials) a.partials += z * a.partials_per_entry;
     if (a.counters) a.counters += z * a.n_chunks;
+    if (z == a.g.batch - 1) {  // parts of one problem's rows: the last part ends with the last row
+      a.g.X -= a.g.last_x_back_bytes;
+      a.g.C = reinterpret_cast<uint8_t*>(a.g.C) - a.g.last_c_back_bytes;
+      a.g.xs -= a.g.last_xs_back;
+    }
   }
 }
 
@@ -331,8 +336,9 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_gemm_transpose_kernel(SmallArg
   const int kb_lo = pair_lo * 2;
   const int kbc = min(g.KB, pair_end * 2) - kb_lo;  // K-blocks of this block
 
-  const uint8_t* const x_base = g.X + z * g.x_batch_bytes;
-  const float* const xs_base = (MODE == kModeBlock) ? g.xs + z * g.xs_batch_stride : nullptr;
+  const bool last_entry = g.batch > 1 && z == g.batch - 1;  // uniform
+  const uint8_t* const x_base = g.X + z * g.x_batch_bytes - (last_entry ? g.last_x_back_bytes : 0);
+  const float* const xs_base = (MODE == kModeBlock) ? g.xs + z * g.xs_batch_stride - (last_entry ? g.last_xs_back : 0) : nullptr;
   const uint32_t xs_cs = (uint32_t)g.xs_cs;
 
   // weight scales: a chunk may begin anywhere, so its rows can lie in two 128-row scale blocks; second[r][i] says

@@ -504,3 +504,37 @@ def test_scale_blocks_of_any_size(M, N, K, block_size, dtype):
     as_cm = As.to(DEV).t().contiguous().t()
     again = flag_gems.w8a8_block_fp8_matmul(A.to(DEV), B.to(DEV), as_cm, Bs.to(DEV), block_size, output_dtype=dtype)
     assert torch.equal(again.view(torch.int8), got.view(torch.int8))
+
+
+@pytest.mark.parametrize("rows,stride,parts,N,K", [(9, 8, 2, 2112, 7168), (16, 15, 2, 6144, 4096), (11, 8, 4, 2112, 7168),
+                                                    (16, 13, 4, 8192, 1536), (13, 9, 8, 1536, 7168), (9, 8, 16, 512, 7168),
+                                                    (16, 11, 32, 1024, 2048)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_parts_that_share_rows_agree_bit_for_bit(rows, stride, parts, N, K, dtype):
+    """17 to 512 rows against small weights run as 2, 4, 8 ... parts of up to 16 rows, the entries of a batch that shares
+    the weights, and the last part starts early so that it ends with the last row: the rows it shares with the part
+    before are computed, and stored, by both.  That is safe because a row's result depends neither on the entry that
+    computes it nor on its place within the entry: here a batch of such entries, `stride` < `rows` rows apart, goes
+    through the C ABI with a buffer per entry, and the rows that neighbours share come out with equal bits (bf16 and
+    fp32, K in one range and split over blocks)."""
+    from flaggems_amd import _lib
+    lib = _lib.load()
+    M = (parts - 1) * stride + rows
+    xq, wq, xs, ws = (t.to(DEV) for t in _quantized_inputs(M, N, K, seed=31))
+    kb = K // 128
+    c = torch.zeros(parts, rows, N, dtype=dtype, device=DEV)
+    need = lib.fg_batched_block_fp8_gemm_workspace_bytes(parts, rows, N, K)
+    wsp = _lib.workspace(torch.device(DEV), need) if need else None
+    rc = lib.fg_batched_block_fp8_gemm(
+        xq.data_ptr(), K, stride * K, wq.data_ptr(), K, 0, xs.data_ptr(), kb, 1, stride * kb, ws.data_ptr(), kb, 1, 0,
+        c.data_ptr(), N, rows * N, _lib.DTYPE_CODE[dtype], parts, rows, N, K, 128, 128,
+        wsp.data_ptr() if need else None, wsp.numel() if need else 0, _lib.current_stream_ptr(torch.device(DEV)))
+    _lib.check(rc, "fg_batched_block_fp8_gemm")
+    torch.cuda.synchronize()
+    want = O.block_fp8_matmul_dequant_ref(xq.cpu(), wq.cpu(), xs.cpu(), ws.cpu(), [128, 128], torch.float32, torch.float64)
+    tol = dict(rtol=1e-4, atol=4e-4) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    shared = rows - stride
+    for z in range(parts):
+        torch.testing.assert_close(c[z].cpu().float(), want[z * stride:z * stride + rows], **tol)
+        if z + 1 < parts:
+            assert torch.equal(c[z][stride:].view(torch.int8), c[z + 1][:shared].view(torch.int8))
